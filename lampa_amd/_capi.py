@@ -1,0 +1,81 @@
+"""ctypes binding of ``liblampa_amd.so`` -- the only route from Python to the gfx950 kernels.
+
+There is no CPU fallback: if the library has not been built the import of any operator raises.
+Every entry point takes raw device pointers, sizes and a HIP stream, and returns 0 or a negative error code.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblampa_amd.so")
+
+_ERRORS = {
+    -1: "invalid argument",
+    -2: "workspace missing or too small",
+    -3: "HIP launch error",
+    -4: "unsupported shape or dtype",
+}
+
+_vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+
+_SIGNATURES = {
+    "lampa_lsh_bucket_workspace_bytes": (_i64, [_i64, _i32, _i32]),
+    "lampa_lsh_bucket_keys": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "lampa_lsh_project_f32": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
+    "lampa_lsh_ordering_keys": (_i32, [_vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp]),
+    "lampa_row_minmax_f32": (_i32, [_vp, _i32, _i64, _vp, _vp]),
+    "lampa_sort_workspace_bytes": (_i64, [_i32, _i64]),
+    "lampa_sort_pairs": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp]),
+    "lampa_gather_rows": (_i32, [_vp, _i32, _i64, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
+    "lampa_scatter_rows": (_i32, [_vp, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
+    "lampa_invert_perm": (_i32, [_vp, _i32, _i32, _i64, _vp, _vp]),
+}
+
+_lib = None
+
+
+class LampaError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises if it has not been built (``python -m lampa_amd.build``)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build the HIP library first (python -m lampa_amd.build). "
+                "lampa_amd has no CPU or PyTorch fallback.")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def check(code: int, what: str):
+    if code < 0:
+        raise LampaError(f"{what} failed: {_ERRORS.get(int(code), 'error')} ({int(code)})")
+    return code
+
+
+def ptr(t):
+    """Device pointer of a tensor (None -> NULL)."""
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def stream_of(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise LampaError("lampa_amd operators run on the GPU only: got a CPU tensor (there is no CPU fallback)")

@@ -1,0 +1,114 @@
+// Row gather / scatter / inverse permutation for the LSH stage on gfx950 (pure HBM-bound data movement).
+//
+// Replaces (reference chengjiang123/Lampa): batched_index_select  models/model_utils/hash_utils.py:83-93
+// (gather with an index tensor expanded over the feature dimension), sort_to_buckets / unsort_from_buckets
+// models/attention/hept.py:9-19, invert_permutation  hash_utils.py:46-57, and the gather / argsort-unsort of
+// LSHOrdering's caller  models/baselines/full_mamba2.py:213-216,678-682.
+#include "common.h"
+
+#define GS_BLOCK 256
+
+template <typename IdxT>
+__device__ __forceinline__ int64_t gs_index(const void* idx, int64_t i) {
+  return (int64_t)reinterpret_cast<const IdxT*>(idx)[i];
+}
+
+// One thread moves one VEC-byte piece of a row. dst[s, n, :] = src[s or 0, idx[s, n], :] when GATHER,
+// dst[s, idx[s, n], :] = src[s, n, :] otherwise.
+template <typename VecT, typename IdxT, bool GATHER>
+__global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restrict__ src, int64_t src_seg_stride,
+                                                          int src_segments, const void* __restrict__ idx, int64_t n, int64_t n_src,
+                                                          int vec_per_row, char* __restrict__ dst, int* bad) {
+  const int seg = blockIdx.y;
+  const int64_t item = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
+  const int64_t row = item / vec_per_row;
+  const int piece = (int)(item - row * vec_per_row);
+  if (row >= n) return;
+  const int64_t other = gs_index<IdxT>(idx, (int64_t)seg * n + row);
+  const int64_t limit = GATHER ? n_src : n;
+  if (other < 0 || other >= limit) {
+    if (bad) *bad = 1;
+    return;
+  }
+  const int64_t row_bytes = (int64_t)vec_per_row * (int64_t)sizeof(VecT);
+  const int64_t from = GATHER ? other : row, to = GATHER ? row : other;
+  const VecT* s = reinterpret_cast<const VecT*>(src + (seg % src_segments) * src_seg_stride + from * row_bytes) + piece;
+  VecT* d = reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + to) * row_bytes) + piece;
+  *d = *s;
+}
+
+template <typename IdxT>
+__global__ void __launch_bounds__(GS_BLOCK) gs_invert_kernel(const IdxT* __restrict__ perm, int64_t n,
+                                                            IdxT* __restrict__ inv) {
+  const int seg = blockIdx.y;
+  const int64_t i = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
+  if (i >= n) return;
+  const int64_t p = (int64_t)perm[(int64_t)seg * n + i];
+  if (p >= 0 && p < n) inv[(int64_t)seg * n + p] = (IdxT)i;
+}
+
+template <typename IdxT, bool GATHER>
+static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, const void* idx, int n_segments, int64_t n,
+                     int64_t n_src, int64_t row_bytes, void* dst, hipStream_t s) {
+  const bool a16 = row_bytes % 16 == 0 && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) &&
+                   src_seg_stride % 16 == 0;
+  const bool a4 = row_bytes % 4 == 0 && ((uintptr_t)src % 4 == 0) && ((uintptr_t)dst % 4 == 0) &&
+                  src_seg_stride % 4 == 0;
+  const int vec = a16 ? 16 : (a4 ? 4 : 1);
+  const int vec_per_row = (int)(row_bytes / vec);
+  const int64_t items = n * vec_per_row;
+  const dim3 grid((unsigned)((items + GS_BLOCK - 1) / GS_BLOCK), n_segments), block(GS_BLOCK);
+  if (vec == 16)
+    hipLaunchKernelGGL((gs_rows_kernel<uint4, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride, src_segments,
+                       idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+  else if (vec == 4)
+    hipLaunchKernelGGL((gs_rows_kernel<uint32_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
+                       src_segments, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+  else
+    hipLaunchKernelGGL((gs_rows_kernel<uint8_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
+                       src_segments, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+  return lampa_launch_status();
+}
+
+// dst [S, n, row_bytes] = rows of src selected by idx [S, n]. src is [src_segments, n_src, row_bytes] and segment s
+// reads source segment s % src_segments (src_segments == S: one source per segment; a divisor of S: the sources
+// are shared round-robin, which is how a [1, batch, ...] tensor broadcasts over [n_hashes, batch, ...] indices). idx_bytes is 4 (int32) or 8 (int64). Out-of-range
+// indices are skipped (the destination row is left untouched).
+extern "C" int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
+                                 int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream) {
+  if (!src || !idx || !dst || n_segments < 1 || n < 0 || n_src < 0 || row_bytes < 1) return LAMPA_ERR_INVALID;
+  if (src_segments < 1 || n_segments % src_segments != 0) return LAMPA_ERR_INVALID;
+  if (idx_bytes != 4 && idx_bytes != 8) return LAMPA_ERR_INVALID;
+  if (n == 0) return LAMPA_OK;
+  const int64_t stride = n_src * row_bytes;
+  if (idx_bytes == 4)
+    return gs_launch<int32_t, true>(src, stride, src_segments, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
+  return gs_launch<int64_t, true>(src, stride, src_segments, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
+}
+
+// dst [S, n, row_bytes]: dst[s, idx[s, i]] = src[s, i] (idx is a permutation of 0..n-1 per segment).
+extern "C" int lampa_scatter_rows(const void* src, const void* idx, int idx_bytes, int n_segments, int64_t n,
+                                  int64_t row_bytes, void* dst, void* stream) {
+  if (!src || !idx || !dst || n_segments < 1 || n < 0 || row_bytes < 1) return LAMPA_ERR_INVALID;
+  if (idx_bytes != 4 && idx_bytes != 8) return LAMPA_ERR_INVALID;
+  if (n == 0) return LAMPA_OK;
+  const int64_t stride = n * row_bytes;
+  if (idx_bytes == 4)
+    return gs_launch<int32_t, false>(src, stride, n_segments, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
+  return gs_launch<int64_t, false>(src, stride, n_segments, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
+}
+
+// inv[s, perm[s, i]] = i
+extern "C" int lampa_invert_perm(const void* perm, int idx_bytes, int n_segments, int64_t n, void* inv, void* stream) {
+  if (!perm || !inv || n_segments < 1 || n < 0) return LAMPA_ERR_INVALID;
+  if (idx_bytes != 4 && idx_bytes != 8) return LAMPA_ERR_INVALID;
+  if (n == 0) return LAMPA_OK;
+  const dim3 grid((unsigned)((n + GS_BLOCK - 1) / GS_BLOCK), n_segments), block(GS_BLOCK);
+  if (idx_bytes == 4)
+    hipLaunchKernelGGL(gs_invert_kernel<int32_t>, grid, block, 0, (hipStream_t)stream, (const int32_t*)perm, n,
+                       (int32_t*)inv);
+  else
+    hipLaunchKernelGGL(gs_invert_kernel<int64_t>, grid, block, 0, (hipStream_t)stream, (const int64_t*)perm, n,
+                       (int64_t*)inv);
+  return lampa_launch_status();
+}

@@ -1,0 +1,307 @@
+// E2LSH hashing of detector hits on gfx950.
+//
+// Arithmetic contract (bit-exact against the CPU oracle): the projection is the left-to-right chain
+// p = fmaf(x[d], a[d], p) starting from 0, the quantisation is floorf((p + b) * inv_w) saturated to int32 with
+// NaN -> INT32_MAX.  Only explicit fmaf / single operations are used so that compiler contraction cannot
+// change a result.
+//
+// Replaces (reference chengjiang123/Lampa): E2LSH.forward  models/model_utils/hash_utils.py:368-371,
+// the hash range of lsh_mapping  hash_utils.py:334-340, the mixed-radix key idiom of get_geo_shift
+// models/attention/hept.py:79-88, and the key/norm of LSHOrdering  models/baselines/full_mamba2.py:181-203.
+#include "common.h"
+
+#define LSH_MAX_DIM 8
+#define LSH_MAX_COLS 64
+#define LSH_MAX_PROJ 8
+#define LSH_BLOCK 256
+
+__device__ __forceinline__ int32_t lsh_quantise(float p, float b, float inv_w) {
+  float t = (p + b) * inv_w;
+  if (t != t) return INT32_MAX;
+  float f = floorf(t);
+  if (f >= 2147483648.0f) return INT32_MAX;
+  if (f <= -2147483648.0f) return INT32_MIN;
+  return (int32_t)f;
+}
+
+template <int DIM>
+__device__ __forceinline__ void lsh_load_coords(const float* __restrict__ coords, int64_t n, int dim, float* x) {
+  if (DIM == 4) {
+    float4 c = *reinterpret_cast<const float4*>(coords + n * 4);
+    x[0] = c.x; x[1] = c.y; x[2] = c.z; x[3] = c.w;
+  } else {
+#pragma unroll
+    for (int d = 0; d < LSH_MAX_DIM; ++d) x[d] = d < dim ? coords[n * dim + d] : 0.0f;
+  }
+}
+
+template <int DIM>
+__device__ __forceinline__ float lsh_dot(const float* x, const float* __restrict__ alpha, int dim, int n_cols, int c) {
+  float acc = 0.0f;
+  if (DIM == 4) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) acc = __builtin_fmaf(x[d], alpha[d * n_cols + c], acc);
+  } else {
+#pragma unroll
+    for (int d = 0; d < LSH_MAX_DIM; ++d)
+      if (d < dim) acc = __builtin_fmaf(x[d], alpha[d * n_cols + c], acc);
+  }
+  return acc;
+}
+
+// ---- pass 1: per-block min / max of every id column over the valid hits -------------------------------
+// partial [gridDim.x, n_cols, 2] (min, max); no atomics, no initialisation needed.
+template <int DIM>
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __restrict__ coords, int64_t n_valid,
+                                                              int dim, const float* __restrict__ alpha,
+                                                              const float* __restrict__ beta, int n_cols,
+                                                              float inv_w, int32_t* __restrict__ partial) {
+  __shared__ int32_t s_min[LSH_BLOCK / 64][LSH_MAX_COLS];
+  __shared__ int32_t s_max[LSH_BLOCK / 64][LSH_MAX_COLS];
+  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
+  const bool valid = n < n_valid;
+  float x[LSH_MAX_DIM];
+  lsh_load_coords<DIM>(coords, valid ? n : 0, dim, x);
+  const int wave = threadIdx.x >> 6;
+  for (int c = 0; c < n_cols; ++c) {
+    int32_t id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
+    int32_t lo = valid ? id : INT32_MAX, hi = valid ? id : INT32_MIN;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      lo = min(lo, __shfl_xor(lo, off));
+      hi = max(hi, __shfl_xor(hi, off));
+    }
+    if (lane_id() == 0) { s_min[wave][c] = lo; s_max[wave][c] = hi; }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < n_cols; c += LSH_BLOCK) {
+    int32_t lo = s_min[0][c], hi = s_max[0][c];
+    for (int w = 1; w < LSH_BLOCK / 64; ++w) { lo = min(lo, s_min[w][c]); hi = max(hi, s_max[w][c]); }
+    partial[((int64_t)blockIdx.x * n_cols + c) * 2 + 0] = lo;
+    partial[((int64_t)blockIdx.x * n_cols + c) * 2 + 1] = hi;
+  }
+}
+
+// ---- pass 2: reduce the partials, derive the mixed-radix strides, pack the keys ------------------------
+// grid (ceil(N / 256), n_tables). meta [n_tables, 2J+3] = lo[J], range[J], total, key_bits, overflow.
+template <int DIM>
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __restrict__ coords, int64_t n_hits,
+                                                            int64_t n_valid, int dim,
+                                                            const float* __restrict__ alpha,
+                                                            const float* __restrict__ beta, int n_tables,
+                                                            int n_proj, float inv_w,
+                                                            const int32_t* __restrict__ partial, int n_partial,
+                                                            int32_t* __restrict__ ids, int32_t* __restrict__ keys,
+                                                            int32_t* __restrict__ meta) {
+  __shared__ int32_t s_red[2][LSH_MAX_PROJ][LSH_BLOCK / 64];
+  __shared__ int32_t s_lo[LSH_MAX_PROJ];
+  __shared__ uint32_t s_stride[LSH_MAX_PROJ];
+  __shared__ uint32_t s_total;
+  const int table = blockIdx.y;
+  const int n_cols = n_tables * n_proj;
+  const int wave = threadIdx.x >> 6;
+  for (int j = 0; j < n_proj; ++j) {
+    const int c = table * n_proj + j;
+    int32_t lo = INT32_MAX, hi = INT32_MIN;
+    for (int b = threadIdx.x; b < n_partial; b += LSH_BLOCK) {
+      lo = min(lo, partial[((int64_t)b * n_cols + c) * 2 + 0]);
+      hi = max(hi, partial[((int64_t)b * n_cols + c) * 2 + 1]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      lo = min(lo, __shfl_xor(lo, off));
+      hi = max(hi, __shfl_xor(hi, off));
+    }
+    if (lane_id() == 0) { s_red[0][j][wave] = lo; s_red[1][j][wave] = hi; }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint64_t total = 1;
+    int overflow = 0;
+    int32_t lo_j[LSH_MAX_PROJ];
+    int64_t range_j[LSH_MAX_PROJ];
+    for (int j = 0; j < n_proj; ++j) {
+      int32_t lo = s_red[0][j][0], hi = s_red[1][j][0];
+      for (int w = 1; w < LSH_BLOCK / 64; ++w) { lo = min(lo, s_red[0][j][w]); hi = max(hi, s_red[1][j][w]); }
+      if (n_valid == 0) { lo = 0; hi = 0; }
+      lo_j[j] = lo;
+      range_j[j] = (int64_t)hi - (int64_t)lo + 1;
+      s_lo[j] = lo;
+      s_stride[j] = (uint32_t)total;
+      total *= (uint64_t)range_j[j];
+      if (total > (uint64_t)INT32_MAX) { overflow = 1; total = (uint64_t)INT32_MAX + 1; }
+    }
+    s_total = (uint32_t)total;
+    if (blockIdx.x == 0) {
+      int32_t* m = meta + (int64_t)table * (2 * n_proj + 3);
+      for (int j = 0; j < n_proj; ++j) {
+        m[j] = lo_j[j];
+        m[n_proj + j] = range_j[j] > INT32_MAX ? INT32_MAX : (int32_t)range_j[j];
+      }
+      uint64_t top = (n_valid < n_hits) ? total : total - 1;
+      int bits = 1;
+      while (bits < 32 && (top >> bits) != 0) ++bits;
+      if (overflow) bits = 32;
+      m[2 * n_proj] = total > (uint64_t)INT32_MAX ? INT32_MAX : (int32_t)total;
+      m[2 * n_proj + 1] = bits;
+      m[2 * n_proj + 2] = overflow;
+    }
+  }
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
+  if (n >= n_hits) return;
+  uint32_t key = s_total;
+  const bool valid = n < n_valid;
+  float x[LSH_MAX_DIM];
+  if (valid) lsh_load_coords<DIM>(coords, n, dim, x);
+  if (valid) key = 0;
+  for (int j = 0; j < n_proj; ++j) {
+    const int c = table * n_proj + j;
+    int32_t id = 0;
+    if (valid) {
+      id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
+      key += ((uint32_t)id - (uint32_t)s_lo[j]) * s_stride[j];
+    }
+    if (ids) ids[(int64_t)c * n_hits + n] = id;
+  }
+  keys[(int64_t)table * n_hits + n] = (int32_t)key;
+}
+
+// ---- plain projection (the reference's E2LSH.forward, a batched [N,dim] x [dim,n_hashes] product) -----
+// vecs [n_heads, N, dim], alpha [n_heads, dim, n_cols]; out element (c, head, n) at
+// c * stride_c + head * stride_h + n * stride_n.
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_project_kernel(const float* __restrict__ vecs, int64_t n_hits,
+                                                               int dim, const float* __restrict__ alpha,
+                                                               int n_cols, float* __restrict__ out,
+                                                               int64_t stride_c, int64_t stride_h,
+                                                               int64_t stride_n) {
+  const int head = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
+  if (n >= n_hits) return;
+  const float* x = vecs + ((int64_t)head * n_hits + n) * dim;
+  const float* a = alpha + (int64_t)head * dim * n_cols;
+  for (int c = 0; c < n_cols; ++c) {
+    float acc = 0.0f;
+    for (int d = 0; d < dim; ++d) acc = __builtin_fmaf(x[d], a[d * n_cols + c], acc);
+    out[c * stride_c + head * stride_h + n * stride_n] = acc;
+  }
+}
+
+// ---- LSHOrdering sort keys: key = ((p_0 + 2 p_1) + 4 p_2) + ..., norm = sqrt(sum x^2) ------------------
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_ordering_keys_kernel(const float* __restrict__ coords,
+                                                                     int64_t n_hits, int dim,
+                                                                     const float* __restrict__ alpha,
+                                                                     int n_hashes, float* __restrict__ key,
+                                                                     float* __restrict__ norm) {
+  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
+  if (n >= n_hits) return;
+  const float* x = coords + n * dim;
+  float k = 0.0f, w = 1.0f;
+  for (int h = 0; h < n_hashes; ++h) {
+    float acc = 0.0f;
+    for (int d = 0; d < dim; ++d) acc = __builtin_fmaf(x[d], alpha[d * n_hashes + h], acc);
+    float term = acc * w;
+    k = (h == 0) ? term : k + term;
+    w *= 2.0f;
+  }
+  float ss = 0.0f;
+  for (int d = 0; d < dim; ++d) ss = __builtin_fmaf(x[d], x[d], ss);
+  key[n] = k;
+  norm[n] = __fsqrt_rn(ss);
+}
+
+// ---- host entry points ----------------------------------------------------------------------------------
+extern "C" int64_t lampa_lsh_bucket_workspace_bytes(int64_t n_hits, int n_tables, int n_proj) {
+  if (n_hits < 0 || n_tables <= 0 || n_proj <= 0) return LAMPA_ERR_INVALID;
+  int64_t blocks = (n_hits + LSH_BLOCK - 1) / LSH_BLOCK;
+  if (blocks < 1) blocks = 1;
+  return lampa_align_up(blocks * n_tables * n_proj * 2 * (int64_t)sizeof(int32_t), 256);
+}
+
+extern "C" int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, int dim,
+                                     const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                                     int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+  if (!coords || !alpha || !beta || !keys_out || !meta_out) return LAMPA_ERR_INVALID;
+  if (n_hits < 0 || n_valid < 0 || n_valid > n_hits || n_hits > INT32_MAX) return LAMPA_ERR_INVALID;
+  if (dim < 1 || dim > LSH_MAX_DIM || n_tables < 1 || n_proj < 1 || n_proj > LSH_MAX_PROJ ||
+      n_tables * n_proj > LSH_MAX_COLS || !(w > 0.0f))
+    return LAMPA_ERR_INVALID;
+  if (!workspace || workspace_bytes < lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj))
+    return LAMPA_ERR_WORKSPACE;
+  if (n_hits == 0) return LAMPA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const float inv_w = 1.0f / w;
+  const int n_cols = n_tables * n_proj;
+  int32_t* partial = (int32_t*)workspace;
+  int blocks_valid = (int)((n_valid + LSH_BLOCK - 1) / LSH_BLOCK);
+  if (blocks_valid < 1) blocks_valid = 1;
+  const int blocks_all = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
+  if (dim == 4) {
+    hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
+                       beta, n_cols, inv_w, partial);
+    hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
+                       meta_out);
+  } else {
+    hipLaunchKernelGGL(lsh_minmax_kernel<0>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
+                       beta, n_cols, inv_w, partial);
+    hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
+                       meta_out);
+  }
+  return lampa_launch_status();
+}
+
+extern "C" int lampa_lsh_project_f32(const float* vecs, int n_heads, int64_t n_hits, int dim, const float* alpha,
+                                     int n_cols, float* out, int64_t stride_c, int64_t stride_h, int64_t stride_n,
+                                     void* stream) {
+  if (!vecs || !alpha || !out || n_heads < 1 || n_hits < 0 || dim < 1 || n_cols < 1) return LAMPA_ERR_INVALID;
+  if (n_hits == 0) return LAMPA_OK;
+  const int blocks = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
+  hipLaunchKernelGGL(lsh_project_kernel, dim3(blocks, n_heads), dim3(LSH_BLOCK), 0, (hipStream_t)stream, vecs,
+                     n_hits, dim, alpha, n_cols, out, stride_c, stride_h, stride_n);
+  return lampa_launch_status();
+}
+
+extern "C" int lampa_lsh_ordering_keys(const float* coords, int64_t n_hits, int dim, const float* alpha,
+                                       int n_hashes, float* key_out, float* norm_out, void* stream) {
+  if (!coords || !alpha || !key_out || !norm_out || n_hits < 0 || dim < 1 || n_hashes < 1) return LAMPA_ERR_INVALID;
+  if (n_hits == 0) return LAMPA_OK;
+  const int blocks = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
+  hipLaunchKernelGGL(lsh_ordering_keys_kernel, dim3(blocks), dim3(LSH_BLOCK), 0, (hipStream_t)stream, coords,
+                     n_hits, dim, alpha, n_hashes, key_out, norm_out);
+  return lampa_launch_status();
+}
+
+// ---- per-row min / max of hashed values (the range used as a radix stride, hash_utils.py:334-340) -----------
+// x [rows, n]; out [rows, 2] = (min, max). NaNs are ignored unless the whole row is NaN.
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_row_minmax_kernel(const float* __restrict__ x, int64_t n,
+                                                                  float* __restrict__ out) {
+  __shared__ float s_lo[LSH_BLOCK / 64], s_hi[LSH_BLOCK / 64];
+  const float* row = x + (int64_t)blockIdx.x * n;
+  float lo = INFINITY, hi = -INFINITY;
+  for (int64_t i = threadIdx.x; i < n; i += LSH_BLOCK) {
+    const float v = row[i];
+    lo = fminf(lo, v);
+    hi = fmaxf(hi, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    lo = fminf(lo, __shfl_xor(lo, off));
+    hi = fmaxf(hi, __shfl_xor(hi, off));
+  }
+  if (lane_id() == 0) { s_lo[threadIdx.x >> 6] = lo; s_hi[threadIdx.x >> 6] = hi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < LSH_BLOCK / 64; ++w) { lo = fminf(lo, s_lo[w]); hi = fmaxf(hi, s_hi[w]); }
+    out[blockIdx.x * 2 + 0] = lo;
+    out[blockIdx.x * 2 + 1] = hi;
+  }
+}
+
+extern "C" int lampa_row_minmax_f32(const float* x, int rows, int64_t n, float* out, void* stream) {
+  if (!x || !out || rows < 1 || n < 1) return LAMPA_ERR_INVALID;
+  hipLaunchKernelGGL(lsh_row_minmax_kernel, dim3(rows), dim3(LSH_BLOCK), 0, (hipStream_t)stream, x, n, out);
+  return lampa_launch_status();
+}

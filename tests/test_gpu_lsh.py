@@ -1,0 +1,149 @@
+"""GPU parity of the LSH stage against the CPU oracle: bit-exact ids, keys, permutations and features."""
+import numpy as np
+import pytest
+import torch
+
+from lampa_amd import lsh, synth
+from oracle import lsh as ol
+
+pytestmark = pytest.mark.gpu
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("n", [1, 63, 2048, 2049, 60000])
+def test_config1_bucket_sort_bit_exact(device, n):
+    coords, feats, _ = synth.collider_event(n, seed=0)
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    want = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy())
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats.to(device))
+    assert np.array_equal(_np(got["ids"]), want["ids"])
+    assert np.array_equal(_np(got["meta"]), want["meta"])
+    assert np.array_equal(_np(got["keys"]), want["keys"])
+    assert np.array_equal(_np(got["perm"]), want["perm"])
+    assert np.array_equal(_np(got["feats"]), want["feats"])
+
+
+def test_bucket_sort_padding_and_dim3(device):
+    coords, feats, _ = synth.collider_event(5000, seed=3)
+    coords = coords[:, :3].contiguous()
+    alpha, beta = synth.lsh_params(3, 2, 3, 0.25, 7)
+    want = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.25, 2, 3, feats.numpy(), n_valid=4321)
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.25, 2, 3, feats.to(device),
+                              n_valid=4321)
+    for name in ("ids", "meta", "keys", "perm", "feats"):
+        assert np.array_equal(_np(got[name]), want[name]), name
+    assert (_np(got["perm"])[:, 4321:] >= 4321).all()  # padding sorts last, in input order
+
+
+def test_bucket_overflow_flag(device):
+    coords = torch.tensor([[0.0, 0, 0, 0], [1e6, 1e6, 0, 0]])
+    alpha = torch.eye(4)[:, :2].contiguous()
+    beta = torch.zeros(2)
+    _, _, meta = lsh.lsh_bucket_keys(coords.to(device), alpha.to(device), beta.to(device), 1.0, 1, 2)
+    ids = ol.bucket_ids(coords.numpy(), alpha.numpy(), beta.numpy(), 1.0)
+    _, want = ol.pack_keys(ids, 1, 2)
+    assert np.array_equal(_np(meta), want) and want[0, -1] == 1
+
+
+@pytest.mark.parametrize("kind", ["i32", "f32", "u32bits"])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 777), (2, 20000), (5, 4096)])
+def test_stable_argsort_matches_torch(device, kind, shape):
+    gen = torch.Generator().manual_seed(hash((kind, shape)) % 1000)
+    if kind == "i32":
+        keys = torch.randint(-300, 300, shape, generator=gen, dtype=torch.int32)  # many ties
+        got = lsh.stable_argsort(keys.to(device))
+    elif kind == "f32":
+        keys = torch.randn(shape, generator=gen)
+        keys[..., ::7] = 0.0
+        keys[..., 3::11] = -0.0
+        if shape[1] > 100:
+            keys[0, 5], keys[0, 17], keys[0, 50], keys[0, 51] = float("inf"), float("-inf"), float("nan"), float("nan")
+        got = lsh.stable_argsort(keys.to(device))
+    else:
+        keys = torch.randint(0, 1 << 13, shape, generator=gen, dtype=torch.int32)
+        got = lsh.stable_argsort(keys.to(device), key_bits=13, unsigned=True)
+    want = torch.sort(keys, dim=-1, stable=True).indices
+    assert torch.equal(got.cpu().long(), want)
+
+
+def test_stable_argsort_full_range_and_values(device):
+    gen = torch.Generator().manual_seed(0)
+    keys = torch.randint(-2**31, 2**31 - 1, (2, 50000), generator=gen, dtype=torch.int64).to(torch.int32)
+    vals = torch.stack([torch.randperm(50000, generator=gen) for _ in range(2)]).to(torch.int32)
+    for passes in (0, 3, 4):
+        got = lsh.stable_argsort(keys.to(device), values=vals.to(device), n_passes=passes)
+        want = torch.gather(vals, 1, torch.sort(keys, dim=-1, stable=True).indices)
+        assert torch.equal(got.cpu(), want)
+    want = ol.stable_argsort(keys.numpy(), ol.KEY_I32)
+    assert np.array_equal(_np(lsh.stable_argsort(keys.to(device))), want)
+
+
+def test_gather_scatter_invert_roundtrip(device):
+    gen = torch.Generator().manual_seed(1)
+    for d, dtype in ((24, torch.float32), (5, torch.float32), (3, torch.int16), (64, torch.bfloat16)):
+        x = torch.randn(4, 3000, d, generator=gen).to(dtype)
+        perm = torch.stack([torch.randperm(3000, generator=gen) for _ in range(4)])
+        for idx in (perm, perm.int()):
+            g = lsh.gather_rows(x.to(device), idx.to(device))
+            assert torch.equal(g.cpu(), torch.gather(x, 1, perm[..., None].expand(-1, -1, d)))
+            inv = lsh.invert_permutation(idx.to(device))
+            assert torch.equal(inv.cpu().long(), torch.argsort(perm, dim=-1))
+            assert torch.equal(lsh.gather_rows(g, inv).cpu(), x)
+            assert torch.equal(lsh.scatter_rows(g, idx.to(device)).cpu(), x)
+    x = torch.randn(3000, 24, generator=gen)
+    assert np.array_equal(_np(lsh.gather_rows(x.to(device), perm.int().to(device))),
+                          ol.gather_rows(x.numpy(), perm.int().numpy()))
+
+
+def test_reference_named_helpers(device):
+    gen = torch.Generator().manual_seed(2)
+    h, b, s, d, bucket = 3, 2, 600, 16, 100
+    x = torch.randn(b, s, d, generator=gen)
+    keys = torch.randn(h, b, s, generator=gen)
+    perm = lsh.stable_argsort(keys.to(device)).long()
+    assert torch.equal(perm.cpu(), keys.argsort(dim=-1, stable=True))
+    sx = lsh.sort_to_buckets(x.to(device), perm, bucket)
+    want = x[None].expand(h, -1, -1, -1).gather(-2, perm.cpu()[..., None].expand(-1, -1, -1, d))
+    assert sx.shape == (h, b, s // bucket, bucket, d) and torch.equal(sx.cpu().reshape(h, b, s, d), want)
+    back = lsh.unsort_from_buckets(sx, lsh.invert_permutation(perm))
+    assert torch.equal(back.cpu(), x[None].expand(h, -1, -1, -1))
+    p = lsh.pad_to_multiple(x, 256, dims=-2, value=float("inf"))
+    assert p.shape == (b, 768, d) and torch.isinf(p[:, 600:]).all()
+
+
+def test_e2lsh_and_lsh_mapping(device):
+    torch.manual_seed(4)
+    e = lsh.E2LSH(n_hashes=3, n_heads=2, dim=10).to(device)
+    q, k = torch.randn(2, 5000, 10), torch.randn(2, 5000, 10)
+    qh, kh, shift = lsh.lsh_mapping(e, q.to(device), k.to(device))
+    a = e.alpha.detach().cpu()
+    want_q = np.stack([ol.project(q[i].numpy(), a[i].numpy()) for i in range(2)], axis=1)  # [n_hashes, heads, N]
+    assert qh.shape == (3, 2, 5000) and np.array_equal(_np(qh), want_q)
+    ref_q, ref_k = torch.bmm(q, a).permute(2, 0, 1), torch.bmm(k, a).permute(2, 0, 1)
+    assert torch.allclose(qh.cpu(), ref_q, atol=1e-5)
+    ref_shift = torch.max(ref_q.max(-1, keepdim=True).values, ref_k.max(-1, keepdim=True).values) - \
+        torch.min(ref_q.min(-1, keepdim=True).values, ref_k.min(-1, keepdim=True).values)
+    assert shift.shape == (3, 2, 1) and torch.allclose(shift.cpu(), ref_shift, atol=1e-5)
+    hh, sh = lsh.lsh_mapping1(e, q.to(device))
+    assert torch.equal(hh, qh) and torch.allclose(sh.cpu(), ref_q.max(-1, keepdim=True).values - ref_q.min(-1, keepdim=True).values, atol=1e-5)
+
+
+def test_lsh_ordering_bit_exact_and_unsort(device):
+    torch.manual_seed(5)
+    B, L, D = 2, 6000, 24
+    mod = lsh.LSHOrdering(input_dim=4, num_hashes=3).to(device)
+    coords = torch.stack([synth.collider_event(L, seed=s)[0] for s in range(B)])
+    points = torch.randn(B, L, D)
+    ordered, idx = mod(points.to(device), coords.to(device))
+    alpha = mod.e2lsh.alpha.detach().cpu()[0].numpy()
+    for b in range(B):
+        want = ol.lsh_ordering(coords[b].numpy(), alpha)
+        assert np.array_equal(_np(idx[b]), want.astype(np.int64))
+    assert idx.dtype == torch.int64
+    assert torch.equal(ordered.cpu(), points.gather(1, idx.cpu()[..., None].expand(-1, -1, D)))
+    inv = lsh.invert_permutation(idx)
+    assert torch.equal(inv.cpu(), idx.cpu().argsort(dim=1))
+    assert torch.equal(lsh.gather_rows(ordered, inv).cpu(), points)
