@@ -31,6 +31,13 @@ _SIGNATURES = {
     "lampa_gather_rows": (_i32, [_vp, _i32, _i64, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
     "lampa_scatter_rows": (_i32, [_vp, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
     "lampa_invert_perm": (_i32, [_vp, _i32, _i32, _i64, _vp, _vp]),
+    "lampa_gdr_recurrent_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32,
+                                       _i32, _i32, _f32, _i32, _vp]),
+    "lampa_gdr_plan_size": (_i64, [_vp, _i32, _i32]),
+    "lampa_gdr_plan_fill": (_i32, [_vp, _i32, _i32, _vp]),
+    "lampa_gdr_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),
+    "lampa_gdr_chunk_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
+                                   _f32, _i32, _vp, _i64, _vp]),
 }
 
 _lib = None

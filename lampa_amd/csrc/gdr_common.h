@@ -1,0 +1,69 @@
+// Types and small device helpers shared by the gated-delta kernels (gfx950, wave64, MFMA 32x32x16 bf16).
+#pragma once
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+
+enum { GDR_BF16 = 0, GDR_FP16 = 1, GDR_FP32 = 2 };
+enum { GDR_L2_NONE = 0, GDR_L2_CHUNK = 1, GDR_L2_RECURRENT = 2 };
+
+// D = A (32x16) * B (16x32) + C on one wave.  Lane l = 32*hh + ln supplies A[row ln][k 8hh..8hh+7] and
+// B[k 8hh..8hh+7][col ln]; accumulator register r of lane l is element (row 8*(r/4) + 4*hh + r%4, col ln).
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// The 8 accumulator registers [base, base+8) of a lane, rounded to bf16, form that lane's share of an MFMA
+// operand whose 16-wide contraction step covers accumulator rows 16*(base/8) .. +15 in the order
+// slot s -> row 8*(s/4) + 4*hh + s%4.  Any operand built from memory for the other side of such a product
+// must use the same slot order (see kappa()).
+__device__ __forceinline__ bf16x8 acc_to_operand(const f32x16& acc, int base) {
+  bf16x8 out;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) out[s] = (__bf16)acc[base + s];
+  return out;
+}
+
+// Offset inside a 16-wide contraction step of slot s for lane half hh.
+__device__ __forceinline__ int kappa(int hh, int s) { return 8 * (s / 4) + 4 * hh + (s % 4); }
+
+__device__ __forceinline__ float bf16_bits_to_float(unsigned short b) { return __uint_as_float((uint32_t)b << 16); }
+
+template <typename T>
+struct GdrElem;
+template <>
+struct GdrElem<__bf16> {
+  static __device__ __forceinline__ float to_float(__bf16 x) { return (float)x; }
+  static __device__ __forceinline__ __bf16 from_float(float x) { return (__bf16)x; }
+};
+template <>
+struct GdrElem<_Float16> {
+  static __device__ __forceinline__ float to_float(_Float16 x) { return (float)x; }
+  static __device__ __forceinline__ _Float16 from_float(float x) { return (_Float16)x; }
+};
+template <>
+struct GdrElem<float> {
+  static __device__ __forceinline__ float to_float(float x) { return x; }
+  static __device__ __forceinline__ float from_float(float x) { return x; }
+};
+
+// Loads 8 consecutive elements (the pointer must be aligned to 8 elements) and widens them to fp32.
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float* out) {
+  if constexpr (sizeof(T) == 2) {
+    typedef T vec8 __attribute__((ext_vector_type(8)));
+    vec8 v = *reinterpret_cast<const vec8*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = GdrElem<T>::to_float(v[i]);
+  } else {
+    f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { out[i] = a[i]; out[4 + i] = b[i]; }
+  }
+}

@@ -1,0 +1,170 @@
+"""Gated-delta-rule forward on the GPU behind the reference's operator signatures.
+
+``chunk_gated_delta_rule`` (reference ``models/hattention/gated_delta_rule_ori.py:236-357``) and
+``fused_recurrent_gated_delta_rule`` (``gated_delta_rule_ori.py:565-667``): same argument names, order,
+defaults, checks and return tuples.  The arithmetic runs in hand-written gfx950 kernels reached through the
+C ABI of ``liblampa_amd.so``; there is no Triton, no PyTorch fallback and no CPU path.
+
+Differences that a caller can observe, all additive:
+* forward only -- ``backward`` raises ``NotImplementedError``;
+* ``allow_fp32=True`` lets ``chunk_gated_delta_rule`` accept float32 q/k/v (the reference rejects them); they
+  are evaluated by the token-serial fp32 kernel;
+* head sizes other than 64 / 128 are evaluated by the token-serial kernel as well (correct, slower).
+"""
+import ctypes
+import math
+import warnings
+from typing import Optional
+
+import torch
+
+from . import _capi
+from ._capi import check, ptr, require_cuda, stream_of
+
+L2_NONE, L2_CHUNK, L2_RECURRENT = 0, 1, 2
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+# Number of 64-token chunks per segment of the split-sequence scan; None picks it from the sequence lengths.
+CHUNKS_PER_SEGMENT: Optional[int] = None
+
+_plan_cache = {}
+
+
+def _default_chunks_per_segment(max_chunks: int) -> int:
+    # serial cost ~ (chunks per segment) + 0.3 * (segments per sequence); minimise over the split
+    return int(min(64, max(4, round(math.sqrt(0.3 * max(max_chunks, 1))))))
+
+
+def _plan(cu_host, device):
+    """Host + device copies of the chunk/segment tables for these sequence boundaries (cached)."""
+    max_chunks = max((b - a + 63) // 64 for a, b in zip(cu_host[:-1], cu_host[1:]))
+    cps = CHUNKS_PER_SEGMENT or _default_chunks_per_segment(max_chunks)
+    key = (tuple(cu_host), cps, str(device))
+    hit = _plan_cache.get(key)
+    if hit is not None:
+        return hit
+    lib = _capi.lib()
+    cu = (ctypes.c_int64 * len(cu_host))(*cu_host)
+    n_seq = len(cu_host) - 1
+    size = check(lib.lampa_gdr_plan_size(cu, n_seq, cps), "lampa_gdr_plan_size")
+    host = torch.empty(size, dtype=torch.int32)
+    check(lib.lampa_gdr_plan_fill(cu, n_seq, cps, ctypes.c_void_p(host.data_ptr())), "lampa_gdr_plan_fill")
+    dev = host.to(device)
+    if len(_plan_cache) > 64:
+        _plan_cache.clear()
+    _plan_cache[key] = (host, dev)
+    return host, dev
+
+
+def _recurrent_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
+    B, T, H, K = q.shape
+    HV, V = v.shape[2], v.shape[3]
+    n_seq = B if cu_seqlens is None else len(cu_seqlens) - 1
+    o = torch.empty_like(v)
+    ht = torch.empty((n_seq, HV, K, V), dtype=torch.float32, device=q.device) if output_final_state else None
+    cu = None if cu_seqlens is None else cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
+    h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+    check(_capi.lib().lampa_gdr_recurrent_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(o), ptr(h0), ptr(ht),
+                                              ptr(cu), n_seq, T, H, HV, K, V, _DTYPES[q.dtype], float(scale), l2norm,
+                                              stream_of(q)), "lampa_gdr_recurrent_fwd")
+    return o, ht
+
+
+def _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
+    B, T, H, K = q.shape
+    HV, V = v.shape[2], v.shape[3]
+    if cu_seqlens is None:
+        cu_host = [i * T for i in range(B + 1)]
+    else:
+        cu_host = [int(c) for c in cu_seqlens.tolist()]
+    n_seq = len(cu_host) - 1
+    plan_host, plan_dev = _plan(cu_host, q.device)
+    chunks, segs = int(plan_host[1]), int(plan_host[2])
+    lib = _capi.lib()
+    ws_bytes = check(lib.lampa_gdr_chunk_workspace_bytes(chunks, segs, HV, K, V), "lampa_gdr_chunk_workspace_bytes")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    o = torch.empty_like(v)
+    ht = torch.empty((n_seq, HV, K, V), dtype=torch.float32, device=q.device) if output_final_state else None
+    h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+    check(lib.lampa_gdr_chunk_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(o), ptr(h0), ptr(ht),
+                                  ctypes.c_void_p(plan_host.data_ptr()), ptr(plan_dev), H, HV, K, V, _DTYPES[q.dtype],
+                                  float(scale), l2norm, ptr(ws), ws_bytes, stream_of(q)), "lampa_gdr_chunk_fwd")
+    return o, ht
+
+
+def _chunk_path_supported(q, v) -> bool:
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] in (64, 128) and v.shape[-1] in (64, 128)
+
+
+class _ForwardOnly(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, launcher, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
+        require_cuda(q, k, v, g, beta, initial_state)
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
+        return launcher(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("lampa_amd gated-delta operators are forward-only")
+
+
+def _check_varlen(q, initial_state, cu_seqlens):
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(
+                f"The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`."
+                f"Please flatten variable-length inputs before processing.")
+        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+            raise ValueError(
+                f"The number of initial states is expected to be equal to the number of input sequences, "
+                f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+
+
+def chunk_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor,
+                           scale: float = None, initial_state: torch.Tensor = None, output_final_state: bool = False,
+                           cu_seqlens: Optional[torch.LongTensor] = None, head_first: bool = False,
+                           use_qk_l2norm_in_kernel: bool = False, *, allow_fp32: bool = False):
+    """q, k [B,T,H,K]; v [B,T,H,V]; g (log-decay, <= 0), beta [B,T,H]; returns (o [B,T,H,V] in q.dtype,
+    final_state [N,H,K,V] fp32 or None). See ``gated_delta_rule_ori.py:236-357`` for the argument contract."""
+    assert q.dtype == k.dtype == v.dtype
+    if not allow_fp32:
+        assert q.dtype != torch.float32, "ChunkGatedDeltaRuleFunction does not support float32. Please use bfloat16."
+    assert len(beta.shape) == 3, "beta must be of shape [B, T, H] if head_first=False, or [B, H, T] otherwise."
+    if head_first:
+        raise DeprecationWarning(
+            "head_first is deprecated and will be removed in a future version. "
+            "Please use head_first=False for now instead.")
+    if q.shape[1] < q.shape[2]:
+        warnings.warn(
+            f"Input tensor shape suggests potential format mismatch: seq_len ({q.shape[1]}) < num_heads ({q.shape[2]}). "
+            "This may indicate the inputs were passed in head-first format [B, H, T, ...] "
+            "when head_first=False was specified. "
+            "Please verify your input tensor format matches the expected shape [B, T, H, ...].")
+    _check_varlen(q, initial_state, cu_seqlens)
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    l2norm = L2_CHUNK if use_qk_l2norm_in_kernel else L2_NONE
+    launcher = _chunk_launch if _chunk_path_supported(q, v) else _recurrent_launch
+    o, final_state = _ForwardOnly.apply(launcher, q, k, v, g, beta, scale, initial_state, output_final_state,
+                                        cu_seqlens, l2norm)
+    return o.to(q.dtype), final_state
+
+
+def fused_recurrent_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
+                                     beta: torch.Tensor = None, scale: float = None,
+                                     initial_state: torch.Tensor = None, output_final_state: bool = False,
+                                     cu_seqlens: Optional[torch.LongTensor] = None,
+                                     use_qk_l2norm_in_kernel: bool = False):
+    """q, k [B,T,H,K]; v [B,T,HV,V]; g, beta [B,T,HV]; grouped value heads when HV > H. Returns (o [B,T,HV,V],
+    final_state [N,HV,K,V] fp32 or None). See ``gated_delta_rule_ori.py:565-667``."""
+    _check_varlen(q, initial_state, cu_seqlens)
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    else:
+        assert scale > 0, "scale must be positive"
+    if beta is None:
+        beta = torch.ones_like(q[..., 0])
+    l2norm = L2_RECURRENT if use_qk_l2norm_in_kernel else L2_NONE
+    return _ForwardOnly.apply(_recurrent_launch, q, k, v, g, beta, scale, initial_state, output_final_state,
+                              cu_seqlens, l2norm)

@@ -1,0 +1,176 @@
+"""GPU parity of the gated-delta operators against the CPU oracle.
+
+Tolerances (from the benchmark contract): bf16 inputs with fp32 accumulation -- max-abs 2e-2 and mean-relative
+5e-3 on outputs and final states; fp32 mode -- 1e-4.
+"""
+import pytest
+import torch
+
+from lampa_amd import gated_delta as gd
+from lampa_amd import synth
+from oracle import gated_delta as og
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_ABS, BF16_MEAN_REL, FP32_TOL = 2e-2, 5e-3, 1e-4
+
+
+def _errors(got, want):
+    got, want = got.detach().float().cpu(), want.float()
+    diff = (got - want).abs()
+    return diff.max().item(), (diff.mean() / want.abs().mean().clamp_min(1e-12)).item()
+
+
+def _assert_bf16_close(got, want, what):
+    max_abs, mean_rel = _errors(got, want)
+    assert max_abs <= BF16_MAX_ABS and mean_rel <= BF16_MEAN_REL, f"{what}: max_abs={max_abs:.3e} mean_rel={mean_rel:.3e}"
+
+
+def _to(dev, *xs):
+    return [None if x is None else x.to(dev) for x in xs]
+
+
+# ------------------------------------------------------------------------------------------------- token-serial
+@pytest.mark.parametrize("K,V,T", [(32, 32, 700), (64, 64, 300), (128, 128, 130), (16, 32, 257)])
+def test_recurrent_fp32_matches_oracle(device, K, V, T):
+    q, k, v, g, beta = synth.gdr_inputs(2, T, 3, K, V, torch.float32, seed=K + T, g_scale=0.1)
+    h0 = torch.randn(2, 3, K, V, generator=torch.Generator().manual_seed(1))
+    for l2, flag in ((og.L2_NONE, False), (og.L2_RECURRENT, True)):
+        want_o, want_s = og.recurrent_c(q * 2, k, v, g, beta, initial_state=h0, l2=l2)
+        o, s = gd.fused_recurrent_gated_delta_rule(*_to(device, q * 2, k, v, g, beta), initial_state=h0.to(device),
+                                                   output_final_state=True, use_qk_l2norm_in_kernel=flag)
+        assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL
+
+
+def test_config0_fp32_plumbing(device):
+    # B=1, H=4, T=8192, d_k=d_v=32, fp32, seed 0, zero initial state
+    q, k, v, g, beta = synth.gdr_inputs(1, 8192, 4, 32, 32, torch.float32, seed=0)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta)
+    o, s = gd.fused_recurrent_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True)
+    assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL
+    o2, s2 = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True, allow_fp32=True)
+    assert _errors(o2, want_o)[0] <= FP32_TOL and _errors(s2, want_s)[0] <= FP32_TOL
+    with pytest.raises(AssertionError):
+        gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta))
+
+
+def test_recurrent_varlen_gva_bf16(device):
+    gen = torch.Generator().manual_seed(3)
+    T, H, HV, K, V = 500, 2, 4, 64, 64
+    q = torch.randn(1, T, H, K, generator=gen).bfloat16()
+    k = torch.nn.functional.normalize(torch.randn(1, T, H, K, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(1, T, HV, V, generator=gen).bfloat16()
+    g = -torch.rand(1, T, HV, generator=gen) * 0.2
+    beta = torch.rand(1, T, HV, generator=gen)
+    cu = torch.tensor([0, 100, 101, 333, 500])
+    h0 = torch.randn(4, HV, K, V, generator=gen)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu, l2=og.L2_RECURRENT)
+    o, s = gd.fused_recurrent_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                               output_final_state=True, cu_seqlens=cu.to(device),
+                                               use_qk_l2norm_in_kernel=True)
+    _assert_bf16_close(o, want_o, "o")
+    assert _errors(s, want_s)[0] <= 1e-3
+    # beta=None means all ones
+    o1, _ = gd.fused_recurrent_gated_delta_rule(*_to(device, q[:, :, :, :], k, v[:, :, :2], g[:, :, :2]))
+    w1, _ = og.recurrent_c(q, k, v[:, :, :2], g[:, :, :2], torch.ones(1, T, 2))
+    _assert_bf16_close(o1, w1, "beta none")
+
+
+# ----------------------------------------------------------------------------------------------------- chunk path
+@pytest.mark.parametrize("T", [1, 64, 65, 200, 1000])
+@pytest.mark.parametrize("g_scale", [1.0, 0.02])
+def test_chunk_bf16_matches_oracle(device, T, g_scale):
+    q, k, v, g, beta = synth.gdr_inputs(2, T, 2, 64, 64, torch.bfloat16, seed=T, g_scale=g_scale)
+    h0 = 0.5 * torch.randn(2, 2, 64, 64, generator=torch.Generator().manual_seed(2))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                     output_final_state=True)
+    assert o.dtype == torch.bfloat16 and s.dtype == torch.float32 and s.shape == (2, 2, 64, 64)
+    _assert_bf16_close(o, want_o, f"o T={T}")
+    _assert_bf16_close(s, want_s, f"state T={T}")
+
+
+@pytest.mark.parametrize("cps", [1, 3, 16])
+def test_chunk_segment_split_is_invisible(device, cps, monkeypatch):
+    monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", cps)
+    q, k, v, g, beta = synth.gdr_inputs(1, 64 * 13 + 7, 2, 64, 64, torch.bfloat16, seed=9, g_scale=0.01)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True)
+    _assert_bf16_close(o, want_o, f"o cps={cps}")
+    _assert_bf16_close(s, want_s, f"state cps={cps}")
+
+
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 128), (128, 64)])
+def test_chunk_other_head_sizes_and_l2norm(device, K, V):
+    q, k, v, g, beta = synth.gdr_inputs(1, 333, 2, K, V, torch.bfloat16, seed=K + V, g_scale=0.05)
+    q, k = (q.float() * 3).bfloat16(), (k.float() * 0.3).bfloat16()
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, l2=og.L2_CHUNK)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True,
+                                     use_qk_l2norm_in_kernel=True)
+    _assert_bf16_close(o, want_o, "o")
+    _assert_bf16_close(s, want_s, "state")
+
+
+def test_chunk_varlen_equals_separate_runs(device):
+    lens = [5, 64, 0, 130, 700, 1]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)))
+    T = int(cu[-1])
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 2, 64, 64, torch.bfloat16, seed=11, g_scale=0.05)
+    h0 = 0.5 * torch.randn(len(lens), 2, 64, 64, generator=torch.Generator().manual_seed(4))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                     output_final_state=True, cu_seqlens=cu.to(device))
+    _assert_bf16_close(o, want_o, "o")
+    _assert_bf16_close(s, want_s, "state")
+    assert torch.equal(s[2].cpu(), h0[2])  # an empty sequence returns its initial state
+    # no final state requested -> None; fp16 inputs accepted
+    o16, none = gd.chunk_gated_delta_rule(*_to(device, q.half(), k.half(), v.half(), g, beta), cu_seqlens=cu.to(device))
+    assert none is None and o16.dtype == torch.float16
+    w16, _ = og.recurrent_c(q.half(), k.half(), v.half(), g, beta, cu_seqlens=cu)
+    _assert_bf16_close(o16, w16, "fp16 o")
+
+
+def test_chunk_argument_checks(device):
+    q, k, v, g, beta = _to(device, *synth.gdr_inputs(2, 128, 2, 64, 64, torch.bfloat16, seed=0))
+    with pytest.raises(ValueError):
+        gd.chunk_gated_delta_rule(q, k, v, g, beta, cu_seqlens=torch.tensor([0, 128], device=device))
+    with pytest.raises(ValueError):
+        gd.chunk_gated_delta_rule(q[:1], k[:1], v[:1], g[:1], beta[:1], cu_seqlens=torch.tensor([0, 100, 128], device=device),
+                                  initial_state=torch.zeros(3, 2, 64, 64, device=device))
+    with pytest.raises(DeprecationWarning):
+        gd.chunk_gated_delta_rule(q, k, v, g, beta, head_first=True)
+    with pytest.warns(UserWarning):
+        gd.chunk_gated_delta_rule(q[:, :1], k[:, :1], v[:, :1], g[:, :1], beta[:, :1])
+    with pytest.raises(Exception):
+        gd.chunk_gated_delta_rule(q.cpu(), k.cpu(), v.cpu(), g.cpu(), beta.cpu())  # no CPU fallback
+
+
+def test_chunk_matches_token_serial_kernel_on_gpu(device):
+    q, k, v, g, beta = _to(device, *synth.gdr_inputs(1, 5000, 4, 64, 64, torch.bfloat16, seed=21, g_scale=0.1))
+    o1, s1 = gd.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    o2, s2 = gd.fused_recurrent_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    _assert_bf16_close(o1, o2.float().cpu(), "o")
+    _assert_bf16_close(s1, s2.cpu(), "state")
+
+
+def test_config2_full_size(device):
+    # B=1, H=8, T=60000, d=64, bf16 q/k/v, fp32 g/beta, tokens in the LSH-sorted order of a config-1 event
+    from lampa_amd import lsh
+
+    q, k, v, g, beta = synth.gdr_inputs(1, 60000, 8, 64, 64, torch.bfloat16, seed=0)
+    coords, _, _ = synth.collider_event(60000, seed=0)
+    alpha, b = synth.lsh_params(4, 3, 4, 0.5, 1)
+    perm = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), b.to(device), 0.5, 3, 4)["perm"][0].long().cpu()
+    q, k, v, g, beta = (x[:, perm].contiguous() for x in (q, k, v, g, beta))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True)
+    _assert_bf16_close(o, want_o, "o")
+    _assert_bf16_close(s, want_s, "state")
+    # size-independent property: splitting the sequence and carrying the state reproduces the one-shot run
+    cut = 64 * 400 + 17
+    oa, sa = gd.chunk_gated_delta_rule(*_to(device, q[:, :cut], k[:, :cut], v[:, :cut], g[:, :cut], beta[:, :cut]),
+                                       output_final_state=True)
+    ob, sb = gd.chunk_gated_delta_rule(*_to(device, q[:, cut:], k[:, cut:], v[:, cut:], g[:, cut:], beta[:, cut:]),
+                                       initial_state=sa, output_final_state=True)
+    _assert_bf16_close(torch.cat([oa, ob], 1), o.float().cpu(), "split o")
+    _assert_bf16_close(sb, s.cpu(), "split state")
