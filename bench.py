@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+A step is one chunkwise gated-delta layer forward (BASELINE config 2: B=1, H=8, T=60000, d_k=d_v=64, C=64, bf16
+q/k/v, fp32 g/beta, tokens in the LSH-sorted order of a config-1 event) with every input resident in HBM.
+Prints one JSON line; see DESIGN.md for how each figure is defined.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+T, H, K, V = 60000, 8, 64, 64
+N_HITS, N_TABLES, N_PROJ, W_BUCKET, FEAT_DIM = 60000, 3, 4, 0.5, 24
+# algorithmic work per unit
+LAYER_BYTES_PER_TOKEN_HEAD = 2 * K + 2 * K + 2 * V + 2 * V + 8                 # q,k,v,o bf16 + g,beta fp32 = 520
+LAYER_FLOP_PER_TOKEN_HEAD = 2 * 64 * (3 * K + 2 * V) + 6 * K * V + (2 * 64 * 64) // 3  # 68.3 kFLOP
+KERNEL_BYTES_PER_TOKEN_HEAD = {            # the part of the 520 B each kernel of the pipeline is responsible for
+    "gdr_prep_kernel": 2 * K + 2 * K + 2 * V + 8,   # reads q, k, v, g, beta
+    "gdr_output_kernel": 2 * V,                     # writes o
+}
+LSH_BYTES_PER_HIT_TABLE = 224
+
+
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def cpu_baseline_gdr(q, k, v, g, beta, sample_tokens):
+    """The reference's CPU path for the layer: a token loop in plain PyTorch (port: oracle.gated_delta.recurrent_delta,
+    fp32) on a prefix of the same inputs, scaled to hits/s."""
+    import torch
+    from oracle import gated_delta as og
+
+    sl = slice(0, sample_tokens)
+    args = [x[:, sl].float() for x in (q, k, v, g, beta)]
+    og.recurrent_delta(*[a[:, :64] for a in args], dtype=torch.float32)  # warm-up
+    t0 = time.perf_counter()
+    og.recurrent_delta(*args, dtype=torch.float32)
+    dt = time.perf_counter() - t0
+    return sample_tokens / dt, dt
+
+
+def cpu_baseline_lsh(coords, feats, alpha):
+    """The reference's CPU path for the LSH stage in plain PyTorch: bmm -> quantise -> pack -> stable sort -> gather."""
+    import torch
+
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        proj = torch.bmm(coords[None], alpha[None])[0]
+        ids = torch.floor(proj / W_BUCKET).to(torch.int64).T.reshape(N_TABLES, N_PROJ, -1)
+        lo = ids.amin(-1, keepdim=True)
+        rng = ids.amax(-1, keepdim=True) - lo + 1
+        stride = torch.cumprod(torch.cat([torch.ones_like(rng[:, :1]), rng[:, :-1]], 1), 1)
+        keys = ((ids - lo) * stride).sum(1)
+        perm = torch.sort(keys, dim=-1, stable=True).indices
+        out = feats[None].expand(N_TABLES, -1, -1).gather(1, perm[..., None].expand(-1, -1, feats.shape[-1]))
+        times.append(time.perf_counter() - t0)
+    del out
+    return _median(times)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
+              "(sharding is described in DESIGN.md, not implemented).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from lampa_amd import _capi
+    from lampa_amd import gated_delta as gd
+    from lampa_amd import lsh, synth
+
+    if not os.path.exists(_capi.LIB_PATH):
+        from lampa_amd import build as lib_build
+        lib_build.build()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---- inputs (synthetic, seeded) ----
+    coords, feats, _ = synth.collider_event(N_HITS, seed=0)
+    alpha, beta_h = synth.lsh_params(4, N_TABLES, N_PROJ, W_BUCKET, 1)
+    q, k, v, g, beta = synth.gdr_inputs(1, T, H, K, V, torch.bfloat16, seed=0)
+    coords_d, feats_d, alpha_d, beta_hd = (x.to(dev) for x in (coords, feats, alpha, beta_h))
+    perm = lsh.lsh_bucket_sort(coords_d, alpha_d, beta_hd, W_BUCKET, N_TABLES, N_PROJ)["perm"][0].long().cpu()
+    q, k, v, g, beta = (x[:, perm].contiguous() for x in (q, k, v, g, beta))
+    qd, kd, vd, gd_, bd = (x.to(dev) for x in (q, k, v, g, beta))
+
+    def step():
+        return gd.chunk_gated_delta_rule(qd, kd, vd, gd_, bd, output_final_state=True)
+
+    # ---- timed region: exactly K steps ----
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    hits_per_s = T / (elapsed / args.steps)
+
+    # ---- per-kernel durations with HIP events on the launch stream (separate pass of the same steps) ----
+    _capi.profile_begin()
+    for _ in range(args.steps):
+        step()
+    prof = _capi.profile_end(max_entries=8 * args.steps + 8)
+    stage = {}
+    for name, ms in prof:
+        stage.setdefault(name, []).append(ms)
+    stage_us = {name: 1e3 * sum(v_) / len(v_) for name, v_ in stage.items()}
+    dominant = max(stage_us, key=stage_us.get)
+    token_heads = T * H
+    dom_bytes = KERNEL_BYTES_PER_TOKEN_HEAD.get(dominant, LAYER_BYTES_PER_TOKEN_HEAD) * token_heads
+    dom_gbs = dom_bytes / (stage_us[dominant] * 1e-6) / 1e9
+    layer_us = ms_per_step * 1e3
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel_us": round(stage_us[dominant], 2), "algorithmic_bytes_per_launch": dom_bytes}
+    layer = {
+        "us_per_layer": round(layer_us, 2),
+        "hbm_frac": round(LAYER_BYTES_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "mfma_frac": round(LAYER_FLOP_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "kernel_us": {n: round(u, 2) for n, u in stage_us.items()},
+    }
+
+    # ---- LSH stage (config 1): ids + keys + stable sort + feature gather, 3 tables ----
+    def lsh_step():
+        return lsh.lsh_bucket_sort(coords_d, alpha_d, beta_hd, W_BUCKET, N_TABLES, N_PROJ, feats_d)
+
+    for _ in range(args.warmup):
+        lsh_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lsh_step()
+    torch.cuda.synchronize()
+    lsh_us = 1e6 * (time.perf_counter() - t0) / args.steps
+    _capi.profile_begin()
+    for _ in range(args.steps):
+        lsh_step()
+    lprof = _capi.profile_end(max_entries=16 * args.steps + 16)
+    lstage = {}
+    for name, ms in lprof:
+        lstage.setdefault(name, []).append(ms)
+    lsh_bytes = LSH_BYTES_PER_HIT_TABLE * N_HITS * N_TABLES
+    lsh_kernel_us = {n: round(1e3 * sum(v_) / args.steps, 2) for n, v_ in lstage.items()}
+    lsh_gpu_us = sum(lsh_kernel_us.values())
+    lsh_info = {
+        "workload": f"config1: N={N_HITS}, {N_TABLES} tables x {N_PROJ} proj, w={W_BUCKET}, {FEAT_DIM} fp32 feats",
+        "us_per_event": round(lsh_us, 2), "hits_per_s": round(N_HITS / (lsh_us * 1e-6), 1),
+        "sum_kernel_us": round(lsh_gpu_us, 2), "kernel_us_per_event": lsh_kernel_us,
+        "roofline": {"bound": "hbm", "achieved": round(lsh_bytes / (lsh_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(lsh_bytes / (lsh_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     "algorithmic_bytes": lsh_bytes},
+    }
+
+    # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
+    cores = torch.get_num_threads()
+    cpu_hits_per_s, cpu_dt = cpu_baseline_gdr(q, k, v, g, beta, args.cpu_sample_tokens)
+    lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha)
+    lsh_info["cpu_baseline_us"] = round(lsh_cpu_s * 1e6, 1)
+    cpu = {"value": round(cpu_hits_per_s, 1), "unit": "hits/s", "cores": cores, "kind": "port",
+           "sample": f"first {args.cpu_sample_tokens} of {T} tokens, all {H} heads, fp32 token loop in PyTorch "
+                     f"({cpu_dt:.2f} s), scaled linearly",
+           "cpu_count": os.cpu_count()}
+
+    out = {
+        "metric": "hits/s per gated-delta layer at T=60k (bf16); % HBM and MFMA roofline",
+        "value": round(hits_per_s, 1), "unit": "hits/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
+                               "g/beta/state, LSH-sorted token order of a config-1 event"},
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,136 @@
+/*
+ * lampa_amd.h -- C ABI of liblampa_amd.so: the MI355X (gfx950) implementation of Lampa's data-parallel hot path,
+ * E2LSH hashing + stable bucket sort + gather of detector hits, then the chunkwise gated-delta-rule forward.
+ *
+ * Conventions
+ *   - every pointer named *_dev or documented as "device" is HIP device memory on the current device; inputs are
+ *     never modified; outputs and workspaces are caller-allocated (query the *_workspace_bytes function first);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all work is enqueued on it and the
+ *     functions return without synchronising;
+ *   - return value: 0 on success, negative on error (LAMPA_ERR_*). No C++ exception crosses the boundary;
+ *   - the library keeps no state between calls apart from the optional profiling recorder.
+ * The reference (chengjiang123/Lampa) is Python over Triton/ATen, so each entry point names the Python operator or
+ * kernel it replaces (file:line in the reference tree).
+ */
+#ifndef LAMPA_AMD_H
+#define LAMPA_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LAMPA_OK 0
+#define LAMPA_ERR_INVALID (-1)     /* bad argument */
+#define LAMPA_ERR_WORKSPACE (-2)   /* workspace missing or too small */
+#define LAMPA_ERR_LAUNCH (-3)      /* HIP reported an error at launch */
+#define LAMPA_ERR_UNSUPPORTED (-4) /* shape / dtype outside what the kernels are built for */
+
+/* key kinds of lampa_sort_pairs */
+#define LAMPA_KEY_U32 0
+#define LAMPA_KEY_I32 1
+#define LAMPA_KEY_F32 2 /* torch.sort order: -0.0 == +0.0, NaN last */
+
+/* element types of q, k, v, o */
+#define LAMPA_BF16 0
+#define LAMPA_FP16 1
+#define LAMPA_FP32 2
+
+/* l2 normalisation of q and k inside the kernel */
+#define LAMPA_L2_NONE 0
+#define LAMPA_L2_CHUNK 1     /* x / sqrt(sum x^2 + 1e-6)      models/hattention/l2norm.py:97-103 */
+#define LAMPA_L2_RECURRENT 2 /* x / (sqrt(sum x^2) + 1e-6)    models/hattention/gated_delta_rule_ori.py:436-438 */
+
+/* ------------------------------------------------------------------------------------------------ LSH stage */
+
+/* E2LSH projection. Replaces E2LSH.forward = torch.bmm(vecs, alpha) + permute
+ * (models/model_utils/hash_utils.py:368-371; models/baselines/full_mamba2.py:136-141).
+ * vecs [n_heads, n_hits, dim] fp32, alpha [n_heads, dim, n_cols] fp32; out element (c, head, n) is written at
+ * out[c*stride_c + head*stride_h + n*stride_n] (so both reference layouts are one call).
+ * Arithmetic: p = fmaf(x[d], a[d], p) for d = 0..dim-1 starting from 0. */
+int lampa_lsh_project_f32(const float* vecs, int n_heads, int64_t n_hits, int dim, const float* alpha, int n_cols,
+                          float* out, int64_t stride_c, int64_t stride_h, int64_t stride_n, void* stream);
+
+/* Per-row (min, max) of x [rows, n] -> out [rows, 2]. Replaces the four max/min reductions of lsh_mapping
+ * (models/model_utils/hash_utils.py:334-340). */
+int lampa_row_minmax_f32(const float* x, int rows, int64_t n, float* out, void* stream);
+
+/* Quantised E2LSH bucket ids and mixed-radix bucket keys of one event.
+ * Replaces the hash + range + key-combination steps of the reference's bucketing front end
+ * (hash_utils.py:333-371, models/attention/hept.py:79-88) with the textbook id floor((a.x + b) / w).
+ * coords [n_hits, dim] fp32 (dim <= 8); alpha [dim, n_tables*n_proj]; beta [n_tables*n_proj]; column
+ * c = table*n_proj + projection. Hits n >= n_valid are padding (ids 0, key = total so that they sort last).
+ * ids_out [n_tables*n_proj, n_hits] int32 (nullable), keys_out [n_tables, n_hits] int32,
+ * meta_out [n_tables, 2*n_proj+3] int32 = lo[n_proj], range[n_proj], total, key_bits, overflow. */
+int64_t lampa_lsh_bucket_workspace_bytes(int64_t n_hits, int n_tables, int n_proj);
+int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, int dim, const float* alpha,
+                          const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
+                          int32_t* meta_out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Sort keys of LSHOrdering: key[n] = sum_h 2^h <coords[n], alpha[:, h]>, norm[n] = |coords[n]|.
+ * Replaces models/baselines/full_mamba2.py:174-203. coords [n_hits, dim], alpha [dim, n_hashes]. */
+int lampa_lsh_ordering_keys(const float* coords, int64_t n_hits, int dim, const float* alpha, int n_hashes,
+                            float* key_out, float* norm_out, void* stream);
+
+/* Stable ascending segmented radix sort of (32-bit key, int32 payload) pairs; payload defaults to the position.
+ * Replaces argsort / sort(stable=True) (models/attention/hept.py:138-139; full_mamba2.py:203,207,678).
+ * keys_in [n_segments, n]; vals_in [n_segments, n] or NULL; vals_out [n_segments, n].
+ * key_bits (1..32) or key_bits_dev (device, element s at key_bits_dev[s*key_bits_stride]) bound the significant
+ * bits of LAMPA_KEY_U32 keys; n_passes 0 = automatic. */
+int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n);
+int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
+                     int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
+                     int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* dst[s, i, :] = src[s % src_segments, idx[s, i], :]. Replaces batched_index_select / sort_to_buckets /
+ * unsort_from_buckets and the points.gather of LSHOrdering (hash_utils.py:83-93; hept.py:9-19;
+ * full_mamba2.py:213-216,679-682). idx_bytes = 4 (int32) or 8 (int64); rows of row_bytes bytes. */
+int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
+                      int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
+
+/* dst[s, idx[s, i], :] = src[s, i, :] (unsort by scatter, the O(n) alternative to full_mamba2.py:678-682). */
+int lampa_scatter_rows(const void* src, const void* idx, int idx_bytes, int n_segments, int64_t n,
+                       int64_t row_bytes, void* dst, void* stream);
+
+/* inv[s, perm[s, i]] = i. Replaces invert_permutation (hash_utils.py:46-57). */
+int lampa_invert_perm(const void* perm, int idx_bytes, int n_segments, int64_t n, void* inv, void* stream);
+
+/* ---------------------------------------------------------------------------------------- gated-delta forward */
+
+/* Token-serial forward with an fp32 state. Replaces fused_recurrent_gated_delta_rule_fwd
+ * (models/hattention/gated_delta_rule_ori.py:372-520); also the fp32 mode of the chunk operator.
+ * q, k [tokens, H, K]; v, o [tokens, HV, V] (dtype LAMPA_BF16/FP16/FP32); g, beta fp32 [tokens, HV];
+ * h0, ht fp32 [n_seq, HV, K, V] (nullable). cu_seqlens: device int64 [n_seq+1] or NULL (n_seq blocks of t_len). */
+int lampa_gdr_recurrent_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta, void* o,
+                            const float* h0, float* ht, const int64_t* cu_seqlens, int n_seq, int64_t t_len, int H,
+                            int HV, int K, int V, int dtype, float scale, int l2norm, void* stream);
+
+/* Chunk / segment tables of the chunkwise forward, built on the host from the sequence boundaries.
+ * Replaces prepare_chunk_indices / prepare_chunk_offsets (models/hattention/index.py:69-83).
+ * cu_seqlens_host: int64 [n_seq+1]; chunks_per_segment: length of a segment of the split-sequence scan in
+ * 64-token chunks. plan[1] = number of chunks, plan[2] = number of segments. */
+int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment);
+int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment, int32_t* plan_host);
+
+/* Chunkwise forward (chunk = 64 tokens). Replaces chunk_gated_delta_rule_fwd and the seven Triton kernels it
+ * launches (models/hattention/gated_delta_rule_ori.py:29-80). Shapes as above with H <= HV; K, V in {64, 128};
+ * dtype LAMPA_BF16 or LAMPA_FP16; plan_host / plan_dev: the same plan in host and device memory. */
+int64_t lampa_gdr_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V);
+int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta, void* o,
+                        const float* h0, float* ht, const int32_t* plan_host, const int32_t* plan_dev, int H, int HV,
+                        int K, int V, int dtype, float scale, int l2norm, void* workspace, int64_t workspace_bytes,
+                        void* stream);
+
+/* ------------------------------------------------------------------------------------------------- profiling */
+
+/* Time every kernel the library launches between begin and end with HIP events on the launch stream (a
+ * benchmarking aid with no counterpart in the reference; one recording at a time, not thread-safe).
+ * lampa_profile_end returns the number of entries written: ms[i] and a static name string per kernel launch. */
+int lampa_profile_begin(void);
+int lampa_profile_end(int max_entries, float* ms, const char** names);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LAMPA_AMD_H */

@@ -33,6 +33,8 @@ _SIGNATURES = {
     "lampa_invert_perm": (_i32, [_vp, _i32, _i32, _i64, _vp, _vp]),
     "lampa_gdr_recurrent_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32,
                                        _i32, _i32, _f32, _i32, _vp]),
+    "lampa_profile_begin": (_i32, []),
+    "lampa_profile_end": (_i32, [_i32, _vp, _vp]),
     "lampa_gdr_plan_size": (_i64, [_vp, _i32, _i32]),
     "lampa_gdr_plan_fill": (_i32, [_vp, _i32, _i32, _vp]),
     "lampa_gdr_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),
@@ -61,6 +63,19 @@ def lib() -> ctypes.CDLL:
             fn.restype, fn.argtypes = res, args
         _lib = handle
     return _lib
+
+
+def profile_begin():
+    """Start timing every kernel launched by the library (HIP events on the launch stream)."""
+    check(lib().lampa_profile_begin(), "lampa_profile_begin")
+
+
+def profile_end(max_entries: int = 256):
+    """Stop timing; returns [(kernel name, milliseconds), ...] in launch order."""
+    ms = (ctypes.c_float * max_entries)()
+    names = (ctypes.c_char_p * max_entries)()
+    n = check(lib().lampa_profile_end(max_entries, ms, names), "lampa_profile_end")
+    return [(names[i].decode(), float(ms[i])) for i in range(n)]
 
 
 def exported_symbols():

@@ -17,3 +17,9 @@ static inline int lampa_launch_status() {
 static inline int64_t lampa_align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+// Optional per-kernel timing with HIP events on the launch stream (see profile.hip). No-ops unless a
+// recording is open; the launchers call LAMPA_PROF(stream, "start") first and LAMPA_PROF(stream, "<kernel>") after
+// each launch.
+void lampa_prof_mark(hipStream_t stream, const char* name);
+#define LAMPA_PROF(stream, name) lampa_prof_mark((stream), (name))

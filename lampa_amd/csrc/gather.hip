@@ -58,6 +58,7 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
   const int vec_per_row = (int)(row_bytes / vec);
   const int64_t items = n * vec_per_row;
   const dim3 grid((unsigned)((items + GS_BLOCK - 1) / GS_BLOCK), n_segments), block(GS_BLOCK);
+  LAMPA_PROF(s, "start");
   if (vec == 16)
     hipLaunchKernelGGL((gs_rows_kernel<uint4, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride, src_segments,
                        idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);

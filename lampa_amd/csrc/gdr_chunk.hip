@@ -661,16 +661,22 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       return LAMPA_ERR_LAUNCH;
     attr_set = true;
   }
+  LAMPA_PROF(s, "start");
   if (chunks > 0) {
     hipLaunchKernelGGL((gdr_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem, s, (const T*)q, (const T*)k,
                        (const T*)v, g, beta, plan_dev, records, decs, H, HV, scale, l2norm);
-    if (segs > n_seq)
+    LAMPA_PROF(s, "gdr_prep_kernel");
+    if (segs > n_seq) {
       hipLaunchKernelGGL((gdr_composite_kernel<KT, VT>), dim3((KT + VT) / 32, segs, HV), dim3(64), 0, s, plan_dev,
                          records, decs, Mc, Nc, HV);
+      LAMPA_PROF(s, "gdr_composite_kernel");
+    }
   }
   hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, plan_dev, Mc, Nc, h0, Si, HV);
+  LAMPA_PROF(s, "gdr_scan_kernel");
   hipLaunchKernelGGL((gdr_output_kernel<T, KT, VT>), dim3(VT / 32, segs, HV), dim3(64), 0, s, plan_dev, records, decs,
                      Si, (T*)o, ht, HV);
+  LAMPA_PROF(s, "gdr_output_kernel");
   return lampa_launch_status();
 }
 

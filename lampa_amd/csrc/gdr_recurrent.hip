@@ -93,6 +93,7 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
                                 void* o, const float* h0, float* ht, const int64_t* cu, int n_seq, int64_t t_len,
                                 int H, int HV, int K, int V, float scale, int l2norm, hipStream_t s) {
   const dim3 grid((V + 63) / 64, n_seq * HV), block(64);
+  LAMPA_PROF(s, "start");
 #define GDR_REC_CASE(KT)                                                                                         \
   hipLaunchKernelGGL((gdr_recurrent_kernel<T, KT>), grid, block, 0, s, (const T*)q, (const T*)k, (const T*)v, g, \
                      beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm)
@@ -100,6 +101,7 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
   else if (K <= 64) GDR_REC_CASE(64);
   else GDR_REC_CASE(128);
 #undef GDR_REC_CASE
+  LAMPA_PROF(s, "gdr_recurrent_kernel");
   return lampa_launch_status();
 }
 

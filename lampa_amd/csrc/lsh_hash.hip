@@ -237,19 +237,23 @@ extern "C" int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_
   int blocks_valid = (int)((n_valid + LSH_BLOCK - 1) / LSH_BLOCK);
   if (blocks_valid < 1) blocks_valid = 1;
   const int blocks_all = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
+  LAMPA_PROF(s, "start");
   if (dim == 4) {
     hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
                        beta, n_cols, inv_w, partial);
+    LAMPA_PROF(s, "lsh_minmax_kernel");
     hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
                        meta_out);
   } else {
     hipLaunchKernelGGL(lsh_minmax_kernel<0>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
                        beta, n_cols, inv_w, partial);
+    LAMPA_PROF(s, "lsh_minmax_kernel");
     hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
                        meta_out);
   }
+  LAMPA_PROF(s, "lsh_pack_kernel");
   return lampa_launch_status();
 }
 

@@ -221,6 +221,7 @@ extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t
   int32_t* vbuf[2] = {(int32_t*)(ws + 2 * pairs), (int32_t*)(ws + 3 * pairs)};
   uint32_t* hist = (uint32_t*)(ws + 4 * pairs);
   const dim3 grid(n_tiles, n_segments), block(RS_BLOCK);
+  LAMPA_PROF(s, "start");
   for (int p = 0; p < n_passes; ++p) {
     const uint32_t* kin = p == 0 ? (const uint32_t*)keys_in : kbuf[(p - 1) & 1];
     const int32_t* vin = p == 0 ? vals_in : vbuf[(p - 1) & 1];
@@ -228,9 +229,11 @@ extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t
     const bool last = p == n_passes - 1;
     hipLaunchKernelGGL(rs_histogram_kernel, grid, block, 0, s, kin, n, kind, key_bits_dev, key_bits_stride, key_bits,
                        p, n_passes, hist);
+    LAMPA_PROF(s, "rs_histogram_kernel");
     hipLaunchKernelGGL(rs_scatter_kernel, grid, block, 0, s, kin, vin, n, kind, key_bits_dev, key_bits_stride,
                        key_bits, p, n_passes, hist, last ? (uint32_t*)nullptr : kbuf[p & 1],
                        last ? vals_out : vbuf[p & 1]);
+    LAMPA_PROF(s, "rs_scatter_kernel");
   }
   return lampa_launch_status();
 }

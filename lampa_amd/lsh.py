@@ -253,7 +253,7 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
     dev = coords.device
     ids = torch.empty((n_tables * n_proj, n), dtype=torch.int32, device=dev) if return_ids else None
     keys = torch.empty((n_tables, n), dtype=torch.int32, device=dev)
-    meta = torch.zeros((n_tables, 2 * n_proj + 3), dtype=torch.int32, device=dev)
+    meta = torch.empty((n_tables, 2 * n_proj + 3), dtype=torch.int32, device=dev)
     lib = _capi.lib()
     ws = _workspace(check(lib.lampa_lsh_bucket_workspace_bytes(n, n_tables, n_proj), "workspace"), dev)
     check(lib.lampa_lsh_bucket_keys(ptr(coords), n, n_valid, dim, ptr(alpha), ptr(beta), n_tables, n_proj, float(w),

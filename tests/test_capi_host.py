@@ -1,0 +1,106 @@
+"""Host-side checks that run without a GPU: the C-ABI library loads, exports every symbol the header declares,
+and its host-only planning logic is right. No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from lampa_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_capi.LIB_PATH):
+        from lampa_amd import build
+
+        build.build(verbose=False)
+    return _capi.lib()
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "lampa_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lampa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = _declared()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in include/lampa_amd.h but not exported"
+    assert sorted(_capi.exported_symbols()) == names  # the ctypes binding covers the whole header
+
+
+def test_workspace_queries_and_argument_errors(lib):
+    assert lib.lampa_sort_workspace_bytes(3, 60000) > 4 * 3 * 60000 * 4
+    assert lib.lampa_sort_workspace_bytes(0, 10) == -1
+    assert lib.lampa_lsh_bucket_workspace_bytes(60000, 3, 4) >= 235 * 12 * 8
+    assert lib.lampa_gdr_chunk_workspace_bytes(938, 60, 8, 64, 64) > 938 * 8 * 40 * 1024
+    assert lib.lampa_gdr_chunk_workspace_bytes(938, 60, 8, 48, 64) == -4  # unsupported head size
+    # null pointers / bad sizes are rejected before any launch
+    assert lib.lampa_sort_pairs(None, 0, None, 1, 10, 32, None, 1, 0, None, None, 0, None) == -1
+    assert lib.lampa_gather_rows(None, 1, 1, None, 4, 1, 1, 4, None, None) == -1
+    assert lib.lampa_gdr_recurrent_fwd(*([None] * 9), 1, 1, 1, 1, 64, 64, 0, 1.0, 0, None) == -1
+
+
+def _plan(lib, cu, cps):
+    arr = (ctypes.c_int64 * len(cu))(*cu)
+    size = lib.lampa_gdr_plan_size(arr, len(cu) - 1, cps)
+    assert size > 0
+    plan = torch.zeros(size, dtype=torch.int32)
+    assert lib.lampa_gdr_plan_fill(arr, len(cu) - 1, cps, ctypes.c_void_p(plan.data_ptr())) == 0
+    return plan.tolist()
+
+
+def test_plan_tables(lib):
+    cu = [0, 5, 69, 69, 199, 60199]
+    p = _plan(lib, cu, 16)
+    n_seq, chunks, segs, cps = p[0:4]
+    lens = [b - a for a, b in zip(cu[:-1], cu[1:])]
+    want_chunks = [(l + 63) // 64 for l in lens]
+    assert (n_seq, chunks, cps) == (5, sum(want_chunks), 16)
+    tok0 = p[p[4]:p[4] + chunks]
+    clen = p[p[5]:p[5] + chunks]
+    seg_c0, seg_nc = p[p[6]:p[6] + segs], p[p[7]:p[7] + segs]
+    seg_seq, seg_flags = p[p[8]:p[8] + segs], p[p[9]:p[9] + segs]
+    seq_seg0, seq_nseg = p[p[10]:p[10] + n_seq], p[p[11]:p[11] + n_seq]
+    # chunks tile every sequence exactly and never straddle a boundary (index.py:69-83)
+    covered = []
+    for t, l in zip(tok0, clen):
+        assert 1 <= l <= 64
+        covered.extend(range(t, t + l))
+    assert covered == list(range(cu[-1]))
+    for t, l in zip(tok0, clen):
+        s = max(i for i in range(n_seq) if cu[i] <= t and lens[i] > 0)
+        assert t + l <= cu[s + 1] and (t - cu[s]) % 64 == 0
+    # segments partition the chunks of their sequence; flags mark first / last
+    assert sum(seg_nc) == chunks and seq_nseg == [max(1, (c + 15) // 16) for c in want_chunks]
+    for s in range(n_seq):
+        mine = [g for g in range(segs) if seg_seq[g] == s]
+        assert mine == list(range(seq_seg0[s], seq_seg0[s] + seq_nseg[s]))
+        assert seg_flags[mine[0]] & 1 and seg_flags[mine[-1]] & 2
+        assert all(seg_nc[g] <= 16 for g in mine) and sum(seg_nc[g] for g in mine) == want_chunks[s]
+    assert p[12] == cu[-1]
+
+
+def test_plan_rejects_bad_input(lib):
+    bad = (ctypes.c_int64 * 3)(0, 10, 5)
+    assert lib.lampa_gdr_plan_size(bad, 2, 4) == -1
+    ok = (ctypes.c_int64 * 2)(0, 10)
+    assert lib.lampa_gdr_plan_size(ok, 1, 0) == -1
+
+
+def test_operators_refuse_cpu_tensors():
+    from lampa_amd import gated_delta as gd
+    from lampa_amd import lsh
+
+    x = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16)
+    g = torch.zeros(1, 64, 2)
+    with pytest.raises(_capi.LampaError):
+        gd.chunk_gated_delta_rule(x, x, x, g, g)
+    with pytest.raises(_capi.LampaError):
+        lsh.stable_argsort(torch.zeros(4, dtype=torch.int32))
