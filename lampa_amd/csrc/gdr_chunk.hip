@@ -145,7 +145,11 @@ __device__ __forceinline__ bf16x8 frag_load(const unsigned char* rec, int frag, 
   return *reinterpret_cast<const bf16x8*>(rec + (size_t)frag * 1024 + lane * 16);
 }
 __device__ __forceinline__ void frag_store(unsigned char* rec, int frag, int lane, bf16x8 v) {
+#ifndef GDR_DBG_SKIP_STORE
   *reinterpret_cast<bf16x8*>(rec + (size_t)frag * 1024 + lane * 16) = v;
+#else
+  if (v[0] == (__bf16)123.456f) *reinterpret_cast<bf16x8*>(rec + (size_t)frag * 1024 + lane * 16) = v;
+#endif
 }
 
 // ---- prep kernel ----------------------------------------------------------------------------------------------
@@ -247,7 +251,9 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
       for (int e = 0; e < 8; ++e) {
         kb[e] = (__bf16)(kf[8 * c + e] * kinv);
         qb[e] = (__bf16)(qf[8 * c + e] * qinv);
+#ifndef GDR_DBG_SKIP_TR
         s_kT[(q4 * EPT + 8 * c + e) * SX + row] = kb[e];
+#endif
       }
       *reinterpret_cast<bf16x8*>(&s_k[row * SK + q4 * EPT + 8 * c]) = kb;
       *reinterpret_cast<bf16x8*>(&s_q[row * SK + q4 * EPT + 8 * c]) = qb;
@@ -264,7 +270,9 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
         for (int e = 0; e < 8; ++e) vf[e] = 0.0f;
       }
 #pragma unroll
+#ifndef GDR_DBG_SKIP_TR
       for (int e = 0; e < 8; ++e) s_vT[(q4 * VPT + 8 * c + e) * SX + row] = (__bf16)vf[e];
+#endif
     }
   }
   __syncthreads();
@@ -295,21 +303,100 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
   __syncthreads();
 
   if (wave == 0) {
-    // (4a) column `lane` of (I + A)^-1 by forward substitution; all lanes read the same A element (LDS broadcast)
-    float x[64];
+    // (4a) T = (I + A)^-1, A strictly lower triangular, as a 2x2 block matrix of 32x32 blocks:
+    //      T11 = (I + A11)^-1, T22 = (I + A22)^-1 by forward substitution -- lane 32b + c owns column c of block b,
+    //      every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
+    //      T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+    const int b = hh, c = ln;
+    const float* Ab = s_A + (32 * b) * SA + 32 * b;
+    float x[32];
+    f32x4 rowbuf[2][8];  // rows i and i+1 of the block, so that the next row loads while this one is reduced
+    rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SA);
+    x[0] = (c == 0) ? 1.0f : 0.0f;
 #pragma unroll
-    for (int i = 0; i < 64; ++i) {
-      float acc = (i == lane) ? 1.0f : 0.0f;
+    for (int i = 1; i < 32; ++i) {
+      if (i + 1 < 32) {
 #pragma unroll
-      for (int j = 0; j < i; ++j) acc = __builtin_fmaf(-s_A[i * SA + j], x[j], acc);
-      x[i] = acc;
+        for (int q = 0; q < (i + 1 + 3) / 4; ++q)
+          rowbuf[(i + 1) & 1][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 1) * SA + 4 * q);
+      }
+      float acc0 = (i == c) ? 1.0f : 0.0f, acc1 = 0.0f;
+#pragma unroll
+      for (int j = 0; j < i; ++j) {
+        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc1);
+        else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
+      }
+      x[i] = acc0 + acc1;
+      // pins the order "loads of row i+1, arithmetic of row i" so the compiler neither serialises every load
+      // behind a wait nor hoists all 124 loads to the top (which spills)
+      asm volatile("" : "+v"(x[i]) : : "memory");
     }
+    __builtin_amdgcn_wave_barrier();
+    // diagonal blocks: fp32 copy in place of A11 / A22 (operands of the merge) and the scaled bf16 outputs;
+    // the upper-right block of T is zero
     const float bc = s_beta[lane];
     const float wc = bc * __expf(s_gamma[lane]);
 #pragma unroll
-    for (int i = 0; i < 64; ++i) {
-      s_TW[i * SX + lane] = (__bf16)(x[i] * wc);
-      s_TU[i * SX + lane] = (__bf16)(x[i] * bc);
+    for (int i = 0; i < 32; ++i) {
+      s_A[(32 * b + i) * SA + lane] = x[i];
+      s_TW[(32 * b + i) * SX + lane] = (__bf16)(x[i] * wc);
+      s_TU[(32 * b + i) * SX + lane] = (__bf16)(x[i] * bc);
+      if (b == 1) {
+        s_TW[i * SX + lane] = (__bf16)0.0f;
+        s_TU[i * SX + lane] = (__bf16)0.0f;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    f32x16 y0, y1, y2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { y0[r] = 0.0f; y1[r] = 0.0f; y2[r] = 0.0f; }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11
+      bf16x8 ahi, alo, bhi, blo;
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 16 * ks + 8 * hh]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 16 * ks + 8 * hh + 4]);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float av = q < 4 ? a0[q % 4] : a1[q % 4];
+        const float bv = s_A[(16 * ks + 8 * hh + q) * SA + ln];
+        const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+        ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+        bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+      }
+      y0 = mfma32(ahi, bhi, y0);
+      y1 = mfma32(alo, bhi, y1);
+      y2 = mfma32(ahi, blo, y2);
+    }
+    f32x16 t0, t1, t2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { y0[r] += y1[r] + y2[r]; t0[r] = 0.0f; t1[r] = 0.0f; t2[r] = 0.0f; }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
+      bf16x8 ahi, alo, bhi, blo;
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 32 + 16 * ks + 4 * hh]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 32 + 16 * ks + 8 + 4 * hh]);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float av = q < 4 ? a0[q % 4] : a1[q % 4];
+        const float bv = y0[8 * ks + q];
+        const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+        ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+        bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+      }
+      t0 = mfma32(ahi, bhi, t0);
+      t1 = mfma32(alo, bhi, t1);
+      t2 = mfma32(ahi, blo, t2);
+    }
+    const float bl = s_beta[ln];
+    const float wl = bl * __expf(s_gamma[ln]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+      const float t21 = -(t0[r] + (t1[r] + t2[r]));
+      s_TW[row * SX + ln] = (__bf16)(t21 * wl);
+      s_TU[row * SX + ln] = (__bf16)(t21 * bl);
     }
     if (lane == 0) decs[(size_t)chunk * HV + hv] = __expf(s_gamma[63]);
   } else {
@@ -408,32 +495,112 @@ __device__ __forceinline__ void state_operands(const f32x16* S, bf16x8* Sb) {
   for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
 }
 
-__device__ __forceinline__ f32x16 utile_load(const unsigned char* rec, int u_off_kib, int tile, int lane) {
-  const unsigned char* up = rec + (size_t)u_off_kib * 1024 + (size_t)tile * 2048 + lane * 32;
-  const bf16x8 a = *reinterpret_cast<const bf16x8*>(up);
-  const bf16x8 b = *reinterpret_cast<const bf16x8*>(up + 16);
+// Operand fragments of one chunk for one wave of the sequential kernels, held in registers so that the next
+// chunk's loads are in flight while the current chunk computes.
+template <int KT, int VT, bool WITH_OUTPUT>
+struct GdrChunkOps {
+  bf16x8 W[2 * (KT / 16)];
+  bf16x8 Kf[(KT / 32) * 4];
+  bf16x8 Q[WITH_OUTPUT ? 2 * (KT / 16) : 1];
+  bf16x8 P[WITH_OUTPUT ? 6 : 1];
+  bf16x8 U[4];  // U tiles tm = 0, 1 of this wave's 32 columns, two halves each
+  float dec;
+};
+
+template <int KT, int VT, bool WITH_OUTPUT>
+__device__ __forceinline__ void chunk_ops_load(GdrChunkOps<KT, VT, WITH_OUTPUT>& ops,
+                                               const unsigned char* __restrict__ rec, const float* __restrict__ decp,
+                                               int lane, int vn, bool with_u) {
+  using REC = GdrRecord<KT, VT>;
+#pragma unroll
+  for (int f = 0; f < 2 * (KT / 16); ++f) ops.W[f] = frag_load(rec, REC::W_OFF + f, lane);
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm) {
+    const unsigned char* up = rec + (size_t)REC::U_OFF * 1024 + (size_t)(tm * (VT / 32) + vn) * 2048 + lane * 32;
+    if (with_u) {
+      ops.U[2 * tm + 0] = *reinterpret_cast<const bf16x8*>(up);
+      ops.U[2 * tm + 1] = *reinterpret_cast<const bf16x8*>(up + 16);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) { ops.U[2 * tm][q] = (__bf16)0.0f; ops.U[2 * tm + 1][q] = (__bf16)0.0f; }
+    }
+  }
+  if constexpr (WITH_OUTPUT) {
+#pragma unroll
+    for (int f = 0; f < 2 * (KT / 16); ++f) ops.Q[f] = frag_load(rec, REC::Q_OFF + f, lane);
+#pragma unroll
+    for (int f = 0; f < 2; ++f) ops.P[f] = frag_load(rec, REC::P_OFF + f, lane);
+#pragma unroll
+    for (int f = 0; f < 4; ++f) ops.P[2 + f] = frag_load(rec, REC::P_OFF + 4 + f, lane);
+  }
+#pragma unroll
+  for (int f = 0; f < (KT / 32) * 4; ++f) ops.Kf[f] = frag_load(rec, REC::K_OFF + f, lane);
+  ops.dec = *decp;
+}
+
+__device__ __forceinline__ f32x16 utile_widen(bf16x8 a, bf16x8 b) {
   f32x16 out;
 #pragma unroll
   for (int s = 0; s < 8; ++s) { out[s] = (float)a[s]; out[8 + s] = (float)b[s]; }
   return out;
 }
 
-// composite: grid ((KT+VT)/32, n_segments, HV). Slabs < KT/32 carry columns of M (start: identity, no U term),
-// the others columns of N (start: zero). Mcomp [seg, HV, KT, KT], Ncomp [seg, HV, KT, VT] fp32 row-major.
+// One chunk of the recurrence on a 32-column slab: v_new = U - W S (Vb = its B-operand fragments),
+// S <- dec S + K~^T v_new. With output: o tile tm = Q~ S + P v_new is handed to `emit(tm, acc)`.
+template <int KT, int VT, bool WITH_OUTPUT, typename Emit>
+__device__ __forceinline__ void chunk_step(const GdrChunkOps<KT, VT, WITH_OUTPUT>& ops, f32x16* S, Emit emit) {
+  bf16x8 Sb[KT / 16];
+  state_operands<KT>(S, Sb);
+  bf16x8 Vb[4];
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm) {
+    f32x16 acc = utile_widen(ops.U[2 * tm], ops.U[2 * tm + 1]);
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(ops.W[tm * (KT / 16) + ks], Sb[ks], acc);
+    Vb[2 * tm + 0] = acc_to_operand(acc, 0);
+    Vb[2 * tm + 1] = acc_to_operand(acc, 8);
+  }
+  if constexpr (WITH_OUTPUT) {
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+      f32x16 acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(ops.Q[tm * (KT / 16) + ks], Sb[ks], acc);
+#pragma unroll
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ops.P[2 * tm + ks], Vb[ks], acc);
+      emit(tm, acc);
+    }
+  }
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[km][r] *= ops.dec;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(ops.Kf[km * 4 + ks], Vb[ks], S[km]);
+  }
+}
+
+// composite: grid (n_segments, HV), one wave per 32-column slab of [M | N] ((KT+VT)/32 waves per workgroup, so the
+// waves that read the same W and K~ fragments share one CU's L1 and one XCD's L2). Slabs < KT/32 carry columns of
+// M (start: identity, no U term), the others columns of N (start: zero).
+// Mcomp [seg, HV, KT, KT], Ncomp [seg, HV, KT, VT] fp32 row-major.
 template <int KT, int VT>
-__global__ void __launch_bounds__(64) gdr_composite_kernel(const int32_t* __restrict__ plan,
+__global__ void __launch_bounds__(2 * (KT + VT)) gdr_composite_kernel(const int32_t* __restrict__ plan,
                                                           const unsigned char* __restrict__ records,
                                                           const float* __restrict__ decs,
                                                           float* __restrict__ Mcomp, float* __restrict__ Ncomp,
                                                           int HV) {
   using REC = GdrRecord<KT, VT>;
-  const int slab = blockIdx.x, seg = blockIdx.y, hv = blockIdx.z;
+  using OPS = GdrChunkOps<KT, VT, false>;
+  const int slab = threadIdx.x >> 6, seg = blockIdx.x, hv = blockIdx.y;
   const int flags = plan[plan[PLAN_OFF_SEG_FLAGS] + seg];
   if (flags & SEG_LAST) return;  // nothing follows the last segment of a sequence
   const int c0 = plan[plan[PLAN_OFF_SEG_CHUNK0] + seg], nc = plan[plan[PLAN_OFF_SEG_NCHUNKS] + seg];
-  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   const bool is_m = slab < KT / 32;
-  const int vn = slab - KT / 32;
+  const int vn = is_m ? 0 : slab - KT / 32;
 
   f32x16 S[KT / 32];
 #pragma unroll
@@ -442,32 +609,18 @@ __global__ void __launch_bounds__(64) gdr_composite_kernel(const int32_t* __rest
     for (int r = 0; r < 16; ++r)
       S[km][r] = (is_m && (32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) == 32 * slab + ln) ? 1.0f : 0.0f;
 
-  for (int c = c0; c < c0 + nc; ++c) {
-    const unsigned char* rec = records + ((size_t)c * HV + hv) * REC::BYTES;
-    const float dec = decs[(size_t)c * HV + hv];
-    bf16x8 Sb[KT / 16];
-    state_operands<KT>(S, Sb);
-    bf16x8 Vb[4];
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm) {
-      f32x16 acc;
-      if (is_m) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-      } else {
-        acc = utile_load(rec, REC::U_OFF, tm * (VT / 32) + vn, lane);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(frag_load(rec, REC::W_OFF + tm * (KT / 16) + ks, lane), Sb[ks], acc);
-      Vb[2 * tm + 0] = acc_to_operand(acc, 0);
-      Vb[2 * tm + 1] = acc_to_operand(acc, 8);
-    }
-#pragma unroll
-    for (int km = 0; km < KT / 32; ++km) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] *= dec;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(frag_load(rec, REC::K_OFF + km * 4 + ks, lane), Vb[ks], S[km]);
+  auto rec_of = [&](int c) { return records + ((size_t)c * HV + hv) * REC::BYTES; };
+  auto dec_of = [&](int c) { return decs + (size_t)c * HV + hv; };
+  auto no_emit = [](int, const f32x16&) {};
+  const int c1 = c0 + nc;
+  OPS a, b;
+  if (nc > 0) chunk_ops_load<KT, VT, false>(a, rec_of(c0), dec_of(c0), lane, vn, !is_m);
+  for (int c = c0; c < c1; c += 2) {
+    if (c + 1 < c1) chunk_ops_load<KT, VT, false>(b, rec_of(c + 1), dec_of(c + 1), lane, vn, !is_m);
+    chunk_step<KT, VT, false>(a, S, no_emit);
+    if (c + 1 < c1) {
+      if (c + 2 < c1) chunk_ops_load<KT, VT, false>(a, rec_of(c + 2), dec_of(c + 2), lane, vn, !is_m);
+      chunk_step<KT, VT, false>(b, S, no_emit);
     }
   }
   float* out = is_m ? Mcomp + ((size_t)seg * HV + hv) * KT * KT : Ncomp + ((size_t)seg * HV + hv) * KT * VT;
@@ -478,90 +631,118 @@ __global__ void __launch_bounds__(64) gdr_composite_kernel(const int32_t* __rest
     for (int r = 0; r < 16; ++r) out[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * ncols + col] = S[km][r];
 }
 
-// scan: grid (VT/32, n_seq, HV). Sinit [seg, HV, KT, VT] fp32 row-major receives the state every segment starts from.
+// scan: grid (VT/32, n_seq, HV), KT/32 waves per workgroup. Wave w owns state rows 32w..32w+31 of a 32-column slab.
+// Per segment: store the state as the segment's initial state, then S <- M S + N with M and S split into bf16
+// high and remainder parts (three MFMA products, close to fp32 accuracy). The waves exchange their share of S as
+// B-operand fragments through a double-buffered LDS array (one barrier per step); the M rows and N tile of the
+// next step are loaded while the current one computes.
+// Sinit [seg, HV, KT, VT] fp32 row-major receives the state every segment starts from.
+template <int KT>
+struct GdrScanRegs {
+  f32x4 m[KT / 16][2];
+  float n[16];
+};
+
 template <int KT, int VT>
-__global__ void __launch_bounds__(64) gdr_scan_kernel(const int32_t* __restrict__ plan,
-                                                     const float* __restrict__ Mcomp,
-                                                     const float* __restrict__ Ncomp, const float* __restrict__ h0,
-                                                     float* __restrict__ Sinit, int HV) {
+__device__ __forceinline__ void scan_load(GdrScanRegs<KT>& r, const float* __restrict__ M,
+                                          const float* __restrict__ N, int wave, int hh, int ln, int col) {
+#pragma unroll
+  for (int ks = 0; ks < KT / 16; ++ks) {
+    const float* mrow = M + (size_t)(32 * wave + ln) * KT + 16 * ks;
+    r.m[ks][0] = *reinterpret_cast<const f32x4*>(mrow + 4 * hh);
+    r.m[ks][1] = *reinterpret_cast<const f32x4*>(mrow + 8 + 4 * hh);
+  }
+#pragma unroll
+  for (int q = 0; q < 16; ++q) r.n[q] = N[(size_t)(32 * wave + 8 * (q / 4) + 4 * hh + (q % 4)) * VT + col];
+}
+
+template <int KT, int VT>
+__global__ void __launch_bounds__(KT * 2) gdr_scan_kernel(const int32_t* __restrict__ plan,
+                                                         const float* __restrict__ Mcomp,
+                                                         const float* __restrict__ Ncomp,
+                                                         const float* __restrict__ h0, float* __restrict__ Sinit,
+                                                         int HV) {
+  __shared__ __align__(16) bf16x8 s_frag[2][2][KT / 16][64];  // [buffer][hi/lo][contraction step][lane]
   const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
   const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
-  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
-  f32x16 S[KT / 32];
+  f32x16 S;
 #pragma unroll
-  for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 32 * km + 8 * (r / 4) + 4 * hh + (r % 4);
-      S[km][r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + row) * VT + col] : 0.0f;
-    }
+  for (int r = 0; r < 16; ++r) {
+    const int row = 32 * wave + 8 * (r / 4) + 4 * hh + (r % 4);
+    S[r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + row) * VT + col] : 0.0f;
+  }
+  GdrScanRegs<KT> nxt;
+  if (nseg > 1)
+    scan_load<KT, VT>(nxt, Mcomp + ((size_t)seg0 * HV + hv) * KT * KT, Ncomp + ((size_t)seg0 * HV + hv) * KT * VT, wave,
+                      hh, ln, col);
   for (int p = 0; p < nseg; ++p) {
     const int seg = seg0 + p;
     float* si = Sinit + ((size_t)seg * HV + hv) * KT * VT;
 #pragma unroll
-    for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) si[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col] = S[km][r];
+    for (int r = 0; r < 16; ++r) si[(size_t)(32 * wave + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col] = S[r];
     if (p == nseg - 1) break;
-    // S <- M S + N with M and S each split into a bf16 high part and a bf16 remainder
-    const float* M = Mcomp + ((size_t)seg * HV + hv) * KT * KT;
-    const float* N = Ncomp + ((size_t)seg * HV + hv) * KT * VT;
-    bf16x8 Shi[KT / 16], Slo[KT / 16];
+    // this step's M rows (hi / lo operand fragments) and N tile arrived in nxt; start fetching the next step's
+    bf16x8 Mhi[KT / 16], Mlo[KT / 16];
+    f32x16 acc0, acc1, acc2;
 #pragma unroll
     for (int ks = 0; ks < KT / 16; ++ks)
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const float x = S[ks / 2][8 * (ks % 2) + s];
+      for (int q = 0; q < 8; ++q) {
+        const float x = nxt.m[ks][q / 4][q % 4];
         const __bf16 hi = (__bf16)x;
-        Shi[ks][s] = hi;
-        Slo[ks][s] = (__bf16)(x - (float)hi);
+        Mhi[ks][q] = hi;
+        Mlo[ks][q] = (__bf16)(x - (float)hi);
       }
-    f32x16 Snew[KT / 32];
 #pragma unroll
-    for (int tm = 0; tm < KT / 32; ++tm) {
-      f32x16 acc;
+    for (int r = 0; r < 16; ++r) { acc0[r] = nxt.n[r]; acc1[r] = 0.0f; acc2[r] = 0.0f; }
+    if (p + 2 < nseg)
+      scan_load<KT, VT>(nxt, Mcomp + ((size_t)(seg + 1) * HV + hv) * KT * KT,
+                        Ncomp + ((size_t)(seg + 1) * HV + hv) * KT * VT, wave, hh, ln, col);
+    // publish this wave's rows of S as B-operand fragments (contraction steps 2*wave and 2*wave+1)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[r] = N[(size_t)(32 * tm + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col];
+    for (int half = 0; half < 2; ++half) {
+      bf16x8 hi, lo;
 #pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) {
-        const float* mrow = M + (size_t)(32 * tm + ln) * KT + 16 * ks;
-        const f32x4 m0 = *reinterpret_cast<const f32x4*>(mrow + 4 * hh);
-        const f32x4 m1 = *reinterpret_cast<const f32x4*>(mrow + 8 + 4 * hh);
-        bf16x8 Mhi, Mlo;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const float x = s < 4 ? m0[s % 4] : m1[s % 4];
-          const __bf16 hi = (__bf16)x;
-          Mhi[s] = hi;
-          Mlo[s] = (__bf16)(x - (float)hi);
-        }
-        acc = mfma32(Mlo, Shi[ks], acc);
-        acc = mfma32(Mhi, Slo[ks], acc);
-        acc = mfma32(Mhi, Shi[ks], acc);
+      for (int q = 0; q < 8; ++q) {
+        const float x = S[8 * half + q];
+        const __bf16 h = (__bf16)x;
+        hi[q] = h;
+        lo[q] = (__bf16)(x - (float)h);
       }
-      Snew[tm] = acc;
+      s_frag[p & 1][0][2 * wave + half][lane] = hi;
+      s_frag[p & 1][1][2 * wave + half][lane] = lo;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) {
+      const bf16x8 Shi = s_frag[p & 1][0][ks][lane];
+      const bf16x8 Slo = s_frag[p & 1][1][ks][lane];
+      acc0 = mfma32(Mhi[ks], Shi, acc0);
+      acc1 = mfma32(Mlo[ks], Shi, acc1);
+      acc2 = mfma32(Mhi[ks], Slo, acc2);
     }
 #pragma unroll
-    for (int km = 0; km < KT / 32; ++km) S[km] = Snew[km];
+    for (int r = 0; r < 16; ++r) S[r] = acc0[r] + (acc1[r] + acc2[r]);
   }
 }
 
-// output: grid (VT/32, n_segments, HV).
+// output: grid (n_segments, HV), one wave per 32 value columns (VT/32 waves per workgroup).
 template <typename T, int KT, int VT>
-__global__ void __launch_bounds__(64) gdr_output_kernel(const int32_t* __restrict__ plan,
+__global__ void __launch_bounds__(2 * VT) gdr_output_kernel(const int32_t* __restrict__ plan,
                                                        const unsigned char* __restrict__ records,
                                                        const float* __restrict__ decs,
                                                        const float* __restrict__ Sinit, T* __restrict__ o,
                                                        float* __restrict__ ht, int HV) {
   using REC = GdrRecord<KT, VT>;
-  const int vn = blockIdx.x, seg = blockIdx.y, hv = blockIdx.z;
+  using OPS = GdrChunkOps<KT, VT, true>;
+  const int vn = threadIdx.x >> 6, seg = blockIdx.x, hv = blockIdx.y;
   const int c0 = plan[plan[PLAN_OFF_SEG_CHUNK0] + seg], nc = plan[plan[PLAN_OFF_SEG_NCHUNKS] + seg];
   const int flags = plan[plan[PLAN_OFF_SEG_FLAGS] + seg], seq = plan[plan[PLAN_OFF_SEG_SEQ] + seg];
   const int* chunk_tok0 = plan + plan[PLAN_OFF_CHUNK_TOK0];
   const int* chunk_len = plan + plan[PLAN_OFF_CHUNK_LEN];
-  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
   f32x16 S[KT / 32];
   {
@@ -571,42 +752,35 @@ __global__ void __launch_bounds__(64) gdr_output_kernel(const int32_t* __restric
 #pragma unroll
       for (int r = 0; r < 16; ++r) S[km][r] = si[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col];
   }
-  for (int c = c0; c < c0 + nc; ++c) {
-    const unsigned char* rec = records + ((size_t)c * HV + hv) * REC::BYTES;
-    const float dec = decs[(size_t)c * HV + hv];
+  auto rec_of = [&](int c) { return records + ((size_t)c * HV + hv) * REC::BYTES; };
+  auto dec_of = [&](int c) { return decs + (size_t)c * HV + hv; };
+  auto run = [&](const OPS& ops, int c) {
     const int tok0 = chunk_tok0[c], len = chunk_len[c];
-    bf16x8 Sb[KT / 16];
-    state_operands<KT>(S, Sb);
-    bf16x8 Vb[4];
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm) {
-      f32x16 acc = utile_load(rec, REC::U_OFF, tm * (VT / 32) + vn, lane);
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(frag_load(rec, REC::W_OFF + tm * (KT / 16) + ks, lane), Sb[ks], acc);
-      Vb[2 * tm + 0] = acc_to_operand(acc, 0);
-      Vb[2 * tm + 1] = acc_to_operand(acc, 8);
-    }
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm) {
-      f32x16 acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(frag_load(rec, REC::Q_OFF + tm * (KT / 16) + ks, lane), Sb[ks], acc);
-#pragma unroll
-      for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(frag_load(rec, REC::P_OFF + tm * 4 + ks, lane), Vb[ks], acc);
+    chunk_step<KT, VT, true>(ops, S, [&](int tm, const f32x16& acc) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int tok = 32 * tm + 8 * (r / 4) + 4 * hh + (r % 4);
         if (tok < len) o[((size_t)(tok0 + tok) * HV + hv) * VT + col] = GdrElem<T>::from_float(acc[r]);
       }
+    });
+  };
+  const int c1 = c0 + nc;
+  if constexpr (KT <= 64) {
+    OPS a, b;  // two register sets: the next chunk's fragments load while the current chunk computes
+    if (nc > 0) chunk_ops_load<KT, VT, true>(a, rec_of(c0), dec_of(c0), lane, vn, true);
+    for (int c = c0; c < c1; c += 2) {
+      if (c + 1 < c1) chunk_ops_load<KT, VT, true>(b, rec_of(c + 1), dec_of(c + 1), lane, vn, true);
+      run(a, c);
+      if (c + 1 < c1) {
+        if (c + 2 < c1) chunk_ops_load<KT, VT, true>(a, rec_of(c + 2), dec_of(c + 2), lane, vn, true);
+        run(b, c + 1);
+      }
     }
-#pragma unroll
-    for (int km = 0; km < KT / 32; ++km) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] *= dec;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(frag_load(rec, REC::K_OFF + km * 4 + ks, lane), Vb[ks], S[km]);
+  } else {
+    for (int c = c0; c < c1; ++c) {
+      OPS a;
+      chunk_ops_load<KT, VT, true>(a, rec_of(c), dec_of(c), lane, vn, true);
+      run(a, c);
     }
   }
   if (ht && (flags & SEG_LAST)) {
@@ -667,15 +841,16 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
                        (const T*)v, g, beta, plan_dev, records, decs, H, HV, scale, l2norm);
     LAMPA_PROF(s, "gdr_prep_kernel");
     if (segs > n_seq) {
-      hipLaunchKernelGGL((gdr_composite_kernel<KT, VT>), dim3((KT + VT) / 32, segs, HV), dim3(64), 0, s, plan_dev,
-                         records, decs, Mc, Nc, HV);
+      hipLaunchKernelGGL((gdr_composite_kernel<KT, VT>), dim3(segs, HV), dim3(2 * (KT + VT)), 0, s, plan_dev, records,
+                         decs, Mc, Nc, HV);
       LAMPA_PROF(s, "gdr_composite_kernel");
     }
   }
-  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, plan_dev, Mc, Nc, h0, Si, HV);
+  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(KT * 2), 0, s, plan_dev, Mc, Nc, h0, Si,
+                     HV);
   LAMPA_PROF(s, "gdr_scan_kernel");
-  hipLaunchKernelGGL((gdr_output_kernel<T, KT, VT>), dim3(VT / 32, segs, HV), dim3(64), 0, s, plan_dev, records, decs,
-                     Si, (T*)o, ht, HV);
+  hipLaunchKernelGGL((gdr_output_kernel<T, KT, VT>), dim3(segs, HV), dim3(2 * VT), 0, s, plan_dev, records, decs, Si,
+                     (T*)o, ht, HV);
   LAMPA_PROF(s, "gdr_output_kernel");
   return lampa_launch_status();
 }
