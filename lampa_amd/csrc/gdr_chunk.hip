@@ -6,201 +6,133 @@
 // recompute_w_u_fwd (wy_fast.py:140-189), chunk_gated_delta_rule_fwd_h (chunk_delta_h.py:34-189) and
 // chunk_fwd_o (chunk_o.py:33-111).
 //
-// Four kernels:
-//   prep       one workgroup per (chunk, head): l2norm, cumulative log-decay, KK^T and QK^T on MFMA, the
-//              unit-lower-triangular inverse by forward substitution in LDS, then W, U.  Everything the
-//              sequential part needs is written as ready-made MFMA operand fragments ("record" of the chunk).
-//   composite  the state map of a chunk is affine, S' = M S + N.  The sequence is cut into segments of a few
-//              chunks; one wave per (segment, head, 32 columns of [M | N]) runs the recurrence on the identity
-//              and on zero to obtain the segment's composite (M, N).
-//   scan       one wave per (sequence, head, 32 value columns) walks the segments: S_{p+1} = M_p S_p + N_p
-//              (hi/lo split bf16 MFMA, fp32 state) and stores every segment's initial state.
-//   output     one wave per (segment, head, 32 value columns) replays its segment from the right initial state:
-//              v_new = U - W S,  o = Q~ S + P v_new,  S <- e^{g_last} S + K~^T v_new.
-// The sequential kernels keep the state in accumulator registers and feed it straight back as the next MFMA's
-// B operand (accumulator rows 8*(r/4) + 4*hh + r%4 become contraction slots), so the state never touches LDS.
+// Per chunk of C = 64 tokens of one head, with gamma the in-chunk cumulative log-decay, rk / rq the l2-norm
+// factors of the raw k / q rows and S the K x V state entering the chunk:
+//   A     = strict_lower( beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j} ),   T = (I + A)^-1
+//   R     = beta_i ( v_i - e^{gamma_i} rk_i (K S)_i )                v_new = T R
+//   o_i   = scale e^{gamma_i} rq_i (Q S)_i + (P v_new)_i,    P_ij = scale rq_i rk_j (q_i . k_j) e^{gamma_i - gamma_j}, j <= i
+//   S'    = e^{gamma_last} S + K^T ( e^{gamma_last - gamma_j} rk_j v_new_j )
+// All per-token factors are applied to accumulator rows in fp32, so the MFMA operands are the RAW bf16 k, q, v
+// tiles and the only intermediate that goes through HBM is T (6 KiB per chunk and head).
+//
+// Kernels:
+//   tinv     workgroup per (chunk, head): K K^T on MFMA, gating, blocked inverse (two 32x32 forward substitutions
+//            in fp32 + an MFMA merge with bf16 high/remainder splits), T written as MFMA A-operand fragments.
+//   segment  workgroup per (segment of chunks, head), one wave per 32 columns. Each chunk's k, q, v tiles are
+//            staged once in LDS (row-major and transposed), the next chunk's global loads are in flight
+//            meanwhile, and every wave runs the recurrence on its columns with the state in accumulator
+//            registers. PASS_A: columns of [M | N] of the segment's affine map S -> M S + N (start identity /
+//            zero). PASS_B: value columns, from the segment's true initial state, writing o (and the final state).
+//   scan     S_{p+1} = M_p S_p + N_p over the segments of a sequence (hi/lo-split bf16 MFMA), storing each
+//            segment's initial state.
+// The state tile is fed back as the next MFMA's B operand straight from the accumulator registers: register r of
+// lane l is row 8*(r/4) + 4*(l/32) + r%4, and since a contraction may visit its index in any order as long as
+// both operands agree, every A operand is read from LDS in that slot order (ld_kappa).
 #include "gdr_common.h"
+#include "gdr_plan.h"
 
-#define GDR_C 64  // chunk length
-
-// ---- plan (host-built tables, int32) -------------------------------------------------------------------------
-enum {
-  PLAN_N_SEQ = 0,
-  PLAN_TOTAL_CHUNKS = 1,
-  PLAN_N_SEGMENTS = 2,
-  PLAN_CHUNKS_PER_SEGMENT = 3,
-  PLAN_OFF_CHUNK_TOK0 = 4,
-  PLAN_OFF_CHUNK_LEN = 5,
-  PLAN_OFF_SEG_CHUNK0 = 6,
-  PLAN_OFF_SEG_NCHUNKS = 7,
-  PLAN_OFF_SEG_SEQ = 8,
-  PLAN_OFF_SEG_FLAGS = 9,
-  PLAN_OFF_SEQ_SEG0 = 10,
-  PLAN_OFF_SEQ_NSEG = 11,
-  PLAN_TOTAL_TOKENS = 12,
-  PLAN_HEADER = 16
-};
-#define SEG_FIRST 1
-#define SEG_LAST 2
-
-static int64_t plan_counts(const int64_t* cu, int n_seq, int cps, int64_t* n_chunks, int64_t* n_segments) {
-  int64_t chunks = 0, segs = 0;
-  for (int s = 0; s < n_seq; ++s) {
-    const int64_t len = cu[s + 1] - cu[s];
-    if (len < 0) return -1;
-    const int64_t nc = (len + GDR_C - 1) / GDR_C;
-    chunks += nc;
-    segs += nc == 0 ? 1 : (nc + cps - 1) / cps;  // an empty sequence still owns one (empty) segment
-  }
-  *n_chunks = chunks;
-  *n_segments = segs;
-  return 0;
-}
-
-// Number of int32 entries of the plan for these sequences (negative on error).
-extern "C" int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment) {
-  if (!cu_seqlens_host || n_seq < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
-  int64_t chunks, segs;
-  if (plan_counts(cu_seqlens_host, n_seq, chunks_per_segment, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
-  if (cu_seqlens_host[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
-  return PLAN_HEADER + 2 * chunks + 4 * segs + 2 * (int64_t)n_seq;
-}
-
-// Fills plan_host (lampa_gdr_plan_size entries). The caller copies it to the device and passes that pointer on.
-extern "C" int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment,
-                                   int32_t* plan_host) {
-  if (!plan_host) return LAMPA_ERR_INVALID;
-  const int64_t size = lampa_gdr_plan_size(cu_seqlens_host, n_seq, chunks_per_segment);
-  if (size < 0) return (int)size;
-  int64_t chunks, segs;
-  plan_counts(cu_seqlens_host, n_seq, chunks_per_segment, &chunks, &segs);
-  int32_t* p = plan_host;
-  for (int i = 0; i < PLAN_HEADER; ++i) p[i] = 0;
-  p[PLAN_N_SEQ] = n_seq;
-  p[PLAN_TOTAL_CHUNKS] = (int32_t)chunks;
-  p[PLAN_N_SEGMENTS] = (int32_t)segs;
-  p[PLAN_CHUNKS_PER_SEGMENT] = chunks_per_segment;
-  p[PLAN_TOTAL_TOKENS] = (int32_t)cu_seqlens_host[n_seq];
-  int64_t off = PLAN_HEADER;
-  p[PLAN_OFF_CHUNK_TOK0] = (int32_t)off; off += chunks;
-  p[PLAN_OFF_CHUNK_LEN] = (int32_t)off; off += chunks;
-  p[PLAN_OFF_SEG_CHUNK0] = (int32_t)off; off += segs;
-  p[PLAN_OFF_SEG_NCHUNKS] = (int32_t)off; off += segs;
-  p[PLAN_OFF_SEG_SEQ] = (int32_t)off; off += segs;
-  p[PLAN_OFF_SEG_FLAGS] = (int32_t)off; off += segs;
-  p[PLAN_OFF_SEQ_SEG0] = (int32_t)off; off += n_seq;
-  p[PLAN_OFF_SEQ_NSEG] = (int32_t)off; off += n_seq;
-  int64_t c = 0, g = 0;
-  for (int s = 0; s < n_seq; ++s) {
-    const int64_t bos = cu_seqlens_host[s], len = cu_seqlens_host[s + 1] - bos;
-    const int64_t nc = (len + GDR_C - 1) / GDR_C;
-    const int64_t ns = nc == 0 ? 1 : (nc + chunks_per_segment - 1) / chunks_per_segment;
-    p[p[PLAN_OFF_SEQ_SEG0] + s] = (int32_t)g;
-    p[p[PLAN_OFF_SEQ_NSEG] + s] = (int32_t)ns;
-    for (int64_t i = 0; i < ns; ++i) {
-      const int64_t c0 = i * chunks_per_segment;
-      const int64_t cn = nc - c0 < chunks_per_segment ? nc - c0 : chunks_per_segment;
-      p[p[PLAN_OFF_SEG_CHUNK0] + g] = (int32_t)(c + c0);
-      p[p[PLAN_OFF_SEG_NCHUNKS] + g] = (int32_t)(cn < 0 ? 0 : cn);
-      p[p[PLAN_OFF_SEG_SEQ] + g] = s;
-      p[p[PLAN_OFF_SEG_FLAGS] + g] = (i == 0 ? SEG_FIRST : 0) | (i == ns - 1 ? SEG_LAST : 0);
-      ++g;
-    }
-    for (int64_t i = 0; i < nc; ++i) {
-      p[p[PLAN_OFF_CHUNK_TOK0] + c] = (int32_t)(bos + i * GDR_C);
-      p[p[PLAN_OFF_CHUNK_LEN] + c] = (int32_t)(len - i * GDR_C < GDR_C ? len - i * GDR_C : GDR_C);
-      ++c;
-    }
-  }
-  return LAMPA_OK;
-}
-
-// ---- record layout ----------------------------------------------------------------------------------------------
-// A fragment is 64 lanes x 8 bf16 (1 KiB): lane l's 16 bytes are its share of one MFMA 32x32x16 A operand.
-//   Wf[tm][ks]   -W rows 32tm..+31 (tokens), contraction step ks over the key dimension     2*(K/16) fragments
-//   Kf[km][ks]   K~^T rows 32km..+31 (key dims), contraction step ks over the tokens         (K/32)*4
-//   Qf[tm][ks]   Q~ rows (tokens), contraction over the key dimension                        2*(K/16)
-//   Pf[tm][ks]   P rows (tokens i), contraction over the tokens j (tm = 0 only needs ks < 2) 2*4
-//   Uf[tm][vn]   U tile in accumulator layout, 16 bf16 per lane (2 KiB)                      2*(V/32)
-template <int KT, int VT>
-struct GdrRecord {
-  static constexpr int W_FRAGS = 2 * (KT / 16);
-  static constexpr int K_FRAGS = (KT / 32) * 4;
-  static constexpr int Q_FRAGS = 2 * (KT / 16);
-  static constexpr int P_FRAGS = 8;
-  static constexpr int U_TILES = 2 * (VT / 32);
-  static constexpr int W_OFF = 0;
-  static constexpr int K_OFF = W_OFF + W_FRAGS;
-  static constexpr int Q_OFF = K_OFF + K_FRAGS;
-  static constexpr int P_OFF = Q_OFF + Q_FRAGS;
-  static constexpr int U_OFF = P_OFF + P_FRAGS;            // in units of 1 KiB
-  static constexpr int BYTES = (U_OFF + 2 * U_TILES) * 1024;
-};
-
-static int64_t gdr_record_bytes(int K, int V) {
-  return (int64_t)(2 * (K / 16) * 2 + (K / 32) * 4 + 8 + 2 * 2 * (V / 32)) * 1024;
-}
-
-__device__ __forceinline__ bf16x8 frag_load(const unsigned char* rec, int frag, int lane) {
-  return *reinterpret_cast<const bf16x8*>(rec + (size_t)frag * 1024 + lane * 16);
-}
-__device__ __forceinline__ void frag_store(unsigned char* rec, int frag, int lane, bf16x8 v) {
-#ifndef GDR_DBG_SKIP_STORE
-  *reinterpret_cast<bf16x8*>(rec + (size_t)frag * 1024 + lane * 16) = v;
-#else
-  if (v[0] == (__bf16)123.456f) *reinterpret_cast<bf16x8*>(rec + (size_t)frag * 1024 + lane * 16) = v;
+#ifndef LB_MIN
+#define LB_MIN 2
 #endif
+#ifndef DBG_TR
+#define DBG_TR
+#endif
+#ifdef DBG_TIMING
+__device__ unsigned long long g_dbg[8192];
+extern "C" int lampa_dbg_read(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), sizeof(unsigned long long) * n);
+}
+#define DBG_T(slot) do { if (dbg_on && lane == 0) g_dbg[dbg_base + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define DBG_T(slot) do { } while (0)
+#endif
+#define T_BYTES (64 * 64 * 2)  // T of one chunk and head in HBM: bf16 [64][64] row-major
+
+__device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
+  return *reinterpret_cast<const bf16x8*>(base + (size_t)frag * 1024 + lane * 16);
+}
+__device__ __forceinline__ void frag_store(unsigned char* base, int frag, int lane, bf16x8 v) {
+  *reinterpret_cast<bf16x8*>(base + (size_t)frag * 1024 + lane * 16) = v;
 }
 
-// ---- prep kernel ----------------------------------------------------------------------------------------------
-template <int KT, int VT>
-struct GdrPrepSmem {
-  static constexpr int SK = KT + 8;  // row stride of the row-major k / q tiles (bf16)
-  static constexpr int SX = 72;      // row stride of the [dim][token] tiles and of the [token][token] tiles (bf16)
-  static constexpr int SA = 68;      // row stride of the fp32 A tile
-  static constexpr int OFF_K = 0;
-  static constexpr int OFF_Q = OFF_K + 64 * SK * 2;
-  static constexpr int OFF_KT = OFF_Q + 64 * SK * 2;
-  static constexpr int OFF_VT = OFF_KT + KT * SX * 2;
-  static constexpr int OFF_A = OFF_VT + VT * SX * 2;
-  static constexpr int OFF_TW = OFF_A + 64 * SA * 4;
-  static constexpr int OFF_TU = OFF_TW + 64 * SX * 2;
-  static constexpr int OFF_GAMMA = OFF_TU + 64 * SX * 2;
-  static constexpr int OFF_BETA = OFF_GAMMA + 64 * 4;
-  static constexpr int BYTES = OFF_BETA + 64 * 4;
+// A-operand fragment (rows row0..row0+31 of a row-major bf16 array with `stride` elements per row, contraction
+// step starting at column col0) in accumulator slot order: slots 0-3 = columns col0 + 4hh + 0..3,
+// slots 4-7 = columns col0 + 8 + 4hh + 0..3.
+__device__ __forceinline__ bf16x8 ld_kappa(const __bf16* arr, int stride, int row, int col0, int hh) {
+  const bf16x4 lo = *reinterpret_cast<const bf16x4*>(arr + row * stride + col0 + 4 * hh);
+  const bf16x4 hi = *reinterpret_cast<const bf16x4*>(arr + row * stride + col0 + 8 + 4 * hh);
+  bf16x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
+__device__ __forceinline__ f32x16 zero16() {
+  f32x16 z;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+  return z;
+}
+
+__device__ __forceinline__ int acc_row(int r, int hh) { return 8 * (r / 4) + 4 * hh + (r % 4); }
+
+__device__ __forceinline__ float l2_factor(float ss, int l2norm) {
+  if (l2norm == GDR_L2_CHUNK) return 1.0f / __fsqrt_rn(ss + 1e-6f);
+  if (l2norm == GDR_L2_RECURRENT) return 1.0f / (__fsqrt_rn(ss) + 1e-6f);
+  return 1.0f;
+}
+
+// 16-byte vector of the input element type
+template <typename T>
+struct Raw8 {
+  typedef T type __attribute__((ext_vector_type(8)));
 };
 
-template <typename T, int KT, int VT>
-__global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, const T* __restrict__ k,
-                                                      const T* __restrict__ v, const float* __restrict__ g,
+// Raw input piece -> bf16 operand piece (+ its sum of squares when the rows get l2-normalised). bf16 inputs are
+// passed through bit for bit; fp16 inputs are rounded to bf16 here.
+template <typename T>
+__device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& ss, bool want_ss) {
+  bf16x8 out;
+  if constexpr (sizeof(T) == 2 && !__is_same(T, _Float16)) {
+    out = __builtin_bit_cast(bf16x8, v);
+    if (want_ss) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)out[e];
+        ss = __builtin_fmaf(f, f, ss);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)v[e];
+      if (want_ss) ss = __builtin_fmaf(f, f, ss);
+      out[e] = (__bf16)f;
+    }
+  }
+  return out;
+}
+
+// ---- T = (I + A)^-1 ------------------------------------------------------------------------------------------
+template <typename T, int KT>
+__global__ void __launch_bounds__(256) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
                                                       const float* __restrict__ beta,
                                                       const int32_t* __restrict__ plan,
-                                                      unsigned char* __restrict__ records,
-                                                      float* __restrict__ decs, int H, int HV, float scale,
+                                                      unsigned char* __restrict__ tmat, int H, int HV,
                                                       int l2norm) {
-  using SM = GdrPrepSmem<KT, VT>;
-  using REC = GdrRecord<KT, VT>;
-  extern __shared__ __align__(16) unsigned char smem[];
-  __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
-  __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
-  __bf16* s_kT = reinterpret_cast<__bf16*>(smem + SM::OFF_KT);
-  __bf16* s_vT = reinterpret_cast<__bf16*>(smem + SM::OFF_VT);
-  float* s_A = reinterpret_cast<float*>(smem + SM::OFF_A);
-  __bf16* s_TW = reinterpret_cast<__bf16*>(smem + SM::OFF_TW);
-  __bf16* s_TU = reinterpret_cast<__bf16*>(smem + SM::OFF_TU);
-  float* s_gamma = reinterpret_cast<float*>(smem + SM::OFF_GAMMA);
-  float* s_beta = reinterpret_cast<float*>(smem + SM::OFF_BETA);
-  constexpr int SK = SM::SK, SX = SM::SX, SA = SM::SA;
+  constexpr int SK = KT + 8, SA = 68, ST = 72;
+  __shared__ __align__(16) __bf16 s_k[64 * SK];
+  __shared__ __align__(16) float s_A[64 * SA];
+  __shared__ __align__(16) __bf16 s_T[64 * ST];
+  __shared__ float s_gamma[64], s_beta[64], s_rk[64];
 
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
   const int tok0 = plan[plan[PLAN_OFF_CHUNK_TOK0] + chunk];
   const int len = plan[plan[PLAN_OFF_CHUNK_LEN] + chunk];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
-  unsigned char* rec = records + ((size_t)chunk * HV + hv) * REC::BYTES;
 
-  // (1) cumulative log-decay and beta of the chunk; rows past the end behave as g = 0, beta = 0, k = v = q = 0
-  if (wave == 0) {
+  if (wave == 0) {  // rows past the end of a partial chunk behave as g = 0, beta = 0, k = 0
     float gv = lane < len ? g[(size_t)(tok0 + lane) * HV + hv] : 0.0f;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -210,80 +142,29 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
     s_gamma[lane] = gv;
     s_beta[lane] = lane < len ? beta[(size_t)(tok0 + lane) * HV + hv] : 0.0f;
   }
-
-  // (2) load, l2-normalise, stage in LDS: k row-major and transposed, q row-major, v transposed
   {
-    const int row = tid >> 2, q4 = tid & 3;
-    const bool valid = row < len;
+    const int row = tid >> 2, part = tid & 3;
     constexpr int EPT = KT / 4;
-    float kf[EPT], qf[EPT];
-    float kss = 0.0f, qss = 0.0f;
-    const T* kp = k + ((size_t)(tok0 + row) * H + h) * KT + q4 * EPT;
-    const T* qp = q + ((size_t)(tok0 + row) * H + h) * KT + q4 * EPT;
+    float ss = 0.0f;
+    const T* kp = k + ((size_t)(tok0 + (row < len ? row : 0)) * H + h) * KT + part * EPT;
 #pragma unroll
     for (int c = 0; c < EPT / 8; ++c) {
-      if (valid) {
-        load8<T>(kp + 8 * c, kf + 8 * c);
-        load8<T>(qp + 8 * c, qf + 8 * c);
-      } else {
+      typename Raw8<T>::type raw;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { kf[8 * c + e] = 0.0f; qf[8 * c + e] = 0.0f; }
-      }
+      for (int e = 0; e < 8; ++e) raw[e] = (T)0.0f;
+      if (row < len) raw = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * c);
+      *reinterpret_cast<bf16x8*>(&s_k[row * SK + part * EPT + 8 * c]) = raw_to_bf16<T>(raw, ss, l2norm != GDR_L2_NONE);
     }
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) { kss += kf[e] * kf[e]; qss += qf[e] * qf[e]; }
-    float kinv = 1.0f, qinv = 1.0f;
-    if (l2norm != GDR_L2_NONE) {
-      kss += __shfl_xor(kss, 1); kss += __shfl_xor(kss, 2);
-      qss += __shfl_xor(qss, 1); qss += __shfl_xor(qss, 2);
-      if (l2norm == GDR_L2_CHUNK) {
-        kinv = 1.0f / __fsqrt_rn(kss + 1e-6f);
-        qinv = 1.0f / __fsqrt_rn(qss + 1e-6f);
-      } else {
-        kinv = 1.0f / (__fsqrt_rn(kss) + 1e-6f);
-        qinv = 1.0f / (__fsqrt_rn(qss) + 1e-6f);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < EPT / 8; ++c) {
-      bf16x8 kb, qb;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        kb[e] = (__bf16)(kf[8 * c + e] * kinv);
-        qb[e] = (__bf16)(qf[8 * c + e] * qinv);
-#ifndef GDR_DBG_SKIP_TR
-        s_kT[(q4 * EPT + 8 * c + e) * SX + row] = kb[e];
-#endif
-      }
-      *reinterpret_cast<bf16x8*>(&s_k[row * SK + q4 * EPT + 8 * c]) = kb;
-      *reinterpret_cast<bf16x8*>(&s_q[row * SK + q4 * EPT + 8 * c]) = qb;
-    }
-    constexpr int VPT = VT / 4;
-    const T* vp = v + ((size_t)(tok0 + row) * HV + hv) * VT + q4 * VPT;
-#pragma unroll
-    for (int c = 0; c < VPT / 8; ++c) {
-      float vf[8];
-      if (valid) {
-        load8<T>(vp + 8 * c, vf);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) vf[e] = 0.0f;
-      }
-#pragma unroll
-#ifndef GDR_DBG_SKIP_TR
-      for (int e = 0; e < 8; ++e) s_vT[(q4 * VPT + 8 * c + e) * SX + row] = (__bf16)vf[e];
-#endif
-    }
+    ss += __shfl_xor(ss, 1);
+    ss += __shfl_xor(ss, 2);
+    if (part == 0) s_rk[row] = l2_factor(ss, l2norm);
   }
   __syncthreads();
 
-  // (3) A = strict_lower(beta_i (k_i . k_j) e^{gamma_i - gamma_j}) -> LDS fp32; one 32x32 tile per wave
-  {
+  {  // A -> LDS fp32; one 32x32 tile per wave, the tile above the diagonal is never read
     const int tm = wave >> 1, tn = wave & 1;
     if (!(tm == 0 && tn == 1)) {
-      f32x16 acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+      f32x16 acc = zero16();
 #pragma unroll
       for (int ks = 0; ks < KT / 16; ++ks) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tm + ln) * SK + 16 * ks + 8 * hh]);
@@ -291,22 +172,20 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
         acc = mfma32(a, b, acc);
       }
       const int j = 32 * tn + ln;
-      const float gj = s_gamma[j];
+      const float gj = s_gamma[j], rj = s_rk[j];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = 32 * tm + 8 * (r / 4) + 4 * hh + (r % 4);
-        const float val = i > j ? acc[r] * s_beta[i] * __expf(s_gamma[i] - gj) : 0.0f;
-        s_A[i * SA + j] = val;
+        const int i = 32 * tm + acc_row(r, hh);
+        s_A[i * SA + j] = i > j ? acc[r] * s_beta[i] * s_rk[i] * rj * __expf(s_gamma[i] - gj) : 0.0f;
       }
     }
   }
   __syncthreads();
 
   if (wave == 0) {
-    // (4a) T = (I + A)^-1, A strictly lower triangular, as a 2x2 block matrix of 32x32 blocks:
-    //      T11 = (I + A11)^-1, T22 = (I + A22)^-1 by forward substitution -- lane 32b + c owns column c of block b,
-    //      every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
-    //      T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+    // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
+    // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
+    // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
     const int b = hh, c = ln;
     const float* Ab = s_A + (32 * b) * SA + 32 * b;
     float x[32];
@@ -327,31 +206,21 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
         else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
       }
       x[i] = acc0 + acc1;
-      // pins the order "loads of row i+1, arithmetic of row i" so the compiler neither serialises every load
-      // behind a wait nor hoists all 124 loads to the top (which spills)
+      // pins the order "loads of row i+1, arithmetic of row i": without it the compiler either serialises every
+      // load behind a wait or hoists all 124 loads to the top and spills
       asm volatile("" : "+v"(x[i]) : : "memory");
     }
     __builtin_amdgcn_wave_barrier();
-    // diagonal blocks: fp32 copy in place of A11 / A22 (operands of the merge) and the scaled bf16 outputs;
-    // the upper-right block of T is zero
-    const float bc = s_beta[lane];
-    const float wc = bc * __expf(s_gamma[lane]);
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      s_A[(32 * b + i) * SA + lane] = x[i];
-      s_TW[(32 * b + i) * SX + lane] = (__bf16)(x[i] * wc);
-      s_TU[(32 * b + i) * SX + lane] = (__bf16)(x[i] * bc);
-      if (b == 1) {
-        s_TW[i * SX + lane] = (__bf16)0.0f;
-        s_TU[i * SX + lane] = (__bf16)0.0f;
-      }
+      s_A[(32 * b + i) * SA + lane] = x[i];  // fp32 diagonal blocks in place of A11 / A22 (operands of the merge)
+      s_T[(32 * b + i) * ST + lane] = (__bf16)x[i];
+      if (b == 1) s_T[i * ST + lane] = (__bf16)0.0f;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    f32x16 y0, y1, y2;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { y0[r] = 0.0f; y1[r] = 0.0f; y2[r] = 0.0f; }
+    f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11
       bf16x8 ahi, alo, bhi, blo;
@@ -369,9 +238,9 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
       y1 = mfma32(alo, bhi, y1);
       y2 = mfma32(ahi, blo, y2);
     }
-    f32x16 t0, t1, t2;
+    f32x16 t0 = zero16(), t1 = zero16(), t2 = zero16();
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { y0[r] += y1[r] + y2[r]; t0[r] = 0.0f; t1[r] = 0.0f; t2[r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) y0[r] += y1[r] + y2[r];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
       bf16x8 ahi, alo, bhi, blo;
@@ -389,422 +258,558 @@ __global__ void __launch_bounds__(256) gdr_prep_kernel(const T* __restrict__ q, 
       t1 = mfma32(alo, bhi, t1);
       t2 = mfma32(ahi, blo, t2);
     }
-    const float bl = s_beta[ln];
-    const float wl = bl * __expf(s_gamma[ln]);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-      const float t21 = -(t0[r] + (t1[r] + t2[r]));
-      s_TW[row * SX + ln] = (__bf16)(t21 * wl);
-      s_TU[row * SX + ln] = (__bf16)(t21 * bl);
-    }
-    if (lane == 0) decs[(size_t)chunk * HV + hv] = __expf(s_gamma[63]);
-  } else {
-    // (4b) meanwhile: P^T tiles, K~^T fragments, Q~ fragments
-    constexpr int N_TASKS = 3 + REC::K_FRAGS + REC::Q_FRAGS;
-    const float g_last = s_gamma[63];
-    for (int task = wave - 1; task < N_TASKS; task += 3) {
-      if (task < 3) {
-        const int jm = task == 2 ? 1 : 0, tn = task == 0 ? 0 : 1;  // tiles (0,0), (0,1), (1,1); (1,0) is all zero
-        f32x16 acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(&s_k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
-          acc = mfma32(a, b, acc);
-        }
-        const int i = 32 * tn + ln;
-        const float gi = s_gamma[i];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int j = 32 * jm + 8 * (r / 4) + 4 * hh + (r % 4);
-          acc[r] = i >= j ? acc[r] * scale * __expf(gi - s_gamma[j]) : 0.0f;
-        }
-        frag_store(rec, REC::P_OFF + tn * 4 + 2 * jm + 0, lane, acc_to_operand(acc, 0));
-        frag_store(rec, REC::P_OFF + tn * 4 + 2 * jm + 1, lane, acc_to_operand(acc, 8));
-      } else if (task < 3 + REC::K_FRAGS) {
-        const int f = task - 3, km = f / 4, ks = f % 4;
-        const int kd = 32 * km + ln;
-        const bf16x4 lo = *reinterpret_cast<const bf16x4*>(&s_kT[kd * SX + 16 * ks + 4 * hh]);
-        const bf16x4 hi = *reinterpret_cast<const bf16x4*>(&s_kT[kd * SX + 16 * ks + 8 + 4 * hh]);
-        bf16x8 out;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const int tok = 16 * ks + kappa(hh, s);
-          const float kv = (float)(s < 4 ? lo[s % 4] : hi[s % 4]);
-          out[s] = (__bf16)(kv * __expf(g_last - s_gamma[tok]));
-        }
-        frag_store(rec, REC::K_OFF + f, lane, out);
-      } else {
-        const int f = task - 3 - REC::K_FRAGS, tm = f / (KT / 16), ks = f % (KT / 16);
-        const int tok = 32 * tm + ln;
-        const bf16x4 lo = *reinterpret_cast<const bf16x4*>(&s_q[tok * SK + 16 * ks + 4 * hh]);
-        const bf16x4 hi = *reinterpret_cast<const bf16x4*>(&s_q[tok * SK + 16 * ks + 8 + 4 * hh]);
-        const float sc = scale * __expf(s_gamma[tok]);
-        bf16x8 out;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) out[s] = (__bf16)((float)(s < 4 ? lo[s % 4] : hi[s % 4]) * sc);
-        frag_store(rec, REC::Q_OFF + f, lane, out);
-      }
-    }
+    for (int r = 0; r < 16; ++r) s_T[(32 + acc_row(r, hh)) * ST + ln] = (__bf16)(-(t0[r] + (t1[r] + t2[r])));
   }
   __syncthreads();
 
-  // (5) -W^T = -(k^T TW^T) -> A fragments of W S;  U = TU v -> accumulator-layout tiles
+  // T row-major bf16 [64][64] (the upper-right 32x32 block is zero)
   {
-    constexpr int W_TILES = (KT / 32) * 2, U_TILES = 2 * (VT / 32);
-    for (int task = wave; task < W_TILES + U_TILES; task += 4) {
-      f32x16 acc;
+    __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * T_BYTES);
+    const int row = tid >> 2, part = tid & 3;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-      if (task < W_TILES) {
-        const int km = task >> 1, tn = task & 1;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(&s_kT[(32 * km + ln) * SX + 16 * ks + 8 * hh]);
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&s_TW[(32 * tn + ln) * SX + 16 * ks + 8 * hh]);
-          acc = mfma32(a, b, acc);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = -acc[r];
-        frag_store(rec, REC::W_OFF + tn * (KT / 16) + 2 * km + 0, lane, acc_to_operand(acc, 0));
-        frag_store(rec, REC::W_OFF + tn * (KT / 16) + 2 * km + 1, lane, acc_to_operand(acc, 8));
-      } else {
-        const int t = task - W_TILES, tm = t / (VT / 32), vn = t % (VT / 32);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(&s_TU[(32 * tm + ln) * SX + 16 * ks + 8 * hh]);
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&s_vT[(32 * vn + ln) * SX + 16 * ks + 8 * hh]);
-          acc = mfma32(a, b, acc);
-        }
-        unsigned char* up = rec + (size_t)REC::U_OFF * 1024 + (size_t)t * 2048 + lane * 32;
-        *reinterpret_cast<bf16x8*>(up) = acc_to_operand(acc, 0);
-        *reinterpret_cast<bf16x8*>(up + 16) = acc_to_operand(acc, 8);
-      }
-    }
+    for (int c = 0; c < 2; ++c)
+      *reinterpret_cast<bf16x8*>(out + row * 64 + part * 16 + 8 * c) =
+          *reinterpret_cast<const bf16x8*>(&s_T[row * ST + part * 16 + 8 * c]);
   }
 }
 
-// ---- sequential kernels -----------------------------------------------------------------------------------------
-// State tile km of a wave: rows 32km..+31 (key dims), 32 columns; register r of lane l = (row 8*(r/4)+4*hh+r%4, col ln).
-template <int KT>
-__device__ __forceinline__ void state_operands(const f32x16* S, bf16x8* Sb) {
-#pragma unroll
-  for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
-}
-
-// Operand fragments of one chunk for one wave of the sequential kernels, held in registers so that the next
-// chunk's loads are in flight while the current chunk computes.
-template <int KT, int VT, bool WITH_OUTPUT>
-struct GdrChunkOps {
-  bf16x8 W[2 * (KT / 16)];
-  bf16x8 Kf[(KT / 32) * 4];
-  bf16x8 Q[WITH_OUTPUT ? 2 * (KT / 16) : 1];
-  bf16x8 P[WITH_OUTPUT ? 6 : 1];
-  bf16x8 U[4];  // U tiles tm = 0, 1 of this wave's 32 columns, two halves each
-  float dec;
+// ---- segment kernel --------------------------------------------------------------------------------------------
+// Workgroup per (segment, head). Waves 0 .. SLABS-1 ("chain" waves) each own 32 columns of the state and run the
+// recurrence; the last two waves ("stagers") load the next chunk's tiles from HBM, stage them in LDS, derive the
+// per-token factors and (PASS_B) build the P fragments. The two roles run separate loops that meet at three
+// LDS-only barriers per chunk, so that the stagers' global loads stay in flight while the chain waves compute and
+// neither role pays for the other's registers.
+template <int KT, int VT, bool PASS_B>
+struct GdrSegSmem {
+  static constexpr int SK = KT + 8;  // row stride of the row-major k / q tiles (bf16 elements)
+  static constexpr int SX = 72;      // row stride of the transposed [dim][token] tiles and of T
+  static constexpr int OFF_K = 0;
+  static constexpr int OFF_KT = OFF_K + 64 * SK * 2;
+  static constexpr int OFF_VT = OFF_KT + KT * SX * 2;
+  static constexpr int OFF_T = OFF_VT + VT * SX * 2;
+  static constexpr int OFF_Q = OFF_T + 64 * SX * 2;
+  static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
+  static constexpr int OFF_SCAL = OFF_P + (PASS_B ? 6 * 1024 : 0);
+  static constexpr int N_SCAL = 8;  // beta, ek, dk, qs, gamma, rk, rq, misc
+  static constexpr int BYTES = OFF_SCAL + N_SCAL * 64 * 4;
 };
 
-template <int KT, int VT, bool WITH_OUTPUT>
-__device__ __forceinline__ void chunk_ops_load(GdrChunkOps<KT, VT, WITH_OUTPUT>& ops,
-                                               const unsigned char* __restrict__ rec, const float* __restrict__ decp,
-                                               int lane, int vn, bool with_u) {
-  using REC = GdrRecord<KT, VT>;
-#pragma unroll
-  for (int f = 0; f < 2 * (KT / 16); ++f) ops.W[f] = frag_load(rec, REC::W_OFF + f, lane);
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
-    const unsigned char* up = rec + (size_t)REC::U_OFF * 1024 + (size_t)(tm * (VT / 32) + vn) * 2048 + lane * 32;
-    if (with_u) {
-      ops.U[2 * tm + 0] = *reinterpret_cast<const bf16x8*>(up);
-      ops.U[2 * tm + 1] = *reinterpret_cast<const bf16x8*>(up + 16);
-    } else {
-#pragma unroll
-      for (int q = 0; q < 8; ++q) { ops.U[2 * tm][q] = (__bf16)0.0f; ops.U[2 * tm + 1][q] = (__bf16)0.0f; }
-    }
-  }
-  if constexpr (WITH_OUTPUT) {
-#pragma unroll
-    for (int f = 0; f < 2 * (KT / 16); ++f) ops.Q[f] = frag_load(rec, REC::Q_OFF + f, lane);
-#pragma unroll
-    for (int f = 0; f < 2; ++f) ops.P[f] = frag_load(rec, REC::P_OFF + f, lane);
-#pragma unroll
-    for (int f = 0; f < 4; ++f) ops.P[2 + f] = frag_load(rec, REC::P_OFF + 4 + f, lane);
-  }
-#pragma unroll
-  for (int f = 0; f < (KT / 32) * 4; ++f) ops.Kf[f] = frag_load(rec, REC::K_OFF + f, lane);
-  ops.dec = *decp;
-}
+template <int KT, int VT, bool PASS_B>
+struct GdrSegShape {
+  static constexpr int SLABS = PASS_B ? VT / 32 : (KT + VT) / 32;  // chain waves
+  static constexpr int WAVES = SLABS + 2;                          // + two stager waves
+};
 
-__device__ __forceinline__ f32x16 utile_widen(bf16x8 a, bf16x8 b) {
-  f32x16 out;
-#pragma unroll
-  for (int s = 0; s < 8; ++s) { out[s] = (float)a[s]; out[8 + s] = (float)b[s]; }
-  return out;
-}
+template <typename T, int KT, int VT, bool PASS_B>
+__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_MIN)
+    gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                       const float* __restrict__ g, const float* __restrict__ beta,
+                       const int32_t* __restrict__ plan, const unsigned char* __restrict__ tmat,
+                       const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
+                       unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o, float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
+  using SM = GdrSegSmem<KT, VT, PASS_B>;
+  constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
+  constexpr int SK = SM::SK, SX = SM::SX;
+  extern __shared__ __align__(16) unsigned char smem[];
+  __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
+  __bf16* s_kT = reinterpret_cast<__bf16*>(smem + SM::OFF_KT);
+  __bf16* s_vT = reinterpret_cast<__bf16*>(smem + SM::OFF_VT);
+  __bf16* s_T = reinterpret_cast<__bf16*>(smem + SM::OFF_T);
+  __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
+  unsigned char* s_P = smem + SM::OFF_P;
+  float* s_beta = reinterpret_cast<float*>(smem + SM::OFF_SCAL);
+  float* s_ek = s_beta + 64;     // e^{gamma_i} rk_i
+  float* s_dk = s_beta + 128;    // e^{gamma_last - gamma_i} rk_i
+  float* s_qs = s_beta + 192;    // scale e^{gamma_i} rq_i
+  float* s_gamma = s_beta + 256;
+  float* s_rk = s_beta + 320;
+  float* s_rq = s_beta + 384;
+  float* s_misc = s_beta + 448;  // [0] = e^{gamma_last}
 
-// One chunk of the recurrence on a 32-column slab: v_new = U - W S (Vb = its B-operand fragments),
-// S <- dec S + K~^T v_new. With output: o tile tm = Q~ S + P v_new is handed to `emit(tm, acc)`.
-template <int KT, int VT, bool WITH_OUTPUT, typename Emit>
-__device__ __forceinline__ void chunk_step(const GdrChunkOps<KT, VT, WITH_OUTPUT>& ops, f32x16* S, Emit emit) {
-  bf16x8 Sb[KT / 16];
-  state_operands<KT>(S, Sb);
-  bf16x8 Vb[4];
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
-    f32x16 acc = utile_widen(ops.U[2 * tm], ops.U[2 * tm + 1]);
-#pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(ops.W[tm * (KT / 16) + ks], Sb[ks], acc);
-    Vb[2 * tm + 0] = acc_to_operand(acc, 0);
-    Vb[2 * tm + 1] = acc_to_operand(acc, 8);
-  }
-  if constexpr (WITH_OUTPUT) {
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm) {
-      f32x16 acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(ops.Q[tm * (KT / 16) + ks], Sb[ks], acc);
-#pragma unroll
-      for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ops.P[2 * tm + ks], Vb[ks], acc);
-      emit(tm, acc);
-    }
-  }
-#pragma unroll
-  for (int km = 0; km < KT / 32; ++km) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) S[km][r] *= ops.dec;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(ops.Kf[km * 4 + ks], Vb[ks], S[km]);
-  }
-}
-
-// composite: grid (n_segments, HV), one wave per 32-column slab of [M | N] ((KT+VT)/32 waves per workgroup, so the
-// waves that read the same W and K~ fragments share one CU's L1 and one XCD's L2). Slabs < KT/32 carry columns of
-// M (start: identity, no U term), the others columns of N (start: zero).
-// Mcomp [seg, HV, KT, KT], Ncomp [seg, HV, KT, VT] fp32 row-major.
-template <int KT, int VT>
-__global__ void __launch_bounds__(2 * (KT + VT)) gdr_composite_kernel(const int32_t* __restrict__ plan,
-                                                          const unsigned char* __restrict__ records,
-                                                          const float* __restrict__ decs,
-                                                          float* __restrict__ Mcomp, float* __restrict__ Ncomp,
-                                                          int HV) {
-  using REC = GdrRecord<KT, VT>;
-  using OPS = GdrChunkOps<KT, VT, false>;
-  const int slab = threadIdx.x >> 6, seg = blockIdx.x, hv = blockIdx.y;
+  const int seg = blockIdx.x, hv = blockIdx.y;
+  const int h = hv / (HV / H);
   const int flags = plan[plan[PLAN_OFF_SEG_FLAGS] + seg];
-  if (flags & SEG_LAST) return;  // nothing follows the last segment of a sequence
+  if (!PASS_B && (flags & SEG_LAST)) return;  // nothing follows the last segment of a sequence
   const int c0 = plan[plan[PLAN_OFF_SEG_CHUNK0] + seg], nc = plan[plan[PLAN_OFF_SEG_NCHUNKS] + seg];
-  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
-  const bool is_m = slab < KT / 32;
-  const int vn = is_m ? 0 : slab - KT / 32;
-
-  f32x16 S[KT / 32];
-#pragma unroll
-  for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-    for (int r = 0; r < 16; ++r)
-      S[km][r] = (is_m && (32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) == 32 * slab + ln) ? 1.0f : 0.0f;
-
-  auto rec_of = [&](int c) { return records + ((size_t)c * HV + hv) * REC::BYTES; };
-  auto dec_of = [&](int c) { return decs + (size_t)c * HV + hv; };
-  auto no_emit = [](int, const f32x16&) {};
   const int c1 = c0 + nc;
-  OPS a, b;
-  if (nc > 0) chunk_ops_load<KT, VT, false>(a, rec_of(c0), dec_of(c0), lane, vn, !is_m);
-  for (int c = c0; c < c1; c += 2) {
-    if (c + 1 < c1) chunk_ops_load<KT, VT, false>(b, rec_of(c + 1), dec_of(c + 1), lane, vn, !is_m);
-    chunk_step<KT, VT, false>(a, S, no_emit);
-    if (c + 1 < c1) {
-      if (c + 2 < c1) chunk_ops_load<KT, VT, false>(a, rec_of(c + 2), dec_of(c + 2), lane, vn, !is_m);
-      chunk_step<KT, VT, false>(b, S, no_emit);
-    }
-  }
-  float* out = is_m ? Mcomp + ((size_t)seg * HV + hv) * KT * KT : Ncomp + ((size_t)seg * HV + hv) * KT * VT;
-  const int ncols = is_m ? KT : VT, col = (is_m ? 32 * slab : 32 * vn) + ln;
-#pragma unroll
-  for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) out[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * ncols + col] = S[km][r];
-}
-
-// scan: grid (VT/32, n_seq, HV), KT/32 waves per workgroup. Wave w owns state rows 32w..32w+31 of a 32-column slab.
-// Per segment: store the state as the segment's initial state, then S <- M S + N with M and S split into bf16
-// high and remainder parts (three MFMA products, close to fp32 accuracy). The waves exchange their share of S as
-// B-operand fragments through a double-buffered LDS array (one barrier per step); the M rows and N tile of the
-// next step are loaded while the current one computes.
-// Sinit [seg, HV, KT, VT] fp32 row-major receives the state every segment starts from.
-template <int KT>
-struct GdrScanRegs {
-  f32x4 m[KT / 16][2];
-  float n[16];
-};
-
-template <int KT, int VT>
-__device__ __forceinline__ void scan_load(GdrScanRegs<KT>& r, const float* __restrict__ M,
-                                          const float* __restrict__ N, int wave, int hh, int ln, int col) {
-#pragma unroll
-  for (int ks = 0; ks < KT / 16; ++ks) {
-    const float* mrow = M + (size_t)(32 * wave + ln) * KT + 16 * ks;
-    r.m[ks][0] = *reinterpret_cast<const f32x4*>(mrow + 4 * hh);
-    r.m[ks][1] = *reinterpret_cast<const f32x4*>(mrow + 8 + 4 * hh);
-  }
-#pragma unroll
-  for (int q = 0; q < 16; ++q) r.n[q] = N[(size_t)(32 * wave + 8 * (q / 4) + 4 * hh + (q % 4)) * VT + col];
-}
-
-template <int KT, int VT>
-__global__ void __launch_bounds__(KT * 2) gdr_scan_kernel(const int32_t* __restrict__ plan,
-                                                         const float* __restrict__ Mcomp,
-                                                         const float* __restrict__ Ncomp,
-                                                         const float* __restrict__ h0, float* __restrict__ Sinit,
-                                                         int HV) {
-  __shared__ __align__(16) bf16x8 s_frag[2][2][KT / 16][64];  // [buffer][hi/lo][contraction step][lane]
-  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
-  const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
-  const int col = 32 * vn + ln;
-  f32x16 S;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = 32 * wave + 8 * (r / 4) + 4 * hh + (r % 4);
-    S[r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + row) * VT + col] : 0.0f;
-  }
-  GdrScanRegs<KT> nxt;
-  if (nseg > 1)
-    scan_load<KT, VT>(nxt, Mcomp + ((size_t)seg0 * HV + hv) * KT * KT, Ncomp + ((size_t)seg0 * HV + hv) * KT * VT, wave,
-                      hh, ln, col);
-  for (int p = 0; p < nseg; ++p) {
-    const int seg = seg0 + p;
-    float* si = Sinit + ((size_t)seg * HV + hv) * KT * VT;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) si[(size_t)(32 * wave + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col] = S[r];
-    if (p == nseg - 1) break;
-    // this step's M rows (hi / lo operand fragments) and N tile arrived in nxt; start fetching the next step's
-    bf16x8 Mhi[KT / 16], Mlo[KT / 16];
-    f32x16 acc0, acc1, acc2;
-#pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks)
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float x = nxt.m[ks][q / 4][q % 4];
-        const __bf16 hi = (__bf16)x;
-        Mhi[ks][q] = hi;
-        Mlo[ks][q] = (__bf16)(x - (float)hi);
-      }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = nxt.n[r]; acc1[r] = 0.0f; acc2[r] = 0.0f; }
-    if (p + 2 < nseg)
-      scan_load<KT, VT>(nxt, Mcomp + ((size_t)(seg + 1) * HV + hv) * KT * KT,
-                        Ncomp + ((size_t)(seg + 1) * HV + hv) * KT * VT, wave, hh, ln, col);
-    // publish this wave's rows of S as B-operand fragments (contraction steps 2*wave and 2*wave+1)
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      bf16x8 hi, lo;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float x = S[8 * half + q];
-        const __bf16 h = (__bf16)x;
-        hi[q] = h;
-        lo[q] = (__bf16)(x - (float)h);
-      }
-      s_frag[p & 1][0][2 * wave + half][lane] = hi;
-      s_frag[p & 1][1][2 * wave + half][lane] = lo;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks) {
-      const bf16x8 Shi = s_frag[p & 1][0][ks][lane];
-      const bf16x8 Slo = s_frag[p & 1][1][ks][lane];
-      acc0 = mfma32(Mhi[ks], Shi, acc0);
-      acc1 = mfma32(Mlo[ks], Shi, acc1);
-      acc2 = mfma32(Mhi[ks], Slo, acc2);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) S[r] = acc0[r] + (acc1[r] + acc2[r]);
-  }
-}
-
-// output: grid (n_segments, HV), one wave per 32 value columns (VT/32 waves per workgroup).
-template <typename T, int KT, int VT>
-__global__ void __launch_bounds__(2 * VT) gdr_output_kernel(const int32_t* __restrict__ plan,
-                                                       const unsigned char* __restrict__ records,
-                                                       const float* __restrict__ decs,
-                                                       const float* __restrict__ Sinit, T* __restrict__ o,
-                                                       float* __restrict__ ht, int HV) {
-  using REC = GdrRecord<KT, VT>;
-  using OPS = GdrChunkOps<KT, VT, true>;
-  const int vn = threadIdx.x >> 6, seg = blockIdx.x, hv = blockIdx.y;
-  const int c0 = plan[plan[PLAN_OFF_SEG_CHUNK0] + seg], nc = plan[plan[PLAN_OFF_SEG_NCHUNKS] + seg];
-  const int flags = plan[plan[PLAN_OFF_SEG_FLAGS] + seg], seq = plan[plan[PLAN_OFF_SEG_SEQ] + seg];
   const int* chunk_tok0 = plan + plan[PLAN_OFF_CHUNK_TOK0];
   const int* chunk_len = plan + plan[PLAN_OFF_CHUNK_LEN];
-  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
-  const int col = 32 * vn + ln;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+
+#ifdef DBG_TIMING
+  const bool dbg_seg = PASS_B && seg == 5 && hv == 0;
+  bool dbg_on = false; int dbg_base = 0;
+#endif
+  if (wave >= NSLAB) {
+    // ================================================ stager ================================================
+    constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
+    const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
+    const int srow = stid >> 1, spart = stid & 1;
+    typename Raw8<T>::type rk_[KU], rv_[VU], rq_[PASS_B ? KU : 1];
+    bf16x8 rt_[4];
+    float rg = 0.0f, rb = 0.0f;
+    // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
+    // a select on a freshly loaded value would make the wave wait for the load at once.
+    auto issue_loads = [&](int c) {
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+      const T* kb = k + ((size_t)tok0 * H + h) * KT;
+      const T* vb = v + ((size_t)tok0 * HV + hv) * VT;
+      const int r = min(srow, len - 1);
+      const int koff = r * H * KT + spart * (KT / 2), voff = r * HV * VT + spart * (VT / 2);
+#pragma unroll
+      for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
+#pragma unroll
+      for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
+      if constexpr (PASS_B) {
+        const T* qb = q + ((size_t)tok0 * H + h) * KT;
+#pragma unroll
+        for (int u = 0; u < KU; ++u) rq_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(qb + koff + 8 * u);
+      }
+      const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * T_BYTES);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rt_[j] = tp[stid + 128 * j];
+      const float* gb = g + (size_t)tok0 * HV + hv;
+      const float* bb = beta + (size_t)tok0 * HV + hv;
+      const int gl = min(lane, len - 1) * HV;
+      rg = gb[gl];
+      rb = bb[gl];
+    };
+    if (nc > 0) issue_loads(c0);
+    for (int c = c0; c < c1; ++c) {
+      const int len = chunk_len[c];
+#ifdef DBG_TIMING
+      dbg_on = dbg_seg && (c - c0) >= 4 && (c - c0) < 8; dbg_base = (wave * 8 + (c - c0)) * 16;
+#endif
+      DBG_T(0);
+      // ---- stage chunk c ----
+      float gv = lane < len ? rg : 0.0f;  // inclusive scan of the log-decay over the chunk
+      const float bv = lane < len ? rb : 0.0f;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const float up = __shfl_up(gv, off);
+        if (lane >= off) gv += up;
+      }
+      const float g_last = __shfl(gv, 63);
+      const bool live = srow < len, want_ss = l2norm != GDR_L2_NONE;
+      float kss = 0.0f, qss = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int piece = stid + 128 * j;  // row piece / 8, columns 8 * (piece % 8) ..
+        *reinterpret_cast<bf16x8*>(&s_T[(piece >> 3) * SX + 8 * (piece & 7)]) = rt_[j];
+      }
+      typename Raw8<T>::type zero;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+#pragma unroll
+      for (int u = 0; u < KU; ++u) {
+        const bf16x8 kb8 = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+        const int e0 = spart * (KT / 2) + 8 * u;
+        *reinterpret_cast<bf16x8*>(&s_k[srow * SK + e0]) = kb8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_kT[(e0 + e) * SX + srow] = kb8[e];
+        if constexpr (PASS_B)
+          *reinterpret_cast<bf16x8*>(&s_q[srow * SK + e0]) = raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
+      }
+#pragma unroll
+      for (int u = 0; u < VU; ++u) {
+        float unused = 0.0f;
+        const bf16x8 vb8 = raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
+        const int e0 = spart * (VT / 2) + 8 * u;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_vT[(e0 + e) * SX + srow] = vb8[e];
+      }
+      kss += __shfl_xor(kss, 1);
+      qss += __shfl_xor(qss, 1);
+      // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
+      const float grow = __shfl(gv, srow), brow = __shfl(bv, srow);
+      if (spart == 0) {
+        const float rk = l2_factor(kss, l2norm), rq = l2_factor(qss, l2norm);
+        const float eg = __expf(grow);
+        s_beta[srow] = brow;
+        s_ek[srow] = eg * rk;
+        s_dk[srow] = __expf(g_last - grow) * rk;
+        s_qs[srow] = scale * eg * rq;
+        s_gamma[srow] = grow;
+        s_rk[srow] = rk;
+        s_rq[srow] = rq;
+        if (srow == 0) s_misc[0] = __expf(g_last);
+      }
+      DBG_T(1);
+      lds_barrier();  // A1: tiles and factors of chunk c are in LDS
+      DBG_T(2);
+      if (c + 1 < c1) issue_loads(c + 1);
+      if constexpr (PASS_B) {
+        for (int t = sw; t < 3; t += 2) {  // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero
+          const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
+          bf16x8 fa[KT / 16], fb[KT / 16];
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) {
+            fa[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
+            fb[ks] = *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
+          }
+          f32x4 gj[4], rj[4];  // gamma_j, rk_j of this lane's 16 accumulator rows
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4) {
+            gj[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * jm + 8 * b4 + 4 * hh]);
+            rj[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * jm + 8 * b4 + 4 * hh]);
+          }
+          const int i = 32 * tn + ln;
+          const float gi = s_gamma[i], fi = scale * s_rq[i];
+          lds_fence();
+          f32x16 acc = zero16();
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int j = 32 * jm + acc_row(r, hh);
+            acc[r] = i >= j ? acc[r] * fi * rj[r / 4][r % 4] * __expf(gi - gj[r / 4][r % 4]) : 0.0f;
+          }
+          const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
+          frag_store(s_P, f0 + 0, lane, acc_to_operand(acc, 0));
+          frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
+        }
+      }
+      DBG_T(3);
+      lds_barrier();  // B: P fragments are in LDS
+      DBG_T(4);
+      lds_barrier();  // C: the chain waves are done with chunk c's tiles
+      DBG_T(5);
+    }
+    return;
+  }
+
+  // ================================================== chain ==================================================
+  // this wave's 32 columns: PASS_B value columns; PASS_A columns of [M | N]
+  const bool is_m = !PASS_B && wave < KT / 32;
+  const int vslab = PASS_B ? wave : (is_m ? 0 : wave - KT / 32);
+  const int col = 32 * vslab + ln;  // value column (unused for M slabs)
+
   f32x16 S[KT / 32];
-  {
+  if (PASS_B) {
     const float* si = Sinit + ((size_t)seg * HV + hv) * KT * VT;
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] = si[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col];
-  }
-  auto rec_of = [&](int c) { return records + ((size_t)c * HV + hv) * REC::BYTES; };
-  auto dec_of = [&](int c) { return decs + (size_t)c * HV + hv; };
-  auto run = [&](const OPS& ops, int c) {
-    const int tok0 = chunk_tok0[c], len = chunk_len[c];
-    chunk_step<KT, VT, true>(ops, S, [&](int tm, const f32x16& acc) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int tok = 32 * tm + 8 * (r / 4) + 4 * hh + (r % 4);
-        if (tok < len) o[((size_t)(tok0 + tok) * HV + hv) * VT + col] = GdrElem<T>::from_float(acc[r]);
-      }
-    });
-  };
-  const int c1 = c0 + nc;
-  if constexpr (KT <= 64) {
-    OPS a, b;  // two register sets: the next chunk's fragments load while the current chunk computes
-    if (nc > 0) chunk_ops_load<KT, VT, true>(a, rec_of(c0), dec_of(c0), lane, vn, true);
-    for (int c = c0; c < c1; c += 2) {
-      if (c + 1 < c1) chunk_ops_load<KT, VT, true>(b, rec_of(c + 1), dec_of(c + 1), lane, vn, true);
-      run(a, c);
-      if (c + 1 < c1) {
-        if (c + 2 < c1) chunk_ops_load<KT, VT, true>(a, rec_of(c + 2), dec_of(c + 2), lane, vn, true);
-        run(b, c + 1);
-      }
-    }
+      for (int r = 0; r < 16; ++r) S[km][r] = si[(size_t)(32 * km + acc_row(r, hh)) * VT + col];
   } else {
-    for (int c = c0; c < c1; ++c) {
-      OPS a;
-      chunk_ops_load<KT, VT, true>(a, rec_of(c), dec_of(c), lane, vn, true);
-      run(a, c);
-    }
-  }
-  if (ht && (flags & SEG_LAST)) {
-    float* out = ht + ((size_t)seq * HV + hv) * KT * VT;
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) out[(size_t)(32 * km + 8 * (r / 4) + 4 * hh + (r % 4)) * VT + col] = S[km][r];
+      for (int r = 0; r < 16; ++r) S[km][r] = (is_m && 32 * km + acc_row(r, hh) == 32 * wave + ln) ? 1.0f : 0.0f;
+  }
+
+  float dtot = 1.0f;  // product of the chunks' decays over the segment (PASS_A)
+  // The LDS operand reads of a stage are issued as one batch one stage ahead of the MFMAs that use them
+  // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
+  // pays the LDS latency once per MFMA.
+  for (int c = c0; c < c1; ++c) {
+#ifdef DBG_TIMING
+    dbg_on = dbg_seg && (c - c0) >= 4 && (c - c0) < 8; dbg_base = (wave * 8 + (c - c0)) * 16;
+#endif
+    DBG_T(0);
+    lds_barrier();  // A
+    DBG_T(1);
+#ifdef DBG_NO_CHAIN
+    lds_barrier(); lds_barrier(); continue;
+#endif
+    bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), later K^T rows (stage 3)
+    bf16x8 ft[6];              // T (stage 2)
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(s_k, SK, 32 * tm + ln, 16 * ks, hh);
+    bf16x8 Sb[KT / 16];
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+    lds_fence();
+    // batch for stage 2: T fragments and the per-token factors / v tile of stage 1's epilogue
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks) ft[2 * tm + ks] = ld_kappa(s_T, SX, 32 * tm + ln, 16 * ks, hh);
+    f32x4 be[8], ek[8];
+    bf16x4 vv[8];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+      const int i0 = 8 * t8 + 4 * hh;
+      be[t8] = *reinterpret_cast<const f32x4*>(&s_beta[i0]);
+      ek[t8] = *reinterpret_cast<const f32x4*>(&s_ek[i0]);
+      if (is_m) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vv[t8][e] = (__bf16)0.0f;
+      } else {
+        vv[t8] = *reinterpret_cast<const bf16x4*>(&s_vT[col * SX + i0]);
+      }
+    }
+    DBG_T(2);
+    bf16x8 Rb[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {  // R = beta (v - ek (K S))
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], acc);
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc[4 * b4 + e] = be[4 * tm + b4][e] * ((float)vv[4 * tm + b4][e] - ek[4 * tm + b4][e] * acc[4 * b4 + e]);
+      Rb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Rb[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    DBG_T(3);
+    lds_fence();
+    // batch for stage 3: K^T fragments and the decay factors
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa(s_kT, SX, 32 * km + ln, 16 * ks, hh);
+    f32x4 dk[8];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&s_dk[8 * t8 + 4 * hh]);
+    const float dec = s_misc[0];
+    bf16x8 Vb[4], Vsb[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {  // v_new = T R (T is lower triangular: tile tm needs 2 (tm + 1) steps)
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ft[2 * tm + ks], Rb[ks], acc);
+      Vb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Vb[2 * tm + 1] = acc_to_operand(acc, 8);
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[4 * b4 + e] *= dk[4 * tm + b4][e];
+      Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    DBG_T(4);
+    lds_fence();
+    dtot *= dec;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) {  // S <- dec S + K^T (dk v_new)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[km][r] *= dec;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(fk[km * 4 + ks], Vsb[ks], S[km]);
+    }
+    DBG_T(5);
+    lds_barrier();  // B
+    DBG_T(6);
+    if constexpr (PASS_B) {
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+      T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
+      const int rs = HV * VT;
+      // batch: Q rows, P fragments, output factors
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+#pragma unroll
+      for (int f = 0; f < 6; ++f) ft[f] = frag_load(s_P, f, lane);
+      f32x4 qs[8];
+#pragma unroll
+      for (int t8 = 0; t8 < 8; ++t8) qs[t8] = *reinterpret_cast<const f32x4*>(&s_qs[8 * t8 + 4 * hh]);
+      lds_fence();
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm) {  // o = qs (Q S_old) + P v_new
+        f32x16 a1 = zero16(), a2 = zero16();
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], a1);
+#pragma unroll
+        for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(ft[2 * tm + ks], Vb[ks], a2);
+        // The offset is (re)computed here in every iteration on purpose: hoisted out of the loop, the 32 row
+        // addresses would occupy 64 registers, spill, and be reloaded from scratch behind a wait each time.
+        int off = (32 * tm + 4 * hh) * rs + col;
+        asm volatile("" : "+v"(off));
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const int t4 = 32 * tm + 8 * b4 + 4 * hh;
+          if (len == GDR_C) {  // full chunk (uniform branch): no per-row guards
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              ob[off + (8 * b4 + e) * rs] = GdrElem<T>::from_float(qs[4 * tm + b4][e] * a1[4 * b4 + e] + a2[4 * b4 + e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (t4 + e < len)
+                ob[off + (8 * b4 + e) * rs] =
+                    GdrElem<T>::from_float(qs[4 * tm + b4][e] * a1[4 * b4 + e] + a2[4 * b4 + e]);
+          }
+        }
+      }
+    }
+    DBG_T(7);
+    lds_barrier();  // C
+    DBG_T(8);
+  }
+
+  // epilogue; the opaque zero keeps the compiler from computing all these addresses before the loop
+  int late = 0;
+  asm volatile("" : "+v"(late));
+  if constexpr (PASS_B) {
+    if (ht && (flags & SEG_LAST)) {
+      const int seq = plan[plan[PLAN_OFF_SEG_SEQ] + seg];
+      float* out = ht + ((size_t)seq * HV + hv) * KT * VT + late;
+#pragma unroll
+      for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[(32 * km + acc_row(r, hh)) * VT + col] = S[km][r];
+    }
+  } else if (is_m) {
+    // M = dtot I + M': M' as bf16 A-operand fragments (rows = state rows, contraction over the columns in
+    // accumulator slot order), element (row, col) -> fragment (row/32, col/16), lane 32*hh' + row%32, slot s
+    unsigned char* out = Mcomp + ((size_t)seg * HV + hv) * (KT * KT * 2) + late;
+    const int mcol = 32 * wave + ln, ks = mcol >> 4, c16 = mcol & 15;
+    const int hs = (c16 >> 2) & 1, slot = 4 * (c16 >> 3) + (c16 & 3);
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * km + acc_row(r, hh);
+        const float val = S[km][r] - (row == mcol ? dtot : 0.0f);
+        *reinterpret_cast<__bf16*>(out + ((size_t)((km * (KT / 16) + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) =
+            (__bf16)val;
+      }
+    if (wave == 0 && lane == 0) Dcomp[(size_t)seg * HV + hv] = dtot;
+  } else {
+    // N slab in accumulator order: tile (vslab, km), plane q (registers 4q..4q+3), lane -> 16 bytes
+    unsigned char* out = Ncomp + (((size_t)seg * HV + hv) * (VT / 32) + vslab) * (KT * 32 * 4) + late;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
+        reinterpret_cast<f32x4*>(out)[(km * 4 + q4) * 64 + lane] = t;
+      }
+  }
+}
+
+// ---- scan ---------------------------------------------------------------------------------------------------------
+// grid (VT/32, n_seq, HV), 8 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column slab
+// of the state; Sinit [seg, HV, KT, VT] fp32 row-major receives the state every segment starts from.
+// The composite pass stores M_p as d_p I + M'_p (d_p = the segment's total decay, exact in fp32) with M' already
+// in bf16 MFMA A-operand fragment order and N_p in accumulator order, so a step is
+//   S <- d S + N + M' S      (one MFMA per fragment; the state feeds the B operand straight from the accumulator)
+// on ONE wave with no exchange of S. The chain is serial in p, so memory latency must not sit on it: all 8 waves
+// keep their 16-byte pieces of the next DEPTH steps in registers (loads issued DEPTH steps ahead) and copy them
+// into a double-buffered LDS slot one step before wave 0 consumes them.
+template <int KT>
+struct GdrScanShape {
+  static constexpr int THREADS = 512;
+  static constexpr int DEPTH = KT <= 64 ? 8 : 3;          // steps held in registers
+  static constexpr int M_BYTES = KT * KT * 2;             // M' fragments (bf16)
+  static constexpr int N_BYTES = KT * 32 * 4;             // one 32-column slab of N (fp32, accumulator order)
+  static constexpr int MP = M_BYTES / 16 / THREADS;       // 16-byte pieces per thread and step
+  static constexpr int NP = N_BYTES / 16 / THREADS;
+  static constexpr int BYTES = 2 * (M_BYTES + N_BYTES);   // two LDS slots
+};
+
+template <int KT, int VT>
+__global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict__ plan,
+                                                      const unsigned char* __restrict__ Mcomp,
+                                                      const unsigned char* __restrict__ Ncomp,
+                                                      const float* __restrict__ Dcomp,
+                                                      const float* __restrict__ h0, float* __restrict__ Sinit,
+                                                      int HV) {
+  using SH = GdrScanShape<KT>;
+  constexpr int D = SH::DEPTH, MP = SH::MP, NP = SH::NP;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
+  const int nsteps = nseg - 1;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int col = 32 * vn + ln;
+  const bool compute = wave == 0;
+
+  f32x16 S[KT / 32];
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km) {
+    S[km] = zero16();
+    if (compute && h0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[km][r] = h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col];
+    }
+  }
+
+  f32x4 rm[D][MP], rn[D][NP];
+  float rd[D];
+  auto issue = [&](int p, f32x4* m, f32x4* n, float& d) {
+    const size_t sh = (size_t)(seg0 + p) * HV + hv;
+    const f32x4* M = reinterpret_cast<const f32x4*>(Mcomp + sh * SH::M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * SH::N_BYTES);
+#pragma unroll
+    for (int j = 0; j < MP; ++j) m[j] = M[tid + SH::THREADS * j];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) n[j] = N[tid + SH::THREADS * j];
+    d = Dcomp[sh];
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nsteps) issue(d, rm[d], rn[d], rd[d]);
+
+  for (int p0 = 0; p0 <= nsteps; p0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int p = p0 + d;
+      if (p > nsteps) break;
+      if (compute) {  // the state segment seg0 + p starts from
+        float* si = Sinit + ((size_t)(seg0 + p) * HV + hv) * KT * VT;
+#pragma unroll
+        for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) si[(size_t)(32 * km + acc_row(r, hh)) * VT + col] = S[km][r];
+      }
+      if (p == nsteps) break;
+      unsigned char* s_M = smem + (p & 1) * (SH::M_BYTES + SH::N_BYTES);
+      unsigned char* s_N = s_M + SH::M_BYTES;
+#pragma unroll
+      for (int j = 0; j < MP; ++j) reinterpret_cast<f32x4*>(s_M)[tid + SH::THREADS * j] = rm[d][j];
+#pragma unroll
+      for (int j = 0; j < NP; ++j) reinterpret_cast<f32x4*>(s_N)[tid + SH::THREADS * j] = rn[d][j];
+      const float dec = rd[d];
+      if (p + D < nsteps) issue(p + D, rm[d], rn[d], rd[d]);
+      lds_barrier();
+      if (compute) {
+        bf16x8 Sb[KT / 16];
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+        f32x16 Snew[KT / 32];
+#pragma unroll
+        for (int tm = 0; tm < KT / 32; ++tm) {
+          f32x16 acc;
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const f32x4 nv = reinterpret_cast<const f32x4*>(s_N)[(tm * 4 + q4) * 64 + lane];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[tm][4 * q4 + e], nv[e]);
+          }
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(frag_load(s_M, tm * (KT / 16) + ks, lane), Sb[ks], acc);
+          Snew[tm] = acc;
+        }
+#pragma unroll
+        for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
+      }
+    }
   }
 }
 
 // ---- host side ------------------------------------------------------------------------------------------------
 struct GdrWorkspace {
-  int64_t off_records, off_decs, off_m, off_n, off_sinit, bytes;
+  int64_t off_t, off_m, off_n, off_d, off_sinit, bytes;
 };
 
 static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, int V) {
   GdrWorkspace w;
   int64_t off = 0;
-  w.off_records = off; off += lampa_align_up(chunks * HV * gdr_record_bytes(K, V), 256);
-  w.off_decs = off;    off += lampa_align_up(chunks * HV * 4, 256);
-  w.off_m = off;       off += lampa_align_up(segs * HV * (int64_t)K * K * 4, 256);
-  w.off_n = off;       off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
-  w.off_sinit = off;   off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
+  w.off_t = off;     off += lampa_align_up(chunks * HV * (int64_t)T_BYTES, 256);
+  w.off_m = off;     off += lampa_align_up(segs * HV * (int64_t)K * K * 2, 256);
+  w.off_n = off;     off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
+  w.off_d = off;     off += lampa_align_up(segs * HV * 4, 256);
+  w.off_sinit = off; off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.bytes = off > 0 ? off : 256;
   return w;
 }
@@ -822,36 +827,42 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
                             const float* h0, float* ht, const int32_t* plan_dev, int n_seq, int chunks, int segs, int H,
                             int HV, float scale, int l2norm, unsigned char* ws, hipStream_t s) {
   const GdrWorkspace w = gdr_workspace(chunks, segs, HV, KT, VT);
-  unsigned char* records = ws + w.off_records;
-  float* decs = (float*)(ws + w.off_decs);
-  float* Mc = (float*)(ws + w.off_m);
-  float* Nc = (float*)(ws + w.off_n);
+  unsigned char* tf = ws + w.off_t;
+  unsigned char* Mc = ws + w.off_m;
+  unsigned char* Nc = ws + w.off_n;
+  float* Dc = (float*)(ws + w.off_d);
   float* Si = (float*)(ws + w.off_sinit);
-  constexpr int smem = GdrPrepSmem<KT, VT>::BYTES;
+  constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_b = GdrSegSmem<KT, VT, true>::BYTES;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gdr_prep_kernel<T, KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize, smem) !=
-        hipSuccess)
+    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
+        hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess ||
+        hipFuncSetAttribute((const void*)gdr_scan_kernel<KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            GdrScanShape<KT>::BYTES) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
     attr_set = true;
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
-    hipLaunchKernelGGL((gdr_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem, s, (const T*)q, (const T*)k,
-                       (const T*)v, g, beta, plan_dev, records, decs, H, HV, scale, l2norm);
-    LAMPA_PROF(s, "gdr_prep_kernel");
+    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(256), 0, s, (const T*)k, g, beta, plan_dev, tf, H,
+                       HV, l2norm);
+    LAMPA_PROF(s, "gdr_tinv_kernel");
     if (segs > n_seq) {
-      hipLaunchKernelGGL((gdr_composite_kernel<KT, VT>), dim3(segs, HV), dim3(2 * (KT + VT)), 0, s, plan_dev, records,
-                         decs, Mc, Nc, HV);
-      LAMPA_PROF(s, "gdr_composite_kernel");
+      hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
+                         (const T*)q, (const T*)k, (const T*)v, g, beta, plan_dev, tf, (const float*)nullptr, Mc, Nc, Dc,
+                         (T*)nullptr, (float*)nullptr, H, HV, scale, l2norm);
+      LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
-  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(KT * 2), 0, s, plan_dev, Mc, Nc, h0, Si,
-                     HV);
+  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
+                     plan_dev, Mc, Nc, Dc, h0, Si, HV);
   LAMPA_PROF(s, "gdr_scan_kernel");
-  hipLaunchKernelGGL((gdr_output_kernel<T, KT, VT>), dim3(segs, HV), dim3(2 * VT), 0, s, plan_dev, records, decs, Si,
-                     (T*)o, ht, HV);
-  LAMPA_PROF(s, "gdr_output_kernel");
+  hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
+                     (const T*)k, (const T*)v, g, beta, plan_dev, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
+                     (float*)nullptr, (T*)o, ht, H, HV, scale, l2norm);
+  LAMPA_PROF(s, "gdr_segment_kernel<output>");
   return lampa_launch_status();
 }
 
@@ -865,6 +876,7 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
   if (!q || !k || !v || !g || !beta || !o || !plan_host || !plan_dev) return LAMPA_ERR_INVALID;
   if (H < 1 || HV < H || HV % H != 0 || l2norm < 0 || l2norm > 2) return LAMPA_ERR_INVALID;
   if (!gdr_chunk_supported(K, V) || (dtype != GDR_BF16 && dtype != GDR_FP16)) return LAMPA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) return LAMPA_ERR_INVALID;
   const int n_seq = plan_host[PLAN_N_SEQ], chunks = plan_host[PLAN_TOTAL_CHUNKS], segs = plan_host[PLAN_N_SEGMENTS];
   if (n_seq < 1 || segs < n_seq) return LAMPA_ERR_INVALID;
   if (!workspace || workspace_bytes < gdr_workspace(chunks, segs, HV, K, V).bytes) return LAMPA_ERR_WORKSPACE;

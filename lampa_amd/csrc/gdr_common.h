@@ -67,3 +67,13 @@ __device__ __forceinline__ void load8(const T* p, float* out) {
     for (int i = 0; i < 4; ++i) { out[i] = a[i]; out[4 + i] = b[i]; }
   }
 }
+
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every outstanding global load
+// and store of the wave (vmcnt(0)), which would serialise the software prefetch of the next chunk behind each
+// barrier; here only the LDS / scalar counter is drained.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Waits for this wave's outstanding LDS reads and keeps the compiler from moving LDS accesses across this point.
+__device__ __forceinline__ void lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
