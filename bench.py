@@ -23,9 +23,10 @@ N_HITS, N_TABLES, N_PROJ, W_BUCKET, FEAT_DIM = 60000, 3, 4, 0.5, 24
 # algorithmic work per unit
 LAYER_BYTES_PER_TOKEN_HEAD = 2 * K + 2 * K + 2 * V + 2 * V + 8                 # q,k,v,o bf16 + g,beta fp32 = 520
 LAYER_FLOP_PER_TOKEN_HEAD = 2 * 64 * (3 * K + 2 * V) + 6 * K * V + (2 * 64 * 64) // 3  # 68.3 kFLOP
-KERNEL_BYTES_PER_TOKEN_HEAD = {            # the part of the 520 B each kernel of the pipeline is responsible for
-    "gdr_prep_kernel": 2 * K + 2 * K + 2 * V + 8,   # reads q, k, v, g, beta
-    "gdr_output_kernel": 2 * V,                     # writes o
+KERNEL_BYTES_PER_TOKEN_HEAD = {            # algorithmic bytes each kernel of the pipeline has to move
+    "gdr_segment_kernel<output>": LAYER_BYTES_PER_TOKEN_HEAD,    # reads q, k, v, g, beta and writes o: the whole 520 B
+    "gdr_segment_kernel<composite>": 2 * K + 2 * V + 8,           # reads k, v, g, beta
+    "gdr_tinv_kernel": 2 * K + 8,                                 # reads k, g, beta
 }
 LSH_BYTES_PER_HIT_TABLE = 224
 

@@ -31,21 +31,6 @@
 #include "gdr_common.h"
 #include "gdr_plan.h"
 
-#ifndef LB_MIN
-#define LB_MIN 2
-#endif
-#ifndef DBG_TR
-#define DBG_TR
-#endif
-#ifdef DBG_TIMING
-__device__ unsigned long long g_dbg[8192];
-extern "C" int lampa_dbg_read(unsigned long long* host, int n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), sizeof(unsigned long long) * n);
-}
-#define DBG_T(slot) do { if (dbg_on && lane == 0) g_dbg[dbg_base + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define DBG_T(slot) do { } while (0)
-#endif
 #define T_BYTES (64 * 64 * 2)  // T of one chunk and head in HBM: bf16 [64][64] row-major
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
@@ -114,122 +99,150 @@ __device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& s
 }
 
 // ---- T = (I + A)^-1 ------------------------------------------------------------------------------------------
+// One WAVE per (chunk, head), one wave per workgroup: the forward substitution is a single-wave job, so the chunk
+// is not shared with idle helper waves; many small workgroups per CU keep every SIMD busy instead. All LDS
+// traffic is wave-private (no barriers; LDS operations of one wave complete in order).
 template <typename T, int KT>
-__global__ void __launch_bounds__(256) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
-                                                      const float* __restrict__ beta,
-                                                      const int32_t* __restrict__ plan,
-                                                      unsigned char* __restrict__ tmat, int H, int HV,
-                                                      int l2norm) {
-  constexpr int SK = KT + 8, SA = 68, ST = 72;
-  __shared__ __align__(16) __bf16 s_k[64 * SK];
-  __shared__ __align__(16) float s_A[64 * SA];
-  __shared__ __align__(16) __bf16 s_T[64 * ST];
+__global__ void __launch_bounds__(64, 2) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
+                                                     const float* __restrict__ beta,
+                                                     const int32_t* __restrict__ plan,
+                                                     unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
+  constexpr int SK = KT + 8, SB = 36, ST = 72;
+  constexpr int KT_BYTES = 64 * SK * 2, TT_BYTES = 64 * ST * 2;
+  __shared__ __align__(16) unsigned char s_kt[KT_BYTES > TT_BYTES ? KT_BYTES : TT_BYTES];  // k tile, later T
+  __shared__ __align__(16) float s_A11[32 * SB], s_A21[32 * SB], s_A22[32 * SB];           // blocks of A, later of T
   __shared__ float s_gamma[64], s_beta[64], s_rk[64];
+  __bf16* s_k = reinterpret_cast<__bf16*>(s_kt);
+  __bf16* s_T = reinterpret_cast<__bf16*>(s_kt);
 
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
   const int tok0 = plan[plan[PLAN_OFF_CHUNK_TOK0] + chunk];
   const int len = plan[plan[PLAN_OFF_CHUNK_LEN] + chunk];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
 
-  if (wave == 0) {  // rows past the end of a partial chunk behave as g = 0, beta = 0, k = 0
-    float gv = lane < len ? g[(size_t)(tok0 + lane) * HV + hv] : 0.0f;
+  {  // rows past the end of a partial chunk behave as g = 0, beta = 0, k = 0
+    const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
+    float gv = g[gi], bv = beta[gi];
+    gv = lane < len ? gv : 0.0f;
+    bv = lane < len ? bv : 0.0f;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       const float up = __shfl_up(gv, off);
       if (lane >= off) gv += up;
     }
     s_gamma[lane] = gv;
-    s_beta[lane] = lane < len ? beta[(size_t)(tok0 + lane) * HV + hv] : 0.0f;
+    s_beta[lane] = bv;
   }
-  {
-    const int row = tid >> 2, part = tid & 3;
+  {  // k tile -> LDS (bf16, row-major), row norms; 4 lanes share a row, 16 rows per pass
+    const int part = lane & 3;
     constexpr int EPT = KT / 4;
-    float ss = 0.0f;
-    const T* kp = k + ((size_t)(tok0 + (row < len ? row : 0)) * H + h) * KT + part * EPT;
+    typename Raw8<T>::type raw[4][EPT / 8];
 #pragma unroll
-    for (int c = 0; c < EPT / 8; ++c) {
-      typename Raw8<T>::type raw;
+    for (int ps = 0; ps < 4; ++ps) {
+      const int row = 16 * ps + (lane >> 2);
+      const T* kp = k + ((size_t)(tok0 + min(row, len - 1)) * H + h) * KT + part * EPT;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) raw[e] = (T)0.0f;
-      if (row < len) raw = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * c);
-      *reinterpret_cast<bf16x8*>(&s_k[row * SK + part * EPT + 8 * c]) = raw_to_bf16<T>(raw, ss, l2norm != GDR_L2_NONE);
+      for (int c = 0; c < EPT / 8; ++c) raw[ps][c] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * c);
     }
-    ss += __shfl_xor(ss, 1);
-    ss += __shfl_xor(ss, 2);
-    if (part == 0) s_rk[row] = l2_factor(ss, l2norm);
-  }
-  __syncthreads();
-
-  {  // A -> LDS fp32; one 32x32 tile per wave, the tile above the diagonal is never read
-    const int tm = wave >> 1, tn = wave & 1;
-    if (!(tm == 0 && tn == 1)) {
-      f32x16 acc = zero16();
+    typename Raw8<T>::type zero;
 #pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tm + ln) * SK + 16 * ks + 8 * hh]);
-        const bf16x8 b = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
-        acc = mfma32(a, b, acc);
-      }
-      const int j = 32 * tn + ln;
-      const float gj = s_gamma[j], rj = s_rk[j];
+    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 32 * tm + acc_row(r, hh);
-        s_A[i * SA + j] = i > j ? acc[r] * s_beta[i] * s_rk[i] * rj * __expf(s_gamma[i] - gj) : 0.0f;
-      }
+    for (int ps = 0; ps < 4; ++ps) {
+      const int row = 16 * ps + (lane >> 2);
+      float ss = 0.0f;
+#pragma unroll
+      for (int c = 0; c < EPT / 8; ++c)
+        *reinterpret_cast<bf16x8*>(&s_k[row * SK + part * EPT + 8 * c]) =
+            raw_to_bf16<T>(row < len ? raw[ps][c] : zero, ss, l2norm != GDR_L2_NONE);
+      ss += __shfl_xor(ss, 1);
+      ss += __shfl_xor(ss, 2);
+      if (part == 0) s_rk[row] = l2_factor(ss, l2norm);
     }
   }
-  __syncthreads();
+  lds_fence();
 
-  if (wave == 0) {
-    // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
-    // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
-    // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+  // A = strict_lower(beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j}) -> three 32x32 fp32 blocks in LDS
+#pragma unroll
+  for (int t = 0; t < 3; ++t) {
+    const int tm = t == 0 ? 0 : 1, tn = t == 2 ? 1 : 0;  // (0,0), (1,0), (1,1)
+    float* blk = t == 0 ? s_A11 : (t == 1 ? s_A21 : s_A22);
+    bf16x8 fa[KT / 16], fb[KT / 16];
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) {
+      fa[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tm + ln) * SK + 16 * ks + 8 * hh]);
+      fb[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
+    }
+    f32x4 gi4[4], bi4[4], ri4[4];
+#pragma unroll
+    for (int b4 = 0; b4 < 4; ++b4) {
+      gi4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tm + 8 * b4 + 4 * hh]);
+      bi4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tm + 8 * b4 + 4 * hh]);
+      ri4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tm + 8 * b4 + 4 * hh]);
+    }
+    const int j = 32 * tn + ln;
+    const float gj = s_gamma[j], rj = s_rk[j];
+    lds_fence();
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int il = acc_row(r, hh), i = 32 * tm + il;
+      blk[il * SB + ln] = i > j ? acc[r] * bi4[r / 4][r % 4] * ri4[r / 4][r % 4] * rj * __expf(gi4[r / 4][r % 4] - gj) : 0.0f;
+    }
+  }
+  lds_fence();
+
+  // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
+  // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
+  // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+  {
     const int b = hh, c = ln;
-    const float* Ab = s_A + (32 * b) * SA + 32 * b;
+    float* Ab = b == 0 ? s_A11 : s_A22;
     float x[32];
-    f32x4 rowbuf[2][8];  // rows i and i+1 of the block, so that the next row loads while this one is reduced
-    rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SA);
+    f32x4 rowbuf[4][8];  // a ring of rows: row i+3 loads while row i is reduced (hides the LDS latency)
+    rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SB);
+    rowbuf[2][0] = *reinterpret_cast<const f32x4*>(Ab + 2 * SB);
+    rowbuf[3][0] = *reinterpret_cast<const f32x4*>(Ab + 3 * SB);
     x[0] = (c == 0) ? 1.0f : 0.0f;
 #pragma unroll
     for (int i = 1; i < 32; ++i) {
-      if (i + 1 < 32) {
-#pragma unroll
-        for (int q = 0; q < (i + 1 + 3) / 4; ++q)
-          rowbuf[(i + 1) & 1][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 1) * SA + 4 * q);
-      }
       float acc0 = (i == c) ? 1.0f : 0.0f, acc1 = 0.0f;
 #pragma unroll
       for (int j = 0; j < i; ++j) {
-        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc1);
-        else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
+        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 3][j / 4][j % 4], x[j], acc1);
+        else acc0 = __builtin_fmaf(-rowbuf[i & 3][j / 4][j % 4], x[j], acc0);
       }
       x[i] = acc0 + acc1;
-      // pins the order "loads of row i+1, arithmetic of row i": without it the compiler either serialises every
+      // pins the order "arithmetic of row i, loads of row i+3": without it the compiler either serialises every
       // load behind a wait or hoists all 124 loads to the top and spills
       asm volatile("" : "+v"(x[i]) : : "memory");
+      if (i + 3 < 32) {
+#pragma unroll
+        for (int q = 0; q < (i + 3 + 3) / 4; ++q)
+          rowbuf[(i + 3) & 3][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 3) * SB + 4 * q);
+      }
     }
-    __builtin_amdgcn_wave_barrier();
+    lds_fence();  // every lane is done reading A11 / A22 (and the k tile) before they are overwritten
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      s_A[(32 * b + i) * SA + lane] = x[i];  // fp32 diagonal blocks in place of A11 / A22 (operands of the merge)
+      Ab[i * SB + c] = x[i];  // fp32 diagonal blocks in place of A11 / A22 (operands of the merge)
       s_T[(32 * b + i) * ST + lane] = (__bf16)x[i];
       if (b == 1) s_T[i * ST + lane] = (__bf16)0.0f;
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    lds_fence();
     f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11
       bf16x8 ahi, alo, bhi, blo;
-      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 16 * ks + 8 * hh]);
-      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 16 * ks + 8 * hh + 4]);
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A21[ln * SB + 16 * ks + 8 * hh]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A21[ln * SB + 16 * ks + 8 * hh + 4]);
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
         const float av = q < 4 ? a0[q % 4] : a1[q % 4];
-        const float bv = s_A[(16 * ks + 8 * hh + q) * SA + ln];
+        const float bv = s_A11[(16 * ks + 8 * hh + q) * SB + ln];
         const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
         ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
         bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
@@ -244,8 +257,8 @@ __global__ void __launch_bounds__(256) gdr_tinv_kernel(const T* __restrict__ k, 
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
       bf16x8 ahi, alo, bhi, blo;
-      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 32 + 16 * ks + 4 * hh]);
-      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A[(32 + ln) * SA + 32 + 16 * ks + 8 + 4 * hh]);
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
         const float av = q < 4 ? a0[q % 4] : a1[q % 4];
@@ -261,16 +274,20 @@ __global__ void __launch_bounds__(256) gdr_tinv_kernel(const T* __restrict__ k, 
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_T[(32 + acc_row(r, hh)) * ST + ln] = (__bf16)(-(t0[r] + (t1[r] + t2[r])));
   }
-  __syncthreads();
+  lds_fence();
 
   // T row-major bf16 [64][64] (the upper-right 32x32 block is zero)
   {
     __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * T_BYTES);
-    const int row = tid >> 2, part = tid & 3;
+    const int part = lane & 3;
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
-      *reinterpret_cast<bf16x8*>(out + row * 64 + part * 16 + 8 * c) =
-          *reinterpret_cast<const bf16x8*>(&s_T[row * ST + part * 16 + 8 * c]);
+    for (int ps = 0; ps < 4; ++ps) {
+      const int row = 16 * ps + (lane >> 2);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        *reinterpret_cast<bf16x8*>(out + row * 64 + part * 16 + 8 * c) =
+            *reinterpret_cast<const bf16x8*>(&s_T[row * ST + part * 16 + 8 * c]);
+    }
   }
 }
 
@@ -302,7 +319,7 @@ struct GdrSegShape {
 };
 
 template <typename T, int KT, int VT, bool PASS_B>
-__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_MIN)
+__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta,
                        const int32_t* __restrict__ plan, const unsigned char* __restrict__ tmat,
@@ -337,10 +354,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
   const int* chunk_len = plan + plan[PLAN_OFF_CHUNK_LEN];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
 
-#ifdef DBG_TIMING
-  const bool dbg_seg = PASS_B && seg == 5 && hv == 0;
-  bool dbg_on = false; int dbg_base = 0;
-#endif
   if (wave >= NSLAB) {
     // ================================================ stager ================================================
     constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
@@ -378,10 +391,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
     if (nc > 0) issue_loads(c0);
     for (int c = c0; c < c1; ++c) {
       const int len = chunk_len[c];
-#ifdef DBG_TIMING
-      dbg_on = dbg_seg && (c - c0) >= 4 && (c - c0) < 8; dbg_base = (wave * 8 + (c - c0)) * 16;
-#endif
-      DBG_T(0);
       // ---- stage chunk c ----
       float gv = lane < len ? rg : 0.0f;  // inclusive scan of the log-decay over the chunk
       const float bv = lane < len ? rb : 0.0f;
@@ -435,9 +444,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
         s_rq[srow] = rq;
         if (srow == 0) s_misc[0] = __expf(g_last);
       }
-      DBG_T(1);
       lds_barrier();  // A1: tiles and factors of chunk c are in LDS
-      DBG_T(2);
       if (c + 1 < c1) issue_loads(c + 1);
       if constexpr (PASS_B) {
         for (int t = sw; t < 3; t += 2) {  // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero
@@ -470,11 +477,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
           frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
         }
       }
-      DBG_T(3);
       lds_barrier();  // B: P fragments are in LDS
-      DBG_T(4);
       lds_barrier();  // C: the chain waves are done with chunk c's tiles
-      DBG_T(5);
     }
     return;
   }
@@ -504,15 +508,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
   // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
   // pays the LDS latency once per MFMA.
   for (int c = c0; c < c1; ++c) {
-#ifdef DBG_TIMING
-    dbg_on = dbg_seg && (c - c0) >= 4 && (c - c0) < 8; dbg_base = (wave * 8 + (c - c0)) * 16;
-#endif
-    DBG_T(0);
     lds_barrier();  // A
-    DBG_T(1);
-#ifdef DBG_NO_CHAIN
-    lds_barrier(); lds_barrier(); continue;
-#endif
     bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), later K^T rows (stage 3)
     bf16x8 ft[6];              // T (stage 2)
 #pragma unroll
@@ -542,7 +538,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
         vv[t8] = *reinterpret_cast<const bf16x4*>(&s_vT[col * SX + i0]);
       }
     }
-    DBG_T(2);
     bf16x8 Rb[4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {  // R = beta (v - ek (K S))
@@ -557,7 +552,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
       Rb[2 * tm + 0] = acc_to_operand(acc, 0);
       Rb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
-    DBG_T(3);
     lds_fence();
     // batch for stage 3: K^T fragments and the decay factors
 #pragma unroll
@@ -583,7 +577,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
       Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
       Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
-    DBG_T(4);
     lds_fence();
     dtot *= dec;
 #pragma unroll
@@ -593,9 +586,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(fk[km * 4 + ks], Vsb[ks], S[km]);
     }
-    DBG_T(5);
     lds_barrier();  // B
-    DBG_T(6);
     if constexpr (PASS_B) {
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
@@ -639,9 +630,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), LB_
         }
       }
     }
-    DBG_T(7);
     lds_barrier();  // C
-    DBG_T(8);
   }
 
   // epilogue; the opaque zero keeps the compiler from computing all these addresses before the loop
@@ -846,7 +835,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
-    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(256), 0, s, (const T*)k, g, beta, plan_dev, tf, H,
+    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, plan_dev, tf, H,
                        HV, l2norm);
     LAMPA_PROF(s, "gdr_tinv_kernel");
     if (segs > n_seq) {
