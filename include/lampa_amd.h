@@ -68,6 +68,16 @@ int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, 
                           const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
                           int32_t* meta_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The whole bucketing stage of one event in one call: lampa_lsh_bucket_keys, then lampa_sort_pairs on the packed
+ * keys (digit widths from meta, read on the device), then lampa_gather_rows of the hit features when feats != NULL.
+ * Replaces the hash -> argsort -> sort_to_buckets sequence of models/attention/hept.py:127-143.
+ * perm_out [n_tables, n_hits] int32; feats [n_hits, feat_row_bytes] -> feats_out [n_tables, n_hits, feat_row_bytes]. */
+int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj);
+int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_t n_valid, int dim, const float* alpha,
+                          const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
+                          int32_t* meta_out, int32_t* perm_out, const void* feats, int64_t feat_row_bytes,
+                          void* feats_out, int n_passes, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Sort keys of LSHOrdering: key[n] = sum_h 2^h <coords[n], alpha[:, h]>, norm[n] = |coords[n]|.
  * Replaces models/baselines/full_mamba2.py:174-203. coords [n_hits, dim], alpha [dim, n_hashes]. */
 int lampa_lsh_ordering_keys(const float* coords, int64_t n_hits, int dim, const float* alpha, int n_hashes,

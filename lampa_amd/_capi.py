@@ -23,6 +23,9 @@ _vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_
 _SIGNATURES = {
     "lampa_lsh_bucket_workspace_bytes": (_i64, [_i64, _i32, _i32]),
     "lampa_lsh_bucket_keys": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "lampa_lsh_bucket_sort_workspace_bytes": (_i64, [_i64, _i32, _i32]),
+    "lampa_lsh_bucket_sort": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp, _vp, _i64,
+                                     _vp, _i32, _vp, _i64, _vp]),
     "lampa_lsh_project_f32": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "lampa_lsh_ordering_keys": (_i32, [_vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp]),
     "lampa_row_minmax_f32": (_i32, [_vp, _i32, _i64, _vp, _vp]),

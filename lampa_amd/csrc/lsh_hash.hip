@@ -8,46 +8,7 @@
 // Replaces (reference chengjiang123/Lampa): E2LSH.forward  models/model_utils/hash_utils.py:368-371,
 // the hash range of lsh_mapping  hash_utils.py:334-340, the mixed-radix key idiom of get_geo_shift
 // models/attention/hept.py:79-88, and the key/norm of LSHOrdering  models/baselines/full_mamba2.py:181-203.
-#include "common.h"
-
-#define LSH_MAX_DIM 8
-#define LSH_MAX_COLS 64
-#define LSH_MAX_PROJ 8
-#define LSH_BLOCK 256
-
-__device__ __forceinline__ int32_t lsh_quantise(float p, float b, float inv_w) {
-  float t = (p + b) * inv_w;
-  if (t != t) return INT32_MAX;
-  float f = floorf(t);
-  if (f >= 2147483648.0f) return INT32_MAX;
-  if (f <= -2147483648.0f) return INT32_MIN;
-  return (int32_t)f;
-}
-
-template <int DIM>
-__device__ __forceinline__ void lsh_load_coords(const float* __restrict__ coords, int64_t n, int dim, float* x) {
-  if (DIM == 4) {
-    float4 c = *reinterpret_cast<const float4*>(coords + n * 4);
-    x[0] = c.x; x[1] = c.y; x[2] = c.z; x[3] = c.w;
-  } else {
-#pragma unroll
-    for (int d = 0; d < LSH_MAX_DIM; ++d) x[d] = d < dim ? coords[n * dim + d] : 0.0f;
-  }
-}
-
-template <int DIM>
-__device__ __forceinline__ float lsh_dot(const float* x, const float* __restrict__ alpha, int dim, int n_cols, int c) {
-  float acc = 0.0f;
-  if (DIM == 4) {
-#pragma unroll
-    for (int d = 0; d < 4; ++d) acc = __builtin_fmaf(x[d], alpha[d * n_cols + c], acc);
-  } else {
-#pragma unroll
-    for (int d = 0; d < LSH_MAX_DIM; ++d)
-      if (d < dim) acc = __builtin_fmaf(x[d], alpha[d * n_cols + c], acc);
-  }
-  return acc;
-}
+#include "lsh_device.h"
 
 // ---- pass 1: per-block min / max of every id column over the valid hits -------------------------------
 // partial [gridDim.x, n_cols, 2] (min, max); no atomics, no initialisation needed.
@@ -308,4 +269,44 @@ extern "C" int lampa_row_minmax_f32(const float* x, int rows, int64_t n, float* 
   if (!x || !out || rows < 1 || n < 1) return LAMPA_ERR_INVALID;
   hipLaunchKernelGGL(lsh_row_minmax_kernel, dim3(rows), dim3(LSH_BLOCK), 0, (hipStream_t)stream, x, n, out);
   return lampa_launch_status();
+}
+
+// ---- whole bucketing stage of one event in one call ---------------------------------------------------------------
+extern "C" int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n);
+extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
+                                int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
+                                int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream);
+extern "C" int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
+                                 int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
+
+extern "C" int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj) {
+  const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
+  const int64_t b = lampa_sort_workspace_bytes(n_tables, n_hits);
+  if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
+  return a + b;
+}
+
+// ids + keys + meta (lampa_lsh_bucket_keys), stable sort permutation of every table (lampa_sort_pairs on the packed
+// keys, digit width taken from meta on the device) and, when feats is given, the hit features in sorted order
+// (lampa_gather_rows): perm_out [n_tables, n_hits] int32, feats_out [n_tables, n_hits, feat_row_bytes].
+extern "C" int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_t n_valid, int dim, const float* alpha,
+                                     const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out,
+                                     int32_t* keys_out, int32_t* meta_out, int32_t* perm_out, const void* feats,
+                                     int64_t feat_row_bytes, void* feats_out, int n_passes, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+  if (!perm_out || (feats && (!feats_out || feat_row_bytes < 1))) return LAMPA_ERR_INVALID;
+  const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
+  const int64_t b = lampa_sort_workspace_bytes(n_tables, n_hits);
+  if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
+  if (!workspace || workspace_bytes < a + b) return LAMPA_ERR_WORKSPACE;
+  int rc = lampa_lsh_bucket_keys(coords, n_hits, n_valid, dim, alpha, beta, n_tables, n_proj, w, ids_out, keys_out,
+                                 meta_out, workspace, a, stream);
+  if (rc != LAMPA_OK) return rc;
+  const int stride = 2 * n_proj + 3;
+  rc = lampa_sort_pairs(keys_out, /*KEY_U32*/ 0, nullptr, n_tables, n_hits, 32, meta_out + 2 * n_proj + 1, stride,
+                        n_passes, perm_out, (char*)workspace + a, b, stream);
+  if (rc != LAMPA_OK) return rc;
+  if (feats)
+    rc = lampa_gather_rows(feats, 1, n_hits, perm_out, 4, n_tables, n_hits, feat_row_bytes, feats_out, stream);
+  return rc;
 }

@@ -264,14 +264,34 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
 
 def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[torch.Tensor] = None,
                     n_valid: Optional[int] = None, return_ids: bool = True, n_passes: int = 0):
-    """E2LSH bucketing of one event: bucket ids -> packed keys -> stable sort permutation per table ->
-    (optionally) the hit features in sorted order. Returns a dict with ids, keys, meta, perm [T, N] int32 and
-    feats [T, N, D]. No host synchronisation: the sort reads the number of key bits from ``meta`` on the device."""
-    ids, keys, meta = lsh_bucket_keys(coords, alpha, beta, w, n_tables, n_proj, n_valid, return_ids)
-    stride = 2 * n_proj + 3
-    bits_dev = meta.view(-1)[2 * n_proj + 1:]
-    perm = stable_argsort(keys, key_bits_dev=bits_dev, key_bits_stride=stride, n_passes=n_passes, unsigned=True)
+    """E2LSH bucketing of one event in one library call: bucket ids -> packed keys -> stable sort permutation per
+    table -> (optionally) the hit features in sorted order. Returns a dict with ids, keys, meta, perm [T, N] int32
+    and feats [T, N, D]. No host synchronisation: the sort reads the number of key bits from ``meta`` on the device."""
+    require_cuda(coords, alpha, beta, feats)
+    coords = coords.contiguous().float()
+    alpha = alpha.contiguous().float()
+    beta = beta.contiguous().float().reshape(-1)
+    n, dim = coords.shape
+    assert alpha.shape == (dim, n_tables * n_proj) and beta.numel() == n_tables * n_proj
+    n_valid = n if n_valid is None else int(n_valid)
+    dev = coords.device
+    ids = torch.empty((n_tables * n_proj, n), dtype=torch.int32, device=dev) if return_ids else None
+    keys = torch.empty((n_tables, n), dtype=torch.int32, device=dev)
+    meta = torch.empty((n_tables, 2 * n_proj + 3), dtype=torch.int32, device=dev)
+    perm = torch.empty((n_tables, n), dtype=torch.int32, device=dev)
     out = {"ids": ids, "keys": keys, "meta": meta, "perm": perm}
+    fo, row_bytes = None, 0
     if feats is not None:
-        out["feats"] = gather_rows(feats, perm)
+        feats = feats.contiguous()
+        assert feats.dim() == 2 and feats.shape[0] == n
+        fo = torch.empty((n_tables, n, feats.shape[1]), dtype=feats.dtype, device=dev)
+        row_bytes = feats.shape[1] * feats.element_size()
+        out["feats"] = fo
+    if n == 0:
+        return out
+    lib = _capi.lib()
+    ws = _workspace(check(lib.lampa_lsh_bucket_sort_workspace_bytes(n, n_tables, n_proj), "workspace"), dev)
+    check(lib.lampa_lsh_bucket_sort(ptr(coords), n, n_valid, dim, ptr(alpha), ptr(beta), n_tables, n_proj, float(w),
+                                    ptr(ids), ptr(keys), ptr(meta), ptr(perm), ptr(feats), row_bytes, ptr(fo), n_passes,
+                                    ptr(ws), ws.numel(), stream_of(coords)), "lampa_lsh_bucket_sort")
     return out
