@@ -76,7 +76,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=T,
+                    help="tokens of the workload the CPU baseline is timed on (default: all of them, about 5-10 s)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (for profiler runs)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="first run one plain device copy of 256 MiB, the known-size kernel that scales a counter run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
@@ -93,6 +97,14 @@ def main():
         lib_build.build()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # 256 MiB read + 256 MiB written by one elementwise copy kernel
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- inputs (synthetic, seeded) ----
     coords, feats, _ = synth.collider_event(N_HITS, seed=0)
@@ -174,14 +186,17 @@ def main():
     }
 
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
-    cores = torch.get_num_threads()
-    cpu_hits_per_s, cpu_dt = cpu_baseline_gdr(q, k, v, g, beta, args.cpu_sample_tokens)
-    lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha)
-    lsh_info["cpu_baseline_us"] = round(lsh_cpu_s * 1e6, 1)
-    cpu = {"value": round(cpu_hits_per_s, 1), "unit": "hits/s", "cores": cores, "kind": "port",
-           "sample": f"first {args.cpu_sample_tokens} of {T} tokens, all {H} heads, fp32 token loop in PyTorch "
-                     f"({cpu_dt:.2f} s), scaled linearly",
-           "cpu_count": os.cpu_count()}
+    cpu = None
+    if not args.no_cpu:
+        cores = torch.get_num_threads()
+        n_cpu = min(T, max(64, args.cpu_sample_tokens))
+        cpu_hits_per_s, cpu_dt = cpu_baseline_gdr(q, k, v, g, beta, n_cpu)
+        lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha)
+        lsh_info["cpu_baseline_us"] = round(lsh_cpu_s * 1e6, 1)
+        cpu = {"value": round(cpu_hits_per_s, 1), "unit": "hits/s", "cores": cores, "kind": "port",
+               "sample": f"first {n_cpu} of {T} tokens, all {H} heads, fp32 token loop in PyTorch ({cpu_dt:.2f} s)"
+                         + ("" if n_cpu == T else ", scaled linearly"),
+               "cpu_count": os.cpu_count()}
 
     out = {
         "metric": "hits/s per gated-delta layer at T=60k (bf16); % HBM and MFMA roofline",

@@ -293,21 +293,29 @@ __global__ void __launch_bounds__(64, 2) gdr_tinv_kernel(const T* __restrict__ k
 
 // ---- segment kernel --------------------------------------------------------------------------------------------
 // Workgroup per (segment, head). Waves 0 .. SLABS-1 ("chain" waves) each own 32 columns of the state and run the
-// recurrence; the last two waves ("stagers") load the next chunk's tiles from HBM, stage them in LDS, derive the
-// per-token factors and (PASS_B) build the P fragments. The two roles run separate loops that meet at three
-// LDS-only barriers per chunk, so that the stagers' global loads stay in flight while the chain waves compute and
-// neither role pays for the other's registers.
+// recurrence; the last two waves ("stagers") load the coming chunks' tiles from HBM, stage them ROW-MAJOR in LDS
+// (16-byte writes only), derive the per-token factors and (PASS_B) build the P fragments. Operands that contract
+// over the tokens (K^T, and v in accumulator layout) are read from the row-major tiles with the transposing LDS
+// load (ds_read_b64_tr_b16), so no transposed copy is ever written.
+//
+// LDS is single-buffered but released early. Per chunk c the two roles meet at three LDS-only barriers:
+//   A(c)  k, v, T, factors and (PASS_B) q of chunk c are staged
+//   X(c)  the chain waves hold every k / v / T operand of chunk c in registers (and P(c) is in LDS)
+//         -> the stagers overwrite the tiles with chunk c+1 while the chain waves finish chunk c
+//   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c -> the stagers write q(c+1)
+// Global loads are issued one full chunk period before their data is staged.
 template <int KT, int VT, bool PASS_B>
 struct GdrSegSmem {
-  static constexpr int SK = KT + 8;  // row stride of the row-major k / q tiles (bf16 elements)
-  static constexpr int SX = 72;      // row stride of the transposed [dim][token] tiles and of T
+  static constexpr int SK = KT + 8;  // row stride of the k / q tiles (bf16 elements)
+  static constexpr int SV = VT + 8;  // row stride of the v and o tiles
+  static constexpr int ST = 72;      // row stride of T
   static constexpr int OFF_K = 0;
-  static constexpr int OFF_KT = OFF_K + 64 * SK * 2;
-  static constexpr int OFF_VT = OFF_KT + KT * SX * 2;
-  static constexpr int OFF_T = OFF_VT + VT * SX * 2;
-  static constexpr int OFF_Q = OFF_T + 64 * SX * 2;
+  static constexpr int OFF_V = OFF_K + 64 * SK * 2;
+  static constexpr int OFF_T = OFF_V + 64 * SV * 2;
+  static constexpr int OFF_Q = OFF_T + 64 * ST * 2;
   static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
-  static constexpr int OFF_SCAL = OFF_P + (PASS_B ? 6 * 1024 : 0);
+  static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
+  static constexpr int OFF_SCAL = OFF_O + (PASS_B ? 64 * SV * 2 : 0);
   static constexpr int N_SCAL = 8;  // beta, ek, dk, qs, gamma, rk, rq, misc
   static constexpr int BYTES = OFF_SCAL + N_SCAL * 64 * 4;
 };
@@ -318,23 +326,50 @@ struct GdrSegShape {
   static constexpr int WAVES = SLABS + 2;                          // + two stager waves
 };
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: lane i of every block of 16 lanes receives element (i % 4) of the four 8-byte rows that
+// lanes i/4, i/4 + 4, i/4 + 8 and i/4 + 12 of its block point at.
+__device__ __forceinline__ bf16x4 lds_read_tr4(const __bf16* p) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p));
+}
+
+// Four consecutive rows row0 + 4hh .. +3 of column col0 + (lane % 32) of a row-major bf16 tile: lane L of a block
+// points at row L / 4, column group L % 4 of the block's 16 columns.
+__device__ __forceinline__ bf16x4 ld_col4(const __bf16* arr, int stride, int col0, int row0, int lane) {
+  const int L = lane & 15, blk = (lane >> 4) & 1, hh = lane >> 5;
+  return lds_read_tr4(arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * (L & 3));
+}
+
+// A-operand fragment of the TRANSPOSE of a row-major tile: operand row = tile column col0 + (lane % 32),
+// contraction over the tile rows row0 .. row0 + 15 in accumulator slot order.
+__device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int col0, int row0, int lane) {
+  const bf16x4 lo = ld_col4(arr, stride, col0, row0, lane), hi = ld_col4(arr, stride, col0, row0 + 8, lane);
+  bf16x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
 template <typename T, int KT, int VT, bool PASS_B>
 __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta,
                        const int32_t* __restrict__ plan, const unsigned char* __restrict__ tmat,
                        const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
-                       unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o, float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
+                       unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o,
+                       float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
   using SM = GdrSegSmem<KT, VT, PASS_B>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
-  constexpr int SK = SM::SK, SX = SM::SX;
+  constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
   extern __shared__ __align__(16) unsigned char smem[];
   __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
-  __bf16* s_kT = reinterpret_cast<__bf16*>(smem + SM::OFF_KT);
-  __bf16* s_vT = reinterpret_cast<__bf16*>(smem + SM::OFF_VT);
+  __bf16* s_v = reinterpret_cast<__bf16*>(smem + SM::OFF_V);
   __bf16* s_T = reinterpret_cast<__bf16*>(smem + SM::OFF_T);
   __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
   unsigned char* s_P = smem + SM::OFF_P;
+  T* s_o = reinterpret_cast<T*>(smem + SM::OFF_O);
   float* s_beta = reinterpret_cast<float*>(smem + SM::OFF_SCAL);
   float* s_ek = s_beta + 64;     // e^{gamma_i} rk_i
   float* s_dk = s_beta + 128;    // e^{gamma_last - gamma_i} rk_i
@@ -362,9 +397,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     typename Raw8<T>::type rk_[KU], rv_[VU], rq_[PASS_B ? KU : 1];
     bf16x8 rt_[4];
     float rg = 0.0f, rb = 0.0f;
+    float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
-    auto issue_loads = [&](int c) {
+    auto issue_tiles = [&](int c) {
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* kb = k + ((size_t)tok0 * H + h) * KT;
       const T* vb = v + ((size_t)tok0 * HV + hv) * VT;
@@ -374,11 +410,6 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
 #pragma unroll
       for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
-      if constexpr (PASS_B) {
-        const T* qb = q + ((size_t)tok0 * H + h) * KT;
-#pragma unroll
-        for (int u = 0; u < KU; ++u) rq_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(qb + koff + 8 * u);
-      }
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * T_BYTES);
 #pragma unroll
       for (int j = 0; j < 4; ++j) rt_[j] = tp[stid + 128 * j];
@@ -388,64 +419,81 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       rg = gb[gl];
       rb = bb[gl];
     };
-    if (nc > 0) issue_loads(c0);
-    for (int c = c0; c < c1; ++c) {
-      const int len = chunk_len[c];
-      // ---- stage chunk c ----
-      float gv = lane < len ? rg : 0.0f;  // inclusive scan of the log-decay over the chunk
-      const float bv = lane < len ? rb : 0.0f;
+    auto issue_q = [&](int c) {
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+      const T* qb = q + ((size_t)tok0 * H + h) * KT;
+      const int koff = min(srow, len - 1) * H * KT + spart * (KT / 2);
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const float up = __shfl_up(gv, off);
-        if (lane >= off) gv += up;
-      }
-      const float g_last = __shfl(gv, 63);
-      const bool live = srow < len, want_ss = l2norm != GDR_L2_NONE;
-      float kss = 0.0f, qss = 0.0f;
+      for (int u = 0; u < KU; ++u) rq_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(qb + koff + 8 * u);
+    };
+    typename Raw8<T>::type zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+    const bool want_ss = l2norm != GDR_L2_NONE;
+
+    auto stage_tiles = [&](int c) {
+      const int len = chunk_len[c];
+      const float bv = lane < len ? rb : 0.0f;
+      const float gv = wave_inclusive_scan(lane < len ? rg : 0.0f);  // in-chunk cumulative log-decay, lane = token
+      const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
+      const bool live = srow < len;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int piece = stid + 128 * j;  // row piece / 8, columns 8 * (piece % 8) ..
-        *reinterpret_cast<bf16x8*>(&s_T[(piece >> 3) * SX + 8 * (piece & 7)]) = rt_[j];
+        *reinterpret_cast<bf16x8*>(&s_T[(piece >> 3) * ST + 8 * (piece & 7)]) = rt_[j];
       }
-      typename Raw8<T>::type zero;
+      float kss = 0.0f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
-#pragma unroll
-      for (int u = 0; u < KU; ++u) {
-        const bf16x8 kb8 = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
-        const int e0 = spart * (KT / 2) + 8 * u;
-        *reinterpret_cast<bf16x8*>(&s_k[srow * SK + e0]) = kb8;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_kT[(e0 + e) * SX + srow] = kb8[e];
-        if constexpr (PASS_B)
-          *reinterpret_cast<bf16x8*>(&s_q[srow * SK + e0]) = raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
-      }
+      for (int u = 0; u < KU; ++u)
+        *reinterpret_cast<bf16x8*>(&s_k[srow * SK + spart * (KT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         float unused = 0.0f;
-        const bf16x8 vb8 = raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
-        const int e0 = spart * (VT / 2) + 8 * u;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_vT[(e0 + e) * SX + srow] = vb8[e];
+        *reinterpret_cast<bf16x8*>(&s_v[srow * SV + spart * (VT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
       }
-      kss += __shfl_xor(kss, 1);
-      qss += __shfl_xor(qss, 1);
+      kss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
       // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
-      const float grow = __shfl(gv, srow), brow = __shfl(bv, srow);
+      grow = __shfl(gv, srow);
+      const float brow = __shfl(bv, srow);
       if (spart == 0) {
-        const float rk = l2_factor(kss, l2norm), rq = l2_factor(qss, l2norm);
-        const float eg = __expf(grow);
+        const float rk = l2_factor(kss, l2norm);
         s_beta[srow] = brow;
-        s_ek[srow] = eg * rk;
+        s_ek[srow] = __expf(grow) * rk;
         s_dk[srow] = __expf(g_last - grow) * rk;
-        s_qs[srow] = scale * eg * rq;
         s_gamma[srow] = grow;
         s_rk[srow] = rk;
-        s_rq[srow] = rq;
         if (srow == 0) s_misc[0] = __expf(g_last);
       }
-      lds_barrier();  // A1: tiles and factors of chunk c are in LDS
-      if (c + 1 < c1) issue_loads(c + 1);
+    };
+    auto stage_q = [&](int c) {
+      const bool live = srow < chunk_len[c];
+      float qss = 0.0f;
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+        *reinterpret_cast<bf16x8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
+      qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
+      if (spart == 0) {
+        const float rq = l2_factor(qss, l2norm);
+        s_qs[srow] = scale * __expf(grow) * rq;
+        s_rq[srow] = rq;
+      }
+    };
+
+    if (nc > 0) {
+      issue_tiles(c0);
+      if constexpr (PASS_B) issue_q(c0);
+      stage_tiles(c0);
+      if (nc > 1) issue_tiles(c0 + 1);
+    }
+    for (int c = c0; c < c1; ++c) {
+      if constexpr (PASS_B) {
+        stage_q(c);
+        if (c + 1 < c1) issue_q(c + 1);
+      }
+      lds_barrier();  // A(c)
       if constexpr (PASS_B) {
         for (int t = sw; t < 3; t += 2) {  // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero
           const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
@@ -468,17 +516,21 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
           for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
+          for (int r = 0; r < 16; ++r) {  // the mask goes on the exponent so that the code stays branch-free
             const int j = 32 * jm + acc_row(r, hh);
-            acc[r] = i >= j ? acc[r] * fi * rj[r / 4][r % 4] * __expf(gi - gj[r / 4][r % 4]) : 0.0f;
+            acc[r] *= fi * rj[r / 4][r % 4] * __expf(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
           }
           const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
           frag_store(s_P, f0 + 0, lane, acc_to_operand(acc, 0));
           frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
         }
       }
-      lds_barrier();  // B: P fragments are in LDS
-      lds_barrier();  // C: the chain waves are done with chunk c's tiles
+      lds_barrier();  // X(c)
+      if (c + 1 < c1) {
+        stage_tiles(c + 1);
+        if (c + 2 < c1) issue_tiles(c + 2);
+      }
+      if constexpr (PASS_B) lds_barrier();  // C(c)
     }
     return;
   }
@@ -488,6 +540,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   const bool is_m = !PASS_B && wave < KT / 32;
   const int vslab = PASS_B ? wave : (is_m ? 0 : wave - KT / 32);
   const int col = 32 * vslab + ln;  // value column (unused for M slabs)
+  const float vmask = is_m ? 0.0f : 1.0f;
 
   f32x16 S[KT / 32];
   if (PASS_B) {
@@ -508,9 +561,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
   // pays the LDS latency once per MFMA.
   for (int c = c0; c < c1; ++c) {
-    lds_barrier();  // A
-    bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), later K^T rows (stage 3)
-    bf16x8 ft[6];              // T (stage 2)
+    lds_barrier();  // A(c)
+    bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+    bf16x8 ft[6];              // T (stage 2), P (output)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
@@ -523,7 +576,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int ks = 0; ks < 2 * (tm + 1); ++ks) ft[2 * tm + ks] = ld_kappa(s_T, SX, 32 * tm + ln, 16 * ks, hh);
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks) ft[2 * tm + ks] = ld_kappa(s_T, ST, 32 * tm + ln, 16 * ks, hh);
     f32x4 be[8], ek[8];
     bf16x4 vv[8];
 #pragma unroll
@@ -531,12 +584,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const int i0 = 8 * t8 + 4 * hh;
       be[t8] = *reinterpret_cast<const f32x4*>(&s_beta[i0]);
       ek[t8] = *reinterpret_cast<const f32x4*>(&s_ek[i0]);
-      if (is_m) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) vv[t8][e] = (__bf16)0.0f;
-      } else {
-        vv[t8] = *reinterpret_cast<const bf16x4*>(&s_vT[col * SX + i0]);
-      }
+      // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
+      // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
+      vv[t8] = ld_col4(s_v, SV, 32 * vslab, 8 * t8, lane);
     }
     bf16x8 Rb[4];
 #pragma unroll
@@ -548,16 +598,17 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          acc[4 * b4 + e] = be[4 * tm + b4][e] * ((float)vv[4 * tm + b4][e] - ek[4 * tm + b4][e] * acc[4 * b4 + e]);
+          acc[4 * b4 + e] =
+              be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ek[4 * tm + b4][e] * acc[4 * b4 + e]);
       Rb[2 * tm + 0] = acc_to_operand(acc, 0);
       Rb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
     lds_fence();
-    // batch for stage 3: K^T fragments and the decay factors
+    // batch for stage 3: K^T fragments (transposing reads of the row-major k tile) and the decay factors
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa(s_kT, SX, 32 * km + ln, 16 * ks, hh);
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(s_k, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&s_dk[8 * t8 + 4 * hh]);
@@ -578,6 +629,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
     lds_fence();
+    lds_barrier();  // X(c): every operand that comes from the k, v and T tiles of chunk c is in registers
     dtot *= dec;
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km) {  // S <- dec S + K^T (dk v_new)
@@ -586,11 +638,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(fk[km * 4 + ks], Vsb[ks], S[km]);
     }
-    lds_barrier();  // B
     if constexpr (PASS_B) {
-      const int tok0 = chunk_tok0[c], len = chunk_len[c];
-      T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
-      const int rs = HV * VT;
       // batch: Q rows, P fragments, output factors
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm)
@@ -602,35 +650,47 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) qs[t8] = *reinterpret_cast<const f32x4*>(&s_qs[8 * t8 + 4 * hh]);
       lds_fence();
+      lds_barrier();  // C(c): the q and P operands of chunk c are in registers
+      // o = qs (Q S_old) + P v_new, packed to the output type two columns at a time: lanes 2j and 2j+1 swap one
+      // value of every adjacent row pair, so the even lane holds both columns of the even row and the odd lane
+      // both columns of the odd row. The slab goes to this wave's own part of the o tile and from there to HBM
+      // in 16-byte pieces.
+      const bool odd = ln & 1;
 #pragma unroll
-      for (int tm = 0; tm < 2; ++tm) {  // o = qs (Q S_old) + P v_new
+      for (int tm = 0; tm < 2; ++tm) {
         f32x16 a1 = zero16(), a2 = zero16();
 #pragma unroll
         for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], a1);
 #pragma unroll
         for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(ft[2 * tm + ks], Vb[ks], a2);
-        // The offset is (re)computed here in every iteration on purpose: hoisted out of the loop, the 32 row
-        // addresses would occupy 64 registers, spill, and be reloaded from scratch behind a wait each time.
-        int off = (32 * tm + 4 * hh) * rs + col;
-        asm volatile("" : "+v"(off));
 #pragma unroll
-        for (int b4 = 0; b4 < 4; ++b4) {
-          const int t4 = 32 * tm + 8 * b4 + 4 * hh;
-          if (len == GDR_C) {  // full chunk (uniform branch): no per-row guards
+        for (int pr = 0; pr < 8; ++pr) {
+          const int r0 = 2 * pr, r1 = r0 + 1;
+          const float x0 = qs[4 * tm + r0 / 4][r0 % 4] * a1[r0] + a2[r0];
+          const float x1 = qs[4 * tm + r1 / 4][r1 % 4] * a1[r1] + a2[r1];
+          const float keep = odd ? x1 : x0;
+          const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
+          typedef T T2 __attribute__((ext_vector_type(2)));
+          T2 pk;
+          pk[0] = GdrElem<T>::from_float(odd ? got : keep);
+          pk[1] = GdrElem<T>::from_float(odd ? keep : got);
+          const int row = 32 * tm + acc_row(r0, hh) + (odd ? 1 : 0);
+          *reinterpret_cast<T2*>(&s_o[row * SV + 32 * vslab + (ln & ~1)]) = pk;
+        }
+      }
+      lds_fence();
+      {
+        const int tok0 = chunk_tok0[c], len = chunk_len[c];
+        T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
+        const int rs = HV * VT;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              ob[off + (8 * b4 + e) * rs] = GdrElem<T>::from_float(qs[4 * tm + b4][e] * a1[4 * b4 + e] + a2[4 * b4 + e]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (t4 + e < len)
-                ob[off + (8 * b4 + e) * rs] =
-                    GdrElem<T>::from_float(qs[4 * tm + b4][e] * a1[4 * b4 + e] + a2[4 * b4 + e]);
-          }
+        for (int j = 0; j < 4; ++j) {
+          const int piece = lane + 64 * j, row = piece >> 2, part = piece & 3;
+          const uint4 val = *reinterpret_cast<const uint4*>(&s_o[row * SV + 32 * vslab + 8 * part]);
+          if (row < len) *reinterpret_cast<uint4*>(ob + row * rs + 32 * vslab + 8 * part) = val;
         }
       }
     }
-    lds_barrier();  // C
   }
 
   // epilogue; the opaque zero keeps the compiler from computing all these addresses before the loop

@@ -68,6 +68,30 @@ __device__ __forceinline__ void load8(const T* p, float* out) {
   }
 }
 
+// Lane exchanges on the VALU data-parallel-primitive path (no LDS round trip, unlike __shfl*).
+// dpp_f32<CTRL, ROW_MASK>(old, x): lane i receives x of the lane CTRL selects; lanes whose row is not in ROW_MASK
+// or whose source lies outside their row of 16 keep `old`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float old, float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(x), CTRL, ROW_MASK, 0xF, false));
+}
+#define GDR_DPP_QUAD_XOR1 0xB1   /* quad_perm [1,0,3,2] */
+#define GDR_DPP_QUAD_XOR2 0x4E   /* quad_perm [2,3,0,1] */
+#define GDR_DPP_ROW_SHR(n) (0x110 + (n))
+#define GDR_DPP_ROW_BCAST15 0x142 /* lane 15 of each row -> every lane of the next row */
+#define GDR_DPP_ROW_BCAST31 0x143 /* lane 31 -> rows 2 and 3 */
+
+// Inclusive prefix sum over the 64 lanes of a wave: Hillis-Steele inside each row of 16, then the row totals.
+__device__ __forceinline__ float wave_inclusive_scan(float x) {
+  x += dpp_f32<GDR_DPP_ROW_SHR(1), 0xF>(0.0f, x);
+  x += dpp_f32<GDR_DPP_ROW_SHR(2), 0xF>(0.0f, x);
+  x += dpp_f32<GDR_DPP_ROW_SHR(4), 0xF>(0.0f, x);
+  x += dpp_f32<GDR_DPP_ROW_SHR(8), 0xF>(0.0f, x);
+  x += dpp_f32<GDR_DPP_ROW_BCAST15, 0xA>(0.0f, x);
+  x += dpp_f32<GDR_DPP_ROW_BCAST31, 0xC>(0.0f, x);
+  return x;
+}
+
 // Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every outstanding global load
 // and store of the wave (vmcnt(0)), which would serialise the software prefetch of the next chunk behind each
 // barrier; here only the LDS / scalar counter is drained.
