@@ -31,7 +31,7 @@
 #include "gdr_common.h"
 #include "gdr_plan.h"
 
-#define T_BYTES (64 * 64 * 2)  // T of one chunk and head in HBM: bf16 [64][64] row-major
+#define T_BYTES (3 * 32 * 32 * 2)  // T of one chunk and head in HBM: bf16 blocks T11 | T21 | T22, 32x32 row-major each
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
   return *reinterpret_cast<const bf16x8*>(base + (size_t)frag * 1024 + lane * 16);
@@ -99,21 +99,19 @@ __device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& s
 }
 
 // ---- T = (I + A)^-1 ------------------------------------------------------------------------------------------
-// One WAVE per (chunk, head), one wave per workgroup: the forward substitution is a single-wave job, so the chunk
-// is not shared with idle helper waves; many small workgroups per CU keep every SIMD busy instead. All LDS
-// traffic is wave-private (no barriers; LDS operations of one wave complete in order).
+// One WAVE per (chunk, head), one wave per workgroup: the forward substitution is a single-wave job, so many small
+// workgroups per CU keep every SIMD busy. The k tile never touches LDS: the MFMA operand fragments of K K^T are
+// 16-byte global loads (lane = row, its half of each 16-wide contraction step). LDS holds only the two diagonal
+// blocks (fp32) and the per-token factors, all wave-private (LDS operations of one wave complete in order).
+// T is stored as three row-major 32x32 bf16 blocks: T11 | T21 | T22 (the upper-right block is zero and not kept).
 template <typename T, int KT>
-__global__ void __launch_bounds__(64, 2) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
-                                                     const float* __restrict__ beta,
-                                                     const int32_t* __restrict__ plan,
-                                                     unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
-  constexpr int SK = KT + 8, SB = 36, ST = 72;
-  constexpr int KT_BYTES = 64 * SK * 2, TT_BYTES = 64 * ST * 2;
-  __shared__ __align__(16) unsigned char s_kt[KT_BYTES > TT_BYTES ? KT_BYTES : TT_BYTES];  // k tile, later T
-  __shared__ __align__(16) float s_A11[32 * SB], s_A21[32 * SB], s_A22[32 * SB];           // blocks of A, later of T
-  __shared__ float s_gamma[64], s_beta[64], s_rk[64];
-  __bf16* s_k = reinterpret_cast<__bf16*>(s_kt);
-  __bf16* s_T = reinterpret_cast<__bf16*>(s_kt);
+__global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
+                                                         const float* __restrict__ beta,
+                                                         const int32_t* __restrict__ plan,
+                                                         unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
+  constexpr int SB = 36, NK = KT / 16;
+  __shared__ __align__(16) float s_A11[32 * SB], s_A22[32 * SB];  // diagonal blocks of A, later of T
+  __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64];
 
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
@@ -121,76 +119,70 @@ __global__ void __launch_bounds__(64, 2) gdr_tinv_kernel(const T* __restrict__ k
   const int len = plan[plan[PLAN_OFF_CHUNK_LEN] + chunk];
   const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
 
-  {  // rows past the end of a partial chunk behave as g = 0, beta = 0, k = 0
-    const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
-    float gv = g[gi], bv = beta[gi];
-    gv = lane < len ? gv : 0.0f;
-    bv = lane < len ? bv : 0.0f;
+  // operand fragments of the k tile: f[tm][ks] = k[32 tm + ln][16 ks + 8 hh .. + 7]; rows past the end of a
+  // partial chunk behave as k = 0, g = 0, beta = 0
+  typename Raw8<T>::type raw[2][NK];
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const float up = __shfl_up(gv, off);
-      if (lane >= off) gv += up;
-    }
-    s_gamma[lane] = gv;
-    s_beta[lane] = bv;
+  for (int tm = 0; tm < 2; ++tm) {
+    const T* kp = k + ((size_t)(tok0 + min(32 * tm + ln, len - 1)) * H + h) * KT + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) raw[tm][ks] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 16 * ks);
   }
-  {  // k tile -> LDS (bf16, row-major), row norms; 4 lanes share a row, 16 rows per pass
-    const int part = lane & 3;
-    constexpr int EPT = KT / 4;
-    typename Raw8<T>::type raw[4][EPT / 8];
-#pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-      const int row = 16 * ps + (lane >> 2);
-      const T* kp = k + ((size_t)(tok0 + min(row, len - 1)) * H + h) * KT + part * EPT;
-#pragma unroll
-      for (int c = 0; c < EPT / 8; ++c) raw[ps][c] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * c);
-    }
+  {
+    const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
+    const float gv = g[gi], bv = beta[gi];
+    s_gamma[lane] = wave_inclusive_scan(lane < len ? gv : 0.0f);
+    s_beta[lane] = lane < len ? bv : 0.0f;
+  }
+  bf16x8 f[2][NK];
+  {
     typename Raw8<T>::type zero;
 #pragma unroll
     for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
 #pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-      const int row = 16 * ps + (lane >> 2);
+    for (int tm = 0; tm < 2; ++tm) {
       float ss = 0.0f;
 #pragma unroll
-      for (int c = 0; c < EPT / 8; ++c)
-        *reinterpret_cast<bf16x8*>(&s_k[row * SK + part * EPT + 8 * c]) =
-            raw_to_bf16<T>(row < len ? raw[ps][c] : zero, ss, l2norm != GDR_L2_NONE);
-      ss += __shfl_xor(ss, 1);
-      ss += __shfl_xor(ss, 2);
-      if (part == 0) s_rk[row] = l2_factor(ss, l2norm);
+      for (int ks = 0; ks < NK; ++ks)
+        f[tm][ks] = raw_to_bf16<T>(32 * tm + ln < len ? raw[tm][ks] : zero, ss, l2norm != GDR_L2_NONE);
+      ss += __shfl_xor(ss, 32);
+      s_rk[32 * tm + ln] = l2_factor(ss, l2norm);
     }
   }
   lds_fence();
 
-  // A = strict_lower(beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j}) -> three 32x32 fp32 blocks in LDS
+  // A = strict_lower(beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j}). The diagonal blocks go to LDS; the
+  // off-diagonal block is computed transposed (rows j < 32, columns i >= 32) and stays in registers, because an
+  // accumulator that holds A21^T is, rounded to bf16, the A operand of A21 X.
+  f32x16 a21t;
 #pragma unroll
   for (int t = 0; t < 3; ++t) {
-    const int tm = t == 0 ? 0 : 1, tn = t == 2 ? 1 : 0;  // (0,0), (1,0), (1,1)
-    float* blk = t == 0 ? s_A11 : (t == 1 ? s_A21 : s_A22);
-    bf16x8 fa[KT / 16], fb[KT / 16];
-#pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks) {
-      fa[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tm + ln) * SK + 16 * ks + 8 * hh]);
-      fb[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
-    }
-    f32x4 gi4[4], bi4[4], ri4[4];
+    const int tr = t == 2 ? 1 : 0, tc = t == 0 ? 0 : 1;  // accumulator rows / columns: (0,0), (0,1) = A21^T, (1,1)
+    f32x4 gr4[4], rr4[4], br4[4];
 #pragma unroll
     for (int b4 = 0; b4 < 4; ++b4) {
-      gi4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tm + 8 * b4 + 4 * hh]);
-      bi4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tm + 8 * b4 + 4 * hh]);
-      ri4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tm + 8 * b4 + 4 * hh]);
+      gr4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tr + 8 * b4 + 4 * hh]);
+      rr4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tr + 8 * b4 + 4 * hh]);
+      br4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tr + 8 * b4 + 4 * hh]);
     }
-    const int j = 32 * tn + ln;
-    const float gj = s_gamma[j], rj = s_rk[j];
+    const int cidx = 32 * tc + ln;
+    const float gc = s_gamma[cidx], rc = s_rk[cidx], bc = s_beta[cidx];
     lds_fence();
     f32x16 acc = zero16();
 #pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
+    for (int ks = 0; ks < NK; ++ks) acc = mfma32(f[tr][ks], f[tc][ks], acc);
+    if (t == 1) {  // rows j (tile 0), columns i (tile 1): i > j always
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int il = acc_row(r, hh), i = 32 * tm + il;
-      blk[il * SB + ln] = i > j ? acc[r] * bi4[r / 4][r % 4] * ri4[r / 4][r % 4] * rj * __expf(gi4[r / 4][r % 4] - gj) : 0.0f;
+      for (int r = 0; r < 16; ++r)
+        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * __expf(gc - gr4[r / 4][r % 4]);
+    } else {       // rows i, columns j of a diagonal block; the mask goes on the exponent (branch-free)
+      float* blk = t == 0 ? s_A11 : s_A22;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int il = acc_row(r, hh);
+        blk[il * SB + ln] = acc[r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
+                            __expf(il > ln ? gr4[r / 4][r % 4] - gc : -1e30f);
+      }
     }
   }
   lds_fence();
@@ -198,95 +190,105 @@ __global__ void __launch_bounds__(64, 2) gdr_tinv_kernel(const T* __restrict__ k
   // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
   // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
   // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+  const int b = hh, c = ln;
+  float* Ab = b == 0 ? s_A11 : s_A22;
   {
-    const int b = hh, c = ln;
-    float* Ab = b == 0 ? s_A11 : s_A22;
     float x[32];
-    f32x4 rowbuf[4][8];  // a ring of rows: row i+3 loads while row i is reduced (hides the LDS latency)
+    f32x4 rowbuf[2][8];  // rows i and i+1: the next row loads while this one is reduced
     rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SB);
-    rowbuf[2][0] = *reinterpret_cast<const f32x4*>(Ab + 2 * SB);
-    rowbuf[3][0] = *reinterpret_cast<const f32x4*>(Ab + 3 * SB);
     x[0] = (c == 0) ? 1.0f : 0.0f;
 #pragma unroll
     for (int i = 1; i < 32; ++i) {
+      if (i + 1 < 32) {
+#pragma unroll
+        for (int q = 0; q < (i + 1 + 3) / 4; ++q)
+          rowbuf[(i + 1) & 1][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 1) * SB + 4 * q);
+      }
       float acc0 = (i == c) ? 1.0f : 0.0f, acc1 = 0.0f;
 #pragma unroll
       for (int j = 0; j < i; ++j) {
-        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 3][j / 4][j % 4], x[j], acc1);
-        else acc0 = __builtin_fmaf(-rowbuf[i & 3][j / 4][j % 4], x[j], acc0);
+        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc1);
+        else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
       }
       x[i] = acc0 + acc1;
-      // pins the order "arithmetic of row i, loads of row i+3": without it the compiler either serialises every
-      // load behind a wait or hoists all 124 loads to the top and spills
+      // pins the order "loads of row i+1, arithmetic of row i": without it the compiler either serialises every
+      // load behind a wait or hoists all the loads to the top and spills
       asm volatile("" : "+v"(x[i]) : : "memory");
-      if (i + 3 < 32) {
-#pragma unroll
-        for (int q = 0; q < (i + 3 + 3) / 4; ++q)
-          rowbuf[(i + 3) & 3][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 3) * SB + 4 * q);
-      }
     }
-    lds_fence();  // every lane is done reading A11 / A22 (and the k tile) before they are overwritten
+    lds_fence();  // every lane is done reading A11 / A22 before they are overwritten
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      Ab[i * SB + c] = x[i];  // fp32 diagonal blocks in place of A11 / A22 (operands of the merge)
-      s_T[(32 * b + i) * ST + lane] = (__bf16)x[i];
-      if (b == 1) s_T[i * ST + lane] = (__bf16)0.0f;
-    }
-    lds_fence();
-    f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11
-      bf16x8 ahi, alo, bhi, blo;
-      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A21[ln * SB + 16 * ks + 8 * hh]);
-      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A21[ln * SB + 16 * ks + 8 * hh + 4]);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float av = q < 4 ? a0[q % 4] : a1[q % 4];
-        const float bv = s_A11[(16 * ks + 8 * hh + q) * SB + ln];
-        const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
-        ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
-        bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
-      }
-      y0 = mfma32(ahi, bhi, y0);
-      y1 = mfma32(alo, bhi, y1);
-      y2 = mfma32(ahi, blo, y2);
-    }
-    f32x16 t0 = zero16(), t1 = zero16(), t2 = zero16();
-#pragma unroll
-    for (int r = 0; r < 16; ++r) y0[r] += y1[r] + y2[r];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
-      bf16x8 ahi, alo, bhi, blo;
-      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
-      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float av = q < 4 ? a0[q % 4] : a1[q % 4];
-        const float bv = y0[8 * ks + q];
-        const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
-        ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
-        bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
-      }
-      t0 = mfma32(ahi, bhi, t0);
-      t1 = mfma32(alo, bhi, t1);
-      t2 = mfma32(ahi, blo, t2);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s_T[(32 + acc_row(r, hh)) * ST + ln] = (__bf16)(-(t0[r] + (t1[r] + t2[r])));
+    for (int i = 0; i < 32; ++i) Ab[i * SB + c] = x[i];  // fp32 T11 / T22 in place of A11 / A22
   }
   lds_fence();
 
-  // T row-major bf16 [64][64] (the upper-right 32x32 block is zero)
+  f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11: A from the A21^T accumulator, T11 rows in the same slot order
+    bf16x8 ahi, alo, bhi, blo;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float av = a21t[8 * ks + q];
+      const float bv = s_A11[(16 * ks + kappa(hh, q)) * SB + ln];
+      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    }
+    y0 = mfma32(ahi, bhi, y0);
+    y1 = mfma32(alo, bhi, y1);
+    y2 = mfma32(ahi, blo, y2);
+  }
+  f32x16 t0 = zero16(), t1 = zero16(), t2 = zero16();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) y0[r] += y1[r] + y2[r];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
+    bf16x8 ahi, alo, bhi, blo;
+    const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
+    const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float av = q < 4 ? a0[q % 4] : a1[q % 4];
+      const float bv = y0[8 * ks + q];
+      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    }
+    t0 = mfma32(ahi, bhi, t0);
+    t1 = mfma32(alo, bhi, t1);
+    t2 = mfma32(ahi, blo, t2);
+  }
+
+  // T -> HBM: the diagonal blocks from LDS in 16-byte pieces; T21 from the accumulator, two columns per store
+  // (lanes 2j and 2j+1 swap one value of every adjacent row pair, as in the segment kernel's output)
+  __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * T_BYTES);
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const float* src = blk == 0 ? s_A11 : s_A22;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int piece = lane + 64 * j, row = piece >> 2, part = piece & 3;
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part]);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part + 4]);
+      bf16x8 pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { pk[e] = (__bf16)lo[e]; pk[4 + e] = (__bf16)hi[e]; }
+      *reinterpret_cast<bf16x8*>(out + (blk == 0 ? 0 : 2048) + row * 32 + 8 * part) = pk;
+    }
+  }
   {
-    __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * T_BYTES);
-    const int part = lane & 3;
+    const bool odd = ln & 1;
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-      const int row = 16 * ps + (lane >> 2);
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-        *reinterpret_cast<bf16x8*>(out + row * 64 + part * 16 + 8 * c) =
-            *reinterpret_cast<const bf16x8*>(&s_T[row * ST + part * 16 + 8 * c]);
+    for (int pr = 0; pr < 8; ++pr) {
+      const int r0 = 2 * pr, r1 = r0 + 1;
+      const float x0 = -(t0[r0] + (t1[r0] + t2[r0])), x1 = -(t0[r1] + (t1[r1] + t2[r1]));
+      const float keep = odd ? x1 : x0;
+      const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
+      bf16x2 pk;
+      pk[0] = (__bf16)(odd ? got : keep);
+      pk[1] = (__bf16)(odd ? keep : got);
+      const int row = acc_row(r0, hh) + (odd ? 1 : 0);
+      *reinterpret_cast<bf16x2*>(out + 1024 + row * 32 + (ln & ~1)) = pk;
     }
   }
 }
@@ -395,7 +397,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
     const int srow = stid >> 1, spart = stid & 1;
     typename Raw8<T>::type rk_[KU], rv_[VU], rq_[PASS_B ? KU : 1];
-    bf16x8 rt_[4];
+    bf16x8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
@@ -412,7 +414,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * T_BYTES);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) rt_[j] = tp[stid + 128 * j];
+      for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
       const float* gb = g + (size_t)tok0 * HV + hv;
       const float* bb = beta + (size_t)tok0 * HV + hv;
       const int gl = min(lane, len - 1) * HV;
@@ -438,10 +440,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
       const bool live = srow < len;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int piece = stid + 128 * j;  // row piece / 8, columns 8 * (piece % 8) ..
-        *reinterpret_cast<bf16x8*>(&s_T[(piece >> 3) * ST + 8 * (piece & 7)]) = rt_[j];
-      }
+      for (int j = 0; j < 3; ++j)  // the upper-right block of s_T is never read
+        *reinterpret_cast<bf16x8*>(&s_T[((j > 0 ? 32 : 0) + (stid >> 2)) * ST + (j == 2 ? 32 : 0) + 8 * (stid & 3)]) = rt_[j];
       float kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
@@ -543,12 +543,16 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   const float vmask = is_m ? 0.0f : 1.0f;
 
   f32x16 S[KT / 32];
-  if (PASS_B) {
-    const float* si = Sinit + ((size_t)seg * HV + hv) * KT * VT;
+  if (PASS_B) {  // the scan leaves every segment's initial state as 32-column slabs in accumulator order
+    const f32x4* si = reinterpret_cast<const f32x4*>(Sinit + (((size_t)seg * HV + hv) * (VT / 32) + vslab) * (KT * 32));
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] = si[(size_t)(32 * km + acc_row(r, hh)) * VT + col];
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const f32x4 t = si[(km * 4 + q4) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[km][4 * q4 + e] = t[e];
+      }
   } else {
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
@@ -804,12 +808,17 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict
     for (int d = 0; d < D; ++d) {
       const int p = p0 + d;
       if (p > nsteps) break;
-      if (compute) {  // the state segment seg0 + p starts from
-        float* si = Sinit + ((size_t)(seg0 + p) * HV + hv) * KT * VT;
+      if (compute) {  // the state segment seg0 + p starts from (accumulator order, like N)
+        f32x4* si = reinterpret_cast<f32x4*>(Sinit + (((size_t)(seg0 + p) * HV + hv) * (VT / 32) + vn) * (KT * 32));
 #pragma unroll
         for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) si[(size_t)(32 * km + acc_row(r, hh)) * VT + col] = S[km][r];
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
+            si[(km * 4 + q4) * 64 + lane] = t;
+          }
       }
       if (p == nsteps) break;
       unsigned char* s_M = smem + (p & 1) * (SH::M_BYTES + SH::N_BYTES);
@@ -842,6 +851,92 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict
 #pragma unroll
         for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
       }
+    }
+  }
+}
+
+// Single-wave variant for KT = 64: one wave per (32-column slab, sequence, head), no LDS and no barrier. The
+// operands of the next DEPTH steps (M' fragments, the N slab and d) sit in registers, loaded straight from HBM in
+// operand order DEPTH steps ahead, so the serial chain is MFMA + conversion latency only.
+template <int KT, int VT, int DEPTH>
+__global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const int32_t* __restrict__ plan,
+                                                             const unsigned char* __restrict__ Mcomp,
+                                                             const unsigned char* __restrict__ Ncomp,
+                                                             const float* __restrict__ Dcomp,
+                                                             const float* __restrict__ h0, float* __restrict__ Sinit,
+                                                             int HV) {
+  constexpr int MF = (KT / 32) * (KT / 16), NF = (KT / 32) * 4;
+  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
+  const int nsteps = nseg - 1;
+  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+  const int col = 32 * vn + ln;
+
+  f32x16 S[KT / 32];
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km) {
+    S[km] = zero16();
+    if (h0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[km][r] = h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col];
+    }
+  }
+
+  bf16x8 rm[DEPTH][MF];
+  f32x4 rn[DEPTH][NF];
+  float rd[DEPTH];
+  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+    const size_t sh = (size_t)(seg0 + p) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * N_BYTES);
+#pragma unroll
+    for (int f = 0; f < MF; ++f) m[f] = M[f * 64 + lane];
+#pragma unroll
+    for (int j = 0; j < NF; ++j) n[j] = N[j * 64 + lane];
+    d = Dcomp[sh];
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (d < nsteps) issue(d, rm[d], rn[d], rd[d]);
+
+  for (int p0 = 0; p0 <= nsteps; p0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int p = p0 + d;
+      if (p > nsteps) break;
+      {  // the state segment seg0 + p starts from
+        f32x4* si = reinterpret_cast<f32x4*>(Sinit + (((size_t)(seg0 + p) * HV + hv) * (VT / 32) + vn) * (KT * 32));
+#pragma unroll
+        for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
+            si[(km * 4 + q4) * 64 + lane] = t;
+          }
+      }
+      if (p == nsteps) break;
+      const float dec = rd[d];
+      bf16x8 Sb[KT / 16];
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+      f32x16 Snew[KT / 32];
+#pragma unroll
+      for (int tm = 0; tm < KT / 32; ++tm) {
+        f32x16 acc;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[tm][4 * q4 + e], rn[d][tm * 4 + q4][e]);
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(rm[d][tm * (KT / 16) + ks], Sb[ks], acc);
+        Snew[tm] = acc;
+      }
+#pragma unroll
+      for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
+      if (p + DEPTH < nsteps) issue(p + DEPTH, rm[d], rn[d], rd[d]);
     }
   }
 }
@@ -905,8 +1000,12 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
-  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
-                     plan_dev, Mc, Nc, Dc, h0, Si, HV);
+  if constexpr (KT == 64)
+    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 3>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, plan_dev, Mc, Nc, Dc,
+                       h0, Si, HV);
+  else
+    hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
+                       plan_dev, Mc, Nc, Dc, h0, Si, HV);
   LAMPA_PROF(s, "gdr_scan_kernel");
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
                      (const T*)k, (const T*)v, g, beta, plan_dev, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,

@@ -39,7 +39,7 @@ def test_workspace_queries_and_argument_errors(lib):
     assert lib.lampa_sort_workspace_bytes(3, 60000) > 4 * 3 * 60000 * 4
     assert lib.lampa_sort_workspace_bytes(0, 10) == -1
     assert lib.lampa_lsh_bucket_workspace_bytes(60000, 3, 4) >= 235 * 12 * 8
-    assert lib.lampa_gdr_chunk_workspace_bytes(938, 60, 8, 64, 64) > 938 * 8 * 64 * 64 * 2  # T of every chunk
+    assert lib.lampa_gdr_chunk_workspace_bytes(938, 60, 8, 64, 64) > 938 * 8 * 3 * 32 * 32 * 2  # three 32x32 blocks of T per chunk and head
     assert lib.lampa_gdr_chunk_workspace_bytes(938, 60, 8, 48, 64) == -4  # unsupported head size
     # null pointers / bad sizes are rejected before any launch
     assert lib.lampa_sort_pairs(None, 0, None, 1, 10, 32, None, 1, 0, None, None, 0, None) == -1
