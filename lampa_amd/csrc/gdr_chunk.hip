@@ -31,6 +31,24 @@
 #include "gdr_common.h"
 #include "gdr_plan.h"
 
+// Device pointers to the tables of the plan (resolved on the host, so that a kernel reaches an entry with one
+// load instead of a dependent pair).
+struct GdrPlanView {
+  const int32_t *chunk_tok0, *chunk_len, *seg_chunk0, *seg_nchunks, *seg_seq, *seg_flags, *seq_seg0, *seq_nseg;
+};
+static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_dev) {
+  GdrPlanView pv;
+  pv.chunk_tok0 = plan_dev + plan_host[PLAN_OFF_CHUNK_TOK0];
+  pv.chunk_len = plan_dev + plan_host[PLAN_OFF_CHUNK_LEN];
+  pv.seg_chunk0 = plan_dev + plan_host[PLAN_OFF_SEG_CHUNK0];
+  pv.seg_nchunks = plan_dev + plan_host[PLAN_OFF_SEG_NCHUNKS];
+  pv.seg_seq = plan_dev + plan_host[PLAN_OFF_SEG_SEQ];
+  pv.seg_flags = plan_dev + plan_host[PLAN_OFF_SEG_FLAGS];
+  pv.seq_seg0 = plan_dev + plan_host[PLAN_OFF_SEQ_SEG0];
+  pv.seq_nseg = plan_dev + plan_host[PLAN_OFF_SEQ_NSEG];
+  return pv;
+}
+
 #define T_BYTES (3 * 32 * 32 * 2)  // T of one chunk and head in HBM: bf16 blocks T11 | T21 | T22, 32x32 row-major each
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
@@ -106,17 +124,20 @@ __device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& s
 // T is stored as three row-major 32x32 bf16 blocks: T11 | T21 | T22 (the upper-right block is zero and not kept).
 template <typename T, int KT>
 __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
-                                                         const float* __restrict__ beta,
-                                                         const int32_t* __restrict__ plan,
+                                                         const float* __restrict__ beta, const GdrPlanView pv,
                                                          unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
   constexpr int SB = 36, NK = KT / 16;
-  __shared__ __align__(16) float s_A11[32 * SB], s_A22[32 * SB];  // diagonal blocks of A, later of T
+  // diagonal blocks of A, later of T. ONE array: the forward substitution indexes it with the lane's block, and
+  // two separate arrays would make the compiler read both and select per value.
+  __shared__ __align__(16) float s_Ad[2 * 32 * SB];
   __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64];
+  float* s_A11 = s_Ad;
+  float* s_A22 = s_Ad + 32 * SB;
 
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
-  const int tok0 = plan[plan[PLAN_OFF_CHUNK_TOK0] + chunk];
-  const int len = plan[plan[PLAN_OFF_CHUNK_LEN] + chunk];
+  const int tok0 = pv.chunk_tok0[chunk];
+  const int len = pv.chunk_len[chunk];
   const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
 
   // operand fragments of the k tile: f[tm][ks] = k[32 tm + ln][16 ks + 8 hh .. + 7]; rows past the end of a
@@ -128,10 +149,10 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) raw[tm][ks] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 16 * ks);
   }
-  {
+  {  // gamma is kept in units of log 2 (exp2 is one instruction)
     const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
     const float gv = g[gi], bv = beta[gi];
-    s_gamma[lane] = wave_inclusive_scan(lane < len ? gv : 0.0f);
+    s_gamma[lane] = 1.44269504f * wave_inclusive_scan(lane < len ? gv : 0.0f);
     s_beta[lane] = lane < len ? bv : 0.0f;
   }
   bf16x8 f[2][NK];
@@ -174,14 +195,14 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
     if (t == 1) {  // rows j (tile 0), columns i (tile 1): i > j always
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * __expf(gc - gr4[r / 4][r % 4]);
+        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * __builtin_amdgcn_exp2f(gc - gr4[r / 4][r % 4]);
     } else {       // rows i, columns j of a diagonal block; the mask goes on the exponent (branch-free)
       float* blk = t == 0 ? s_A11 : s_A22;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int il = acc_row(r, hh);
         blk[il * SB + ln] = acc[r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
-                            __expf(il > ln ? gr4[r / 4][r % 4] - gc : -1e30f);
+                            __builtin_amdgcn_exp2f(il > ln ? gr4[r / 4][r % 4] - gc : -1e30f);
       }
     }
   }
@@ -191,7 +212,7 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
   // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
   // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
   const int b = hh, c = ln;
-  float* Ab = b == 0 ? s_A11 : s_A22;
+  float* Ab = s_Ad + b * (32 * SB);
   {
     float x[32];
     f32x4 rowbuf[2][8];  // rows i and i+1: the next row loads while this one is reduced
@@ -357,8 +378,9 @@ __device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int
 template <typename T, int KT, int VT, bool PASS_B>
 __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-                       const float* __restrict__ g, const float* __restrict__ beta,
-                       const int32_t* __restrict__ plan, const unsigned char* __restrict__ tmat,
+                       const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
+                       const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
+                       const unsigned char* __restrict__ tmat,
                        const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
                        unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o,
                        float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
@@ -383,12 +405,12 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 
   const int seg = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
-  const int flags = plan[plan[PLAN_OFF_SEG_FLAGS] + seg];
+  const int flags = pv.seg_flags[seg];
   if (!PASS_B && (flags & SEG_LAST)) return;  // nothing follows the last segment of a sequence
-  const int c0 = plan[plan[PLAN_OFF_SEG_CHUNK0] + seg], nc = plan[plan[PLAN_OFF_SEG_NCHUNKS] + seg];
+  const int c0 = pv.seg_chunk0[seg], nc = pv.seg_nchunks[seg];
   const int c1 = c0 + nc;
-  const int* chunk_tok0 = plan + plan[PLAN_OFF_CHUNK_TOK0];
-  const int* chunk_len = plan + plan[PLAN_OFF_CHUNK_LEN];
+  // (the per-chunk tables are separate restrict parameters: read through the view they could alias the kernel's
+  // stores, would be fetched with vector loads and would sit in the same queue as the stagers' prefetches)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
 
   if (wave >= NSLAB) {
@@ -702,7 +724,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   asm volatile("" : "+v"(late));
   if constexpr (PASS_B) {
     if (ht && (flags & SEG_LAST)) {
-      const int seq = plan[plan[PLAN_OFF_SEG_SEQ] + seg];
+      const int seq = pv.seg_seq[seg];
       float* out = ht + ((size_t)seq * HV + hv) * KT * VT + late;
 #pragma unroll
       for (int km = 0; km < KT / 32; ++km)
@@ -761,7 +783,7 @@ struct GdrScanShape {
 };
 
 template <int KT, int VT>
-__global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict__ plan,
+__global__ void __launch_bounds__(512) gdr_scan_kernel(const GdrPlanView pv,
                                                       const unsigned char* __restrict__ Mcomp,
                                                       const unsigned char* __restrict__ Ncomp,
                                                       const float* __restrict__ Dcomp,
@@ -771,7 +793,7 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict
   constexpr int D = SH::DEPTH, MP = SH::MP, NP = SH::NP;
   extern __shared__ __align__(16) unsigned char smem[];
   const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
-  const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
   const int nsteps = nseg - 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
@@ -859,7 +881,7 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const int32_t* __restrict
 // operands of the next DEPTH steps (M' fragments, the N slab and d) sit in registers, loaded straight from HBM in
 // operand order DEPTH steps ahead, so the serial chain is MFMA + conversion latency only.
 template <int KT, int VT, int DEPTH>
-__global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const int32_t* __restrict__ plan,
+__global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const GdrPlanView pv,
                                                              const unsigned char* __restrict__ Mcomp,
                                                              const unsigned char* __restrict__ Ncomp,
                                                              const float* __restrict__ Dcomp,
@@ -868,7 +890,7 @@ __global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const int32_t* __r
   constexpr int MF = (KT / 32) * (KT / 16), NF = (KT / 32) * 4;
   constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
   const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
-  const int seg0 = plan[plan[PLAN_OFF_SEQ_SEG0] + seq], nseg = plan[plan[PLAN_OFF_SEQ_NSEG] + seq];
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
   const int nsteps = nseg - 1;
   const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
@@ -968,7 +990,7 @@ extern "C" int64_t lampa_gdr_chunk_workspace_bytes(int64_t total_chunks, int64_t
 
 template <typename T, int KT, int VT>
 static int gdr_chunk_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, void* o,
-                            const float* h0, float* ht, const int32_t* plan_dev, int n_seq, int chunks, int segs, int H,
+                            const float* h0, float* ht, const GdrPlanView pv, int n_seq, int chunks, int segs, int H,
                             int HV, float scale, int l2norm, unsigned char* ws, hipStream_t s) {
   const GdrWorkspace w = gdr_workspace(chunks, segs, HV, KT, VT);
   unsigned char* tf = ws + w.off_t;
@@ -990,25 +1012,25 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
-    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, plan_dev, tf, H,
-                       HV, l2norm);
+    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv, tf, H, HV,
+                       l2norm);
     LAMPA_PROF(s, "gdr_tinv_kernel");
     if (segs > n_seq) {
       hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
-                         (const T*)q, (const T*)k, (const T*)v, g, beta, plan_dev, tf, (const float*)nullptr, Mc, Nc, Dc,
+                         (const T*)q, (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nc, Dc,
                          (T*)nullptr, (float*)nullptr, H, HV, scale, l2norm);
       LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
   if constexpr (KT == 64)
-    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 3>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, plan_dev, Mc, Nc, Dc,
+    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 3>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, pv, Mc, Nc, Dc,
                        h0, Si, HV);
   else
     hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
-                       plan_dev, Mc, Nc, Dc, h0, Si, HV);
+                       pv, Mc, Nc, Dc, h0, Si, HV);
   LAMPA_PROF(s, "gdr_scan_kernel");
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
-                     (const T*)k, (const T*)v, g, beta, plan_dev, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
+                     (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
                      (float*)nullptr, (T*)o, ht, H, HV, scale, l2norm);
   LAMPA_PROF(s, "gdr_segment_kernel<output>");
   return lampa_launch_status();
@@ -1030,8 +1052,9 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
   if (!workspace || workspace_bytes < gdr_workspace(chunks, segs, HV, K, V).bytes) return LAMPA_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   unsigned char* ws = (unsigned char*)workspace;
+  const GdrPlanView pv = gdr_plan_view(plan_host, plan_dev);
 #define GDR_CASE(TT, KK, VV)                                                                                       \
-  return gdr_chunk_launch<TT, KK, VV>(q, k, v, g, beta, o, h0, ht, plan_dev, n_seq, chunks, segs, H, HV, scale, \
+  return gdr_chunk_launch<TT, KK, VV>(q, k, v, g, beta, o, h0, ht, pv, n_seq, chunks, segs, H, HV, scale, \
                                       l2norm, ws, s)
   if (dtype == GDR_BF16) {
     if (K == 64 && V == 64) GDR_CASE(__bf16, 64, 64);
