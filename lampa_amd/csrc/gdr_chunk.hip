@@ -77,6 +77,10 @@ __device__ __forceinline__ f32x16 zero16() {
   return z;
 }
 
+// Tells the compiler that x is the same in every lane, so that a table lookup with it becomes a scalar load: a
+// vector load would join the queue of the prefetches and its wait would drain all of them.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
 __device__ __forceinline__ int acc_row(int r, int hh) { return 8 * (r / 4) + 4 * hh + (r % 4); }
 
 __device__ __forceinline__ float l2_factor(float ss, int l2norm) {
@@ -418,13 +422,15 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
     const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
     const int srow = stid >> 1, spart = stid & 1;
-    typename Raw8<T>::type rk_[KU], rv_[VU], rq_[PASS_B ? KU : 1];
+    typename Raw8<T>::type rk_[KU], rv_[VU];
+    typename Raw8<T>::type rq0_[PASS_B ? KU : 1], rq1_[PASS_B ? KU : 1];  // q of even / odd chunks of the segment
     bf16x8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
     auto issue_tiles = [&](int c) {
+      c = uniform(c);
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* kb = k + ((size_t)tok0 * H + h) * KT;
       const T* vb = v + ((size_t)tok0 * HV + hv) * VT;
@@ -443,7 +449,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       rg = gb[gl];
       rb = bb[gl];
     };
-    auto issue_q = [&](int c) {
+    auto issue_q = [&](int c, typename Raw8<T>::type* rq_) {
+      c = uniform(c);
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* qb = q + ((size_t)tok0 * H + h) * KT;
       const int koff = min(srow, len - 1) * H * KT + spart * (KT / 2);
@@ -455,16 +462,14 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
     const bool want_ss = l2norm != GDR_L2_NONE;
 
-    auto stage_tiles = [&](int c) {
-      const int len = chunk_len[c];
-      const float bv = lane < len ? rb : 0.0f;
-      const float gv = wave_inclusive_scan(lane < len ? rg : 0.0f);  // in-chunk cumulative log-decay, lane = token
-      const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
-      const bool live = srow < len;
+    float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
+    // k, v and T of chunk c from the registers to LDS
+    auto stage_data = [&](int c) {
+      const bool live = srow < chunk_len[uniform(c)];
 #pragma unroll
       for (int j = 0; j < 3; ++j)  // the upper-right block of s_T is never read
         *reinterpret_cast<bf16x8*>(&s_T[((j > 0 ? 32 : 0) + (stid >> 2)) * ST + (j == 2 ? 32 : 0) + 8 * (stid & 3)]) = rt_[j];
-      float kss = 0.0f;
+      kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
         *reinterpret_cast<bf16x8*>(&s_k[srow * SK + spart * (KT / 2) + 8 * u]) =
@@ -475,22 +480,30 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         *reinterpret_cast<bf16x8*>(&s_v[srow * SV + spart * (VT / 2) + 8 * u]) =
             raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
       }
-      kss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
+    };
+    // per-token factors of chunk c (gate, beta, norms)
+    auto stage_factors = [&](int c) {
+      const int len = chunk_len[uniform(c)];
+      const float bv = lane < len ? rb : 0.0f;
+      // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction), lane = token
+      const float gv = 1.44269504f * wave_inclusive_scan(lane < len ? rg : 0.0f);
+      const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
+      const float kss2 = kss + dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
       // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
       grow = __shfl(gv, srow);
       const float brow = __shfl(bv, srow);
       if (spart == 0) {
-        const float rk = l2_factor(kss, l2norm);
+        const float rk = l2_factor(kss2, l2norm);
         s_beta[srow] = brow;
-        s_ek[srow] = __expf(grow) * rk;
-        s_dk[srow] = __expf(g_last - grow) * rk;
+        s_ek[srow] = __builtin_amdgcn_exp2f(grow) * rk;
+        s_dk[srow] = __builtin_amdgcn_exp2f(g_last - grow) * rk;
         s_gamma[srow] = grow;
         s_rk[srow] = rk;
-        if (srow == 0) s_misc[0] = __expf(g_last);
+        if (srow == 0) s_misc[0] = __builtin_amdgcn_exp2f(g_last);
       }
     };
-    auto stage_q = [&](int c) {
-      const bool live = srow < chunk_len[c];
+    auto stage_q = [&](int c, const typename Raw8<T>::type* rq_) {
+      const bool live = srow < chunk_len[uniform(c)];
       float qss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
@@ -499,25 +512,25 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
       if (spart == 0) {
         const float rq = l2_factor(qss, l2norm);
-        s_qs[srow] = scale * __expf(grow) * rq;
+        s_qs[srow] = scale * __builtin_amdgcn_exp2f(grow) * rq;
         s_rq[srow] = rq;
       }
     };
 
-    if (nc > 0) {
-      issue_tiles(c0);
-      if constexpr (PASS_B) issue_q(c0);
-      stage_tiles(c0);
-      if (nc > 1) issue_tiles(c0 + 1);
-    }
-    for (int c = c0; c < c1; ++c) {
+    // All loads of a chunk (k, v, T, g, beta and q) are issued at ONE point, a full chunk period before the wait
+    // that precedes the staging of its tiles, so no wait ever has to leave younger loads in flight (the compiler
+    // drains the whole queue at such waits as soon as the control flow between issue and use is not trivial).
+    // q is staged half a period after the tiles, hence two q register sets, used by even and odd chunks in turn.
+    // The chunk index is clamped at the end of the segment (the last chunk is fetched again for nothing).
+    auto issue_chunk = [&](int c, typename Raw8<T>::type* rq_) {
+      issue_tiles(c);
+      if constexpr (PASS_B) issue_q(c, rq_);
+    };
+    auto build_p = [&]() {
       if constexpr (PASS_B) {
-        stage_q(c);
-        if (c + 1 < c1) issue_q(c + 1);
-      }
-      lds_barrier();  // A(c)
-      if constexpr (PASS_B) {
-        for (int t = sw; t < 3; t += 2) {  // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero
+        // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tiles 0 and 2, stager 1
+        // tile 1.
+        auto p_tile = [&](int t) {
           const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
           bf16x8 fa[KT / 16], fb[KT / 16];
 #pragma unroll
@@ -540,19 +553,53 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {  // the mask goes on the exponent so that the code stays branch-free
             const int j = 32 * jm + acc_row(r, hh);
-            acc[r] *= fi * rj[r / 4][r % 4] * __expf(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
+            acc[r] *= fi * rj[r / 4][r % 4] * __builtin_amdgcn_exp2f(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
           }
           const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
           frag_store(s_P, f0 + 0, lane, acc_to_operand(acc, 0));
           frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
-        }
+        };
+        p_tile(sw);
+        if (sw == 0) p_tile(2);
       }
-      lds_barrier();  // X(c)
-      if (c + 1 < c1) {
-        stage_tiles(c + 1);
-        if (c + 2 < c1) issue_tiles(c + 2);
+    };
+    // What a stager does between X(c) and X(c+1), spread over the three intervals so that in each of them it needs
+    // no longer than the chain waves (every barrier is a rendezvous: an interval lasts as long as its slower side).
+    // The loop below starts at a point where the loads that were issued one period ago have to have arrived
+    // anyway. Returns false after the last chunk. q(c) / q(c+2) use rq_same, q(c+1) uses rq_other.
+    auto half_step = [&](int c, typename Raw8<T>::type* rq_same, typename Raw8<T>::type* rq_other) -> bool {
+      const int cn = min(c + 1, c1 - 1), cnn = min(c + 2, c1 - 1);  // (clamped: the last chunk is fetched again)
+      stage_data(cn);
+      if constexpr (PASS_B) {
+        lds_barrier();  // C(c)
+        if (c + 1 >= c1) return false;
+        stage_factors(cn);
+        stage_q(cn, rq_other);
+        issue_chunk(cnn, rq_same);
+        lds_barrier();  // A(c+1)
+        build_p();
+      } else {
+        if (c + 1 >= c1) return false;
+        stage_factors(cn);
+        lds_barrier();  // A(c+1)
+        issue_chunk(cnn, rq_same);
       }
-      if constexpr (PASS_B) lds_barrier();  // C(c)
+      lds_barrier();  // X(c+1)
+      return true;
+    };
+    if (nc > 0) {
+      issue_chunk(c0, rq0_);
+      stage_data(c0);
+      stage_factors(c0);
+      if constexpr (PASS_B) stage_q(c0, rq0_);
+      issue_chunk(min(c0 + 1, c1 - 1), rq1_);
+      lds_barrier();  // A(c0)
+      build_p();
+      lds_barrier();  // X(c0)
+      for (int c = c0;; c += 2) {
+        if (!half_step(c, rq0_, rq1_)) break;
+        if (!half_step(c + 1, rq1_, rq0_)) break;
+      }
     }
     return;
   }
@@ -706,7 +753,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       }
       lds_fence();
       {
-        const int tok0 = chunk_tok0[c], len = chunk_len[c];
+        const int cu = uniform(c), tok0 = chunk_tok0[cu], len = chunk_len[cu];
         T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
         const int rs = HV * VT;
 #pragma unroll
@@ -823,7 +870,7 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const GdrPlanView pv,
   };
 #pragma unroll
   for (int d = 0; d < D; ++d)
-    if (d < nsteps) issue(d, rm[d], rn[d], rd[d]);
+    issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
 
   for (int p0 = 0; p0 <= nsteps; p0 += D) {
 #pragma unroll
@@ -850,7 +897,7 @@ __global__ void __launch_bounds__(512) gdr_scan_kernel(const GdrPlanView pv,
 #pragma unroll
       for (int j = 0; j < NP; ++j) reinterpret_cast<f32x4*>(s_N)[tid + SH::THREADS * j] = rn[d][j];
       const float dec = rd[d];
-      if (p + D < nsteps) issue(p + D, rm[d], rn[d], rd[d]);
+      issue(min(p + D, nsteps - 1), rm[d], rn[d], rd[d]);  // unconditional: keeps the load count per step fixed
       lds_barrier();
       if (compute) {
         bf16x8 Sb[KT / 16];
@@ -919,8 +966,7 @@ __global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const GdrPlanView 
     d = Dcomp[sh];
   };
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if (d < nsteps) issue(d, rm[d], rn[d], rd[d]);
+  for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
 
   for (int p0 = 0; p0 <= nsteps; p0 += DEPTH) {
 #pragma unroll
@@ -958,7 +1004,7 @@ __global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const GdrPlanView 
       }
 #pragma unroll
       for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
-      if (p + DEPTH < nsteps) issue(p + DEPTH, rm[d], rn[d], rd[d]);
+      issue(min(p + DEPTH, nsteps - 1), rm[d], rn[d], rd[d]);  // unconditional: keeps the load count per step fixed
     }
   }
 }

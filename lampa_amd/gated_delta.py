@@ -30,15 +30,25 @@ CHUNKS_PER_SEGMENT: Optional[int] = None
 _plan_cache = {}
 
 
-def _default_chunks_per_segment(max_chunks: int) -> int:
-    # serial cost ~ (chunks per segment) + 0.3 * (segments per sequence); minimise over the split
-    return int(min(64, max(4, round(math.sqrt(0.3 * max(max_chunks, 1))))))
+def _default_chunks_per_segment(chunks_per_seq, n_value_heads: int, slots: int) -> int:
+    """Segment length of the split-sequence scan. One workgroup walks one (segment, head) chunk by chunk, so the two
+    segment kernels take (chunks per segment) chunk periods as long as all workgroups are resident at once
+    (``slots`` = workgroups the chip holds), and the scan in between is serial in the segments per sequence:
+    the shortest segments that still fit are best."""
+    cps = 4
+    while cps < 64 and sum((n + cps - 1) // cps for n in chunks_per_seq) * n_value_heads > slots:
+        cps += 1
+    return cps
 
 
-def _plan(cu_host, device):
+def _plan(cu_host, device, n_value_heads: int, head_dims):
     """Host + device copies of the chunk/segment tables for these sequence boundaries (cached)."""
-    max_chunks = max((b - a + 63) // 64 for a, b in zip(cu_host[:-1], cu_host[1:]))
-    cps = CHUNKS_PER_SEGMENT or _default_chunks_per_segment(max_chunks)
+    cps = CHUNKS_PER_SEGMENT
+    if not cps:
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        per_cu = 2 if max(head_dims) <= 64 else 1  # workgroups of the segment kernels a CU holds (LDS, registers)
+        chunks_per_seq = [(b - a + 63) // 64 for a, b in zip(cu_host[:-1], cu_host[1:])]
+        cps = _default_chunks_per_segment(chunks_per_seq, n_value_heads, per_cu * cus)
     key = (tuple(cu_host), cps, str(device))
     hit = _plan_cache.get(key)
     if hit is not None:
@@ -78,7 +88,7 @@ def _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu
     else:
         cu_host = [int(c) for c in cu_seqlens.tolist()]
     n_seq = len(cu_host) - 1
-    plan_host, plan_dev = _plan(cu_host, q.device)
+    plan_host, plan_dev = _plan(cu_host, q.device, HV, (K, V))
     chunks, segs = int(plan_host[1]), int(plan_host[2])
     lib = _capi.lib()
     ws_bytes = check(lib.lampa_gdr_chunk_workspace_bytes(chunks, segs, HV, K, V), "lampa_gdr_chunk_workspace_bytes")
