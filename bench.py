@@ -29,6 +29,14 @@ KERNEL_BYTES_PER_TOKEN_HEAD = {            # algorithmic bytes each kernel of th
     "gdr_tinv_kernel": 2 * K + 8,                                 # reads k, g, beta
 }
 LSH_BYTES_PER_HIT_TABLE = 224
+# HBM bytes per launch at config 2 from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a plain
+# 256 MiB copy gives): profiles/gdr_chunk_fwd_config2_hbm_traffic_pmc.md. Counters cannot be read from inside a run.
+MEASURED_TRAFFIC_BYTES = {
+    "gdr_segment_kernel<output>": 331.8e6,
+    "gdr_segment_kernel<composite>": 210.7e6,
+    "gdr_tinv_kernel": 138.1e6,
+    "gdr_scan_kernel": 24.7e6,
+}
 
 
 def _median(xs):
@@ -145,7 +153,7 @@ def main():
     dom_gbs = dom_bytes / (stage_us[dominant] * 1e-6) / 1e9
     layer_us = ms_per_step * 1e3
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "kernel_us": round(stage_us[dominant], 2), "algorithmic_bytes_per_launch": dom_bytes}
     layer = {
         "us_per_layer": round(layer_us, 2),
