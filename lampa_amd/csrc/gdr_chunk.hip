@@ -16,15 +16,16 @@
 // tiles and the only intermediate that goes through HBM is T (6 KiB per chunk and head).
 //
 // Kernels:
-//   tinv     workgroup per (chunk, head): K K^T on MFMA, gating, blocked inverse (two 32x32 forward substitutions
-//            in fp32 + an MFMA merge with bf16 high/remainder splits), T written as MFMA A-operand fragments.
-//   segment  workgroup per (segment of chunks, head), one wave per 32 columns. Each chunk's k, q, v tiles are
-//            staged once in LDS (row-major and transposed), the next chunk's global loads are in flight
-//            meanwhile, and every wave runs the recurrence on its columns with the state in accumulator
-//            registers. PASS_A: columns of [M | N] of the segment's affine map S -> M S + N (start identity /
-//            zero). PASS_B: value columns, from the segment's true initial state, writing o (and the final state).
-//   scan     S_{p+1} = M_p S_p + N_p over the segments of a sequence (hi/lo-split bf16 MFMA), storing each
-//            segment's initial state.
+//   tinv     wave per (chunk, head): K K^T on MFMA with operand fragments loaded straight from HBM, gating, blocked
+//            inverse (two 32x32 forward substitutions in fp32 + an MFMA merge with bf16 high/remainder splits);
+//            T goes to HBM as three 32x32 bf16 blocks.
+//   segment  workgroup per (segment of chunks, head), one "chain" wave per 32 columns plus two "stager" waves. Each
+//            chunk's k, v, q, T tiles are staged once in LDS (row-major only), the coming chunks' global loads are
+//            in flight meanwhile, and every chain wave runs the recurrence on its columns with the state in
+//            accumulator registers. PASS_A: columns of [M | N] of the segment's affine map S -> M S + N (start
+//            identity / zero). PASS_B: value columns, from the segment's true initial state, writing o (and the
+//            final state).
+//   scan     S_{p+1} = M_p S_p + N_p over the segments of a sequence, storing each segment's initial state.
 // The state tile is fed back as the next MFMA's B operand straight from the accumulator registers: register r of
 // lane l is row 8*(r/4) + 4*(l/32) + r%4, and since a contraction may visit its index in any order as long as
 // both operands agree, every A operand is read from LDS in that slot order (ld_kappa).
