@@ -1070,7 +1070,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
     }
   }
   if constexpr (KT == 64)
-    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 3>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, pv, Mc, Nc, Dc,
+    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 5>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, pv, Mc, Nc, Dc,
                        h0, Si, HV);
   else
     hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
