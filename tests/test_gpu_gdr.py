@@ -174,3 +174,28 @@ def test_config2_full_size(device):
                                        initial_state=sa, output_final_state=True)
     _assert_bf16_close(torch.cat([oa, ob], 1), o.float().cpu(), "split o")
     _assert_bf16_close(sb, s.cpu(), "split state")
+
+
+def test_config4_varlen_batch_d128(device):
+    # 16 events of U[6000, 60000] hits packed with cu_seqlens, H=8, d_k=d_v=128, bf16 (about 528k tokens)
+    lens, cu = synth.varlen_lengths(16, 6000, 60000, seed=0)
+    T = int(cu[-1])
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 8, 128, 128, torch.bfloat16, seed=4)
+    dq, dk, dv, dg, db = _to(device, q, k, v, g, beta)
+    cud = cu.to(device)
+    o, s = gd.chunk_gated_delta_rule(dq, dk, dv, dg, db, output_final_state=True, cu_seqlens=cud)
+    assert o.shape == (1, T, 8, 128) and s.shape == (16, 8, 128, 128)
+    # the whole batch against the token-serial kernel (fp32 state, itself checked against the oracle above)
+    o2, s2 = gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db, output_final_state=True, cu_seqlens=cud)
+    _assert_bf16_close(o, o2.float().cpu(), "o vs token-serial")
+    _assert_bf16_close(s, s2.cpu(), "state vs token-serial")
+    # the shortest event against the CPU oracle
+    i = int(torch.argmin(lens))
+    a, b = int(cu[i]), int(cu[i + 1])
+    want_o, want_s = og.recurrent_c(q[:, a:b], k[:, a:b], v[:, a:b], g[:, a:b], beta[:, a:b])
+    _assert_bf16_close(o[:, a:b], want_o, "o vs oracle")
+    _assert_bf16_close(s[i:i + 1], want_s, "state vs oracle")
+    # packing is invisible: the same event run alone gives the same result
+    o1, s1 = gd.chunk_gated_delta_rule(dq[:, a:b], dk[:, a:b], dv[:, a:b], dg[:, a:b], db[:, a:b], output_final_state=True)
+    _assert_bf16_close(o[:, a:b], o1.float().cpu(), "o alone")
+    _assert_bf16_close(s[i:i + 1], s1.cpu(), "state alone")
