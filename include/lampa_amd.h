@@ -78,6 +78,18 @@ int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_t n_valid, 
                           int32_t* meta_out, int32_t* perm_out, const void* feats, int64_t feat_row_bytes,
                           void* feats_out, int n_passes, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same stage for a batch of events in one set of launches (events are independent: own id ranges, own key
+ * width; the sort runs over n_events * n_tables segments). This is the data-parallel form of the loop over events
+ * around hept.py:127-143. coords [n_events, n_hits, dim]; n_valid_dev: device int32 [n_events] or NULL (all valid);
+ * ids_out [E, T*J, N] (nullable), keys_out / perm_out [E, T, N], meta_out [E, T, 2J+3],
+ * feats [E, N, feat_row_bytes] -> feats_out [E, T, N, feat_row_bytes]. */
+int64_t lampa_lsh_bucket_sort_batch_workspace_bytes(int n_events, int64_t n_hits, int n_tables, int n_proj);
+int lampa_lsh_bucket_sort_batch(const float* coords, int n_events, int64_t n_hits, const int32_t* n_valid_dev, int dim,
+                                const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                                int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, int32_t* perm_out,
+                                const void* feats, int64_t feat_row_bytes, void* feats_out, int n_passes,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Sort keys of LSHOrdering: key[n] = sum_h 2^h <coords[n], alpha[:, h]>, norm[n] = |coords[n]|.
  * Replaces models/baselines/full_mamba2.py:174-203. coords [n_hits, dim], alpha [dim, n_hashes]. */
 int lampa_lsh_ordering_keys(const float* coords, int64_t n_hits, int dim, const float* alpha, int n_hashes,

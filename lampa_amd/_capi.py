@@ -26,6 +26,9 @@ _SIGNATURES = {
     "lampa_lsh_bucket_sort_workspace_bytes": (_i64, [_i64, _i32, _i32]),
     "lampa_lsh_bucket_sort": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp, _vp, _i64,
                                      _vp, _i32, _vp, _i64, _vp]),
+    "lampa_lsh_bucket_sort_batch_workspace_bytes": (_i64, [_i32, _i64, _i32, _i32]),
+    "lampa_lsh_bucket_sort_batch": (_i32, [_vp, _i32, _i64, _vp, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp,
+                                           _vp, _i64, _vp, _i32, _vp, _i64, _vp]),
     "lampa_lsh_project_f32": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "lampa_lsh_ordering_keys": (_i32, [_vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp]),
     "lampa_row_minmax_f32": (_i32, [_vp, _i32, _i64, _vp, _vp]),

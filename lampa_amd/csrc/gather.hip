@@ -17,8 +17,8 @@ __device__ __forceinline__ int64_t gs_index(const void* idx, int64_t i) {
 // dst[s, idx[s, n], :] = src[s, n, :] otherwise.
 template <typename VecT, typename IdxT, bool GATHER>
 __global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restrict__ src, int64_t src_seg_stride,
-                                                          int src_segments, const void* __restrict__ idx, int64_t n, int64_t n_src,
-                                                          int vec_per_row, char* __restrict__ dst, int* bad) {
+                                                          int src_segments, int group, const void* __restrict__ idx, int64_t n,
+                                                          int64_t n_src, int vec_per_row, char* __restrict__ dst, int* bad) {
   const int seg = blockIdx.y;
   const int64_t item = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
   const int64_t row = item / vec_per_row;
@@ -32,7 +32,7 @@ __global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restric
   }
   const int64_t row_bytes = (int64_t)vec_per_row * (int64_t)sizeof(VecT);
   const int64_t from = GATHER ? other : row, to = GATHER ? row : other;
-  const VecT* s = reinterpret_cast<const VecT*>(src + (seg % src_segments) * src_seg_stride + from * row_bytes) + piece;
+  const VecT* s = reinterpret_cast<const VecT*>(src + ((seg / group) % src_segments) * src_seg_stride + from * row_bytes) + piece;
   VecT* d = reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + to) * row_bytes) + piece;
   *d = *s;
 }
@@ -48,7 +48,7 @@ __global__ void __launch_bounds__(GS_BLOCK) gs_invert_kernel(const IdxT* __restr
 }
 
 template <typename IdxT, bool GATHER>
-static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, const void* idx, int n_segments, int64_t n,
+static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, int group, const void* idx, int n_segments, int64_t n,
                      int64_t n_src, int64_t row_bytes, void* dst, hipStream_t s) {
   const bool a16 = row_bytes % 16 == 0 && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) &&
                    src_seg_stride % 16 == 0;
@@ -61,13 +61,13 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
   LAMPA_PROF(s, "start");
   if (vec == 16)
     hipLaunchKernelGGL((gs_rows_kernel<uint4, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride, src_segments,
-                       idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
   else if (vec == 4)
     hipLaunchKernelGGL((gs_rows_kernel<uint32_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
-                       src_segments, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
   else
     hipLaunchKernelGGL((gs_rows_kernel<uint8_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
-                       src_segments, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
   return lampa_launch_status();
 }
 
@@ -75,16 +75,23 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
 // reads source segment s % src_segments (src_segments == S: one source per segment; a divisor of S: the sources
 // are shared round-robin, which is how a [1, batch, ...] tensor broadcasts over [n_hashes, batch, ...] indices). idx_bytes is 4 (int32) or 8 (int64). Out-of-range
 // indices are skipped (the destination row is left untouched).
-extern "C" int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
-                                 int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream) {
-  if (!src || !idx || !dst || n_segments < 1 || n < 0 || n_src < 0 || row_bytes < 1) return LAMPA_ERR_INVALID;
+// Segment s reads source segment (s / group) % src_segments (group = 1: the exported behaviour; group = tables per
+// event: a batch of events whose tables share the event's rows).
+int lampa_gather_rows_grouped(const void* src, int src_segments, int group, int64_t n_src, const void* idx,
+                              int idx_bytes, int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream) {
+  if (!src || !idx || !dst || n_segments < 1 || n < 0 || n_src < 0 || row_bytes < 1 || group < 1) return LAMPA_ERR_INVALID;
   if (src_segments < 1 || n_segments % src_segments != 0) return LAMPA_ERR_INVALID;
   if (idx_bytes != 4 && idx_bytes != 8) return LAMPA_ERR_INVALID;
   if (n == 0) return LAMPA_OK;
   const int64_t stride = n_src * row_bytes;
   if (idx_bytes == 4)
-    return gs_launch<int32_t, true>(src, stride, src_segments, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
-  return gs_launch<int64_t, true>(src, stride, src_segments, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
+    return gs_launch<int32_t, true>(src, stride, src_segments, group, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
+  return gs_launch<int64_t, true>(src, stride, src_segments, group, idx, n_segments, n, n_src, row_bytes, dst, (hipStream_t)stream);
+}
+
+extern "C" int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
+                                 int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream) {
+  return lampa_gather_rows_grouped(src, src_segments, 1, n_src, idx, idx_bytes, n_segments, n, row_bytes, dst, stream);
 }
 
 // dst [S, n, row_bytes]: dst[s, idx[s, i]] = src[s, i] (idx is a permutation of 0..n-1 per segment).
@@ -95,8 +102,8 @@ extern "C" int lampa_scatter_rows(const void* src, const void* idx, int idx_byte
   if (n == 0) return LAMPA_OK;
   const int64_t stride = n * row_bytes;
   if (idx_bytes == 4)
-    return gs_launch<int32_t, false>(src, stride, n_segments, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
-  return gs_launch<int64_t, false>(src, stride, n_segments, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
+    return gs_launch<int32_t, false>(src, stride, n_segments, 1, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
+  return gs_launch<int64_t, false>(src, stride, n_segments, 1, idx, n_segments, n, n, row_bytes, dst, (hipStream_t)stream);
 }
 
 // inv[s, perm[s, i]] = i

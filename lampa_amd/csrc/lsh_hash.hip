@@ -13,12 +13,18 @@
 // ---- pass 1: per-block min / max of every id column over the valid hits -------------------------------
 // partial [gridDim.x, n_cols, 2] (min, max); no atomics, no initialisation needed.
 template <int DIM>
-__global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __restrict__ coords, int64_t n_valid,
-                                                              int dim, const float* __restrict__ alpha,
+__global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __restrict__ coords, int64_t n_hits,
+                                                              int64_t n_valid,
+                                                              const int32_t* __restrict__ n_valid_dev, int dim,
+                                                              const float* __restrict__ alpha,
                                                               const float* __restrict__ beta, int n_cols,
                                                               float inv_w, int32_t* __restrict__ partial) {
   __shared__ int32_t s_min[LSH_BLOCK / 64][LSH_MAX_COLS];
   __shared__ int32_t s_max[LSH_BLOCK / 64][LSH_MAX_COLS];
+  // blockIdx.z = event of a batch: its own coords, valid count and partials
+  coords += (int64_t)blockIdx.z * n_hits * dim;
+  partial += (int64_t)blockIdx.z * gridDim.x * n_cols * 2;
+  if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
   const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
   const bool valid = n < n_valid;
   float x[LSH_MAX_DIM];
@@ -47,13 +53,21 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
 // grid (ceil(N / 256), n_tables). meta [n_tables, 2J+3] = lo[J], range[J], total, key_bits, overflow.
 template <int DIM>
 __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __restrict__ coords, int64_t n_hits,
-                                                            int64_t n_valid, int dim,
+                                                            int64_t n_valid,
+                                                            const int32_t* __restrict__ n_valid_dev, int dim,
                                                             const float* __restrict__ alpha,
                                                             const float* __restrict__ beta, int n_tables,
                                                             int n_proj, float inv_w,
                                                             const int32_t* __restrict__ partial, int n_partial,
                                                             int32_t* __restrict__ ids, int32_t* __restrict__ keys,
                                                             int32_t* __restrict__ meta) {
+  // blockIdx.z = event of a batch
+  coords += (int64_t)blockIdx.z * n_hits * dim;
+  partial += (int64_t)blockIdx.z * n_partial * (n_tables * n_proj) * 2;
+  if (ids) ids += (int64_t)blockIdx.z * (n_tables * n_proj) * n_hits;
+  keys += (int64_t)blockIdx.z * n_tables * n_hits;
+  meta += (int64_t)blockIdx.z * n_tables * (2 * n_proj + 3);
+  if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
   __shared__ int32_t s_red[2][LSH_MAX_PROJ][LSH_BLOCK / 64];
   __shared__ int32_t s_lo[LSH_MAX_PROJ];
   __shared__ uint32_t s_stride[LSH_MAX_PROJ];
@@ -179,43 +193,55 @@ extern "C" int64_t lampa_lsh_bucket_workspace_bytes(int64_t n_hits, int n_tables
   return lampa_align_up(blocks * n_tables * n_proj * 2 * (int64_t)sizeof(int32_t), 256);
 }
 
-extern "C" int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, int dim,
-                                     const float* alpha, const float* beta, int n_tables, int n_proj, float w,
-                                     int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, void* workspace,
-                                     int64_t workspace_bytes, void* stream) {
+// ids, keys and meta of n_events events of n_hits hits each (event e at offset e * n_hits rows); the valid count of
+// an event is n_valid_dev[e] (device) when given, else n_valid for all of them.
+static int lsh_bucket_keys_batch(const float* coords, int n_events, int64_t n_hits, int64_t n_valid,
+                                 const int32_t* n_valid_dev, int dim, const float* alpha, const float* beta,
+                                 int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
+                                 int32_t* meta_out, void* workspace, int64_t workspace_bytes, hipStream_t s) {
   if (!coords || !alpha || !beta || !keys_out || !meta_out) return LAMPA_ERR_INVALID;
-  if (n_hits < 0 || n_valid < 0 || n_valid > n_hits || n_hits > INT32_MAX) return LAMPA_ERR_INVALID;
+  if (n_events < 1 || n_events > 65535 || n_hits < 0 || n_valid < 0 || n_valid > n_hits || n_hits > INT32_MAX)
+    return LAMPA_ERR_INVALID;
   if (dim < 1 || dim > LSH_MAX_DIM || n_tables < 1 || n_proj < 1 || n_proj > LSH_MAX_PROJ ||
       n_tables * n_proj > LSH_MAX_COLS || !(w > 0.0f))
     return LAMPA_ERR_INVALID;
-  if (!workspace || workspace_bytes < lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj))
+  if (!workspace || workspace_bytes < n_events * lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj))
     return LAMPA_ERR_WORKSPACE;
   if (n_hits == 0) return LAMPA_OK;
-  hipStream_t s = (hipStream_t)stream;
   const float inv_w = 1.0f / w;
   const int n_cols = n_tables * n_proj;
   int32_t* partial = (int32_t*)workspace;
-  int blocks_valid = (int)((n_valid + LSH_BLOCK - 1) / LSH_BLOCK);
+  // with per-event counts on the device every block of the event takes part (blocks past the count contribute
+  // the neutral elements)
+  int blocks_valid = (int)(((n_valid_dev ? n_hits : n_valid) + LSH_BLOCK - 1) / LSH_BLOCK);
   if (blocks_valid < 1) blocks_valid = 1;
   const int blocks_all = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
   LAMPA_PROF(s, "start");
   if (dim == 4) {
-    hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
-                       beta, n_cols, inv_w, partial);
+    hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, n_valid_dev, dim, alpha, beta, n_cols, inv_w, partial);
     LAMPA_PROF(s, "lsh_minmax_kernel");
-    hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
-                       n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
-                       meta_out);
+    hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, n_tables, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, n_valid_dev, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out,
+                       keys_out, meta_out);
   } else {
-    hipLaunchKernelGGL(lsh_minmax_kernel<0>, dim3(blocks_valid), dim3(LSH_BLOCK), 0, s, coords, n_valid, dim, alpha,
-                       beta, n_cols, inv_w, partial);
+    hipLaunchKernelGGL(lsh_minmax_kernel<0>, dim3(blocks_valid, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, n_valid_dev, dim, alpha, beta, n_cols, inv_w, partial);
     LAMPA_PROF(s, "lsh_minmax_kernel");
-    hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, n_tables), dim3(LSH_BLOCK), 0, s, coords, n_hits,
-                       n_valid, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out, keys_out,
-                       meta_out);
+    hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, n_tables, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+                       n_valid, n_valid_dev, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out,
+                       keys_out, meta_out);
   }
   LAMPA_PROF(s, "lsh_pack_kernel");
   return lampa_launch_status();
+}
+
+extern "C" int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, int dim,
+                                     const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                                     int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+  return lsh_bucket_keys_batch(coords, 1, n_hits, n_valid, nullptr, dim, alpha, beta, n_tables, n_proj, w, ids_out,
+                               keys_out, meta_out, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int lampa_lsh_project_f32(const float* vecs, int n_heads, int64_t n_hits, int dim, const float* alpha,
@@ -276,14 +302,48 @@ extern "C" int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n);
 extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
                                 int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
                                 int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream);
-extern "C" int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
-                                 int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
+int lampa_gather_rows_grouped(const void* src, int src_segments, int group, int64_t n_src, const void* idx,
+                              int idx_bytes, int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
+
+extern "C" int64_t lampa_lsh_bucket_sort_batch_workspace_bytes(int n_events, int64_t n_hits, int n_tables, int n_proj) {
+  if (n_events < 1) return LAMPA_ERR_INVALID;
+  const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
+  const int64_t b = lampa_sort_workspace_bytes(n_events * n_tables, n_hits);
+  if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
+  return n_events * a + b;
+}
 
 extern "C" int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj) {
+  return lampa_lsh_bucket_sort_batch_workspace_bytes(1, n_hits, n_tables, n_proj);
+}
+
+// A batch of events in one set of launches: coords [n_events, n_hits, dim]; n_valid_dev: device int32 [n_events]
+// (NULL = every hit valid); outputs as for one event with a leading event dimension: ids [E, T*J, N], keys / perm
+// [E, T, N], meta [E, T, 2J+3], feats [E, N, row] -> feats_out [E, T, N, row]. Events are independent
+// (each has its own id ranges and key width); the sort runs over E*T segments.
+extern "C" int lampa_lsh_bucket_sort_batch(const float* coords, int n_events, int64_t n_hits,
+                                           const int32_t* n_valid_dev, int dim, const float* alpha, const float* beta,
+                                           int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
+                                           int32_t* meta_out, int32_t* perm_out, const void* feats,
+                                           int64_t feat_row_bytes, void* feats_out, int n_passes, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+  if (!perm_out || (feats && (!feats_out || feat_row_bytes < 1)) || n_events < 1) return LAMPA_ERR_INVALID;
   const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
-  const int64_t b = lampa_sort_workspace_bytes(n_tables, n_hits);
-  if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
-  return a + b;
+  if (a < 0) return LAMPA_ERR_INVALID;
+  const int64_t b = lampa_sort_workspace_bytes(n_events * n_tables, n_hits);
+  if (b < 0) return LAMPA_ERR_INVALID;
+  if (!workspace || workspace_bytes < n_events * a + b) return LAMPA_ERR_WORKSPACE;
+  int rc = lsh_bucket_keys_batch(coords, n_events, n_hits, n_hits, n_valid_dev, dim, alpha, beta, n_tables, n_proj, w,
+                                 ids_out, keys_out, meta_out, workspace, n_events * a, (hipStream_t)stream);
+  if (rc != LAMPA_OK) return rc;
+  const int stride = 2 * n_proj + 3;
+  rc = lampa_sort_pairs(keys_out, /*KEY_U32*/ 0, nullptr, n_events * n_tables, n_hits, 32, meta_out + 2 * n_proj + 1,
+                        stride, n_passes, perm_out, (char*)workspace + n_events * a, b, stream);
+  if (rc != LAMPA_OK) return rc;
+  if (feats)
+    rc = lampa_gather_rows_grouped(feats, n_events, n_tables, n_hits, perm_out, 4, n_events * n_tables, n_hits,
+                                   feat_row_bytes, feats_out, stream);
+  return rc;
 }
 
 // ids + keys + meta (lampa_lsh_bucket_keys), stable sort permutation of every table (lampa_sort_pairs on the packed
@@ -307,6 +367,6 @@ extern "C" int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_
                         n_passes, perm_out, (char*)workspace + a, b, stream);
   if (rc != LAMPA_OK) return rc;
   if (feats)
-    rc = lampa_gather_rows(feats, 1, n_hits, perm_out, 4, n_tables, n_hits, feat_row_bytes, feats_out, stream);
+    rc = lampa_gather_rows_grouped(feats, 1, 1, n_hits, perm_out, 4, n_tables, n_hits, feat_row_bytes, feats_out, stream);
   return rc;
 }

@@ -263,33 +263,54 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
 
 
 def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[torch.Tensor] = None,
-                    n_valid: Optional[int] = None, return_ids: bool = True, n_passes: int = 0):
-    """E2LSH bucketing of one event in one library call: bucket ids -> packed keys -> stable sort permutation per
-    table -> (optionally) the hit features in sorted order. Returns a dict with ids, keys, meta, perm [T, N] int32
-    and feats [T, N, D]. No host synchronisation: the sort reads the number of key bits from ``meta`` on the device."""
+                    n_valid=None, return_ids: bool = True, n_passes: int = 0):
+    """E2LSH bucketing in one library call: bucket ids -> packed keys -> stable sort permutation per table ->
+    (optionally) the hit features in sorted order. No host synchronisation: the sort reads the number of key bits
+    from ``meta`` on the device.
+
+    One event: coords [N, dim], feats [N, D], n_valid an int -> dict with ids [T*J, N], keys / perm [T, N] int32,
+    meta [T, 2J+3], feats [T, N, D].
+    A batch of events of N hits each (pad shorter ones): coords [E, N, dim], feats [E, N, D], n_valid an int32
+    tensor [E] on the device (or None) -> the same entries with a leading event dimension; one set of launches for
+    the whole batch."""
     require_cuda(coords, alpha, beta, feats)
     coords = coords.contiguous().float()
     alpha = alpha.contiguous().float()
     beta = beta.contiguous().float().reshape(-1)
-    n, dim = coords.shape
+    batched = coords.dim() == 3
+    n, dim = coords.shape[-2:]
+    n_events = coords.shape[0] if batched else 1
+    lead = (n_events,) if batched else ()
     assert alpha.shape == (dim, n_tables * n_proj) and beta.numel() == n_tables * n_proj
-    n_valid = n if n_valid is None else int(n_valid)
     dev = coords.device
-    ids = torch.empty((n_tables * n_proj, n), dtype=torch.int32, device=dev) if return_ids else None
-    keys = torch.empty((n_tables, n), dtype=torch.int32, device=dev)
-    meta = torch.empty((n_tables, 2 * n_proj + 3), dtype=torch.int32, device=dev)
-    perm = torch.empty((n_tables, n), dtype=torch.int32, device=dev)
+    ids = torch.empty(lead + (n_tables * n_proj, n), dtype=torch.int32, device=dev) if return_ids else None
+    keys = torch.empty(lead + (n_tables, n), dtype=torch.int32, device=dev)
+    meta = torch.empty(lead + (n_tables, 2 * n_proj + 3), dtype=torch.int32, device=dev)
+    perm = torch.empty(lead + (n_tables, n), dtype=torch.int32, device=dev)
     out = {"ids": ids, "keys": keys, "meta": meta, "perm": perm}
     fo, row_bytes = None, 0
     if feats is not None:
         feats = feats.contiguous()
-        assert feats.dim() == 2 and feats.shape[0] == n
-        fo = torch.empty((n_tables, n, feats.shape[1]), dtype=feats.dtype, device=dev)
-        row_bytes = feats.shape[1] * feats.element_size()
+        assert feats.shape[:-1] == coords.shape[:-1]
+        fo = torch.empty(lead + (n_tables, n, feats.shape[-1]), dtype=feats.dtype, device=dev)
+        row_bytes = feats.shape[-1] * feats.element_size()
         out["feats"] = fo
-    if n == 0:
+    if n == 0 or n_events == 0:
         return out
     lib = _capi.lib()
+    if batched:
+        nv = None
+        if n_valid is not None:
+            nv = torch.as_tensor(n_valid, dtype=torch.int32, device=dev).contiguous()
+            assert nv.shape == (n_events,)
+        ws = _workspace(check(lib.lampa_lsh_bucket_sort_batch_workspace_bytes(n_events, n, n_tables, n_proj),
+                              "workspace"), dev)
+        check(lib.lampa_lsh_bucket_sort_batch(ptr(coords), n_events, n, ptr(nv), dim, ptr(alpha), ptr(beta), n_tables,
+                                              n_proj, float(w), ptr(ids), ptr(keys), ptr(meta), ptr(perm), ptr(feats),
+                                              row_bytes, ptr(fo), n_passes, ptr(ws), ws.numel(), stream_of(coords)),
+              "lampa_lsh_bucket_sort_batch")
+        return out
+    n_valid = n if n_valid is None else int(n_valid)
     ws = _workspace(check(lib.lampa_lsh_bucket_sort_workspace_bytes(n, n_tables, n_proj), "workspace"), dev)
     check(lib.lampa_lsh_bucket_sort(ptr(coords), n, n_valid, dim, ptr(alpha), ptr(beta), n_tables, n_proj, float(w),
                                     ptr(ids), ptr(keys), ptr(meta), ptr(perm), ptr(feats), row_bytes, ptr(fo), n_passes,

@@ -147,3 +147,24 @@ def test_lsh_ordering_bit_exact_and_unsort(device):
     inv = lsh.invert_permutation(idx)
     assert torch.equal(inv.cpu(), idx.cpu().argsort(dim=1))
     assert torch.equal(lsh.gather_rows(ordered, inv).cpu(), points)
+
+
+def test_bucket_sort_batch_of_events_bit_exact(device):
+    """A batch of padded events in one set of launches equals the events one by one (and the oracle)."""
+    n_max, lens = 7000, [7000, 1, 4097, 0, 6999]
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    coords = torch.zeros(len(lens), n_max, 4)
+    feats = torch.zeros(len(lens), n_max, 24)
+    for e, n in enumerate(lens):
+        c, f, _ = synth.collider_event(n_max, seed=10 + e)
+        coords[e], feats[e] = c, f
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats.to(device),
+                              n_valid=torch.tensor(lens, dtype=torch.int32))
+    for e, n in enumerate(lens):
+        want = ol.bucket_sort(coords[e].numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats[e].numpy(), n_valid=n)
+        for name in ("ids", "meta", "keys", "perm", "feats"):
+            assert np.array_equal(_np(got[name][e]), want[name]), (name, e)
+    full = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats.to(device))
+    one = lsh.lsh_bucket_sort(coords[2].to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats[2].to(device))
+    for name in ("ids", "meta", "keys", "perm", "feats"):
+        assert torch.equal(full[name][2], one[name]), name
