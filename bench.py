@@ -193,6 +193,35 @@ def main():
                      "algorithmic_bytes": lsh_bytes},
     }
 
+    # ---- the same stage on a batch of events in one set of launches (throughput form of config 1) ----
+    n_batch = 32
+    bc, bf = [], []
+    for e in range(n_batch):
+        c_e, f_e, _ = synth.collider_event(N_HITS, seed=e)
+        bc.append(c_e)
+        bf.append(f_e)
+    bc_d, bf_d = torch.stack(bc).to(dev), torch.stack(bf).to(dev)
+
+    def lsh_batch_step():
+        return lsh.lsh_bucket_sort(bc_d, alpha_d, beta_hd, W_BUCKET, N_TABLES, N_PROJ, bf_d)
+
+    for _ in range(3):
+        lsh_batch_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        lsh_batch_step()
+    torch.cuda.synchronize()
+    batch_us = 1e6 * (time.perf_counter() - t0) / 10
+    lsh_info["batch"] = {
+        "events": n_batch, "us_per_event": round(batch_us / n_batch, 2),
+        "hits_per_s": round(n_batch * N_HITS / (batch_us * 1e-6), 1),
+        "roofline": {"bound": "hbm", "achieved": round(n_batch * lsh_bytes / (batch_us * 1e-6) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(n_batch * lsh_bytes / (batch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    del bc_d, bf_d
+
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
     if not args.no_cpu:

@@ -1,4 +1,4 @@
-// Device helpers of the E2LSH hash shared by the separate kernels and the fused single-launch kernel.
+// Device helpers of the E2LSH hash.
 // Arithmetic contract: p = fmaf(x[d], a[d], p) left to right from 0; id = floorf((p + b) * inv_w) saturated to
 // int32, NaN -> INT32_MAX. Only explicit fmaf / single operations, so compiler contraction cannot change a bit.
 #pragma once
@@ -43,3 +43,25 @@ __device__ __forceinline__ float lsh_dot(const float* x, const float* __restrict
   return acc;
 }
 
+
+// Wave-wide min / max on the VALU data-parallel-primitive path (no LDS round trips); the result is valid in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int32_t lsh_dpp(int32_t x) {
+  return __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xF, false);  // lanes without a source keep their own x
+}
+template <bool MAX>
+__device__ __forceinline__ int32_t lsh_wave_extreme(int32_t v) {
+#define LSH_STEP(CTRL, ROWS)                      \
+  {                                               \
+    const int32_t o = lsh_dpp<CTRL, ROWS>(v);     \
+    v = MAX ? max(v, o) : min(v, o);              \
+  }
+  LSH_STEP(0xB1, 0xF)   // quad_perm [1,0,3,2]
+  LSH_STEP(0x4E, 0xF)   // quad_perm [2,3,0,1]
+  LSH_STEP(0x141, 0xF)  // row_half_mirror
+  LSH_STEP(0x140, 0xF)  // row_mirror: every lane of a row of 16 holds the row's extreme
+  LSH_STEP(0x142, 0xA)  // row_bcast15 into rows 1 and 3
+  LSH_STEP(0x143, 0xC)  // row_bcast31 into rows 2 and 3
+#undef LSH_STEP
+  return v;
+}

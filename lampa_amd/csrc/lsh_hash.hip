@@ -11,7 +11,9 @@
 #include "lsh_device.h"
 
 // ---- pass 1: per-block min / max of every id column over the valid hits -------------------------------
-// partial [gridDim.x, n_cols, 2] (min, max); no atomics, no initialisation needed.
+// A block covers LSH_MM_ITEMS * 256 hits (all coordinate loads of a thread are independent). partial
+// [gridDim.x, n_cols, 2] (min, max) per event; no atomics, no initialisation needed.
+#define LSH_MM_ITEMS 8
 template <int DIM>
 __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __restrict__ coords, int64_t n_hits,
                                                               int64_t n_valid,
@@ -25,20 +27,27 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
   coords += (int64_t)blockIdx.z * n_hits * dim;
   partial += (int64_t)blockIdx.z * gridDim.x * n_cols * 2;
   if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
-  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
-  const bool valid = n < n_valid;
-  float x[LSH_MAX_DIM];
-  lsh_load_coords<DIM>(coords, valid ? n : 0, dim, x);
+  float x[LSH_MM_ITEMS][LSH_MAX_DIM];
+  bool valid[LSH_MM_ITEMS];
+#pragma unroll
+  for (int i = 0; i < LSH_MM_ITEMS; ++i) {
+    const int64_t n = ((int64_t)blockIdx.x * LSH_MM_ITEMS + i) * LSH_BLOCK + threadIdx.x;
+    valid[i] = n < n_valid;
+    lsh_load_coords<DIM>(coords, valid[i] ? n : 0, dim, x[i]);
+  }
   const int wave = threadIdx.x >> 6;
   for (int c = 0; c < n_cols; ++c) {
-    int32_t id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
-    int32_t lo = valid ? id : INT32_MAX, hi = valid ? id : INT32_MIN;
+    int32_t lo = INT32_MAX, hi = INT32_MIN;
+    const float b = beta[c];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      lo = min(lo, __shfl_xor(lo, off));
-      hi = max(hi, __shfl_xor(hi, off));
+    for (int i = 0; i < LSH_MM_ITEMS; ++i) {
+      const int32_t id = lsh_quantise(lsh_dot<DIM>(x[i], alpha, dim, n_cols, c), b, inv_w);
+      lo = valid[i] ? min(lo, id) : lo;
+      hi = valid[i] ? max(hi, id) : hi;
     }
-    if (lane_id() == 0) { s_min[wave][c] = lo; s_max[wave][c] = hi; }
+    lo = lsh_wave_extreme<false>(lo);
+    hi = lsh_wave_extreme<true>(hi);
+    if (lane_id() == 63) { s_min[wave][c] = lo; s_max[wave][c] = hi; }
   }
   __syncthreads();
   for (int c = threadIdx.x; c < n_cols; c += LSH_BLOCK) {
@@ -49,8 +58,9 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
   }
 }
 
-// ---- pass 2: reduce the partials, derive the mixed-radix strides, pack the keys ------------------------
-// grid (ceil(N / 256), n_tables). meta [n_tables, 2J+3] = lo[J], range[J], total, key_bits, overflow.
+// ---- pass 2: reduce the partials, derive the mixed-radix strides, pack the keys of every table ---------
+// grid (ceil(N / 256), 1, events): a hit's coordinates are read once for all tables.
+// meta [n_tables, 2J+3] = lo[J], range[J], total, key_bits, overflow.
 template <int DIM>
 __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __restrict__ coords, int64_t n_hits,
                                                             int64_t n_valid,
@@ -61,58 +71,49 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
                                                             const int32_t* __restrict__ partial, int n_partial,
                                                             int32_t* __restrict__ ids, int32_t* __restrict__ keys,
                                                             int32_t* __restrict__ meta) {
+  const int n_cols = n_tables * n_proj;
   // blockIdx.z = event of a batch
   coords += (int64_t)blockIdx.z * n_hits * dim;
-  partial += (int64_t)blockIdx.z * n_partial * (n_tables * n_proj) * 2;
-  if (ids) ids += (int64_t)blockIdx.z * (n_tables * n_proj) * n_hits;
+  partial += (int64_t)blockIdx.z * n_partial * n_cols * 2;
+  if (ids) ids += (int64_t)blockIdx.z * n_cols * n_hits;
   keys += (int64_t)blockIdx.z * n_tables * n_hits;
   meta += (int64_t)blockIdx.z * n_tables * (2 * n_proj + 3);
   if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
-  __shared__ int32_t s_red[2][LSH_MAX_PROJ][LSH_BLOCK / 64];
-  __shared__ int32_t s_lo[LSH_MAX_PROJ];
-  __shared__ uint32_t s_stride[LSH_MAX_PROJ];
-  __shared__ uint32_t s_total;
-  const int table = blockIdx.y;
-  const int n_cols = n_tables * n_proj;
-  const int wave = threadIdx.x >> 6;
-  for (int j = 0; j < n_proj; ++j) {
-    const int c = table * n_proj + j;
+  __shared__ int32_t s_lo[LSH_MAX_COLS], s_hi[LSH_MAX_COLS];
+  __shared__ uint32_t s_stride[LSH_MAX_COLS];
+  __shared__ uint32_t s_total[LSH_MAX_COLS];  // per table
+  // column c is reduced by the four threads 4c .. 4c+3 (n_cols <= 64)
+  {
+    const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
     int32_t lo = INT32_MAX, hi = INT32_MIN;
-    for (int b = threadIdx.x; b < n_partial; b += LSH_BLOCK) {
-      lo = min(lo, partial[((int64_t)b * n_cols + c) * 2 + 0]);
-      hi = max(hi, partial[((int64_t)b * n_cols + c) * 2 + 1]);
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      lo = min(lo, __shfl_xor(lo, off));
-      hi = max(hi, __shfl_xor(hi, off));
-    }
-    if (lane_id() == 0) { s_red[0][j][wave] = lo; s_red[1][j][wave] = hi; }
+    if (c < n_cols)
+      for (int b = part; b < n_partial; b += 4) {
+        lo = min(lo, partial[((int64_t)b * n_cols + c) * 2 + 0]);
+        hi = max(hi, partial[((int64_t)b * n_cols + c) * 2 + 1]);
+      }
+    lo = min(lo, __shfl_xor(lo, 1)); hi = max(hi, __shfl_xor(hi, 1));
+    lo = min(lo, __shfl_xor(lo, 2)); hi = max(hi, __shfl_xor(hi, 2));
+    if (c < n_cols && part == 0) { s_lo[c] = n_valid == 0 ? 0 : lo; s_hi[c] = n_valid == 0 ? 0 : hi; }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (threadIdx.x < n_tables) {
+    const int table = threadIdx.x;
     uint64_t total = 1;
     int overflow = 0;
-    int32_t lo_j[LSH_MAX_PROJ];
-    int64_t range_j[LSH_MAX_PROJ];
+    int32_t* m = meta + (int64_t)table * (2 * n_proj + 3);
     for (int j = 0; j < n_proj; ++j) {
-      int32_t lo = s_red[0][j][0], hi = s_red[1][j][0];
-      for (int w = 1; w < LSH_BLOCK / 64; ++w) { lo = min(lo, s_red[0][j][w]); hi = max(hi, s_red[1][j][w]); }
-      if (n_valid == 0) { lo = 0; hi = 0; }
-      lo_j[j] = lo;
-      range_j[j] = (int64_t)hi - (int64_t)lo + 1;
-      s_lo[j] = lo;
-      s_stride[j] = (uint32_t)total;
-      total *= (uint64_t)range_j[j];
+      const int c = table * n_proj + j;
+      const int64_t range = (int64_t)s_hi[c] - (int64_t)s_lo[c] + 1;
+      s_stride[c] = (uint32_t)total;
+      total *= (uint64_t)range;
       if (total > (uint64_t)INT32_MAX) { overflow = 1; total = (uint64_t)INT32_MAX + 1; }
-    }
-    s_total = (uint32_t)total;
-    if (blockIdx.x == 0) {
-      int32_t* m = meta + (int64_t)table * (2 * n_proj + 3);
-      for (int j = 0; j < n_proj; ++j) {
-        m[j] = lo_j[j];
-        m[n_proj + j] = range_j[j] > INT32_MAX ? INT32_MAX : (int32_t)range_j[j];
+      if (blockIdx.x == 0) {
+        m[j] = s_lo[c];
+        m[n_proj + j] = range > INT32_MAX ? INT32_MAX : (int32_t)range;
       }
+    }
+    s_total[table] = (uint32_t)total;
+    if (blockIdx.x == 0) {
       uint64_t top = (n_valid < n_hits) ? total : total - 1;
       int bits = 1;
       while (bits < 32 && (top >> bits) != 0) ++bits;
@@ -125,21 +126,22 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
   __syncthreads();
   const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
   if (n >= n_hits) return;
-  uint32_t key = s_total;
   const bool valid = n < n_valid;
   float x[LSH_MAX_DIM];
-  if (valid) lsh_load_coords<DIM>(coords, n, dim, x);
-  if (valid) key = 0;
-  for (int j = 0; j < n_proj; ++j) {
-    const int c = table * n_proj + j;
-    int32_t id = 0;
-    if (valid) {
-      id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
-      key += ((uint32_t)id - (uint32_t)s_lo[j]) * s_stride[j];
+  lsh_load_coords<DIM>(coords, valid ? n : 0, dim, x);
+  for (int table = 0; table < n_tables; ++table) {
+    uint32_t key = valid ? 0u : s_total[table];
+    for (int j = 0; j < n_proj; ++j) {
+      const int c = table * n_proj + j;
+      int32_t id = 0;
+      if (valid) {
+        id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
+        key += ((uint32_t)id - (uint32_t)s_lo[c]) * s_stride[c];
+      }
+      if (ids) ids[(int64_t)c * n_hits + n] = id;
     }
-    if (ids) ids[(int64_t)c * n_hits + n] = id;
+    keys[(int64_t)table * n_hits + n] = (int32_t)key;
   }
-  keys[(int64_t)table * n_hits + n] = (int32_t)key;
 }
 
 // ---- plain projection (the reference's E2LSH.forward, a batched [N,dim] x [dim,n_hashes] product) -----
@@ -213,7 +215,8 @@ static int lsh_bucket_keys_batch(const float* coords, int n_events, int64_t n_hi
   int32_t* partial = (int32_t*)workspace;
   // with per-event counts on the device every block of the event takes part (blocks past the count contribute
   // the neutral elements)
-  int blocks_valid = (int)(((n_valid_dev ? n_hits : n_valid) + LSH_BLOCK - 1) / LSH_BLOCK);
+  const int64_t per_block = (int64_t)LSH_BLOCK * LSH_MM_ITEMS;
+  int blocks_valid = (int)(((n_valid_dev ? n_hits : n_valid) + per_block - 1) / per_block);
   if (blocks_valid < 1) blocks_valid = 1;
   const int blocks_all = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
   LAMPA_PROF(s, "start");
@@ -221,14 +224,14 @@ static int lsh_bucket_keys_batch(const float* coords, int n_events, int64_t n_hi
     hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, n_valid_dev, dim, alpha, beta, n_cols, inv_w, partial);
     LAMPA_PROF(s, "lsh_minmax_kernel");
-    hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, n_tables, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+    hipLaunchKernelGGL(lsh_pack_kernel<4>, dim3(blocks_all, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, n_valid_dev, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out,
                        keys_out, meta_out);
   } else {
     hipLaunchKernelGGL(lsh_minmax_kernel<0>, dim3(blocks_valid, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, n_valid_dev, dim, alpha, beta, n_cols, inv_w, partial);
     LAMPA_PROF(s, "lsh_minmax_kernel");
-    hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, n_tables, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
+    hipLaunchKernelGGL(lsh_pack_kernel<0>, dim3(blocks_all, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,
                        n_valid, n_valid_dev, dim, alpha, beta, n_tables, n_proj, inv_w, partial, blocks_valid, ids_out,
                        keys_out, meta_out);
   }
