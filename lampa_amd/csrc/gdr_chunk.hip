@@ -811,202 +811,99 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 }
 
 // ---- scan ---------------------------------------------------------------------------------------------------------
-// grid (VT/32, n_seq, HV), 8 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column slab
-// of the state; Sinit [seg, HV, KT, VT] fp32 row-major receives the state every segment starts from.
-// The composite pass stores M_p as d_p I + M'_p (d_p = the segment's total decay, exact in fp32) with M' already
-// in bf16 MFMA A-operand fragment order and N_p in accumulator order, so a step is
-//   S <- d S + N + M' S      (one MFMA per fragment; the state feeds the B operand straight from the accumulator)
-// on ONE wave with no exchange of S. The chain is serial in p, so memory latency must not sit on it: all 8 waves
-// keep their 16-byte pieces of the next DEPTH steps in registers (loads issued DEPTH steps ahead) and copy them
-// into a double-buffered LDS slot one step before wave 0 consumes them.
-template <int KT>
-struct GdrScanShape {
-  static constexpr int THREADS = 512;
-  static constexpr int DEPTH = KT <= 64 ? 8 : 3;          // steps held in registers
-  static constexpr int M_BYTES = KT * KT * 2;             // M' fragments (bf16)
-  static constexpr int N_BYTES = KT * 32 * 4;             // one 32-column slab of N (fp32, accumulator order)
-  static constexpr int MP = M_BYTES / 16 / THREADS;       // 16-byte pieces per thread and step
-  static constexpr int NP = N_BYTES / 16 / THREADS;
-  static constexpr int BYTES = 2 * (M_BYTES + N_BYTES);   // two LDS slots
-};
-
-template <int KT, int VT>
-__global__ void __launch_bounds__(512) gdr_scan_kernel(const GdrPlanView pv,
-                                                      const unsigned char* __restrict__ Mcomp,
-                                                      const unsigned char* __restrict__ Ncomp,
-                                                      const float* __restrict__ Dcomp,
-                                                      const float* __restrict__ h0, float* __restrict__ Sinit,
-                                                      int HV) {
-  using SH = GdrScanShape<KT>;
-  constexpr int D = SH::DEPTH, MP = SH::MP, NP = SH::NP;
-  extern __shared__ __align__(16) unsigned char smem[];
+// grid (VT/32, n_seq, HV), KT/32 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column
+// slab of the state; Sinit receives the state every segment starts from, as 32-column slabs in accumulator order
+// (the layout the output pass loads with 16-byte reads).
+// The composite pass stores M_p as d_p I + M'_p (d_p = the segment's total decay, exact in fp32) with M' in bf16
+// MFMA A-operand fragment order and N_p in accumulator order, so a step is
+//   S <- d S + N + M' S      (one MFMA per fragment; the state feeds the B operand straight from the accumulator).
+// The chain is serial in p, so nothing else may sit on it. Wave w owns rows 32w .. 32w+31 of the slab: it loads
+// only its own row tile of M' and N (DEPTH steps ahead, straight into registers in operand order: no staging) and
+// needs the other waves' rows of the state only as B operand: every wave publishes its two operand fragments in
+// LDS (double-buffered by step parity, one LDS-only barrier per step) and starts the step's MFMAs with its own
+// fragments while the others' are on their way.
+template <int KT, int VT, int DEPTH>
+__global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanView pv,
+                                                                 const unsigned char* __restrict__ Mcomp,
+                                                                 const unsigned char* __restrict__ Ncomp,
+                                                                 const float* __restrict__ Dcomp,
+                                                                 const float* __restrict__ h0,
+                                                                 float* __restrict__ Sinit, int HV, int n_segments) {
+  constexpr int NKS = KT / 16;
+  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
   const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
   const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
   const int nsteps = nseg - 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
-  const bool compute = wave == 0;
 
-  f32x16 S[KT / 32];
+  f32x16 S = zero16();
+  if (h0) {
 #pragma unroll
-  for (int km = 0; km < KT / 32; ++km) {
-    S[km] = zero16();
-    if (compute && h0) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] = h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col];
-    }
+    for (int r = 0; r < 16; ++r) S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + col];
   }
 
-  f32x4 rm[D][MP], rn[D][NP];
-  float rd[D];
-  auto issue = [&](int p, f32x4* m, f32x4* n, float& d) {
-    const size_t sh = (size_t)(seg0 + p) * HV + hv;
-    const f32x4* M = reinterpret_cast<const f32x4*>(Mcomp + sh * SH::M_BYTES);
-    const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * SH::N_BYTES);
-#pragma unroll
-    for (int j = 0; j < MP; ++j) m[j] = M[tid + SH::THREADS * j];
-#pragma unroll
-    for (int j = 0; j < NP; ++j) n[j] = N[tid + SH::THREADS * j];
-    d = Dcomp[sh];
-  };
-#pragma unroll
-  for (int d = 0; d < D; ++d)
-    issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
-
-  for (int p0 = 0; p0 <= nsteps; p0 += D) {
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int p = p0 + d;
-      if (p > nsteps) break;
-      if (compute) {  // the state segment seg0 + p starts from (accumulator order, like N)
-        f32x4* si = reinterpret_cast<f32x4*>(Sinit + (((size_t)(seg0 + p) * HV + hv) * (VT / 32) + vn) * (KT * 32));
-#pragma unroll
-        for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 t;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
-            si[(km * 4 + q4) * 64 + lane] = t;
-          }
-      }
-      if (p == nsteps) break;
-      unsigned char* s_M = smem + (p & 1) * (SH::M_BYTES + SH::N_BYTES);
-      unsigned char* s_N = s_M + SH::M_BYTES;
-#pragma unroll
-      for (int j = 0; j < MP; ++j) reinterpret_cast<f32x4*>(s_M)[tid + SH::THREADS * j] = rm[d][j];
-#pragma unroll
-      for (int j = 0; j < NP; ++j) reinterpret_cast<f32x4*>(s_N)[tid + SH::THREADS * j] = rn[d][j];
-      const float dec = rd[d];
-      issue(min(p + D, nsteps - 1), rm[d], rn[d], rd[d]);  // unconditional: keeps the load count per step fixed
-      lds_barrier();
-      if (compute) {
-        bf16x8 Sb[KT / 16];
-#pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
-        f32x16 Snew[KT / 32];
-#pragma unroll
-        for (int tm = 0; tm < KT / 32; ++tm) {
-          f32x16 acc;
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const f32x4 nv = reinterpret_cast<const f32x4*>(s_N)[(tm * 4 + q4) * 64 + lane];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[tm][4 * q4 + e], nv[e]);
-          }
-#pragma unroll
-          for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(frag_load(s_M, tm * (KT / 16) + ks, lane), Sb[ks], acc);
-          Snew[tm] = acc;
-        }
-#pragma unroll
-        for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
-      }
-    }
-  }
-}
-
-// Single-wave variant for KT = 64: one wave per (32-column slab, sequence, head), no LDS and no barrier. The
-// operands of the next DEPTH steps (M' fragments, the N slab and d) sit in registers, loaded straight from HBM in
-// operand order DEPTH steps ahead, so the serial chain is MFMA + conversion latency only.
-template <int KT, int VT, int DEPTH>
-__global__ void __launch_bounds__(64, 1) gdr_scan_wave_kernel(const GdrPlanView pv,
-                                                             const unsigned char* __restrict__ Mcomp,
-                                                             const unsigned char* __restrict__ Ncomp,
-                                                             const float* __restrict__ Dcomp,
-                                                             const float* __restrict__ h0, float* __restrict__ Sinit,
-                                                             int HV) {
-  constexpr int MF = (KT / 32) * (KT / 16), NF = (KT / 32) * 4;
-  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
-  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
-  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
-  const int nsteps = nseg - 1;
-  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
-  const int col = 32 * vn + ln;
-
-  f32x16 S[KT / 32];
-#pragma unroll
-  for (int km = 0; km < KT / 32; ++km) {
-    S[km] = zero16();
-    if (h0) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[km][r] = h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col];
-    }
-  }
-
-  bf16x8 rm[DEPTH][MF];
-  f32x4 rn[DEPTH][NF];
+  bf16x8 rm[DEPTH][NKS];
+  f32x4 rn[DEPTH][4];
   float rd[DEPTH];
   auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
     const size_t sh = (size_t)(seg0 + p) * HV + hv;
     const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
     const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * N_BYTES);
 #pragma unroll
-    for (int f = 0; f < MF; ++f) m[f] = M[f * 64 + lane];
+    for (int j = 0; j < NKS; ++j) m[j] = M[(wave * NKS + (2 * wave + j) % NKS) * 64 + lane];  // own fragments first
 #pragma unroll
-    for (int j = 0; j < NF; ++j) n[j] = N[j * 64 + lane];
+    for (int q4 = 0; q4 < 4; ++q4) n[q4] = N[(wave * 4 + q4) * 64 + lane];
     d = Dcomp[sh];
   };
+  // (every step issues the same loads, clamped at the end, so that the waits can leave younger loads in flight)
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
 
-  for (int p0 = 0; p0 <= nsteps; p0 += DEPTH) {
+  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+    {  // the state segment seg0 + p starts from; steps past the end write to the spare slot behind the last segment
+      const size_t slot = p <= nsteps ? (size_t)(seg0 + p) : (size_t)n_segments;
+      f32x4* si = reinterpret_cast<f32x4*>(Sinit + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int p = p0 + d;
-      if (p > nsteps) break;
-      {  // the state segment seg0 + p starts from
-        f32x4* si = reinterpret_cast<f32x4*>(Sinit + (((size_t)(seg0 + p) * HV + hv) * (VT / 32) + vn) * (KT * 32));
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
 #pragma unroll
-        for (int km = 0; km < KT / 32; ++km)
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 t;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
-            si[(km * 4 + q4) * 64 + lane] = t;
-          }
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        si[(wave * 4 + q4) * 64 + lane] = t;
       }
-      if (p == nsteps) break;
-      const float dec = rd[d];
-      bf16x8 Sb[KT / 16];
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
-      f32x16 Snew[KT / 32];
-#pragma unroll
-      for (int tm = 0; tm < KT / 32; ++tm) {
-        f32x16 acc;
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[tm][4 * q4 + e], rn[d][tm * 4 + q4][e]);
-#pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(rm[d][tm * (KT / 16) + ks], Sb[ks], acc);
-        Snew[tm] = acc;
-      }
-#pragma unroll
-      for (int tm = 0; tm < KT / 32; ++tm) S[tm] = Snew[tm];
-      issue(min(p + DEPTH, nsteps - 1), rm[d], rn[d], rd[d]);  // unconditional: keeps the load count per step fixed
     }
+    const float dec = dd;
+    unsigned char* xbuf = s_x[p & 1];
+    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
+    frag_store(xbuf, 2 * wave + 0, lane, own0);
+    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    f32x16 acc;
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[4 * q4 + e], n[q4][e]);
+    acc = mfma32(m[0], own0, acc);
+    acc = mfma32(m[1], own1, acc);
+    lds_barrier();
+#pragma unroll
+    for (int j = 2; j < NKS; ++j) acc = mfma32(m[j], frag_load(xbuf, (2 * wave + j) % NKS, lane), acc);
+    S = acc;
+    issue(max(0, min(p + DEPTH, nsteps - 1)), m, n, dd);
+  };
+  // The step loops have NO early exit: they run in whole groups, and the steps past the last segment work on clamped
+  // operands and store to the spare slot. With a branch around a step the compiler can no longer count the loads in
+  // flight and waits for all of them at every step; and since it drains the queue at every loop header anyway (the
+  // ring registers are loaded in one iteration and used in the next), the main loop covers LONG groups of steps.
+  constexpr int LONG = 4 * DEPTH;
+  int p0 = 0;
+  for (; p0 + LONG <= nsteps + 1; p0 += LONG) {
+#pragma unroll
+    for (int u = 0; u < LONG; ++u) step(p0 + u, rm[u % DEPTH], rn[u % DEPTH], rd[u % DEPTH]);
+  }
+  for (; p0 <= nsteps; p0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) step(p0 + d, rm[d], rn[d], rd[d]);
   }
 }
 
@@ -1022,7 +919,7 @@ static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, i
   w.off_m = off;     off += lampa_align_up(segs * HV * (int64_t)K * K * 2, 256);
   w.off_n = off;     off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.off_d = off;     off += lampa_align_up(segs * HV * 4, 256);
-  w.off_sinit = off; off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
+  w.off_sinit = off; off += lampa_align_up((segs + 1) * HV * (int64_t)K * V * 4, 256);  // + a spare slot (scan)
   w.bytes = off > 0 ? off : 256;
   return w;
 }
@@ -1051,9 +948,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
     if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
         hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, true>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess ||
-        hipFuncSetAttribute((const void*)gdr_scan_kernel<KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            GdrScanShape<KT>::BYTES) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
     attr_set = true;
   }
@@ -1069,12 +964,8 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
-  if constexpr (KT == 64)
-    hipLaunchKernelGGL((gdr_scan_wave_kernel<KT, VT, 5>), dim3(VT / 32, n_seq, HV), dim3(64), 0, s, pv, Mc, Nc, Dc,
-                       h0, Si, HV);
-  else
-    hipLaunchKernelGGL((gdr_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(512), GdrScanShape<KT>::BYTES, s,
-                       pv, Mc, Nc, Dc, h0, Si, HV);
+  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
+                     pv, Mc, Nc, Dc, h0, Si, HV, segs);
   LAMPA_PROF(s, "gdr_scan_kernel");
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
                      (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
