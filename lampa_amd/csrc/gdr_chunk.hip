@@ -326,26 +326,38 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
 // over the tokens (K^T, and v in accumulator layout) are read from the row-major tiles with the transposing LDS
 // load (ds_read_b64_tr_b16), so no transposed copy is ever written.
 //
-// LDS is single-buffered but released early. Per chunk c the two roles meet at three LDS-only barriers:
-//   A(c)  k, v, T, factors and (PASS_B) q of chunk c are staged
-//   X(c)  the chain waves hold every k / v / T operand of chunk c in registers (and P(c) is in LDS)
-//         -> the stagers overwrite the tiles with chunk c+1 while the chain waves finish chunk c
-//   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c -> the stagers write q(c+1)
-// Global loads are issued one full chunk period before their data is staged.
+// The k, v, T tiles and the per-token factors are DOUBLE-buffered in LDS, so the stagers fill the tiles of chunk c+1
+// while the chain waves work on chunk c; q, P and the o tile exist once. LDS-only barriers per chunk (every barrier is
+// a rendezvous of all waves, so the stagers' work is spread such that they are never the slower side):
+//   Qb(c) (PASS_B) q(c) is staged                         -> the stagers build P(c)
+//   B(c)  the chain waves hold every k / v / T operand of chunk c in registers, and tiles (c+1) [PASS_A: also its
+//         factors] and P(c) are complete                   -> buffer c%2 is free for chunk c+2
+//   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
+//                                                          -> the stagers may write q(c+1)
+// Global loads are issued about one chunk period before their data is staged.
 template <int KT, int VT, bool PASS_B>
 struct GdrSegSmem {
   static constexpr int SK = KT + 8;  // row stride of the k / q tiles (bf16 elements)
   static constexpr int SV = VT + 8;  // row stride of the v and o tiles
-  static constexpr int ST = 72;      // row stride of T
-  static constexpr int OFF_K = 0;
-  static constexpr int OFF_V = OFF_K + 64 * SK * 2;
-  static constexpr int OFF_T = OFF_V + 64 * SV * 2;
-  static constexpr int OFF_Q = OFF_T + 64 * ST * 2;
+  static constexpr int ST = 40;      // row stride of a 32x32 block of T (blocks T11, T21, T22)
+  // one set of tiles (two of them)
+  static constexpr int T_OFF_K = 0;
+  static constexpr int T_OFF_V = T_OFF_K + 64 * SK * 2;
+  static constexpr int T_OFF_T = T_OFF_V + 64 * SV * 2;
+  static constexpr int T_OFF_F = T_OFF_T + 3 * 32 * ST * 2;
+  static constexpr int N_FACT = 6;  // beta, ek, dk, gamma, rk, misc
+  static constexpr int TILE_BYTES = T_OFF_F + N_FACT * 64 * 4;
+  static constexpr int OFF_Q = 2 * TILE_BYTES;
   static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
   static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
-  static constexpr int OFF_SCAL = OFF_O + (PASS_B ? 64 * SV * 2 : 0);
-  static constexpr int N_SCAL = 8;  // beta, ek, dk, qs, gamma, rk, rq, misc
-  static constexpr int BYTES = OFF_SCAL + N_SCAL * 64 * 4;
+  static constexpr int OFF_QF = OFF_O + (PASS_B ? 64 * SV * 2 : 0);  // qs, rq
+  static constexpr int BYTES = OFF_QF + (PASS_B ? 2 * 64 * 4 : 0);
+};
+
+// pointers into one of the two tile sets
+struct GdrTiles {
+  __bf16 *k, *v, *t;
+  float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
 };
 
 template <int KT, int VT, bool PASS_B>
@@ -393,20 +405,25 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
   extern __shared__ __align__(16) unsigned char smem[];
-  __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
-  __bf16* s_v = reinterpret_cast<__bf16*>(smem + SM::OFF_V);
-  __bf16* s_T = reinterpret_cast<__bf16*>(smem + SM::OFF_T);
+  auto tiles = [&](int par) {
+    unsigned char* base = smem + par * SM::TILE_BYTES;
+    GdrTiles t;
+    t.k = reinterpret_cast<__bf16*>(base + SM::T_OFF_K);
+    t.v = reinterpret_cast<__bf16*>(base + SM::T_OFF_V);
+    t.t = reinterpret_cast<__bf16*>(base + SM::T_OFF_T);
+    t.beta = reinterpret_cast<float*>(base + SM::T_OFF_F);
+    t.ek = t.beta + 64;
+    t.dk = t.beta + 128;
+    t.gamma = t.beta + 192;
+    t.rk = t.beta + 256;
+    t.misc = t.beta + 320;
+    return t;
+  };
   __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
   unsigned char* s_P = smem + SM::OFF_P;
   T* s_o = reinterpret_cast<T*>(smem + SM::OFF_O);
-  float* s_beta = reinterpret_cast<float*>(smem + SM::OFF_SCAL);
-  float* s_ek = s_beta + 64;     // e^{gamma_i} rk_i
-  float* s_dk = s_beta + 128;    // e^{gamma_last - gamma_i} rk_i
-  float* s_qs = s_beta + 192;    // scale e^{gamma_i} rq_i
-  float* s_gamma = s_beta + 256;
-  float* s_rk = s_beta + 320;
-  float* s_rq = s_beta + 384;
-  float* s_misc = s_beta + 448;  // [0] = e^{gamma_last}
+  float* s_qs = reinterpret_cast<float*>(smem + SM::OFF_QF);  // scale e^{gamma_i} rq_i
+  float* s_rq = s_qs + 64;
 
   const int seg = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
@@ -430,7 +447,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
-    auto issue_tiles = [&](int c) {
+    auto issue_tiles = [&](int c) {  // k, v, T
       c = uniform(c);
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* kb = k + ((size_t)tok0 * H + h) * KT;
@@ -444,11 +461,13 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * T_BYTES);
 #pragma unroll
       for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
-      const float* gb = g + (size_t)tok0 * HV + hv;
-      const float* bb = beta + (size_t)tok0 * HV + hv;
+    };
+    auto issue_gb = [&](int c) {  // g, beta (lane = token)
+      c = uniform(c);
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const int gl = min(lane, len - 1) * HV;
-      rg = gb[gl];
-      rb = bb[gl];
+      rg = (g + (size_t)tok0 * HV + hv)[gl];
+      rb = (beta + (size_t)tok0 * HV + hv)[gl];
     };
     auto issue_q = [&](int c, typename Raw8<T>::type* rq_) {
       c = uniform(c);
@@ -464,26 +483,28 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     const bool want_ss = l2norm != GDR_L2_NONE;
 
     float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
-    // k, v and T of chunk c from the registers to LDS
-    auto stage_data = [&](int c) {
+    // k, v and T of chunk c from the registers to tile set par
+    auto stage_data = [&](int c, int par) {
+      const GdrTiles tl = tiles(par);
       const bool live = srow < chunk_len[uniform(c)];
 #pragma unroll
-      for (int j = 0; j < 3; ++j)  // the upper-right block of s_T is never read
-        *reinterpret_cast<bf16x8*>(&s_T[((j > 0 ? 32 : 0) + (stid >> 2)) * ST + (j == 2 ? 32 : 0) + 8 * (stid & 3)]) = rt_[j];
+      for (int j = 0; j < 3; ++j)
+        *reinterpret_cast<bf16x8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
       kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
-        *reinterpret_cast<bf16x8*>(&s_k[srow * SK + spart * (KT / 2) + 8 * u]) =
+        *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) =
             raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         float unused = 0.0f;
-        *reinterpret_cast<bf16x8*>(&s_v[srow * SV + spart * (VT / 2) + 8 * u]) =
+        *reinterpret_cast<bf16x8*>(&tl.v[srow * SV + spart * (VT / 2) + 8 * u]) =
             raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
       }
     };
-    // per-token factors of chunk c (gate, beta, norms)
-    auto stage_factors = [&](int c) {
+    // per-token factors of chunk c (gate, beta, norms) into tile set par
+    auto stage_factors = [&](int c, int par) {
+      const GdrTiles tl = tiles(par);
       const int len = chunk_len[uniform(c)];
       const float bv = lane < len ? rb : 0.0f;
       // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction), lane = token
@@ -495,12 +516,12 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const float brow = __shfl(bv, srow);
       if (spart == 0) {
         const float rk = l2_factor(kss2, l2norm);
-        s_beta[srow] = brow;
-        s_ek[srow] = __builtin_amdgcn_exp2f(grow) * rk;
-        s_dk[srow] = __builtin_amdgcn_exp2f(g_last - grow) * rk;
-        s_gamma[srow] = grow;
-        s_rk[srow] = rk;
-        if (srow == 0) s_misc[0] = __builtin_amdgcn_exp2f(g_last);
+        tl.beta[srow] = brow;
+        tl.ek[srow] = __builtin_amdgcn_exp2f(grow) * rk;
+        tl.dk[srow] = __builtin_amdgcn_exp2f(g_last - grow) * rk;
+        tl.gamma[srow] = grow;
+        tl.rk[srow] = rk;
+        if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
       }
     };
     auto stage_q = [&](int c, const typename Raw8<T>::type* rq_) {
@@ -518,88 +539,81 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       }
     };
 
-    // All loads of a chunk (k, v, T, g, beta and q) are issued at ONE point, a full chunk period before the wait
-    // that precedes the staging of its tiles, so no wait ever has to leave younger loads in flight (the compiler
-    // drains the whole queue at such waits as soon as the control flow between issue and use is not trivial).
-    // q is staged half a period after the tiles, hence two q register sets, used by even and odd chunks in turn.
-    // The chunk index is clamped at the end of the segment (the last chunk is fetched again for nothing).
-    auto issue_chunk = [&](int c, typename Raw8<T>::type* rq_) {
-      issue_tiles(c);
-      if constexpr (PASS_B) issue_q(c, rq_);
-    };
-    auto build_p = [&]() {
+    auto build_p = [&](int par) {
       if constexpr (PASS_B) {
-        // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tiles 0 and 2, stager 1
-        // tile 1.
-        auto p_tile = [&](int t) {
+        const GdrTiles tl = tiles(par);
+        // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tile 0, stager 1 tile 2,
+        // and they share tile 1: both run its four MFMAs, each finishes and stores one of its two fragments.
+        auto p_tile = [&](int t, int half) {  // half: -1 = whole tile, 0 / 1 = accumulator registers 0-7 / 8-15
           const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
           bf16x8 fa[KT / 16], fb[KT / 16];
 #pragma unroll
           for (int ks = 0; ks < KT / 16; ++ks) {
-            fa[ks] = *reinterpret_cast<const bf16x8*>(&s_k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
+            fa[ks] = *reinterpret_cast<const bf16x8*>(&tl.k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
             fb[ks] = *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
           }
           f32x4 gj[4], rj[4];  // gamma_j, rk_j of this lane's 16 accumulator rows
 #pragma unroll
           for (int b4 = 0; b4 < 4; ++b4) {
-            gj[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * jm + 8 * b4 + 4 * hh]);
-            rj[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * jm + 8 * b4 + 4 * hh]);
+            gj[b4] = *reinterpret_cast<const f32x4*>(&tl.gamma[32 * jm + 8 * b4 + 4 * hh]);
+            rj[b4] = *reinterpret_cast<const f32x4*>(&tl.rk[32 * jm + 8 * b4 + 4 * hh]);
           }
           const int i = 32 * tn + ln;
-          const float gi = s_gamma[i], fi = scale * s_rq[i];
+          const float gi = tl.gamma[i], fi = scale * s_rq[i];
           lds_fence();
           f32x16 acc = zero16();
 #pragma unroll
           for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {  // the mask goes on the exponent so that the code stays branch-free
-            const int j = 32 * jm + acc_row(r, hh);
-            acc[r] *= fi * rj[r / 4][r % 4] * __builtin_amdgcn_exp2f(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
-          }
           const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
-          frag_store(s_P, f0 + 0, lane, acc_to_operand(acc, 0));
-          frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
+#pragma unroll
+          for (int part = 0; part < 2; ++part) {
+            if (half >= 0 && half != part) continue;
+#pragma unroll
+            for (int r = 8 * part; r < 8 * part + 8; ++r) {  // the mask goes on the exponent: branch-free
+              const int j = 32 * jm + acc_row(r, hh);
+              acc[r] *= fi * rj[r / 4][r % 4] * __builtin_amdgcn_exp2f(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
+            }
+            frag_store(s_P, f0 + part, lane, acc_to_operand(acc, 8 * part));
+          }
         };
-        p_tile(sw);
-        if (sw == 0) p_tile(2);
+        p_tile(sw == 0 ? 0 : 2, -1);
+        p_tile(1, sw);
       }
     };
-    // What a stager does between X(c) and X(c+1), spread over the three intervals so that in each of them it needs
-    // no longer than the chain waves (every barrier is a rendezvous: an interval lasts as long as its slower side).
-    // The loop below starts at a point where the loads that were issued one period ago have to have arrived
-    // anyway. Returns false after the last chunk. q(c) / q(c+2) use rq_same, q(c+1) uses rq_other.
-    auto half_step = [&](int c, typename Raw8<T>::type* rq_same, typename Raw8<T>::type* rq_other) -> bool {
-      const int cn = min(c + 1, c1 - 1), cnn = min(c + 2, c1 - 1);  // (clamped: the last chunk is fetched again)
-      stage_data(cn);
-      if constexpr (PASS_B) {
-        lds_barrier();  // C(c)
-        if (c + 1 >= c1) return false;
-        stage_factors(cn);
-        stage_q(cn, rq_other);
-        issue_chunk(cnn, rq_same);
-        lds_barrier();  // A(c+1)
-        build_p();
-      } else {
-        if (c + 1 >= c1) return false;
-        stage_factors(cn);
-        lds_barrier();  // A(c+1)
-        issue_chunk(cnn, rq_same);
-      }
-      lds_barrier();  // X(c+1)
-      return true;
-    };
+    // Chunk indices past the end of the segment are clamped (the last chunk is fetched again for nothing), so that
+    // every iteration issues the same loads: with conditional issues the compiler could not count the loads in
+    // flight any more and would drain the queue at every wait. q(c) / q(c+2) share a register set.
+    const int cl = c1 - 1;
     if (nc > 0) {
-      issue_chunk(c0, rq0_);
-      stage_data(c0);
-      stage_factors(c0);
-      if constexpr (PASS_B) stage_q(c0, rq0_);
-      issue_chunk(min(c0 + 1, c1 - 1), rq1_);
-      lds_barrier();  // A(c0)
-      build_p();
-      lds_barrier();  // X(c0)
-      for (int c = c0;; c += 2) {
-        if (!half_step(c, rq0_, rq1_)) break;
-        if (!half_step(c + 1, rq1_, rq0_)) break;
+      issue_tiles(c0);
+      issue_gb(c0);
+      if constexpr (PASS_B) { issue_q(c0, rq0_); issue_q(min(c0 + 1, cl), rq1_); }
+      stage_data(c0, 0);
+      stage_factors(c0, 0);
+      issue_tiles(min(c0 + 1, cl));
+      issue_gb(min(c0 + 1, cl));
+      lds_barrier();  // tiles (c0) are ready
+      auto one_chunk = [&](int c, int par, typename Raw8<T>::type* rq_) {
+        if (c + 1 < c1) stage_data(c + 1, par ^ 1);
+        issue_tiles(min(c + 2, cl));
+        if constexpr (PASS_B) {
+          stage_q(c, rq_);
+          issue_q(min(c + 2, cl), rq_);
+          lds_barrier();  // Qb(c)
+          build_p(par);
+          lds_barrier();  // B(c)
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          issue_gb(min(c + 2, cl));
+          lds_barrier();  // C(c)
+        } else {
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          issue_gb(min(c + 2, cl));
+          lds_barrier();  // B(c)
+        }
+      };
+      for (int c = c0; c < c1; c += 2) {
+        one_chunk(c, 0, rq0_);
+        if (c + 1 < c1) one_chunk(c + 1, 1, rq1_);
       }
     }
     return;
@@ -634,14 +648,16 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   // The LDS operand reads of a stage are issued as one batch one stage ahead of the MFMAs that use them
   // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
   // pays the LDS latency once per MFMA.
+  if (nc > 0) lds_barrier();  // tiles (c0) are ready
   for (int c = c0; c < c1; ++c) {
-    lds_barrier();  // A(c)
+    const GdrTiles tl = tiles((c - c0) & 1);
+    if constexpr (PASS_B) lds_barrier();  // Qb(c) (the chain waves only take part)
     bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
     bf16x8 ft[6];              // T (stage 2), P (output)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(s_k, SK, 32 * tm + ln, 16 * ks, hh);
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
     bf16x8 Sb[KT / 16];
 #pragma unroll
     for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
@@ -650,17 +666,18 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int ks = 0; ks < 2 * (tm + 1); ++ks) ft[2 * tm + ks] = ld_kappa(s_T, ST, 32 * tm + ln, 16 * ks, hh);
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks)  // blocks T11 | T21, T22
+        ft[2 * tm + ks] = ld_kappa(tl.t + (tm == 0 ? 0 : (ks < 2 ? 1 : 2)) * 32 * ST, ST, ln, 16 * (ks & 1), hh);
     f32x4 be[8], ek[8];
     bf16x4 vv[8];
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
       const int i0 = 8 * t8 + 4 * hh;
-      be[t8] = *reinterpret_cast<const f32x4*>(&s_beta[i0]);
-      ek[t8] = *reinterpret_cast<const f32x4*>(&s_ek[i0]);
+      be[t8] = *reinterpret_cast<const f32x4*>(&tl.beta[i0]);
+      ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
       // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
       // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
-      vv[t8] = ld_col4(s_v, SV, 32 * vslab, 8 * t8, lane);
+      vv[t8] = ld_col4(tl.v, SV, 32 * vslab, 8 * t8, lane);
     }
     bf16x8 Rb[4];
 #pragma unroll
@@ -682,11 +699,11 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(s_k, SK, 32 * km, 16 * ks, lane);
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.k, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
 #pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&s_dk[8 * t8 + 4 * hh]);
-    const float dec = s_misc[0];
+    for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
+    const float dec = tl.misc[0];
     bf16x8 Vb[4], Vsb[4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {  // v_new = T R (T is lower triangular: tile tm needs 2 (tm + 1) steps)
@@ -703,7 +720,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
     lds_fence();
-    lds_barrier();  // X(c): every operand that comes from the k, v and T tiles of chunk c is in registers
+    lds_barrier();  // B(c): every operand that comes from the k, v and T tiles of chunk c is in registers
     dtot *= dec;
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km) {  // S <- dec S + K^T (dk v_new)
