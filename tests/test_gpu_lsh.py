@@ -81,6 +81,30 @@ def test_stable_argsort_full_range_and_values(device):
     assert np.array_equal(_np(lsh.stable_argsort(keys.to(device))), want)
 
 
+def test_stable_argsort_per_segment_device_bits(device):
+    """Segments whose significant key bits differ (read from device memory) take different numbers of radix passes in
+    the same launch: 1-bit, one-digit, just over one digit, two digits and just over, three digits and 32-bit keys."""
+    gen = torch.Generator().manual_seed(7)
+    bits = [1, 5, 11, 12, 22, 23, 32]
+    n = 9000
+    rows = []
+    for b in bits:
+        r = torch.randint(0, 1 << min(b, 31), (n,), generator=gen, dtype=torch.int64)
+        if b == 32:
+            r = r * 2 + torch.randint(0, 2, (n,), generator=gen, dtype=torch.int64)
+        rows.append(r)
+    keys64 = torch.stack(rows)
+    keys = keys64.to(torch.int32) if max(bits) < 32 else (keys64 - ((keys64 >> 31) << 32)).to(torch.int32)
+    want = torch.sort(keys64, dim=-1, stable=True).indices
+    # stride 2: the bit counts sit in every other element, as in the per-table meta rows of the bucket keys
+    bits_dev = torch.zeros(len(bits) * 2, dtype=torch.int32)
+    bits_dev[::2] = torch.tensor(bits, dtype=torch.int32)
+    for passes in (0, 3, 4):
+        got = lsh.stable_argsort(keys.to(device), key_bits_dev=bits_dev.to(device), key_bits_stride=2,
+                                 n_passes=passes, unsigned=True)
+        assert torch.equal(got.cpu().long(), want), passes
+
+
 def test_gather_scatter_invert_roundtrip(device):
     gen = torch.Generator().manual_seed(1)
     for d, dtype in ((24, torch.float32), (5, torch.float32), (3, torch.int16), (64, torch.bfloat16)):
