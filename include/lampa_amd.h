@@ -118,6 +118,25 @@ int lampa_scatter_rows(const void* src, const void* idx, int idx_bytes, int n_se
 /* inv[s, perm[s, i]] = i. Replaces invert_permutation (hash_utils.py:46-57). */
 int lampa_invert_perm(const void* perm, int idx_bytes, int n_segments, int64_t n, void* inv, void* stream);
 
+/* 1-based quantile region of every hit for each row's number of regions. Replaces quantile_partition
+ * (models/model_utils/hash_utils.py:14-26). rank [n] (idx_bytes 4 or 8): position of the hit in the coordinate order
+ * (inverse of the argsort); regions [n_rows] device float32 > 0; out [n_rows, n] float32 =
+ * floor(rank / ceil(n / regions[r])) + 1. n <= 2^24. */
+int lampa_quantile_regions(const void* rank, int idx_bytes, int64_t n, const float* regions, int n_rows, float* out,
+                           void* stream);
+
+/* Region shift of the AND-hash. Replaces get_geo_shift (models/attention/hept.py:78-88).
+ * out [n_rows, n] = (region_phi * hash_shift[r]) * (ceil(regions_eta[r]) + 1) + region_eta * hash_shift[r]. */
+int lampa_geo_shift(const float* region_eta, const float* region_phi, const float* hash_shift,
+                    const float* regions_eta, int n_rows, int64_t n, float* out, void* stream);
+
+/* Sort keys of the HEPT bucketing in one pass. Replaces the arithmetic between lsh_mapping and argsort in
+ * HEPTAttention.forward (models/attention/hept.py:127-136) without materialising the region indices.
+ * hashed, keys [n_rows, n]; rank_eta, rank_phi [n] int32; regions [2, n_rows] (eta row, then phi row);
+ * hash_shift [n_rows]; hits at or beyond n_raw get +inf before the shift is added. n <= 2^24. */
+int lampa_hept_sort_keys(const float* hashed, const int32_t* rank_eta, const int32_t* rank_phi, const float* regions,
+                         const float* hash_shift, int n_rows, int64_t n, int64_t n_raw, float* keys, void* stream);
+
 /* ---------------------------------------------------------------------------------------- gated-delta forward */
 
 /* Token-serial forward with an fp32 state. Replaces fused_recurrent_gated_delta_rule_fwd

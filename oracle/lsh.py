@@ -1,8 +1,8 @@
 """CPU oracle for the LSH stage (TEST INFRASTRUCTURE ONLY).
 
 Thin numpy front-ends to ``lsh_oracle.c`` plus independent brute-force restatements used to pin it.
-Reference lines restated: ``models/model_utils/hash_utils.py:46-57,83-93,333-371``,
-``models/attention/hept.py:9-19,79-88``, ``models/baselines/full_mamba2.py:155-218,678-682``.
+Reference lines restated: ``models/model_utils/hash_utils.py:14-26,46-57,83-93,333-371``,
+``models/attention/hept.py:9-19,78-88,130-136``, ``models/baselines/full_mamba2.py:155-218,678-682``.
 """
 import ctypes
 
@@ -125,3 +125,34 @@ def bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats=None, n_valid=No
     if feats is not None:
         out["feats"] = gather_rows(feats, perm)
     return out
+
+
+# ------------------------------------------------------------------------------- HEPT region (AND-hash) front end
+def quantile_regions(sorted_indices: np.ndarray, regions: np.ndarray) -> np.ndarray:
+    """``hash_utils.py:14-26``: out[r, n] = floor(rank[n] / ceil(N / regions[r])) + 1 in float32, where rank is the
+    inverse of ``sorted_indices`` (the position of hit n in the coordinate order)."""
+    sorted_indices = np.asarray(sorted_indices, np.int64)
+    n = sorted_indices.shape[-1]
+    rank = np.empty(n, np.int64)
+    rank[sorted_indices] = np.arange(n)
+    size = np.ceil(np.float32(n) / np.asarray(regions, np.float32).reshape(-1, 1))
+    return (np.floor(rank.astype(np.float32)[None] / size) + np.float32(1)).astype(np.float32)
+
+
+def geo_shift(regions_eta: np.ndarray, hash_shift: np.ndarray, region_eta: np.ndarray, region_phi: np.ndarray):
+    """``hept.py:78-88``: (region_phi * shift) * (ceil(regions_eta) + 1) + region_eta * shift, each product and the
+    sum rounded once to float32. regions_eta, hash_shift [R]; region_* [R, N]."""
+    shift = np.asarray(hash_shift, np.float32).reshape(-1, 1)
+    mult = np.ceil(np.asarray(regions_eta, np.float32).reshape(-1, 1)) + np.float32(1)
+    a = (np.asarray(region_phi, np.float32) * shift) * mult
+    b = np.asarray(region_eta, np.float32) * shift
+    return (a + b).astype(np.float32)
+
+
+def hept_sort_keys(hashed: np.ndarray, sorted_eta, sorted_phi, regions: np.ndarray, hash_shift, n_raw: int):
+    """``hept.py:130-136``: hashed [R, N] with +inf at and beyond n_raw, plus the region shift. regions [2, R]."""
+    h = np.array(hashed, np.float32, copy=True)
+    h[:, n_raw:] = np.inf
+    reg_eta = quantile_regions(sorted_eta, regions[0])
+    reg_phi = quantile_regions(sorted_phi, regions[1])
+    return (h + geo_shift(regions[0], hash_shift, reg_eta, reg_phi)).astype(np.float32)

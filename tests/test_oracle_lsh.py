@@ -145,3 +145,74 @@ def test_config1_pipeline_properties():
         assert np.all(np.diff(out["perm"][t])[ties] > 0)  # stability: equal keys keep input order
         assert np.array_equal(np.sort(out["perm"][t]), np.arange(60000))
         assert np.array_equal(out["feats"][t], feats[out["perm"][t]])
+
+
+# ------------------------------------------------------------------------------- HEPT region (AND-hash) front end
+def test_quantile_regions_against_python_integers_and_invariants():
+    rng = np.random.default_rng(3)
+    n = 1003
+    coord = rng.permutation(n).astype(np.float64)            # distinct values: the rank is a plain count
+    order = np.argsort(coord, kind="stable")
+    regions = np.array([1.0, 2.0, 7.0, 10.0, 3 + 1 / 3, 6 + 2 / 3, 1003.0, 5000.0], np.float32)
+    got = ol.quantile_regions(order, regions)
+    assert got.shape == (len(regions), n) and got.dtype == np.float32
+    for r, reg in enumerate(regions):
+        # exact integer restatement: hits with a smaller coordinate // ceil(N / regions) + 1; the rational N / regions
+        # is taken on the float32 value actually stored (thirds are not exact) and is far from an integer here
+        from fractions import Fraction
+        size = -((-Fraction(n)) // Fraction(float(reg)))      # ceil
+        want = [int(sum(coord < c)) // int(size) + 1 for c in coord]
+        assert got[r].tolist() == [float(w) for w in want], reg
+        # invariants: 1-based, monotone along the coordinate, every region but the last holds exactly `size` hits
+        along = got[r][order]
+        assert along[0] == 1 and np.all(np.diff(along) >= 0) and np.all(np.diff(along) <= 1)
+        counts = np.bincount(got[r].astype(np.int64))[1:]
+        assert np.all(counts[:-1] == int(size)) and 0 < counts[-1] <= int(size)
+    # a rank array that is not the identity: the region follows the hit, not the position
+    assert not np.array_equal(got[2], got[2][order])
+
+
+def test_geo_shift_orders_lexicographically_by_phi_region_eta_region_hash():
+    # With integer-valued inputs every float32 operation is exact, so the key must equal the Python-integer
+    # mixed-radix value, and sorting by it must equal a lexicographic sort on (phi region, eta region, hash).
+    rng = np.random.default_rng(4)
+    rows, n = 3, 500
+    regions_eta = np.array([2.0, 3 + 1 / 3, 5.0], np.float32)     # ceil -> 2, 4, 5 eta regions at most
+    reg_eta = np.stack([rng.integers(1, int(np.ceil(r)) + 1, n) for r in regions_eta]).astype(np.float32)
+    reg_phi = rng.integers(1, 5, (rows, n)).astype(np.float32)
+    hashed = rng.integers(-40, 41, (rows, n)).astype(np.float32)
+    shift = np.array([81.0, 90.0, 200.0], np.float32)             # strictly above the hash range: no boundary ties
+    got = ol.geo_shift(regions_eta, shift, reg_eta, reg_phi)
+    for r in range(rows):
+        mult = int(np.ceil(regions_eta[r])) + 1
+        want = [int(p) * int(shift[r]) * mult + int(e) * int(shift[r]) for e, p in zip(reg_eta[r], reg_phi[r])]
+        assert got[r].tolist() == [float(w) for w in want]
+        key = hashed[r] + got[r]
+        order = np.argsort(key, kind="stable")
+        lex = np.lexsort((np.arange(n), hashed[r], reg_eta[r], reg_phi[r]))
+        assert np.array_equal(order, lex)
+    # asymmetry pins the operand roles: swapping eta and phi regions changes the result
+    assert not np.array_equal(got, ol.geo_shift(regions_eta, shift, reg_phi, reg_eta))
+
+
+def test_hept_sort_keys_padding_and_composition():
+    rng = np.random.default_rng(5)
+    rows, n, n_raw = 4, 300, 257
+    eta, phi = rng.normal(size=n), rng.uniform(-3, 3, n)
+    eta[n_raw:], phi[n_raw:] = np.inf, np.inf
+    s_eta, s_phi = np.argsort(eta, kind="stable"), np.argsort(phi, kind="stable")
+    regions = np.array([[2.0, 3.0, 4 + 1 / 3, 6.0], [5.0, 3 + 2 / 3, 3.0, 2.0]], np.float32)
+    hashed = rng.normal(size=(rows, n)).astype(np.float32)
+    shift = (hashed.max(1) - hashed.min(1)).astype(np.float32)
+    keys = ol.hept_sort_keys(hashed, s_eta, s_phi, regions, shift, n_raw)
+    assert np.all(np.isinf(keys[:, n_raw:])) and np.all(np.isfinite(keys[:, :n_raw]))
+    # padded hits sort last and keep their order; real hits of a lower (phi, eta) region pair never follow a higher one
+    reg_eta, reg_phi = ol.quantile_regions(s_eta, regions[0]), ol.quantile_regions(s_phi, regions[1])
+    for r in range(rows):
+        order = np.argsort(keys[r], kind="stable")
+        assert np.array_equal(order[n_raw:], np.arange(n_raw, n))
+        pair = reg_phi[r][order[:n_raw]] * 100 + reg_eta[r][order[:n_raw]]
+        # float rounding can only swap neighbours at a region boundary whose hashes sit at opposite ends of the range
+        assert np.mean(np.diff(pair) < 0) < 0.02
+    # the input hashes are not modified
+    assert np.all(np.isfinite(hashed))
