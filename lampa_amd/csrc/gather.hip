@@ -68,6 +68,7 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
   else
     hipLaunchKernelGGL((gs_rows_kernel<uint8_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
                        src_segments, group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+  LAMPA_PROF(s, "gs_rows_kernel");
   return lampa_launch_status();
 }
 

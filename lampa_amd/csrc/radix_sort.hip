@@ -6,8 +6,8 @@
 // bk.sort(stable=True)  models/baselines/full_mamba2.py:203,207, perm.argsort(dim=1)  full_mamba2.py:678.
 //
 // Each pass = a histogram kernel (LDS histogram per tile of 2048 keys, written to HBM per tile), an offsets kernel
-// (per-tile histograms -> output offsets, one block per segment) and a scatter kernel (per-wave ranks from wavefront
-// ballots added to the tile's offsets).  The number of
+// (per digit: prefix of the tile counts over the tiles of the segment, and the digit's total) and a scatter kernel
+// (scan of the digit totals, per-wave ranks from wavefront ballots, both added to the tile's offsets).  The number of
 // passes is fixed by the host; the digit width of a segment is at most 11 bits. key_bits may live in device memory
 // (written by the key-packing kernel) so that no host synchronisation is needed: then the host launches the worst
 // case and each segment uses only the launches its keys need (see rs_digit).
@@ -60,142 +60,183 @@ __device__ __forceinline__ RsDigit rs_digit(const int32_t* bits_dev, int bits_st
   return d;
 }
 
-// grid (n_tiles, S). hist [S, n_tiles, RS_MAX_BINS] (only the first 2^nbits entries of a row are used).
+// Block -> (segment, tile) for the 1-D grids of the histogram and scatter kernels. Workgroups go to the 8 XCDs round
+// robin by their linear id, and each XCD has its own L2: with 8 or more segments all tiles of a segment are given to
+// one XCD, so that the scattered 4-byte writes into the segment's output range meet in one L2 and leave it as full
+// lines. Fewer segments are spread over all XCDs instead. Returns false for the padding blocks of the grid.
+#define RS_XCDS 8
+static int rs_grid_blocks(int n_tiles, int n_segments) {
+  if (n_segments < RS_XCDS) return n_tiles * n_segments;
+  return RS_XCDS * ((n_segments + RS_XCDS - 1) / RS_XCDS) * n_tiles;
+}
+__device__ __forceinline__ bool rs_block_to_tile(int n_tiles, int n_segments, int& seg, int& tile) {
+  const int b = blockIdx.x;
+  if (n_segments < RS_XCDS) {
+    seg = b / n_tiles;
+    tile = b - seg * n_tiles;
+    return true;
+  }
+  const int xcd = b % RS_XCDS, i = b / RS_XCDS;
+  seg = xcd + RS_XCDS * (i / n_tiles);
+  tile = i % n_tiles;
+  return seg < n_segments;
+}
+
+// 1-D grid of rs_grid_blocks(n_tiles, S) blocks. hist [S, n_tiles, RS_MAX_BINS] (only the first 2^nbits entries of a row are used).
 __global__ void __launch_bounds__(RS_BLOCK) rs_histogram_kernel(const uint32_t* __restrict__ keys_orig,
-                                                               const uint32_t* __restrict__ keys_buf, int64_t n,
+                                                               const uint2* __restrict__ pairs_buf, int64_t n,
                                                                int kind_orig, const int32_t* bits_dev, int bits_stride,
-                                                               int host_bits, int pass, int n_passes,
-                                                               uint32_t* __restrict__ hist) {
+                                                               int host_bits, int pass, int n_passes, int n_tiles,
+                                                               int n_segments, uint32_t* __restrict__ hist) {
   __shared__ uint32_t s_hist[RS_MAX_BINS];
-  const int seg = blockIdx.y, tile = blockIdx.x, n_tiles = gridDim.x;
+  int seg, tile;
+  if (!rs_block_to_tile(n_tiles, n_segments, seg, tile)) return;
   const RsDigit dg = rs_digit(bits_dev, bits_stride, host_bits, seg, pass, n_passes);
   if (dg.skip) return;
-  const uint32_t* keys = dg.first ? keys_orig : keys_buf;
-  const int kind = dg.first ? kind_orig : KEY_U32;  // the buffers hold ordered keys
   const int bins = 1 << dg.nbits;
   const uint32_t mask = (uint32_t)bins - 1u;
   for (int d = threadIdx.x; d < bins; d += RS_BLOCK) s_hist[d] = 0;
   __syncthreads();
-  const uint32_t* kseg = keys + (int64_t)seg * n;
-  const int64_t base = (int64_t)tile * RS_TILE;
+  const int64_t base = (int64_t)seg * n, first = (int64_t)tile * RS_TILE;
 #pragma unroll
   for (int i = 0; i < RS_ITEMS; ++i) {
-    const int64_t idx = base + i * RS_BLOCK + threadIdx.x;
-    if (idx < n) atomicAdd(&s_hist[(rs_ordered(kseg[idx], kind) >> dg.shift) & mask], 1u);
+    const int64_t idx = first + i * RS_BLOCK + threadIdx.x;
+    if (idx < n) {
+      // the ping-pong buffers hold (ordered key, payload) pairs
+      const uint32_t k = dg.first ? rs_ordered(keys_orig[base + idx], kind_orig) : pairs_buf[base + idx].x;
+      atomicAdd(&s_hist[(k >> dg.shift) & mask], 1u);
+    }
   }
   __syncthreads();
   uint32_t* out = hist + ((int64_t)seg * n_tiles + tile) * RS_MAX_BINS;
   for (int d = threadIdx.x; d < bins; d += RS_BLOCK) out[d] = s_hist[d];
 }
 
-// grid (S), 1024 threads. Turns the per-tile histograms of a segment into output offsets, in place:
-// hist[tile][d] <- (keys of the segment with a smaller digit) + (keys with digit d in earlier tiles).
-// One pass over the [n_tiles, bins] counts per segment; without it every tile of the scatter would have to re-read
-// all of them (n_tiles times the traffic and a chain of dependent loads per tile).
-#define RS_OFFS_BLOCK 1024
-__global__ void __launch_bounds__(RS_OFFS_BLOCK) rs_offsets_kernel(const int32_t* bits_dev, int bits_stride, int host_bits,
-                                                                  int pass, int n_passes, int n_tiles,
-                                                                  uint32_t* __restrict__ hist) {
-  __shared__ uint32_t s_wsum[RS_OFFS_BLOCK / 64];
-  const int seg = blockIdx.x;
+// grid (RS_MAX_BINS / RS_BLOCK, S). One thread per digit: exclusive prefix of the digit's counts over the tiles of the
+// segment, in place (hist[tile][d] <- keys with digit d in earlier tiles), and the digit's total to tot[seg][d].
+// The scan of the totals over the digits is left to the scatter kernel, so this kernel is one short chain of
+// independent, coalesced loads per thread.
+__global__ void __launch_bounds__(RS_BLOCK) rs_offsets_kernel(const int32_t* bits_dev, int bits_stride, int host_bits,
+                                                             int pass, int n_passes, int n_tiles,
+                                                             uint32_t* __restrict__ hist, uint32_t* __restrict__ tot) {
+  const int seg = blockIdx.y;
+  const RsDigit dg = rs_digit(bits_dev, bits_stride, host_bits, seg, pass, n_passes);
+  if (dg.skip) return;
+  const int d = blockIdx.x * RS_BLOCK + threadIdx.x;
+  if (d >= (1 << dg.nbits)) return;
+  uint32_t* hcol = hist + (int64_t)seg * n_tiles * RS_MAX_BINS + d;
+  uint32_t run = 0;
+  for (int t0 = 0; t0 < n_tiles; t0 += 8) {
+    uint32_t c[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) c[u] = hcol[(int64_t)min(t0 + u, n_tiles - 1) * RS_MAX_BINS];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (t0 + u < n_tiles) {
+        hcol[(int64_t)(t0 + u) * RS_MAX_BINS] = run;
+        run += c[u];
+      }
+  }
+  tot[(int64_t)seg * RS_MAX_BINS + d] = run;
+}
+
+// 1-D grid of rs_grid_blocks(n_tiles, S) blocks. Element order inside a tile: wave w owns [w*512, (w+1)*512), item i
+// of lane l is at w*512 + i*64 + l, so (item, lane) order within a wave is input order and the scatter is stable.
+__global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __restrict__ keys_orig,
+                                                             const int32_t* __restrict__ vals_orig,
+                                                             const uint2* __restrict__ pairs_in, int64_t n,
+                                                             int kind_orig, const int32_t* bits_dev, int bits_stride,
+                                                             int host_bits, int pass, int n_passes, int n_tiles,
+                                                             int n_segments, const uint32_t* __restrict__ hist,
+                                                             const uint32_t* __restrict__ tot,
+                                                             uint2* __restrict__ pairs_out,
+                                                             int32_t* __restrict__ vals_out) {
+  // Row 0 starts at the number of keys of the segment with a smaller digit, the other rows at zero; after the
+  // ranking the rows become the output bases of the waves.
+  __shared__ uint32_t s_bin[RS_WAVES][RS_MAX_BINS];
+  __shared__ uint32_t s_wsum[RS_WAVES];
+  int seg, tile;
+  if (!rs_block_to_tile(n_tiles, n_segments, seg, tile)) return;
+  const int wave = threadIdx.x >> 6, lane = lane_id();
   const RsDigit dg = rs_digit(bits_dev, bits_stride, host_bits, seg, pass, n_passes);
   if (dg.skip) return;
   const int bins = 1 << dg.nbits;
-  uint32_t* hseg = hist + (int64_t)seg * n_tiles * RS_MAX_BINS;
-  const int lane = lane_id(), wave = threadIdx.x >> 6;
-  // each thread owns digits d0 = tid and d1 = tid + 1024 (bins <= 2048): exclusive prefix over the tiles
-  uint32_t tot[2] = {0, 0};
+  const uint32_t mask = (uint32_t)bins - 1u;
+
+  // digit totals of the segment: thread t owns digits 8t .. 8t+7; entries beyond the digit range are stale
+  constexpr int DPT = RS_MAX_BINS / RS_BLOCK;
+  uint32_t dt[DPT];
+  {
+    const uint32_t* trow = tot + (int64_t)seg * RS_MAX_BINS + threadIdx.x * DPT;
+    const bool live = (int)threadIdx.x * DPT < bins;
+    const uint4 a = live ? *reinterpret_cast<const uint4*>(trow) : make_uint4(0, 0, 0, 0);
+    const uint4 b = live ? *reinterpret_cast<const uint4*>(trow + 4) : make_uint4(0, 0, 0, 0);
+    dt[0] = a.x; dt[1] = a.y; dt[2] = a.z; dt[3] = a.w; dt[4] = b.x; dt[5] = b.y; dt[6] = b.z; dt[7] = b.w;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int d = threadIdx.x + h * RS_OFFS_BLOCK;
-    if (d < bins) {
-      uint32_t run = 0;
-      for (int t0 = 0; t0 < n_tiles; t0 += 8) {
-        uint32_t c[8];
+    for (int j = 0; j < DPT; ++j)
+      if ((int)threadIdx.x * DPT + j >= bins) dt[j] = 0;
+  }
+
+  const int64_t sbase = (int64_t)seg * n;
+  const int64_t wbase = (int64_t)tile * RS_TILE + wave * (RS_TILE / RS_WAVES);
+  uint32_t key[RS_ITEMS], rank[RS_ITEMS];
+  int32_t val[RS_ITEMS];
+  bool valid[RS_ITEMS];
+  if (dg.first) {  // the caller's keys and payload (or the position)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) c[u] = hseg[(int64_t)min(t0 + u, n_tiles - 1) * RS_MAX_BINS + d];
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      const int64_t idx = wbase + i * 64 + lane;
+      valid[i] = idx < n;
+      key[i] = valid[i] ? rs_ordered(keys_orig[sbase + idx], kind_orig) : 0xFFFFFFFFu;
+      val[i] = valid[i] ? (vals_orig ? vals_orig[sbase + idx] : (int32_t)idx) : 0;
+    }
+  } else {  // (ordered key, payload) pairs of the previous pass
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (t0 + u < n_tiles) {
-            hseg[(int64_t)(t0 + u) * RS_MAX_BINS + d] = run;
-            run += c[u];
-          }
-      }
-      tot[h] = run;
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      const int64_t idx = wbase + i * 64 + lane;
+      valid[i] = idx < n;
+      const uint2 kv = valid[i] ? pairs_in[sbase + idx] : make_uint2(0xFFFFFFFFu, 0u);
+      key[i] = kv.x;
+      val[i] = (int32_t)kv.y;
     }
   }
-  // exclusive scan of the digit totals over d = 0 .. bins-1 (digit order: first all d0 of the block, then all d1)
-  uint32_t base[2];
-  uint32_t carry = 0;
+  // this tile's offsets within each digit (written by rs_offsets_kernel); used after the ranking
+  const uint32_t* hrow = hist + ((int64_t)seg * n_tiles + tile) * RS_MAX_BINS;
+  uint32_t hoff[DPT];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    uint32_t incl = tot[h];
+  for (int j = 0; j < DPT; ++j) {
+    const int d = threadIdx.x + j * RS_BLOCK;
+    hoff[j] = d < bins ? hrow[d] : 0u;
+  }
+
+  // exclusive scan of the digit totals over the block -> row 0 of s_bin; rows 1.. start at zero
+  {
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) mine += dt[j];
+    uint32_t incl = mine;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       const uint32_t up = __shfl_up(incl, off);
       if (lane >= off) incl += up;
     }
-    __syncthreads();
     if (lane == 63) s_wsum[wave] = incl;
-    __syncthreads();
-    uint32_t woff = 0, all = 0;
-    for (int w = 0; w < RS_OFFS_BLOCK / 64; ++w) {
-      const uint32_t v = s_wsum[w];
-      woff += w < wave ? v : 0u;
-      all += v;
+    for (int d = threadIdx.x; d < bins; d += RS_BLOCK) {
+#pragma unroll
+      for (int w = 1; w < RS_WAVES; ++w) s_bin[w][d] = 0;
     }
-    base[h] = carry + woff + incl - tot[h];
-    carry += all;
-  }
+    __syncthreads();
+    uint32_t run = incl - mine;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int d = threadIdx.x + h * RS_OFFS_BLOCK;
-    if (d < bins)
-      for (int t = 0; t < n_tiles; ++t) hseg[(int64_t)t * RS_MAX_BINS + d] += base[h];
-  }
-}
-
-// grid (n_tiles, S). Element order inside a tile: wave w owns [w*512, (w+1)*512), item i of lane l is at
-// w*512 + i*64 + l, so (item, lane) order within a wave is input order and the scatter is stable.
-__global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __restrict__ keys_orig,
-                                                             const int32_t* __restrict__ vals_orig,
-                                                             const uint32_t* __restrict__ keys_buf,
-                                                             const int32_t* __restrict__ vals_buf, int64_t n,
-                                                             int kind_orig, const int32_t* bits_dev, int bits_stride,
-                                                             int host_bits, int pass, int n_passes,
-                                                             const uint32_t* __restrict__ hist,
-                                                             uint32_t* __restrict__ keys_out,
-                                                             int32_t* __restrict__ vals_out) {
-  __shared__ uint32_t s_bin[RS_WAVES][RS_MAX_BINS];  // per-wave counts, then per-wave output bases
-  const int seg = blockIdx.y, tile = blockIdx.x, n_tiles = gridDim.x;
-  const int wave = threadIdx.x >> 6, lane = lane_id();
-  const RsDigit dg = rs_digit(bits_dev, bits_stride, host_bits, seg, pass, n_passes);
-  if (dg.skip) return;
-  const uint32_t* keys_in = dg.first ? keys_orig : keys_buf;
-  const int32_t* vals_in = dg.first ? vals_orig : vals_buf;
-  const int kind = dg.first ? kind_orig : KEY_U32;
-  const int bins = 1 << dg.nbits;
-  const uint32_t mask = (uint32_t)bins - 1u;
-
-  for (int d = threadIdx.x; d < bins; d += RS_BLOCK) {
+    for (int w = 0; w < RS_WAVES; ++w) run += w < wave ? s_wsum[w] : 0u;
 #pragma unroll
-    for (int w = 0; w < RS_WAVES; ++w) s_bin[w][d] = 0;
+    for (int j = 0; j < DPT; ++j) {
+      if ((int)threadIdx.x * DPT + j < bins) s_bin[0][threadIdx.x * DPT + j] = run;
+      run += dt[j];
+    }
   }
   __syncthreads();
 
-  const uint32_t* kseg = keys_in + (int64_t)seg * n;
-  const int32_t* vseg = vals_in ? vals_in + (int64_t)seg * n : nullptr;
-  const int64_t wbase = (int64_t)tile * RS_TILE + wave * (RS_TILE / RS_WAVES);
-  uint32_t key[RS_ITEMS], rank[RS_ITEMS];
-  int32_t val[RS_ITEMS];
-  bool valid[RS_ITEMS];
-#pragma unroll
-  for (int i = 0; i < RS_ITEMS; ++i) {
-    const int64_t idx = wbase + i * 64 + lane;
-    valid[i] = idx < n;
-    key[i] = valid[i] ? rs_ordered(kseg[idx], kind) : 0xFFFFFFFFu;
-    val[i] = valid[i] ? (vseg ? vseg[idx] : (int32_t)idx) : 0;
-  }
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
 #pragma unroll
   for (int i = 0; i < RS_ITEMS; ++i) {
@@ -214,28 +255,31 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __
   }
   __syncthreads();
 
-  // output base of every digit for this tile (rs_offsets_kernel), then of every wave of the tile
-  const uint32_t* hrow = hist + ((int64_t)seg * n_tiles + tile) * RS_MAX_BINS;
-  for (int d = threadIdx.x; d < bins; d += RS_BLOCK) {
-    uint32_t run = hrow[d];
+  // output base of every wave of the tile for every digit: tile offset, then the waves in order. Row 0 holds
+  // (smaller digits + keys of wave 0), which carries the digit base into the running sum.
 #pragma unroll
-    for (int w = 0; w < RS_WAVES; ++w) {
-      const uint32_t c = s_bin[w][d];
-      s_bin[w][d] = run;
-      run += c;
+  for (int j = 0; j < DPT; ++j) {
+    const int d = threadIdx.x + j * RS_BLOCK;
+    if (d < bins) {
+      uint32_t run = hoff[j];
+#pragma unroll
+      for (int w = 0; w < RS_WAVES; ++w) {
+        const uint32_t c = s_bin[w][d];
+        s_bin[w][d] = run;
+        run += c;
+      }
     }
   }
   __syncthreads();
 
-  uint32_t* kout = keys_out ? keys_out + (int64_t)seg * n : nullptr;
-  int32_t* vout = vals_out + (int64_t)seg * n;
+  // one scattered store per key: an 8-byte (key, payload) pair between passes, the payload alone after the last
 #pragma unroll
   for (int i = 0; i < RS_ITEMS; ++i) {
     if (valid[i]) {
       const uint32_t d = (key[i] >> dg.shift) & mask;
-      const uint32_t pos = s_bin[wave][d] + rank[i];
-      if (kout) kout[pos] = key[i];
-      vout[pos] = val[i];
+      const int64_t pos = sbase + s_bin[wave][d] + rank[i];
+      if (pairs_out) pairs_out[pos] = make_uint2(key[i], (uint32_t)val[i]);
+      else vals_out[pos] = val[i];
     }
   }
 }
@@ -244,7 +288,7 @@ extern "C" int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n) {
   if (n_segments < 1 || n < 0) return LAMPA_ERR_INVALID;
   const int64_t n_tiles = (n + RS_TILE - 1) / RS_TILE > 0 ? (n + RS_TILE - 1) / RS_TILE : 1;
   const int64_t pairs = lampa_align_up((int64_t)n_segments * n * 4, 256);
-  const int64_t hist = lampa_align_up((int64_t)n_segments * n_tiles * RS_MAX_BINS * 4, 256);
+  const int64_t hist = lampa_align_up((int64_t)n_segments * (n_tiles + 1) * RS_MAX_BINS * 4, 256);  // + digit totals
   return 4 * pairs + hist;
 }
 
@@ -270,24 +314,23 @@ extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t
   const int n_tiles = (int)((n + RS_TILE - 1) / RS_TILE);
   const int64_t pairs = lampa_align_up((int64_t)n_segments * n * 4, 256);
   char* ws = (char*)workspace;
-  uint32_t* kbuf[2] = {(uint32_t*)ws, (uint32_t*)(ws + pairs)};
-  int32_t* vbuf[2] = {(int32_t*)(ws + 2 * pairs), (int32_t*)(ws + 3 * pairs)};
+  uint2* pbuf[2] = {(uint2*)ws, (uint2*)(ws + 2 * pairs)};
   uint32_t* hist = (uint32_t*)(ws + 4 * pairs);
-  const dim3 grid(n_tiles, n_segments), block(RS_BLOCK);
+  uint32_t* tot = hist + (int64_t)n_segments * n_tiles * RS_MAX_BINS;
+  const dim3 grid(rs_grid_blocks(n_tiles, n_segments)), block(RS_BLOCK);
   LAMPA_PROF(s, "start");
   for (int p = 0; p < n_passes; ++p) {
-    const uint32_t* kbuf_in = p == 0 ? (const uint32_t*)keys_in : kbuf[(p - 1) & 1];
-    const int32_t* vbuf_in = p == 0 ? vals_in : vbuf[(p - 1) & 1];
+    const uint2* pairs_in = pbuf[(p + 1) & 1];  // written by the previous launch (never read by the first)
     const bool last = p == n_passes - 1;
-    hipLaunchKernelGGL(rs_histogram_kernel, grid, block, 0, s, (const uint32_t*)keys_in, kbuf_in, n, key_kind,
-                       key_bits_dev, key_bits_stride, key_bits, p, n_passes, hist);
+    hipLaunchKernelGGL(rs_histogram_kernel, grid, block, 0, s, (const uint32_t*)keys_in, pairs_in, n, key_kind,
+                       key_bits_dev, key_bits_stride, key_bits, p, n_passes, n_tiles, n_segments, hist);
     LAMPA_PROF(s, "rs_histogram_kernel");
-    hipLaunchKernelGGL(rs_offsets_kernel, dim3(n_segments), dim3(RS_OFFS_BLOCK), 0, s, key_bits_dev, key_bits_stride,
-                       key_bits, p, n_passes, n_tiles, hist);
+    hipLaunchKernelGGL(rs_offsets_kernel, dim3(RS_MAX_BINS / RS_BLOCK, n_segments), block, 0, s, key_bits_dev,
+                       key_bits_stride, key_bits, p, n_passes, n_tiles, hist, tot);
     LAMPA_PROF(s, "rs_offsets_kernel");
-    hipLaunchKernelGGL(rs_scatter_kernel, grid, block, 0, s, (const uint32_t*)keys_in, vals_in, kbuf_in, vbuf_in, n,
-                       key_kind, key_bits_dev, key_bits_stride, key_bits, p, n_passes, hist,
-                       last ? (uint32_t*)nullptr : kbuf[p & 1], last ? vals_out : vbuf[p & 1]);
+    hipLaunchKernelGGL(rs_scatter_kernel, grid, block, 0, s, (const uint32_t*)keys_in, vals_in, pairs_in, n,
+                       key_kind, key_bits_dev, key_bits_stride, key_bits, p, n_passes, n_tiles, n_segments, hist, tot,
+                       last ? (uint2*)nullptr : pbuf[p & 1], vals_out);
     LAMPA_PROF(s, "rs_scatter_kernel");
   }
   return lampa_launch_status();
