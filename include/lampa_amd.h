@@ -137,6 +137,27 @@ int lampa_geo_shift(const float* region_eta, const float* region_phi, const floa
 int lampa_hept_sort_keys(const float* hashed, const int32_t* rank_eta, const int32_t* rank_phi, const float* regions,
                          const float* hash_shift, int n_rows, int64_t n, int64_t n_raw, float* keys, void* stream);
 
+/* ------------------------------------------------------------------------------ operators around the forward */
+
+/* Depthwise causal short convolution with optional bias, SiLU and residual. Replaces causal_conv1d_fwd
+ * (models/hattention/short_convolution.py:39-99,262-300). y[t, d] = act(bias[d] + sum_j weight[d, j] *
+ * x[t - (W-1) + j, d]) + residual[t, d]; taps before the start of the token's sequence are zero.
+ * x, residual, y [n_tokens, D] of dtype (LAMPA_BF16/FP16/FP32) with row strides in elements; weight fp32 [D, W],
+ * bias fp32 [D] or NULL; cu_seqlens device int64 [n_seq+1] or NULL (then n_tokens / t_len sequences of t_len tokens);
+ * activation 0 none, 1 SiLU. D and the strides multiples of 8, pointers 16-byte aligned, W <= 8. */
+int lampa_causal_conv1d_fwd(const void* x, int64_t x_stride, int64_t n_tokens, int D, int W, const float* weight,
+                            const float* bias, const void* residual, int64_t res_stride, const int64_t* cu_seqlens,
+                            int n_seq, int64_t t_len, int activation, int dtype, void* y, int64_t y_stride, void* stream);
+
+/* RMS norm over the last dimension with optional residual add, weight, bias and output gate. Replaces
+ * layer_norm_gated_fwd / layer_norm_fwd with is_rms_norm (models/hattention/fused_norm.py:40-111,456-531,1436-1506).
+ * s = x + residual; residual_out = s; y = s / sqrt(mean(s^2) + eps) * weight + bias; with g: y *= g * sigmoid(g)
+ * (activation 1) or sigmoid(g) (activation 2). x, g, y [rows, D] of dtype; residual, residual_out of res_dtype;
+ * weight, bias fp32 [D]; rstd_out fp32 [rows]; every pointer but x and y may be NULL. D % 8 == 0, D <= 2048. */
+int lampa_rms_norm_fwd(const void* x, const void* g, const float* weight, const float* bias, const void* residual,
+                       void* residual_out, void* y, float* rstd_out, int64_t rows, int D, float eps, int activation,
+                       int dtype, int res_dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------- gated-delta forward */
 
 /* Token-serial forward with an fp32 state. Replaces fused_recurrent_gated_delta_rule_fwd

@@ -1,0 +1,258 @@
+"""The operators either side of the gated-delta forward in a layer: the depthwise causal short convolution and the
+(gated) RMS norm, as gfx950 kernels behind the reference's names.
+
+Mirrors ``causal_conv1d`` / ``ShortConvolution`` (``models/hattention/short_convolution.py:426-458,528-721``) and
+``rms_norm_gated`` / ``rms_norm`` / ``FusedRMSNormGated`` / ``FusedRMSNormSwishGate`` / ``RMSNorm``
+(``models/hattention/fused_norm.py:856-878,1003-1104,2094-2354``). Forward only; GPU tensors only (no CPU fallback).
+"""
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import _capi
+from ._capi import check, ptr, require_cuda, stream_of
+
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+_ACT = {None: 0, "silu": 1, "swish": 1, "sigmoid": 2}
+
+
+class _ForwardOnly(torch.autograd.Function):
+    """Lets the operators take part in a graph that is never differentiated; backward raises."""
+
+    @staticmethod
+    def forward(ctx, fn, *tensors):
+        return fn()
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("lampa_amd implements the forward pass of this operator only")
+
+
+def _code(dtype) -> int:
+    if dtype not in _DTYPES:
+        raise TypeError(f"lampa_amd: unsupported dtype {dtype} (bfloat16, float16 or float32)")
+    return _DTYPES[dtype]
+
+
+def _f32(t: Optional[torch.Tensor], device) -> Optional[torch.Tensor]:
+    return None if t is None else t.detach().to(device=device, dtype=torch.float32).contiguous()
+
+
+# ----------------------------------------------------------------------------------------------- short convolution
+@torch.no_grad()
+def _conv_launch(x2: torch.Tensor, weight, bias, residual2, activation, cu_seqlens, t_len: int) -> torch.Tensor:
+    """x2 [tokens, D] (last dim contiguous, any row stride) -> y [tokens, D] contiguous."""
+    n, D = x2.shape
+    W = weight.shape[-1]
+    y = torch.empty((n, D), dtype=x2.dtype, device=x2.device)
+    if n == 0:
+        return y
+    cu = None if cu_seqlens is None else cu_seqlens.to(device=x2.device, dtype=torch.int64).contiguous()
+    check(_capi.lib().lampa_causal_conv1d_fwd(
+        ptr(x2), x2.stride(0), n, D, W, ptr(weight), ptr(bias), ptr(residual2),
+        0 if residual2 is None else residual2.stride(0), ptr(cu), 0 if cu is None else cu.numel() - 1, t_len,
+        _ACT[activation], _code(x2.dtype), ptr(y), D, stream_of(x2)), "lampa_causal_conv1d_fwd")
+    return y
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """[B, T, D] -> [B*T, D] view with a contiguous last dimension (copies only when it has to)."""
+    B, T, D = t.shape
+    if t.stride(-1) != 1 or (B > 1 and t.stride(0) != T * t.stride(1)) or t.stride(1) % 8 or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t.as_strided((B * T, D), (t.stride(1), 1))
+
+
+def causal_conv1d(x: torch.Tensor, weight: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                  residual: Optional[torch.Tensor] = None, activation: Optional[str] = None,
+                  cu_seqlens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``short_convolution.py:426-458``: x [B, T, D], weight [D, W] (tap W-1 on the current token), bias [D],
+    residual [B, T, D]; activation ``None`` / ``'silu'`` / ``'swish'``; with ``cu_seqlens`` B must be 1 and taps never
+    cross a sequence start. Returns [B, T, D] in x's dtype (fp32 arithmetic)."""
+    require_cuda(x, weight, bias, residual, cu_seqlens)
+    if activation not in (None, "silu", "swish"):
+        raise ValueError(f"Activation `{activation}` not supported yet.")
+    if x.dim() != 3:
+        raise ValueError("causal_conv1d: x must be [B, T, D]")
+    B, T, D = x.shape
+    if cu_seqlens is not None and B != 1:
+        raise ValueError("causal_conv1d: batch size must be 1 when cu_seqlens is given")
+    if weight is None:
+        weight = torch.ones(D, 1, device=x.device)
+    w32, b32 = _f32(weight.reshape(D, -1), x.device), _f32(bias, x.device)
+    res2 = None if residual is None else _rows(residual.to(x.dtype))
+    x2 = _rows(x)
+    fn = lambda: _conv_launch(x2, w32, b32, res2, activation, cu_seqlens, max(T, 1)).view(B, T, D)  # noqa: E731
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias, residual)):
+        return _ForwardOnly.apply(fn, x, weight)
+    return fn()
+
+
+class ShortConvolution(nn.Conv1d):
+    """``short_convolution.py:528-721``: depthwise causal convolution over the time axis of a [B, T, D] tensor with
+    an optional SiLU, a cache of the last W inputs per sequence ([N, D, W]) and a one-token ``step``."""
+
+    def __init__(self, hidden_size: int, kernel_size: int, bias: bool = False, activation: Optional[str] = 'silu',
+                 use_fast_conv1d: Optional[bool] = True, device=None, dtype=None, **kwargs):
+        super().__init__(in_channels=hidden_size, out_channels=hidden_size, kernel_size=kernel_size, groups=hidden_size,
+                         bias=bias, padding=kernel_size - 1, device=device, dtype=dtype)
+        self.hidden_size = hidden_size
+        self.activation = None
+        if kernel_size % 2 != 0:
+            raise ValueError("Kernel size must be the power of 2")
+        if activation is not None:
+            assert activation in ['silu', 'swish'], f"Activation `{activation}` not supported yet."
+            self.activation = activation
+        self.use_fast_conv1d = False  # one implementation here: the HIP kernel
+
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None,
+                cache: Optional[torch.Tensor] = None, output_final_state: bool = False,
+                cu_seqlens: Optional[torch.LongTensor] = None, **kwargs) -> Tuple[torch.Tensor, torch.Tensor]:
+        B, T, D, W = *x.shape, self.kernel_size[0]
+        N = B if cu_seqlens is None else len(cu_seqlens) - 1
+        if mask is not None:
+            if cu_seqlens is not None:
+                raise ValueError("`mask` and `cu_seqlens` cannot be provided at the same time")
+            x = x.mul_(mask.unsqueeze(-1))
+        if output_final_state and cache is None:
+            cache = x.new_zeros(N, D, W)
+        if cache is not None and B * T == N:
+            return self.step(x, residual, cache, cu_seqlens)
+        if cache is not None:
+            with torch.no_grad():
+                if cu_seqlens is not None:
+                    cu = cu_seqlens.to(x.device).long()
+                    idx = cu[1:, None] - W + torch.arange(W, device=x.device)[None]          # [N, W]
+                    ok = idx >= torch.maximum(cu[:-1], cu[1:] - W)[:, None]
+                    rows = x[0][idx.clamp(min=0)] * ok[..., None].to(x.dtype)                # [N, W, D]
+                    cache.copy_(rows.transpose(1, 2))
+                else:
+                    cache[:, :, -min(W, T):].copy_(x[..., -min(W, T):, :].transpose(1, 2))
+        y = causal_conv1d(x=x, weight=self.weight.reshape(D, W), bias=self.bias, residual=residual,
+                          activation=self.activation, cu_seqlens=cu_seqlens)
+        return y, cache
+
+    def step(self, x: torch.Tensor, residual: Optional[torch.Tensor], cache: torch.Tensor,
+             cu_seqlens: Optional[torch.LongTensor] = None):
+        """One token per sequence: the cache is rolled in place, then the convolution runs over its W columns."""
+        shape = x.shape
+        D, W = self.hidden_size, self.kernel_size[0]
+        xt = x.reshape(-1, D)
+        with torch.no_grad():
+            cache.copy_(cache.roll(shifts=-1, dims=-1))
+            cache[:, :, -1] = xt
+            window = cache.transpose(1, 2).contiguous()                                       # [N, W, D]
+        y = causal_conv1d(x=window, weight=self.weight.reshape(D, W), bias=self.bias, activation=self.activation)
+        y = y[:, -1].reshape(shape)
+        if residual is not None:
+            y = y + residual
+        return y, cache
+
+    @property
+    def state_size(self) -> int:
+        return self.hidden_size * self.kernel_size
+
+
+# ------------------------------------------------------------------------------------------------------ RMS norm
+@torch.no_grad()
+def _norm_launch(x2, g2, weight, bias, residual2, residual_dtype, eps, activation):
+    rows, D = x2.shape
+    y = torch.empty_like(x2)
+    want_res_out = residual2 is not None or (residual_dtype is not None and residual_dtype != x2.dtype)
+    res_out = torch.empty((rows, D), dtype=residual_dtype, device=x2.device) if want_res_out else None
+    if rows:
+        check(_capi.lib().lampa_rms_norm_fwd(
+            ptr(x2), ptr(g2), ptr(weight), ptr(bias), ptr(residual2), ptr(res_out), ptr(y), None, rows, D, float(eps),
+            _ACT[activation] if g2 is not None else 0, _code(x2.dtype),
+            _code(residual_dtype) if want_res_out else _code(x2.dtype), stream_of(x2)), "lampa_rms_norm_fwd")
+    return y, (res_out if res_out is not None else x2)
+
+
+def _rms_norm_any(x, g, weight, bias, activation, residual, eps, prenorm, residual_in_fp32):
+    require_cuda(x, g, weight, bias, residual)
+    shape = x.shape
+    D = shape[-1]
+    x2 = x.reshape(-1, D).contiguous()
+    g2 = None if g is None else g.reshape(-1, D).to(x.dtype).contiguous()
+    if residual is not None:
+        assert residual.shape == shape
+    res2 = None if residual is None else residual.reshape(-1, D).contiguous()
+    residual_dtype = res2.dtype if res2 is not None else (torch.float32 if residual_in_fp32 else None)
+    w32, b32 = _f32(weight, x.device), _f32(bias, x.device)
+
+    def fn():
+        y, res_out = _norm_launch(x2, g2, w32, b32, res2, residual_dtype, eps, activation)
+        return (y.reshape(shape), res_out.reshape(shape)) if prenorm else y.reshape(shape)
+
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, g, weight, bias, residual)):
+        return _ForwardOnly.apply(fn, x)
+    return fn()
+
+
+def rms_norm_gated(x: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, activation: str = 'swish',
+                   residual: Optional[torch.Tensor] = None, prenorm: bool = False, residual_in_fp32: bool = False,
+                   eps: float = 1e-6):
+    """``fused_norm.py:856-878``: y = rmsnorm(x + residual) * weight + bias, times ``g * sigmoid(g)`` ('swish' /
+    'silu') or ``sigmoid(g)`` ('sigmoid'); the norm runs over the last dimension. ``prenorm`` also returns x + residual."""
+    if activation not in ('swish', 'silu', 'sigmoid'):
+        raise ValueError(f"Unsupported activation: {activation}")
+    return _rms_norm_any(x, g, weight, bias, activation, residual, eps, prenorm, residual_in_fp32)
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, residual: torch.Tensor = None, eps: float = 1e-5,
+             prenorm: bool = False, residual_in_fp32: bool = False):
+    """``fused_norm.py:2094-2112``: y = rmsnorm(x + residual) * weight + bias; ``prenorm`` also returns x + residual."""
+    return _rms_norm_any(x, None, weight, bias, None, residual, eps, prenorm, residual_in_fp32)
+
+
+class FusedRMSNormGated(nn.Module):
+    """``fused_norm.py:1003-1064``."""
+
+    def __init__(self, hidden_size: int, elementwise_affine: bool = True, eps: float = 1e-5, activation: str = 'swish',
+                 device=None, dtype=None):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.elementwise_affine = elementwise_affine
+        self.eps = eps
+        self.activation = activation
+        if self.activation not in ['swish', 'silu', 'sigmoid']:
+            raise ValueError(f"Unsupported activation: {self.activation}")
+        if elementwise_affine:
+            self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
+        else:
+            self.register_parameter("weight", None)
+        self.register_parameter("bias", None)
+
+    def forward(self, x: torch.Tensor, g: torch.Tensor, residual: Optional[torch.Tensor] = None, prenorm: bool = False,
+                residual_in_fp32: bool = False) -> torch.Tensor:
+        return rms_norm_gated(x, g, self.weight, self.bias, self.activation, residual=residual, eps=self.eps,
+                              prenorm=prenorm, residual_in_fp32=residual_in_fp32)
+
+
+class FusedRMSNormSwishGate(FusedRMSNormGated):
+    """``fused_norm.py:1088-1104``."""
+
+    def __init__(self, hidden_size: int, elementwise_affine: bool = True, eps: float = 1e-5, device=None, dtype=None):
+        super().__init__(hidden_size=hidden_size, elementwise_affine=elementwise_affine, eps=eps, device=device,
+                         dtype=dtype)
+
+
+class RMSNorm(nn.Module):
+    """``fused_norm.py:2307-2354``."""
+
+    def __init__(self, hidden_size: int, elementwise_affine: bool = True, bias: bool = False, eps: float = 1e-5):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.elementwise_affine = elementwise_affine
+        self.eps = eps
+        self.register_parameter("weight", None)
+        self.register_parameter("bias", None)
+        if elementwise_affine:
+            self.weight = nn.Parameter(torch.ones(hidden_size))
+            if bias:
+                self.bias = nn.Parameter(torch.zeros(hidden_size))
+
+    def forward(self, x, residual=None, prenorm=False, residual_in_fp32=False):
+        return rms_norm(x, self.weight, self.bias, residual=residual, eps=self.eps, prenorm=prenorm,
+                        residual_in_fp32=residual_in_fp32)
