@@ -144,19 +144,33 @@ int lampa_hept_sort_keys(const float* hashed, const int32_t* rank_eta, const int
  * x[t - (W-1) + j, d]) + residual[t, d]; taps before the start of the token's sequence are zero.
  * x, residual, y [n_tokens, D] of dtype (LAMPA_BF16/FP16/FP32) with row strides in elements; weight fp32 [D, W],
  * bias fp32 [D] or NULL; cu_seqlens device int64 [n_seq+1] or NULL (then n_tokens / t_len sequences of t_len tokens);
- * activation 0 none, 1 SiLU. D and the strides multiples of 8, pointers 16-byte aligned, W <= 8. */
+ * activation 0 none, 1 SiLU. D and the strides multiples of 8, pointers 16-byte aligned, W <= 8.
+ * y_split in (0, D): output columns [i*y_split, (i+1)*y_split) go to the i-th of D / y_split tensors
+ * [n_tokens, y_split] that lie y_split_stride elements apart (one launch over the q|k|v columns of a fused projection
+ * writing q, k and v); y_split <= 0: one [n_tokens, D] output. */
 int lampa_causal_conv1d_fwd(const void* x, int64_t x_stride, int64_t n_tokens, int D, int W, const float* weight,
                             const float* bias, const void* residual, int64_t res_stride, const int64_t* cu_seqlens,
-                            int n_seq, int64_t t_len, int activation, int dtype, void* y, int64_t y_stride, void* stream);
+                            int n_seq, int64_t t_len, int activation, int dtype, void* y, int64_t y_stride, int y_split,
+                            int64_t y_split_stride, void* stream);
 
 /* RMS norm over the last dimension with optional residual add, weight, bias and output gate. Replaces
  * layer_norm_gated_fwd / layer_norm_fwd with is_rms_norm (models/hattention/fused_norm.py:40-111,456-531,1436-1506).
  * s = x + residual; residual_out = s; y = s / sqrt(mean(s^2) + eps) * weight + bias; with g: y *= g * sigmoid(g)
  * (activation 1) or sigmoid(g) (activation 2). x, g, y [rows, D] of dtype; residual, residual_out of res_dtype;
- * weight, bias fp32 [D]; rstd_out fp32 [rows]; every pointer but x and y may be NULL. D % 8 == 0, D <= 2048. */
+ * weight, bias fp32 [D]; rstd_out fp32 [rows]; every pointer but x and y may be NULL. D % 8 == 0, D <= 2048.
+ * g_group > 0: g is a slice of a wider tensor with g_group rows of D channels per token and g_group_stride elements
+ * between tokens (the g_proj columns of a fused projection output); g_group <= 0: g is [rows, D] contiguous. */
 int lampa_rms_norm_fwd(const void* x, const void* g, const float* weight, const float* bias, const void* residual,
                        void* residual_out, void* y, float* rstd_out, int64_t rows, int D, float eps, int activation,
-                       int dtype, int res_dtype, void* stream);
+                       int dtype, int res_dtype, int g_group, int64_t g_group_stride, void* stream);
+
+/* Decay and write gates of a gated-delta layer. Replaces the elementwise tail of GatedDeltaProduct.forward
+ * (models/hattention/modeling_gated_deltaproduct.py:541-547,568-570): g = -exp(A_log) * softplus(a + dt_bias),
+ * beta = sigmoid(b) * beta_scale (2 with allow_neg_eigval). a, b [n_tokens, H] of dtype, row strides in elements;
+ * A_log, dt_bias fp32 [H]; g, beta fp32 [n_tokens, H]. */
+int lampa_gdr_gates_fwd(const void* a, int64_t a_stride, const void* b, int64_t b_stride, const float* A_log,
+                        const float* dt_bias, int64_t n_tokens, int H, float beta_scale, int dtype, float* g, float* beta,
+                        void* stream);
 
 /* ---------------------------------------------------------------------------------------- gated-delta forward */
 

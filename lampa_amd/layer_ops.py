@@ -5,6 +5,7 @@ Mirrors ``causal_conv1d`` / ``ShortConvolution`` (``models/hattention/short_conv
 ``rms_norm_gated`` / ``rms_norm`` / ``FusedRMSNormGated`` / ``FusedRMSNormSwishGate`` / ``RMSNorm``
 (``models/hattention/fused_norm.py:856-878,1003-1104,2094-2354``). Forward only; GPU tensors only (no CPU fallback).
 """
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -35,24 +36,72 @@ def _code(dtype) -> int:
     return _DTYPES[dtype]
 
 
+_F32_CACHE = {}
+
+
+def _root(t: torch.Tensor) -> torch.Tensor:
+    return t._base if t._base is not None else t
+
+
+def _stamp(t: torch.Tensor):
+    r = _root(t)
+    return (id(r), tuple(t.shape), tuple(t.stride()), t.storage_offset())
+
+
+def _fresh(entry, parts) -> bool:
+    """A remembered copy is valid while every source object is alive, unmoved and unmodified in place."""
+    return entry is not None and all(ref() is _root(p) and ver == _root(p)._version and addr == p.data_ptr()
+                                     for (ref, ver, addr), p in zip(entry[0], parts))
+
+
+def _remember(key, parts, value):
+    if len(_F32_CACHE) > 512:
+        _F32_CACHE.clear()
+    _F32_CACHE[key] = ([(weakref.ref(_root(p)), _root(p)._version, p.data_ptr()) for p in parts], value)
+    return value
+
+
 def _f32(t: Optional[torch.Tensor], device) -> Optional[torch.Tensor]:
-    return None if t is None else t.detach().to(device=device, dtype=torch.float32).contiguous()
+    """fp32 contiguous copy of a small parameter on ``device``. Copies are remembered per source tensor object and
+    dropped when it is modified in place, moved or freed, so a layer does not convert its weights on every call
+    (edits made through ``.data`` bypass the version counter and are not noticed)."""
+    if t is None:
+        return None
+    if t.dtype == torch.float32 and t.is_contiguous() and t.device == torch.device(device):
+        return t.detach()
+    key = ("one", _stamp(t), str(device))
+    entry = _F32_CACHE.get(key)
+    if _fresh(entry, [t]):
+        return entry[1]
+    return _remember(key, [t], t.detach().to(device=device, dtype=torch.float32).contiguous())
+
+
+def _cat_f32(parts, device) -> torch.Tensor:
+    key = ("cat", tuple(_stamp(p) for p in parts), str(device))
+    entry = _F32_CACHE.get(key)
+    if _fresh(entry, parts):
+        return entry[1]
+    return _remember(key, parts,
+                     torch.cat([p.detach().to(device=device, dtype=torch.float32) for p in parts]).contiguous())
 
 
 # ----------------------------------------------------------------------------------------------- short convolution
 @torch.no_grad()
-def _conv_launch(x2: torch.Tensor, weight, bias, residual2, activation, cu_seqlens, t_len: int) -> torch.Tensor:
-    """x2 [tokens, D] (last dim contiguous, any row stride) -> y [tokens, D] contiguous."""
+def _conv_launch(x2: torch.Tensor, weight, bias, residual2, activation, cu_seqlens, t_len: int, parts: int = 1):
+    """x2 [tokens, D] (last dim contiguous, any row stride) -> y [tokens, D] contiguous, or [parts, tokens, D / parts]
+    when the columns are split over ``parts`` output tensors."""
     n, D = x2.shape
     W = weight.shape[-1]
-    y = torch.empty((n, D), dtype=x2.dtype, device=x2.device)
+    split = D // parts
+    y = torch.empty((n, D) if parts == 1 else (parts, n, split), dtype=x2.dtype, device=x2.device)
     if n == 0:
         return y
     cu = None if cu_seqlens is None else cu_seqlens.to(device=x2.device, dtype=torch.int64).contiguous()
     check(_capi.lib().lampa_causal_conv1d_fwd(
         ptr(x2), x2.stride(0), n, D, W, ptr(weight), ptr(bias), ptr(residual2),
         0 if residual2 is None else residual2.stride(0), ptr(cu), 0 if cu is None else cu.numel() - 1, t_len,
-        _ACT[activation], _code(x2.dtype), ptr(y), D, stream_of(x2)), "lampa_causal_conv1d_fwd")
+        _ACT[activation], _code(x2.dtype), ptr(y), split, split if parts > 1 else 0, n * split, stream_of(x2)),
+        "lampa_causal_conv1d_fwd")
     return y
 
 
@@ -87,6 +136,26 @@ def causal_conv1d(x: torch.Tensor, weight: Optional[torch.Tensor] = None, bias: 
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias, residual)):
         return _ForwardOnly.apply(fn, x, weight)
     return fn()
+
+
+@torch.no_grad()
+def causal_conv1d_split(x: torch.Tensor, weights, biases=None, activation: Optional[str] = None,
+                        cu_seqlens: Optional[torch.Tensor] = None):
+    """One launch for several convolutions of equal width over adjacent column blocks of x [B, T, n * D] (the q | k | v
+    columns of a fused projection): weights = n tensors [D, W] (or [D, 1, W]), biases = None or n tensors [D].
+    Returns n contiguous tensors [B, T, D]. Same arithmetic as ``causal_conv1d`` on each block."""
+    require_cuda(x, cu_seqlens, *weights)
+    B, T, Dall = x.shape
+    n = len(weights)
+    D = Dall // n
+    if Dall != n * D or any(w.numel() != weights[0].numel() or w.shape[0] != D for w in weights):
+        raise ValueError("causal_conv1d_split: the column blocks must have equal width")
+    if cu_seqlens is not None and B != 1:
+        raise ValueError("causal_conv1d_split: batch size must be 1 when cu_seqlens is given")
+    w32 = _cat_f32([w.reshape(D, -1) for w in weights], x.device)
+    b32 = None if biases is None or biases[0] is None else _cat_f32(list(biases), x.device)
+    y = _conv_launch(_rows(x), w32, b32, None, activation, cu_seqlens, max(T, 1), parts=n)
+    return tuple(y[i].view(B, T, D) for i in range(n))
 
 
 class ShortConvolution(nn.Conv1d):
@@ -156,7 +225,7 @@ class ShortConvolution(nn.Conv1d):
 
 # ------------------------------------------------------------------------------------------------------ RMS norm
 @torch.no_grad()
-def _norm_launch(x2, g2, weight, bias, residual2, residual_dtype, eps, activation):
+def _norm_launch(x2, g2, weight, bias, residual2, residual_dtype, eps, activation, g_group=0, g_group_stride=0):
     rows, D = x2.shape
     y = torch.empty_like(x2)
     want_res_out = residual2 is not None or (residual_dtype is not None and residual_dtype != x2.dtype)
@@ -165,7 +234,8 @@ def _norm_launch(x2, g2, weight, bias, residual2, residual_dtype, eps, activatio
         check(_capi.lib().lampa_rms_norm_fwd(
             ptr(x2), ptr(g2), ptr(weight), ptr(bias), ptr(residual2), ptr(res_out), ptr(y), None, rows, D, float(eps),
             _ACT[activation] if g2 is not None else 0, _code(x2.dtype),
-            _code(residual_dtype) if want_res_out else _code(x2.dtype), stream_of(x2)), "lampa_rms_norm_fwd")
+            _code(residual_dtype) if want_res_out else _code(x2.dtype), g_group, g_group_stride, stream_of(x2)),
+            "lampa_rms_norm_fwd")
     return y, (res_out if res_out is not None else x2)
 
 
@@ -174,7 +244,16 @@ def _rms_norm_any(x, g, weight, bias, activation, residual, eps, prenorm, residu
     shape = x.shape
     D = shape[-1]
     x2 = x.reshape(-1, D).contiguous()
-    g2 = None if g is None else g.reshape(-1, D).to(x.dtype).contiguous()
+    g2, g_group, g_group_stride = None, 0, 0
+    if g is not None:
+        g = g.to(x.dtype)
+        # [..., T, H, D] view of the g_proj columns of a wider projection output: read in place
+        if (g.dim() >= 3 and not g.is_contiguous() and g.stride(-1) == 1 and g.stride(-2) == D and g.stride(-3) % 8 == 0
+                and g.data_ptr() % 16 == 0 and g.stride(-3) >= g.shape[-2] * D
+                and all(g.stride(i) == g.stride(i + 1) * g.shape[i + 1] for i in range(g.dim() - 3))):
+            g2, g_group, g_group_stride = g, g.shape[-2], g.stride(-3)
+        else:
+            g2 = g.reshape(-1, D).contiguous()
     if residual is not None:
         assert residual.shape == shape
     res2 = None if residual is None else residual.reshape(-1, D).contiguous()
@@ -182,7 +261,7 @@ def _rms_norm_any(x, g, weight, bias, activation, residual, eps, prenorm, residu
     w32, b32 = _f32(weight, x.device), _f32(bias, x.device)
 
     def fn():
-        y, res_out = _norm_launch(x2, g2, w32, b32, res2, residual_dtype, eps, activation)
+        y, res_out = _norm_launch(x2, g2, w32, b32, res2, residual_dtype, eps, activation, g_group, g_group_stride)
         return (y.reshape(shape), res_out.reshape(shape)) if prenorm else y.reshape(shape)
 
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, g, weight, bias, residual)):
@@ -256,3 +335,32 @@ class RMSNorm(nn.Module):
     def forward(self, x, residual=None, prenorm=False, residual_in_fp32=False):
         return rms_norm(x, self.weight, self.bias, residual=residual, eps=self.eps, prenorm=prenorm,
                         residual_in_fp32=residual_in_fp32)
+
+
+# ----------------------------------------------------------------------------------------- decay and write gates
+@torch.no_grad()
+def gdr_gates(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, beta_scale: float = 1.0):
+    """``modeling_gated_deltaproduct.py:541-547,568-570``: g = -exp(A_log) * softplus(a + dt_bias) and
+    beta = sigmoid(b) * beta_scale, both fp32 [..., H]. a, b [..., H] may be column slices of a wider projection."""
+    require_cuda(a, b, A_log, dt_bias)
+    H = a.shape[-1]
+    assert b.shape == a.shape and a.dtype == b.dtype
+
+    def rows(t):
+        if t.dim() >= 2 and t.stride(-1) == 1 and all(t.stride(i) == t.stride(i + 1) * t.shape[i + 1]
+                                                      for i in range(t.dim() - 2)):
+            return t, t.stride(-2) if t.dim() >= 2 else H
+        t = t.contiguous()
+        return t, H
+
+    a2, a_stride = rows(a)
+    b2, b_stride = rows(b)
+    n = a.numel() // H
+    g = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    beta = torch.empty_like(g)
+    A32, dt32 = _f32(A_log, a.device), _f32(dt_bias, a.device)  # named: they must outlive the launch call
+    if n:
+        check(_capi.lib().lampa_gdr_gates_fwd(ptr(a2), a_stride, ptr(b2), b_stride, ptr(A32), ptr(dt32), n, H,
+                                              float(beta_scale), _code(a.dtype), ptr(g), ptr(beta), stream_of(a)),
+              "lampa_gdr_gates_fwd")
+    return g, beta

@@ -60,6 +60,25 @@ def test_causal_conv1d_varlen_strided_and_config_shape(device):
         lo.causal_conv1d(proj[..., :D], w.to(device), activation="gelu")
 
 
+def test_causal_conv1d_split_equals_separate_calls(device):
+    gen = torch.Generator().manual_seed(6)
+    T, D = 3001, 128
+    proj = torch.randn(1, T, 3 * D + 16, generator=gen).to(torch.bfloat16).to(device)
+    ws = [(torch.randn(D, 1, 4, generator=gen) * 0.5).to(torch.bfloat16).to(device) for _ in range(3)]
+    bs = [torch.randn(D, generator=gen).to(torch.bfloat16).to(device) for _ in range(3)]
+    cu = torch.tensor([0, 5, 1000, 3001], device=device)
+    for biases, cu_t in ((None, None), (bs, cu)):
+        outs = lo.causal_conv1d_split(proj[..., :3 * D], ws, biases, "silu", cu_t)
+        for i, y in enumerate(outs):
+            one = lo.causal_conv1d(proj[..., i * D:(i + 1) * D], ws[i].reshape(D, 4), None if biases is None else bs[i],
+                                   None, "silu", cu_t)
+            assert y.is_contiguous() and torch.equal(y, one)
+    with torch.no_grad():                                   # remembered fp32 copies follow in-place weight updates
+        ws[0].mul_(2.0)
+    again = lo.causal_conv1d_split(proj[..., :3 * D], ws, None, "silu")[0]
+    assert torch.equal(again, lo.causal_conv1d(proj[..., :D].contiguous(), ws[0].reshape(D, 4).clone(), None, None, "silu"))
+
+
 def test_short_convolution_module_cache_and_step(device):
     torch.manual_seed(4)
     D, W, T = 64, 4, 19
