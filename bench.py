@@ -222,6 +222,33 @@ def main():
     }
     del bc_d, bf_d
 
+    # ---- config 3: the 4-layer block on one event (input linear, LSH sort, layers, unsort, head), bf16 weights seed 2 ----
+    from lampa_amd import block as lblock
+    torch.manual_seed(2)
+    blk = lblock.LshgdBlock().to(dev).to(torch.bfloat16)
+    for _ in range(3):
+        blk(feats_d, coords_d)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        blk(feats_d, coords_d)
+    torch.cuda.synchronize()
+    block_us = 1e6 * (time.perf_counter() - t0) / 10
+    _capi.profile_begin()
+    blk(feats_d, coords_d)
+    bstage = {}
+    for name, ms in _capi.profile_end(max_entries=512):
+        bstage[name] = bstage.get(name, 0.0) + 1e3 * ms
+    block_info = {
+        "workload": f"config3: N={N_HITS} hits, linear 24->128, LSH sort, 4 gated-delta layers (H=8, d=64, conv 4, SiLU "
+                    "gate, RMS norm), unsort, head 128->24; bf16 weights, seed 2",
+        "us_per_event": round(block_us, 1), "hits_per_s": round(N_HITS / (block_us * 1e-6), 1),
+        "own_kernel_us": {n: round(v_, 1) for n, v_ in bstage.items()},
+        "note": "own_kernel_us: this package's kernels with HIP events; the rest of the time is the library GEMMs "
+                "(projections) and launch gaps",
+    }
+    del blk
+
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
     if not args.no_cpu:
@@ -242,7 +269,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info,
     }
     print(json.dumps(out))
 
