@@ -192,3 +192,18 @@ def test_bucket_sort_batch_of_events_bit_exact(device):
     one = lsh.lsh_bucket_sort(coords[2].to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats[2].to(device))
     for name in ("ids", "meta", "keys", "perm", "feats"):
         assert torch.equal(full[name][2], one[name]), name
+
+
+def test_bucket_sort_batch_of_nine_events_matches_single_events(device):
+    """Eight or more events take the launch forms that keep an event (and a sort segment) on one XCD."""
+    n, n_events = 5000, 9
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    coords = torch.stack([synth.collider_event(n, seed=20 + e)[0] for e in range(n_events)])
+    feats = torch.stack([synth.collider_event(n, seed=20 + e)[1] for e in range(n_events)])
+    lens = torch.tensor([5000, 4999, 1, 0, 2048, 2049, 5000, 77, 4096], dtype=torch.int32)
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats.to(device), n_valid=lens)
+    for e in range(n_events):
+        want = ol.bucket_sort(coords[e].numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats[e].numpy(),
+                              n_valid=int(lens[e]))
+        for name in ("ids", "meta", "keys", "perm", "feats"):
+            assert np.array_equal(_np(got[name][e]), want[name]), (name, e)
