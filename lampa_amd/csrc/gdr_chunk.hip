@@ -925,8 +925,164 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 }
 
 // ---- host side ------------------------------------------------------------------------------------------------
+// ---- two-level scan ------------------------------------------------------------------------------------------------
+// A long sequence has many segments and the scan above walks them one after the other (0.45 us per step, a chain of
+// dependent MFMA / LDS-exchange stages with 16 workgroups on the whole chip). With groups of G segments the serial
+// depth drops from n to about n / G + 2 G:
+//   GROUP  every group but the last of a sequence, in parallel: the composite of its G segments, i.e. the scan step
+//          applied to the KT + VT columns [P_M | P_N] starting from [I | 0]; written as a segment composite is
+//          (D = product of the decays, M' = P_M - D I as bf16 A-operand fragments, N = P_N in accumulator order);
+//   TOP    per sequence, serial over the groups with these composites: the state every group starts from;
+//   LEAF   every group in parallel: from its start state over its segments, writing the state every segment starts
+//          from (what the single-level scan writes).
+// Same step code in the three modes; loops are branch free with clamped operands and a spare store slot as above.
+enum { SCAN_GROUP = 1, SCAN_TOP = 2, SCAN_LEAF = 3 };
+#define GDR_SCAN_GROUP 8  // segments per group; a multiple of the ring depth
+
+template <int KT, int VT, int DEPTH, int MODE>
+__global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlanView pv,
+                                                                  const unsigned char* __restrict__ Msrc,
+                                                                  const unsigned char* __restrict__ Nsrc,
+                                                                  const float* __restrict__ Dsrc,
+                                                                  const float* __restrict__ h0,
+                                                                  const float* __restrict__ init_slab,
+                                                                  float* __restrict__ dst, unsigned char* __restrict__ Mout,
+                                                                  unsigned char* __restrict__ Nout, float* __restrict__ Dout,
+                                                                  int HV, int spare_slot, int gmax) {
+  constexpr int G = GDR_SCAN_GROUP;
+  static_assert(G % DEPTH == 0, "a group must be a whole number of ring rounds");
+  constexpr int NKS = KT / 16;
+  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  constexpr int NCB = MODE == SCAN_GROUP ? (KT + VT) / 32 : VT / 32;  // 32-column blocks per item of the grid
+  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
+  const int vn = blockIdx.x % NCB, j = blockIdx.x / NCB, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
+  const int ngroups = (nseg + G - 1) / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  // items = the maps this workgroup applies, slots = where it stores the running state before each of them
+  int item0, nsteps, slot0;
+  if (MODE == SCAN_GROUP) {
+    if (j >= ngroups - 1) return;  // the composite of a sequence's last group is never needed
+    item0 = seg0 + j * G; nsteps = G - 1; slot0 = 0;
+  } else if (MODE == SCAN_TOP) {
+    item0 = seq * gmax; nsteps = ngroups - 1; slot0 = item0;
+  } else {
+    if (j >= ngroups) return;
+    item0 = seg0 + j * G; nsteps = min(G, nseg - j * G) - 1; slot0 = item0;
+  }
+  const int last = MODE == SCAN_GROUP ? nsteps : nsteps - 1;   // last map that is really applied (prefetches are clamped to it)
+  const bool is_pm = MODE == SCAN_GROUP && vn < KT / 32;       // a block of P_M: no additive term, starts from I
+  const int nblk = MODE == SCAN_GROUP ? max(vn - KT / 32, 0) : vn;  // 32-column block of N / of the state
+
+  f32x16 S = zero16();
+  if (MODE == SCAN_GROUP) {
+    if (is_pm) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[r] = (32 * wave + acc_row(r, hh) == 32 * vn + ln) ? 1.0f : 0.0f;
+    }
+  } else if (MODE == SCAN_LEAF) {
+    const f32x4* src = reinterpret_cast<const f32x4*>(init_slab + (((size_t)(seq * gmax + j) * HV + hv) * (VT / 32) + vn) * (KT * 32));
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 t = src[(wave * 4 + q4) * 64 + lane];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) S[4 * q4 + e] = t[e];
+    }
+  } else if (h0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + 32 * vn + ln];
+  }
+
+  bf16x8 rm[DEPTH][NKS];
+  f32x4 rn[DEPTH][4];
+  float rd[DEPTH];
+  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+    const size_t sh = (size_t)(item0 + p) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>(Msrc + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>(Nsrc + (sh * (VT / 32) + nblk) * N_BYTES);
+#pragma unroll
+    for (int f = 0; f < NKS; ++f) m[f] = M[(wave * NKS + (2 * wave + f) % NKS) * 64 + lane];  // own fragments first
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) n[q4] = N[(wave * 4 + q4) * 64 + lane];
+    d = Dsrc[sh];
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, last)), rm[d], rn[d], rd[d]);
+
+  float dprod = 1.0f;
+  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+    if (MODE != SCAN_GROUP) {
+      const size_t slot = p <= nsteps ? (size_t)(slot0 + p) : (size_t)spare_slot;
+      f32x4* si = reinterpret_cast<f32x4*>(dst + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        si[(wave * 4 + q4) * 64 + lane] = t;
+      }
+    }
+    const float dec = dd;
+    dprod *= dec;
+    unsigned char* xbuf = s_x[p & 1];
+    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
+    frag_store(xbuf, 2 * wave + 0, lane, own0);
+    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    f32x16 acc;
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[4 * q4 + e], is_pm ? 0.0f : n[q4][e]);
+    acc = mfma32(m[0], own0, acc);
+    acc = mfma32(m[1], own1, acc);
+    lds_barrier();
+#pragma unroll
+    for (int f = 2; f < NKS; ++f) acc = mfma32(m[f], frag_load(xbuf, (2 * wave + f) % NKS, lane), acc);
+    S = acc;
+    issue(max(0, min(p + DEPTH, last)), m, n, dd);
+  };
+  constexpr int LONG = 4 * DEPTH;
+  int p0 = 0;
+  if (MODE != SCAN_GROUP) {
+    for (; p0 + LONG <= nsteps + 1; p0 += LONG) {
+#pragma unroll
+      for (int u = 0; u < LONG; ++u) step(p0 + u, rm[u % DEPTH], rn[u % DEPTH], rd[u % DEPTH]);
+    }
+  }
+  for (; p0 <= nsteps; p0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) step(p0 + d, rm[d], rn[d], rd[d]);
+  }
+
+  if (MODE == SCAN_GROUP) {  // exactly G maps were applied (G is a multiple of DEPTH): store the composite
+    const size_t gh = (size_t)(seq * gmax + j) * HV + hv;
+    if (is_pm) {
+      unsigned char* out = Mout + gh * M_BYTES;
+      const int mcol = 32 * vn + ln, ks = mcol >> 4, c16 = mcol & 15;
+      const int hs = (c16 >> 2) & 1, slot = 4 * (c16 >> 3) + (c16 & 3);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * wave + acc_row(r, hh);
+        const float val = S[r] - (row == mcol ? dprod : 0.0f);
+        *reinterpret_cast<__bf16*>(out + ((size_t)((wave * NKS + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) = (__bf16)val;
+      }
+      if (vn == 0 && tid == 0) Dout[gh] = dprod;
+    } else {
+      f32x4* out = reinterpret_cast<f32x4*>(Nout + (gh * (VT / 32) + nblk) * N_BYTES);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        out[(wave * 4 + q4) * 64 + lane] = t;
+      }
+    }
+  }
+}
+
 struct GdrWorkspace {
-  int64_t off_t, off_m, off_n, off_d, off_sinit, bytes;
+  int64_t off_t, off_m, off_n, off_d, off_sinit, off_gm, off_gn, off_gd, off_gs, max_groups, bytes;
 };
 
 static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, int V) {
@@ -937,6 +1093,12 @@ static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, i
   w.off_n = off;     off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.off_d = off;     off += lampa_align_up(segs * HV * 4, 256);
   w.off_sinit = off; off += lampa_align_up((segs + 1) * HV * (int64_t)K * V * 4, 256);  // + a spare slot (scan)
+  // two-level scan: composites and start states of the groups of GDR_SCAN_GROUP segments (+ a spare state slot)
+  w.max_groups = segs / GDR_SCAN_GROUP + 2;
+  w.off_gm = off;    off += lampa_align_up(w.max_groups * HV * (int64_t)K * K * 2, 256);
+  w.off_gn = off;    off += lampa_align_up(w.max_groups * HV * (int64_t)K * V * 4, 256);
+  w.off_gd = off;    off += lampa_align_up(w.max_groups * HV * 4, 256);
+  w.off_gs = off;    off += lampa_align_up((w.max_groups + 1) * HV * (int64_t)K * V * 4, 256);
   w.bytes = off > 0 ? off : 256;
   return w;
 }
@@ -951,8 +1113,8 @@ extern "C" int64_t lampa_gdr_chunk_workspace_bytes(int64_t total_chunks, int64_t
 
 template <typename T, int KT, int VT>
 static int gdr_chunk_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, void* o,
-                            const float* h0, float* ht, const GdrPlanView pv, int n_seq, int chunks, int segs, int H,
-                            int HV, float scale, int l2norm, unsigned char* ws, hipStream_t s) {
+                            const float* h0, float* ht, const GdrPlanView pv, int n_seq, int chunks, int segs, int max_nseg,
+                            int H, int HV, float scale, int l2norm, unsigned char* ws, hipStream_t s) {
   const GdrWorkspace w = gdr_workspace(chunks, segs, HV, KT, VT);
   unsigned char* tf = ws + w.off_t;
   unsigned char* Mc = ws + w.off_m;
@@ -981,9 +1143,30 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
-  hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
-                     pv, Mc, Nc, Dc, h0, Si, HV, segs);
-  LAMPA_PROF(s, "gdr_scan_kernel");
+  const int gmax = (max_nseg + GDR_SCAN_GROUP - 1) / GDR_SCAN_GROUP;
+  if (max_nseg >= 3 * GDR_SCAN_GROUP && (int64_t)n_seq * gmax <= w.max_groups) {
+    // long sequences: group composites, scan over the groups, scan inside the groups
+    unsigned char* Gm = ws + w.off_gm;
+    unsigned char* Gn = ws + w.off_gn;
+    float* Gd = (float*)(ws + w.off_gd);
+    float* Gs = (float*)(ws + w.off_gs);
+    const dim3 block(64 * (KT / 32));
+    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
+                       Nc, Dc, (const float*)nullptr, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
+    LAMPA_PROF(s, "gdr_scan2_kernel<group>");
+    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_TOP>), dim3(VT / 32, n_seq, HV), block, 0, s, pv, Gm, Gn, Gd, h0,
+                       (const float*)nullptr, Gs, (unsigned char*)nullptr, (unsigned char*)nullptr, (float*)nullptr, HV,
+                       (int)w.max_groups, gmax);
+    LAMPA_PROF(s, "gdr_scan2_kernel<top>");
+    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc, Dc,
+                       (const float*)nullptr, Gs, Si, (unsigned char*)nullptr, (unsigned char*)nullptr, (float*)nullptr,
+                       HV, segs, gmax);
+    LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
+  } else {
+    hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
+                       pv, Mc, Nc, Dc, h0, Si, HV, segs);
+    LAMPA_PROF(s, "gdr_scan_kernel");
+  }
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
                      (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
                      (float*)nullptr, (T*)o, ht, H, HV, scale, l2norm);
@@ -1008,8 +1191,10 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
   hipStream_t s = (hipStream_t)stream;
   unsigned char* ws = (unsigned char*)workspace;
   const GdrPlanView pv = gdr_plan_view(plan_host, plan_dev);
+  int max_nseg = 0;
+  for (int i = 0; i < n_seq; ++i) max_nseg = plan_host[plan_host[PLAN_OFF_SEQ_NSEG] + i] > max_nseg ? plan_host[plan_host[PLAN_OFF_SEQ_NSEG] + i] : max_nseg;
 #define GDR_CASE(TT, KK, VV)                                                                                       \
-  return gdr_chunk_launch<TT, KK, VV>(q, k, v, g, beta, o, h0, ht, pv, n_seq, chunks, segs, H, HV, scale, \
+  return gdr_chunk_launch<TT, KK, VV>(q, k, v, g, beta, o, h0, ht, pv, n_seq, chunks, segs, max_nseg, H, HV, scale, \
                                       l2norm, ws, s)
   if (dtype == GDR_BF16) {
     if (K == 64 && V == 64) GDR_CASE(__bf16, 64, 64);

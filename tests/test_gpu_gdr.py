@@ -3,6 +3,7 @@
 Tolerances (from the benchmark contract): bf16 inputs with fp32 accumulation -- max-abs 2e-2 and mean-relative
 5e-3 on outputs and final states; fp32 mode -- 1e-4.
 """
+import numpy as np
 import pytest
 import torch
 
@@ -98,6 +99,38 @@ def test_chunk_segment_split_is_invisible(device, cps, monkeypatch):
     o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True)
     _assert_bf16_close(o, want_o, f"o cps={cps}")
     _assert_bf16_close(s, want_s, f"state cps={cps}")
+
+
+@pytest.mark.parametrize("K,V,n_chunks", [(64, 64, 24), (64, 64, 27), (64, 64, 63), (128, 128, 41), (64, 128, 33)])
+def test_two_level_scan_over_many_segments(device, K, V, n_chunks, monkeypatch):
+    """One chunk per segment makes 24 or more segments per sequence: the scan then runs as group composites, a scan
+    over the groups and a scan inside the groups (groups of 8; 27 / 41 / 33 leave a ragged last group). Weak decay, so
+    that the state really travels through all the levels; initial state and final state included."""
+    monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", 1)
+    T = 64 * n_chunks - 5
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 2, K, V, torch.bfloat16, seed=n_chunks, g_scale=0.003)
+    h0 = 0.5 * torch.randn(1, 2, K, V, generator=torch.Generator().manual_seed(3))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, l2=og.L2_CHUNK)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device), output_final_state=True,
+                                     use_qk_l2norm_in_kernel=True)
+    _assert_bf16_close(o, want_o, f"o chunks={n_chunks}")
+    _assert_bf16_close(s, want_s, f"state chunks={n_chunks}")
+
+
+def test_two_level_scan_varlen_mixed_lengths(device, monkeypatch):
+    """Packed sequences of very different lengths: the long ones take the grouped scan, the short and the empty one
+    ride along in the same launches (their groups beyond the first do nothing)."""
+    monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", 1)
+    lens = [64 * 30 + 1, 5, 0, 64 * 9, 64 * 26 - 1]
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.long)
+    T = int(cu[-1])
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 2, 64, 64, torch.bfloat16, seed=11, g_scale=0.003)
+    h0 = 0.5 * torch.randn(len(lens), 2, 64, 64, generator=torch.Generator().manual_seed(4))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device), output_final_state=True,
+                                     cu_seqlens=cu.to(device))
+    _assert_bf16_close(o, want_o, "o varlen")
+    _assert_bf16_close(s, want_s, "state varlen")
 
 
 @pytest.mark.parametrize("K,V", [(128, 128), (64, 128), (128, 64)])
