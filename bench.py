@@ -82,8 +82,9 @@ def cpu_baseline_lsh(coords, feats, alpha):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # defaults long enough for the GPU clocks to settle (a layer is ~0.16 ms: 50 + 200 steps take 40 ms)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-sample-tokens", type=int, default=T,
                     help="tokens of the workload the CPU baseline is timed on (default: all of them, about 5-10 s)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (for profiler runs)")

@@ -4,7 +4,7 @@
 
 #include <string.h>
 
-#define PROF_MAX 256
+#define PROF_MAX 4096
 
 static bool g_recording = false;
 static int g_count = 0;
