@@ -934,9 +934,11 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 //          (D = product of the decays, M' = P_M - D I as bf16 A-operand fragments, N = P_N in accumulator order);
 //   TOP    per sequence, serial over the groups with these composites: the state every group starts from;
 //   LEAF   every group in parallel: from its start state over its segments, writing the state every segment starts
-//          from (what the single-level scan writes).
+//          from (what the single-level scan writes);
+//   LEAF2  TOP and LEAF in one launch: the workgroup of group j first walks the composites of groups 0 .. j-1 itself
+//          (at most gmax - 1 redundant steps) and then its own segments; one launch and one serial phase less.
 // Same step code in the three modes; loops are branch free with clamped operands and a spare store slot as above.
-enum { SCAN_GROUP = 1, SCAN_TOP = 2, SCAN_LEAF = 3 };
+enum { SCAN_GROUP = 1, SCAN_TOP = 2, SCAN_LEAF = 3, SCAN_LEAF2 = 4 };
 #define GDR_SCAN_GROUP 8  // segments per group; a multiple of the ring depth
 
 template <int KT, int VT, int DEPTH, int MODE>
@@ -960,8 +962,11 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   const int ngroups = (nseg + G - 1) / G;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   // items = the maps this workgroup applies, slots = where it stores the running state before each of them
-  int item0, nsteps, slot0;
-  if (MODE == SCAN_GROUP) {
+  int item0, nsteps, slot0, lead = 0;  // lead: group-level maps walked before the workgroup's own items (LEAF2)
+  if (MODE == SCAN_LEAF2) {
+    if (j >= ngroups) return;
+    item0 = seg0 + j * G; lead = j; nsteps = lead + min(G, nseg - j * G) - 1; slot0 = item0;
+  } else if (MODE == SCAN_GROUP) {
     if (j >= ngroups - 1) return;  // the composite of a sequence's last group is never needed
     item0 = seg0 + j * G; nsteps = G - 1; slot0 = 0;
   } else if (MODE == SCAN_TOP) {
@@ -998,14 +1003,15 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   f32x4 rn[DEPTH][4];
   float rd[DEPTH];
   auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
-    const size_t sh = (size_t)(item0 + p) * HV + hv;
-    const bf16x8* M = reinterpret_cast<const bf16x8*>(Msrc + sh * M_BYTES);
-    const f32x4* N = reinterpret_cast<const f32x4*>(Nsrc + (sh * (VT / 32) + nblk) * N_BYTES);
+    const bool top = MODE == SCAN_LEAF2 && p < lead;  // a group composite (read through the *out pointers)
+    const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mout : Msrc) + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>((top ? Nout : Nsrc) + (sh * (VT / 32) + nblk) * N_BYTES);
 #pragma unroll
     for (int f = 0; f < NKS; ++f) m[f] = M[(wave * NKS + (2 * wave + f) % NKS) * 64 + lane];  // own fragments first
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) n[q4] = N[(wave * 4 + q4) * 64 + lane];
-    d = Dsrc[sh];
+    d = (top ? Dout : Dsrc)[sh];
   };
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, last)), rm[d], rn[d], rd[d]);
@@ -1013,7 +1019,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   float dprod = 1.0f;
   auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
     if (MODE != SCAN_GROUP) {
-      const size_t slot = p <= nsteps ? (size_t)(slot0 + p) : (size_t)spare_slot;
+      const size_t slot = (p >= lead && p <= nsteps) ? (size_t)(slot0 + (p - lead)) : (size_t)spare_slot;
       f32x4* si = reinterpret_cast<f32x4*>(dst + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
@@ -1082,7 +1088,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
 }
 
 struct GdrWorkspace {
-  int64_t off_t, off_m, off_n, off_d, off_sinit, off_gm, off_gn, off_gd, off_gs, max_groups, bytes;
+  int64_t off_t, off_m, off_n, off_d, off_sinit, off_gm, off_gn, off_gd, max_groups, bytes;
 };
 
 static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, int V) {
@@ -1093,12 +1099,11 @@ static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, i
   w.off_n = off;     off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.off_d = off;     off += lampa_align_up(segs * HV * 4, 256);
   w.off_sinit = off; off += lampa_align_up((segs + 1) * HV * (int64_t)K * V * 4, 256);  // + a spare slot (scan)
-  // two-level scan: composites and start states of the groups of GDR_SCAN_GROUP segments (+ a spare state slot)
+  // two-level scan: composites of the groups of GDR_SCAN_GROUP segments
   w.max_groups = segs / GDR_SCAN_GROUP + 2;
   w.off_gm = off;    off += lampa_align_up(w.max_groups * HV * (int64_t)K * K * 2, 256);
   w.off_gn = off;    off += lampa_align_up(w.max_groups * HV * (int64_t)K * V * 4, 256);
   w.off_gd = off;    off += lampa_align_up(w.max_groups * HV * 4, 256);
-  w.off_gs = off;    off += lampa_align_up((w.max_groups + 1) * HV * (int64_t)K * V * 4, 256);
   w.bytes = off > 0 ? off : 256;
   return w;
 }
@@ -1149,18 +1154,12 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
     unsigned char* Gm = ws + w.off_gm;
     unsigned char* Gn = ws + w.off_gn;
     float* Gd = (float*)(ws + w.off_gd);
-    float* Gs = (float*)(ws + w.off_gs);
     const dim3 block(64 * (KT / 32));
     hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
                        Nc, Dc, (const float*)nullptr, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<group>");
-    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_TOP>), dim3(VT / 32, n_seq, HV), block, 0, s, pv, Gm, Gn, Gd, h0,
-                       (const float*)nullptr, Gs, (unsigned char*)nullptr, (unsigned char*)nullptr, (float*)nullptr, HV,
-                       (int)w.max_groups, gmax);
-    LAMPA_PROF(s, "gdr_scan2_kernel<top>");
-    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc, Dc,
-                       (const float*)nullptr, Gs, Si, (unsigned char*)nullptr, (unsigned char*)nullptr, (float*)nullptr,
-                       HV, segs, gmax);
+    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF2>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc,
+                       Dc, h0, (const float*)nullptr, Si, Gm, Gn, Gd, HV, segs, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
   } else {
     hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
