@@ -137,6 +137,15 @@ int lampa_geo_shift(const float* region_eta, const float* region_phi, const floa
 int lampa_hept_sort_keys(const float* hashed, const int32_t* rank_eta, const int32_t* rank_phi, const float* regions,
                          const float* hash_shift, int n_rows, int64_t n, int64_t n_raw, float* keys, void* stream);
 
+/* Hash inputs of the HEPT bucketing. Replaces prep_qk and the rearrange + zeroing of the padded rows after it
+ * (models/attention/hept.py:54-62,118-128): q_hat = [query | sqrt(2 qw) * coords] with qw[h, r] =
+ * sum_k exp(min(sum_d w[h, d, r, k], 50)) and the first appended column reusing qw[h, 0]. query, key [n, H, d];
+ * w [H, d, R, Kw]; coords [n, R + 1]; scale_ws: H * (R + 1) floats of device scratch; q_hat, k_hat [n, H, d + R + 1]
+ * (heads_first 0) or [H, n, d + R + 1] (heads_first 1); rows at or beyond n_raw are zero. All fp32. */
+int lampa_hept_prep_qk(const float* query, const float* key, const float* w, const float* coords, int64_t n, int64_t n_raw,
+                       int H, int d, int R, int Kw, int heads_first, float* scale_ws, float* q_hat, float* k_hat,
+                       void* stream);
+
 /* ------------------------------------------------------------------------------ operators around the forward */
 
 /* Depthwise causal short convolution with optional bias, SiLU and residual. Replaces causal_conv1d_fwd

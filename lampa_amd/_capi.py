@@ -40,6 +40,7 @@ _SIGNATURES = {
     "lampa_quantile_regions": (_i32, [_vp, _i32, _i64, _vp, _i32, _vp, _vp]),
     "lampa_geo_shift": (_i32, [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp]),
     "lampa_hept_sort_keys": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _vp]),
+    "lampa_hept_prep_qk": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp]),
     "lampa_causal_conv1d_fwd": (_i32, [_vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _vp, _i32, _i64, _i32, _i32, _vp,
                                        _i64, _i32, _i64, _vp]),
     "lampa_rms_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _f32, _i32, _i32, _i32, _i32, _i64,

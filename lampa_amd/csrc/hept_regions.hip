@@ -166,3 +166,58 @@ extern "C" int lampa_hept_sort_keys(const float* hashed, const int32_t* rank_eta
   LAMPA_PROF((hipStream_t)stream, "hr_sort_keys_kernel");
   return lampa_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------- prep_qk
+// scale[h, c] = sqrt(2 * qw[h, max(c - 1, 0)]), qw[h, r] = sum_k exp(min(sum_d w[h, d, r, k], 50))   (hept.py:55-58)
+__global__ void hr_prep_scale_kernel(const float* __restrict__ w, int H, int d, int R, int Kw, float* __restrict__ scale) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= H * (R + 1)) return;
+  const int h = i / (R + 1), c = i % (R + 1), r = c > 0 ? c - 1 : 0;
+  float qw = 0.0f;
+  for (int k = 0; k < Kw; ++k) {
+    float sum = 0.0f;
+    for (int j = 0; j < d; ++j) sum += w[(((int64_t)h * d + j) * R + r) * Kw + k];
+    qw += expf(fminf(sum, 50.0f));
+  }
+  scale[i] = sqrtf(2.0f * qw);
+}
+
+// out[(n, h) or (h, n)][j] = x[n, h, j] for j < d, scale[h, j - d] * coords[n, j - d] for the R + 1 appended columns;
+// rows at or beyond n_raw are zero. blockIdx.y selects query / key.
+__global__ void __launch_bounds__(HR_BLOCK) hr_prep_qk_kernel(const float* __restrict__ query, const float* __restrict__ key,
+                                                             const float* __restrict__ coords, const float* __restrict__ scale,
+                                                             int64_t n, int64_t n_raw, int H, int d, int C, int heads_first,
+                                                             float* __restrict__ q_hat, float* __restrict__ k_hat) {
+  const int D = d + C;
+  const int64_t i = (int64_t)blockIdx.x * HR_BLOCK + threadIdx.x;
+  if (i >= n * H * D) return;
+  const int j = (int)(i % D);
+  const int64_t nh = i / D;
+  const int h = (int)(nh % H);
+  const int64_t t = nh / H;
+  const float* x = blockIdx.y == 0 ? query : key;
+  float* out = blockIdx.y == 0 ? q_hat : k_hat;
+  float v = 0.0f;
+  if (t < n_raw) v = j < d ? x[(t * H + h) * d + j] : __fmul_rn(scale[h * C + (j - d)], coords[t * C + (j - d)]);
+  out[heads_first ? ((int64_t)h * n + t) * D + j : i] = v;
+}
+
+// query, key [n, H, d] fp32; w [H, d, R, Kw] fp32; coords [n, R + 1] fp32; scale_ws: R + 1 floats per head (device).
+// q_hat, k_hat [n, H, d + R + 1] (heads_first 0) or [H, n, d + R + 1] (heads_first 1); rows from n_raw on are zero.
+// Replaces prep_qk and the rearrange + zeroing that follows it (models/attention/hept.py:54-62,118-128).
+extern "C" int lampa_hept_prep_qk(const float* query, const float* key, const float* w, const float* coords, int64_t n,
+                                  int64_t n_raw, int H, int d, int R, int Kw, int heads_first, float* scale_ws, float* q_hat,
+                                  float* k_hat, void* stream) {
+  if (!query || !key || !w || !coords || !scale_ws || !q_hat || !k_hat) return LAMPA_ERR_INVALID;
+  if (n < 0 || n_raw < 0 || n_raw > n || H < 1 || d < 1 || R < 1 || Kw < 1) return LAMPA_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  const int C = R + 1;
+  hipLaunchKernelGGL(hr_prep_scale_kernel, dim3((H * C + 63) / 64), dim3(64), 0, s, w, H, d, R, Kw, scale_ws);
+  if (n == 0) return lampa_launch_status();
+  const int64_t items = n * H * (d + C);
+  LAMPA_PROF(s, "start");
+  hipLaunchKernelGGL(hr_prep_qk_kernel, dim3((unsigned)((items + HR_BLOCK - 1) / HR_BLOCK), 2), dim3(HR_BLOCK), 0, s, query,
+                     key, coords, scale_ws, n, n_raw, H, d, C, heads_first, q_hat, k_hat);
+  LAMPA_PROF(s, "hr_prep_qk_kernel");
+  return lampa_launch_status();
+}

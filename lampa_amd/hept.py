@@ -3,8 +3,8 @@ region shift, and the sort that turns hashes plus shifts into bucket positions.
 
 Mirrors the reference's names and argument orders: ``quantile_partition`` / ``get_regions``
 (``models/model_utils/hash_utils.py:14-43``), ``get_geo_shift`` (``models/attention/hept.py:78-88``),
-``prepare_input`` (``models/hattention/modeling_gated_deltaproduct.py:1201-1223``). ``hept_positions`` is the fused
-form of ``hept.py:127-139``. GPU tensors only; there is no CPU fallback.
+``prepare_input`` (``models/hattention/modeling_gated_deltaproduct.py:1201-1223``), ``prep_qk`` (``hept.py:54-62``).
+``hept_positions`` is the fused form of ``hept.py:127-139``, ``prep_qk_heads`` of ``hept.py:118-128``. GPU tensors only; there is no CPU fallback.
 """
 from typing import Optional
 
@@ -94,6 +94,38 @@ def hept_sort_keys(hashed: torch.Tensor, rank_eta: torch.Tensor, rank_phi: torch
                                                n if raw_size is None else int(raw_size), ptr(keys), stream_of(keys)),
               "lampa_hept_sort_keys")
     return keys
+
+
+@torch.no_grad()
+def _prep(query, key, w, coords, raw_size, heads_first):
+    require_cuda(query, key, w, coords)
+    n, H, d = query.shape
+    R, Kw = w.shape[2], w.shape[3]
+    if key.shape != query.shape or w.shape[:2] != (H, d) or coords.shape != (n, R + 1):
+        raise ValueError("prep_qk: query/key [n, H, d], w [H, d, R, K] and coords [n, R + 1] disagree on shapes")
+    query, key, w, coords = (t.detach().float().contiguous() for t in (query, key, w, coords))
+    D = d + R + 1
+    shape = (H, n, D) if heads_first else (n, H, D)
+    q_hat = torch.empty(shape, dtype=torch.float32, device=query.device)
+    k_hat = torch.empty_like(q_hat)
+    scale = torch.empty(H * (R + 1), dtype=torch.float32, device=query.device)
+    check(_capi.lib().lampa_hept_prep_qk(ptr(query), ptr(key), ptr(w), ptr(coords), n, n if raw_size is None else int(raw_size),
+                                         H, d, R, Kw, int(heads_first), ptr(scale), ptr(q_hat), ptr(k_hat), stream_of(query)),
+          "lampa_hept_prep_qk")
+    return q_hat, k_hat
+
+
+def prep_qk(query: torch.Tensor, key: torch.Tensor, w: torch.Tensor, coords: torch.Tensor):
+    """``hept.py:54-62``: query, key [n, H, d], w [H, d, R, K], coords [n, R + 1] -> (q_hat, k_hat) [n, H, d + R + 1]:
+    the inputs with ``sqrt(2 qw) * coords`` appended, qw[h, r] = sum_k exp(min(sum_d w[h, d, r, k], 50)) and the first
+    appended column reusing qw[h, 0]."""
+    return _prep(query, key, w, coords, None, False)
+
+
+def prep_qk_heads(query, key, w, coords, raw_size: Optional[int] = None):
+    """``prep_qk`` followed by the rearrange to [H, n, D] and the zeroing of the rows from ``raw_size`` on
+    (``hept.py:118-128``) in one pass: the form ``hept_positions`` and ``E2LSH`` take."""
+    return _prep(query, key, w, coords, raw_size, True)
 
 
 @torch.no_grad()

@@ -156,3 +156,13 @@ def hept_sort_keys(hashed: np.ndarray, sorted_eta, sorted_phi, regions: np.ndarr
     reg_eta = quantile_regions(sorted_eta, regions[0])
     reg_phi = quantile_regions(sorted_phi, regions[1])
     return (h + geo_shift(regions[0], hash_shift, reg_eta, reg_phi)).astype(np.float32)
+
+
+def prep_qk(query, key, w, coords):
+    """``hept.py:54-62`` in float64: query, key [n, H, d], w [H, d, R, K], coords [n, R + 1] -> q_hat, k_hat
+    [n, H, d + R + 1]."""
+    query, key, w, coords = (np.asarray(t, np.float64) for t in (query, key, w, coords))
+    qw = np.exp(np.minimum(w.sum(axis=1), 50.0)).sum(axis=-1)               # [H, R]
+    expand = np.concatenate([qw[:, :1], qw], axis=-1)                       # [H, R + 1]
+    extra = np.sqrt(2.0 * expand)[None] * coords[:, None]                   # [n, H, R + 1]
+    return np.concatenate([query, extra], axis=-1), np.concatenate([key, extra], axis=-1)

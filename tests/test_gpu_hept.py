@@ -97,3 +97,22 @@ def test_prepare_input_matches_oracle(device):
     for a in range(2):
         order = torch.sort(padded[:, a], stable=True).indices.numpy()
         assert np.array_equal(_np(kw["region_indices"][a]), ol.quantile_regions(order, regions_h[a].numpy()))
+
+
+@pytest.mark.parametrize("n,n_raw", [(1, 1), (1000, 1000), (4100, 4001)])
+def test_prep_qk_against_oracle(device, n, n_raw):
+    gen = torch.Generator().manual_seed(n)
+    H, d, R, K = 8, 24, 2, 3
+    q, k = torch.randn(n, H, d, generator=gen), torch.randn(n, H, d, generator=gen)
+    w, coords = torch.randn(H, d, R, K, generator=gen) * 0.2, torch.randn(n, R + 1, generator=gen)
+    w[1, :, 0, 0] = 40.0                                     # one weight sum beyond the clamp at 50
+    want_q, want_k = ol.prep_qk(q.numpy(), k.numpy(), w.numpy(), coords.numpy())
+    q_hat, k_hat = hept.prep_qk(q.to(device), k.to(device), w.to(device), coords.to(device))
+    assert q_hat.shape == (n, H, d + R + 1) and q_hat.dtype == torch.float32
+    for got, want in ((q_hat, want_q), (k_hat, want_k)):
+        assert np.allclose(_np(got), want, rtol=3e-6, atol=1e-6)
+        assert np.array_equal(_np(got)[..., :d], want[..., :d].astype(np.float32))      # the copied part is exact
+    qh, kh = hept.prep_qk_heads(q.to(device), k.to(device), w.to(device), coords.to(device), n_raw)
+    assert qh.shape == (H, n, d + R + 1)
+    assert torch.equal(qh[:, :n_raw], q_hat.permute(1, 0, 2)[:, :n_raw]) and (qh[:, n_raw:] == 0).all()
+    assert torch.equal(kh[:, :n_raw], k_hat.permute(1, 0, 2)[:, :n_raw]) and (kh[:, n_raw:] == 0).all()

@@ -216,3 +216,28 @@ def test_hept_sort_keys_padding_and_composition():
         assert np.mean(np.diff(pair) < 0) < 0.02
     # the input hashes are not modified
     assert np.all(np.isfinite(hashed))
+
+
+def test_prep_qk_distance_identity_and_column_roles():
+    # The appended columns turn a weighted coordinate distance into part of the Euclidean one:
+    # |q_hat_i - k_hat_j|^2 = |q_i - k_j|^2 + sum_c 2 qw'[h, c] (coords_i,c - coords_j,c)^2, qw' = [qw_0, qw_0, qw_1, ...].
+    rng = np.random.default_rng(6)
+    n, H, d, R, K = 9, 3, 5, 2, 4
+    q, k = rng.normal(size=(n, H, d)), rng.normal(size=(n, H, d))
+    w, coords = rng.normal(size=(H, d, R, K)) * 0.3, rng.normal(size=(n, R + 1))
+    q_hat, k_hat = ol.prep_qk(q, k, w, coords)
+    assert q_hat.shape == (n, H, d + R + 1) and np.array_equal(q_hat[..., :d], q) and np.array_equal(k_hat[..., :d], k)
+    wt = torch.from_numpy(w)
+    qw = wt.sum(dim=1).clamp(max=50).exp().sum(dim=-1).numpy()                   # library evaluation, [H, R]
+    qwx = np.concatenate([qw[:, :1], qw], axis=1)
+    for h in range(H):
+        lhs = ((q_hat[:, None, h] - k_hat[None, :, h]) ** 2).sum(-1)
+        rhs = ((q[:, None, h] - k[None, :, h]) ** 2).sum(-1) + \
+            (2 * qwx[h] * (coords[:, None] - coords[None]) ** 2).sum(-1)
+        assert np.abs(lhs - rhs).max() < 1e-10
+    # the clamp: a huge weight sum saturates at exp(50) instead of overflowing
+    w_big = w.copy()
+    w_big[0, :, 1, 2] = 100.0
+    big, _ = ol.prep_qk(q, k, w_big, coords)
+    assert np.all(np.isfinite(big)) and big[0, 0, d + 2] != q_hat[0, 0, d + 2]
+    assert np.array_equal(big[:, 1:], q_hat[:, 1:])                              # other heads untouched
