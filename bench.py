@@ -1,9 +1,12 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-A step is one chunkwise gated-delta layer forward (BASELINE config 2: B=1, H=8, T=60000, d_k=d_v=64, C=64, bf16
-q/k/v, fp32 g/beta, tokens in the LSH-sorted order of a config-1 event) with every input resident in HBM.
-Prints one JSON line; see DESIGN.md for how each figure is defined.
+A step is one chunkwise gated-delta layer forward (B=1, H=8, T=60000, d_k=d_v=64, C=64, bf16 q/k/v, fp32 g/beta,
+tokens in the LSH-sorted order of a 60000-hit event) with every input resident in HBM.
+Prints one JSON line: `value` = hits/s over the timed steps (wall clock), `roofline` = the slowest kernel of the layer
+against the HBM peak on its algorithmic bytes (duration from HIP events on the launch stream), `cpu_baseline` = the
+pure-PyTorch token loop on this box's host cores, `layer` / `lsh` / `block` = per-kernel times, the LSH stage on one
+event and on a batch, and the 4-layer block.
 """
 import argparse
 import json
@@ -95,7 +98,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
-              "(sharding is described in DESIGN.md, not implemented).", file=sys.stderr)
+              "(heads, sequences and segments would shard across GPUs; that is not implemented).", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -932,13 +932,12 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 //   GROUP  every group but the last of a sequence, in parallel: the composite of its G segments, i.e. the scan step
 //          applied to the KT + VT columns [P_M | P_N] starting from [I | 0]; written as a segment composite is
 //          (D = product of the decays, M' = P_M - D I as bf16 A-operand fragments, N = P_N in accumulator order);
-//   TOP    per sequence, serial over the groups with these composites: the state every group starts from;
-//   LEAF   every group in parallel: from its start state over its segments, writing the state every segment starts
-//          from (what the single-level scan writes);
-//   LEAF2  TOP and LEAF in one launch: the workgroup of group j first walks the composites of groups 0 .. j-1 itself
-//          (at most gmax - 1 redundant steps) and then its own segments; one launch and one serial phase less.
-// Same step code in the three modes; loops are branch free with clamped operands and a spare store slot as above.
-enum { SCAN_GROUP = 1, SCAN_TOP = 2, SCAN_LEAF = 3, SCAN_LEAF2 = 4 };
+//   LEAF   every group in parallel: the workgroup of group j first walks the composites of groups 0 .. j-1 from the
+//          sequence's initial state (at most gmax - 1 redundant steps; a separate serial pass over the groups would
+//          cost a launch more), then its own segments, writing the state every segment starts from (what the
+//          single-level scan writes).
+// Same step code in both modes; loops are branch free with clamped operands and a spare store slot as above.
+enum { SCAN_GROUP = 1, SCAN_LEAF = 2 };
 #define GDR_SCAN_GROUP 8  // segments per group; a multiple of the ring depth
 
 template <int KT, int VT, int DEPTH, int MODE>
@@ -947,7 +946,6 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
                                                                   const unsigned char* __restrict__ Nsrc,
                                                                   const float* __restrict__ Dsrc,
                                                                   const float* __restrict__ h0,
-                                                                  const float* __restrict__ init_slab,
                                                                   float* __restrict__ dst, unsigned char* __restrict__ Mout,
                                                                   unsigned char* __restrict__ Nout, float* __restrict__ Dout,
                                                                   int HV, int spare_slot, int gmax) {
@@ -962,18 +960,13 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   const int ngroups = (nseg + G - 1) / G;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   // items = the maps this workgroup applies, slots = where it stores the running state before each of them
-  int item0, nsteps, slot0, lead = 0;  // lead: group-level maps walked before the workgroup's own items (LEAF2)
-  if (MODE == SCAN_LEAF2) {
-    if (j >= ngroups) return;
-    item0 = seg0 + j * G; lead = j; nsteps = lead + min(G, nseg - j * G) - 1; slot0 = item0;
-  } else if (MODE == SCAN_GROUP) {
+  int item0, nsteps, slot0, lead = 0;  // lead: group-level maps walked before the workgroup's own items (LEAF)
+  if (MODE == SCAN_GROUP) {
     if (j >= ngroups - 1) return;  // the composite of a sequence's last group is never needed
     item0 = seg0 + j * G; nsteps = G - 1; slot0 = 0;
-  } else if (MODE == SCAN_TOP) {
-    item0 = seq * gmax; nsteps = ngroups - 1; slot0 = item0;
   } else {
     if (j >= ngroups) return;
-    item0 = seg0 + j * G; nsteps = min(G, nseg - j * G) - 1; slot0 = item0;
+    item0 = seg0 + j * G; lead = j; nsteps = lead + min(G, nseg - j * G) - 1; slot0 = item0;
   }
   const int last = MODE == SCAN_GROUP ? nsteps : nsteps - 1;   // last map that is really applied (prefetches are clamped to it)
   const bool is_pm = MODE == SCAN_GROUP && vn < KT / 32;       // a block of P_M: no additive term, starts from I
@@ -985,14 +978,6 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
 #pragma unroll
       for (int r = 0; r < 16; ++r) S[r] = (32 * wave + acc_row(r, hh) == 32 * vn + ln) ? 1.0f : 0.0f;
     }
-  } else if (MODE == SCAN_LEAF) {
-    const f32x4* src = reinterpret_cast<const f32x4*>(init_slab + (((size_t)(seq * gmax + j) * HV + hv) * (VT / 32) + vn) * (KT * 32));
-#pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const f32x4 t = src[(wave * 4 + q4) * 64 + lane];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) S[4 * q4 + e] = t[e];
-    }
   } else if (h0) {
 #pragma unroll
     for (int r = 0; r < 16; ++r)
@@ -1003,7 +988,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   f32x4 rn[DEPTH][4];
   float rd[DEPTH];
   auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
-    const bool top = MODE == SCAN_LEAF2 && p < lead;  // a group composite (read through the *out pointers)
+    const bool top = MODE == SCAN_LEAF && p < lead;  // a group composite (read through the *out pointers)
     const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
     const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mout : Msrc) + sh * M_BYTES);
     const f32x4* N = reinterpret_cast<const f32x4*>((top ? Nout : Nsrc) + (sh * (VT / 32) + nblk) * N_BYTES);
@@ -1150,16 +1135,16 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   const int gmax = (max_nseg + GDR_SCAN_GROUP - 1) / GDR_SCAN_GROUP;
   if (max_nseg >= 3 * GDR_SCAN_GROUP && (int64_t)n_seq * gmax <= w.max_groups) {
-    // long sequences: group composites, scan over the groups, scan inside the groups
+    // long sequences: group composites, then every group's scan (which walks the earlier groups' composites first)
     unsigned char* Gm = ws + w.off_gm;
     unsigned char* Gn = ws + w.off_gn;
     float* Gd = (float*)(ws + w.off_gd);
     const dim3 block(64 * (KT / 32));
     hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
-                       Nc, Dc, (const float*)nullptr, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
+                       Nc, Dc, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<group>");
-    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF2>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc,
-                       Dc, h0, (const float*)nullptr, Si, Gm, Gn, Gd, HV, segs, gmax);
+    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc, Dc,
+                       h0, Si, Gm, Gn, Gd, HV, segs, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
   } else {
     hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
