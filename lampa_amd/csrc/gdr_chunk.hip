@@ -51,6 +51,10 @@ static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_d
 }
 
 #define T_BYTES (3 * 32 * 32 * 2)  // T of one chunk and head in HBM: bf16 blocks T11 | T21 | T22, 32x32 row-major each
+// Record of one chunk and head: T, then the chunk's cumulative log-decay (units of log 2) and beta per token, fp32
+// [64] each. The segment kernels take the two factor rows from here: in g and beta themselves a head's 64 values sit
+// 4 bytes apart in rows that interleave all heads, so every workgroup would fetch the sectors of all of them.
+#define REC_BYTES (T_BYTES + 2 * 64 * 4)
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
   return *reinterpret_cast<const bf16x8*>(base + (size_t)frag * 1024 + lane * 16);
@@ -157,8 +161,12 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
   {  // gamma is kept in units of log 2 (exp2 is one instruction)
     const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
     const float gv = g[gi], bv = beta[gi];
-    s_gamma[lane] = 1.44269504f * wave_inclusive_scan(lane < len ? gv : 0.0f);
-    s_beta[lane] = lane < len ? bv : 0.0f;
+    const float gcum = 1.44269504f * wave_inclusive_scan(lane < len ? gv : 0.0f), bz = lane < len ? bv : 0.0f;
+    s_gamma[lane] = gcum;
+    s_beta[lane] = bz;
+    float* fact = reinterpret_cast<float*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES + T_BYTES);
+    fact[lane] = gcum;
+    fact[64 + lane] = bz;
   }
   bf16x8 f[2][NK];
   {
@@ -286,7 +294,7 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
 
   // T -> HBM: the diagonal blocks from LDS in 16-byte pieces; T21 from the accumulator, two columns per store
   // (lanes 2j and 2j+1 swap one value of every adjacent row pair, as in the segment kernel's output)
-  __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * T_BYTES);
+  __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES);
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
     const float* src = blk == 0 ? s_A11 : s_A22;
@@ -458,16 +466,15 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
 #pragma unroll
       for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
-      const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * T_BYTES);
+      const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * REC_BYTES);
 #pragma unroll
       for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
     };
-    auto issue_gb = [&](int c) {  // g, beta (lane = token)
+    auto issue_gb = [&](int c) {  // cumulative log-decay and beta of the chunk's tokens (lane = token)
       c = uniform(c);
-      const int tok0 = chunk_tok0[c], len = chunk_len[c];
-      const int gl = min(lane, len - 1) * HV;
-      rg = (g + (size_t)tok0 * HV + hv)[gl];
-      rb = (beta + (size_t)tok0 * HV + hv)[gl];
+      const float* fact = reinterpret_cast<const float*>(tmat + ((size_t)c * HV + hv) * REC_BYTES + T_BYTES);
+      rg = fact[lane];
+      rb = fact[64 + lane];
     };
     auto issue_q = [&](int c, typename Raw8<T>::type* rq_) {
       c = uniform(c);
@@ -506,9 +513,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     auto stage_factors = [&](int c, int par) {
       const GdrTiles tl = tiles(par);
       const int len = chunk_len[uniform(c)];
-      const float bv = lane < len ? rb : 0.0f;
-      // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction), lane = token
-      const float gv = 1.44269504f * wave_inclusive_scan(lane < len ? rg : 0.0f);
+      // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction) and beta, lane = token; both
+      // come ready from the chunk's record (zero decay increment and zero beta past the end of a partial chunk)
+      const float bv = rb, gv = rg;
       const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
       const float kss2 = kss + dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
       // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
@@ -1079,7 +1086,7 @@ struct GdrWorkspace {
 static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, int V) {
   GdrWorkspace w;
   int64_t off = 0;
-  w.off_t = off;     off += lampa_align_up(chunks * HV * (int64_t)T_BYTES, 256);
+  w.off_t = off;     off += lampa_align_up(chunks * HV * (int64_t)REC_BYTES, 256);
   w.off_m = off;     off += lampa_align_up(segs * HV * (int64_t)K * K * 2, 256);
   w.off_n = off;     off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.off_d = off;     off += lampa_align_up(segs * HV * 4, 256);
