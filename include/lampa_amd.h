@@ -162,6 +162,20 @@ int lampa_causal_conv1d_fwd(const void* x, int64_t x_stride, int64_t n_tokens, i
                             int n_seq, int64_t t_len, int activation, int dtype, void* y, int64_t y_stride, int y_split,
                             int64_t y_split_stride, void* stream);
 
+/* Fused input projections + short convolution + SiLU of a gated-delta layer (bf16, hidden size K = 128). Replaces
+ * the bias-free nn.Linear projections and the ShortConvolution calls after them
+ * (models/hattention/modeling_gated_deltaproduct.py:505-547; models/hattention/short_convolution.py:39-99) without
+ * writing the projection output to memory. x [n_tokens, K] bf16 (row stride x_stride), n_tokens / t_len dense sequences;
+ * W [n_cols, K] bf16 = the projection weights one after the other. The first n_conv columns: y = silu(conv_b +
+ * sum_j conv_w[n, j] * pre[t - 3 + j, n]) (4 taps, zero before a sequence start; the projection output rounded to bf16
+ * first, as a bf16 linear layer's is), written as n_conv / conv_split tensors [n_tokens, conv_split] one after the
+ * other at conv_out; the next plain_cols columns go to plain_out [n_tokens, plain_cols] as they are, the last
+ * tail_cols (< 256, a multiple of 8) to tail_out [n_tokens, tail_cols]. n_conv, conv_split, plain_cols multiples of
+ * 256. tokens_per_wg: tokens per workgroup run (0 = default). */
+int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_tokens, int64_t t_len, int K, const void* W, int n_cols,
+                        const float* conv_w, const float* conv_b, int n_conv, int conv_split, void* conv_out,
+                        int plain_cols, void* plain_out, int tail_cols, void* tail_out, int tokens_per_wg, void* stream);
+
 /* RMS norm over the last dimension with optional residual add, weight, bias and output gate. Replaces
  * layer_norm_gated_fwd / layer_norm_fwd with is_rms_norm (models/hattention/fused_norm.py:40-111,456-531,1436-1506).
  * s = x + residual; residual_out = s; y = s / sqrt(mean(s^2) + eps) * weight + bias; with g: y *= g * sigmoid(g)

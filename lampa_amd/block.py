@@ -16,8 +16,8 @@ import torch.nn.functional as F
 
 from . import lsh
 from .gated_delta import chunk_gated_delta_rule
-from .layer_ops import (FusedRMSNormSwishGate, RMSNorm, ShortConvolution, causal_conv1d, causal_conv1d_split,
-                        gdr_gates)
+from .layer_ops import (PROJ_CONV_HIDDEN, FusedRMSNormSwishGate, RMSNorm, ShortConvolution, causal_conv1d,
+                        causal_conv1d_split, gdr_gates, proj_conv)
 
 
 class GatedDeltaLayer(nn.Module):
@@ -60,16 +60,23 @@ class GatedDeltaLayer(nn.Module):
         """hidden_states [B, T, hidden] -> (o [B, T, hidden], final_state or None)."""
         B, T, _ = hidden_states.shape
         H, dk, dv, kd, vd = self.num_heads, self.head_dim, self.head_v_dim, self.key_dim, self.value_dim
-        proj = F.linear(hidden_states, self._fused_weight())                     # [B, T, 2 kd + 2 vd + 2 H]
-        cols = [0, kd, 2 * kd, 2 * kd + vd, 2 * kd + 2 * vd, 2 * kd + 2 * vd + H, 2 * kd + 2 * vd + 2 * H]
-        xq, xk, xv, xg, xb, xa = (proj[..., cols[i]:cols[i + 1]] for i in range(6))
         convs = (self.q_conv1d, self.k_conv1d, self.v_conv1d)
-        if kd == vd:                                                             # one launch over the q | k | v columns
-            q, k, v = causal_conv1d_split(proj[..., :cols[3]], [c.weight for c in convs], [c.bias for c in convs], "silu",
-                                          cu_seqlens)
+        fused = (cu_seqlens is None and hidden_states.dtype == torch.bfloat16 and self.hidden_size == PROJ_CONV_HIDDEN
+                 and kd == vd and kd % 256 == 0 and (2 * H) % 8 == 0)
+        if fused:  # projections, convolutions and SiLU in one kernel: the projection output never reaches memory
+            (q, k, v), xg, xba = proj_conv(hidden_states, self._fused_weight(), [c.weight for c in convs],
+                                           [c.bias for c in convs], kd, vd)
+            xb, xa = xba[..., :H], xba[..., H:]
         else:
-            q, k, v = (causal_conv1d(t, c.weight.reshape(t.shape[-1], -1), c.bias, None, "silu", cu_seqlens)
-                       for t, c in zip((xq, xk, xv), convs))
+            proj = F.linear(hidden_states, self._fused_weight())                 # [B, T, 2 kd + 2 vd + 2 H]
+            cols = [0, kd, 2 * kd, 2 * kd + vd, 2 * kd + 2 * vd, 2 * kd + 2 * vd + H, 2 * kd + 2 * vd + 2 * H]
+            xq, xk, xv, xg, xb, xa = (proj[..., cols[i]:cols[i + 1]] for i in range(6))
+            if kd == vd:                                                         # one launch over the q | k | v columns
+                q, k, v = causal_conv1d_split(proj[..., :cols[3]], [c.weight for c in convs], [c.bias for c in convs],
+                                              "silu", cu_seqlens)
+            else:
+                q, k, v = (causal_conv1d(t, c.weight.reshape(t.shape[-1], -1), c.bias, None, "silu", cu_seqlens)
+                           for t, c in zip((xq, xk, xv), convs))
         g, beta = gdr_gates(xa, xb, self.A_log, self.dt_bias, 2.0 if self.allow_neg_eigval else 1.0)
         o, state = chunk_gated_delta_rule(q.view(B, T, H, dk), k.view(B, T, H, dk), v.view(B, T, H, dv), g, beta,
                                           initial_state=initial_state, output_final_state=output_final_state,

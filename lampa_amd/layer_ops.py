@@ -158,6 +158,41 @@ def causal_conv1d_split(x: torch.Tensor, weights, biases=None, activation: Optio
     return tuple(y[i].view(B, T, D) for i in range(n))
 
 
+PROJ_CONV_HIDDEN = 128  # contraction length the fused projection kernel is built for
+
+
+@torch.no_grad()
+def proj_conv(x: torch.Tensor, weight: torch.Tensor, conv_weights, conv_biases, conv_split: int, plain_cols: int,
+              tokens_per_wg: int = 0):
+    """Fused bias-free projections + short convolution (4 taps) + SiLU: x [B, T, 128] bf16, weight [n_cols, 128] bf16
+    (the projection weights one after the other), conv_weights = tensors [conv_split, 4] (or [conv_split, 1, 4]) for
+    the first len(conv_weights) * conv_split columns, conv_biases = None or matching tensors. Returns
+    (conv outputs: tuple of [B, T, conv_split], plain [B, T, plain_cols], tail [B, T, rest]); the projection output
+    itself is never written. Same arithmetic as ``F.linear`` in bf16 followed by ``causal_conv1d(..., 'silu')``."""
+    require_cuda(x, weight, *conv_weights)
+    B, T, K = x.shape
+    n_cols = weight.shape[0]
+    n_conv = len(conv_weights) * conv_split
+    tail = n_cols - n_conv - plain_cols
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or K != PROJ_CONV_HIDDEN or weight.shape[1] != K:
+        raise ValueError("proj_conv: bf16 x [B, T, 128] and weight [n_cols, 128] expected")
+    if any(w.shape[0] != conv_split or w.shape[-1] != 4 for w in conv_weights) or tail < 0:
+        raise ValueError("proj_conv: conv_weights must be [conv_split, 4] each and fit the columns of weight")
+    x2 = _rows(x)
+    weight = weight.detach().contiguous()
+    cw = _cat_f32([w.reshape(conv_split, 4) for w in conv_weights], x.device)
+    cb = None if conv_biases is None or conv_biases[0] is None else _cat_f32(list(conv_biases), x.device)
+    n = B * T
+    y_conv = torch.empty((len(conv_weights), n, conv_split), dtype=x.dtype, device=x.device)
+    y_plain = torch.empty((n, plain_cols), dtype=x.dtype, device=x.device)
+    y_tail = torch.empty((n, tail), dtype=x.dtype, device=x.device)
+    check(_capi.lib().lampa_proj_conv_fwd(ptr(x2), x2.stride(0), n, max(T, 1), K, ptr(weight), n_cols, ptr(cw), ptr(cb), n_conv,
+                                          conv_split, ptr(y_conv), plain_cols, ptr(y_plain) if plain_cols else None, tail,
+                                          ptr(y_tail) if tail else None, tokens_per_wg, stream_of(x)), "lampa_proj_conv_fwd")
+    return (tuple(y_conv[i].view(B, T, conv_split) for i in range(len(conv_weights))), y_plain.view(B, T, plain_cols),
+            y_tail.view(B, T, tail))
+
+
 class ShortConvolution(nn.Conv1d):
     """``short_convolution.py:528-721``: depthwise causal convolution over the time axis of a [B, T, D] tensor with
     an optional SiLU, a cache of the last W inputs per sequence ([N, D, W]) and a one-token ``step``."""

@@ -79,6 +79,39 @@ def test_causal_conv1d_split_equals_separate_calls(device):
     assert torch.equal(again, lo.causal_conv1d(proj[..., :D].contiguous(), ws[0].reshape(D, 4).clone(), None, None, "silu"))
 
 
+@pytest.mark.parametrize("B,T,tokens_per_wg", [(1, 1, 0), (1, 31, 0), (2, 700, 64), (1, 5000, 512), (3, 333, 96)])
+def test_fused_projection_convolution(device, B, T, tokens_per_wg):
+    """One kernel for projections + convolution + SiLU against the float64 oracle (tolerance: the projection output is
+    rounded to bf16 before the convolution, as a bf16 linear layer's is, then one more rounding of the result) and
+    against the two-step route on the GPU (same roundings, different summation order inside the GEMM)."""
+    gen = torch.Generator().manual_seed(B * 100 + T)
+    x = torch.randn(B, T, 128, generator=gen).to(torch.bfloat16)
+    W = (torch.randn(3 * 512 + 512 + 16, 128, generator=gen) * 0.1).to(torch.bfloat16)
+    cws = [(torch.randn(512, 1, 4, generator=gen) * 0.5).to(torch.bfloat16) for _ in range(3)]
+    cbs = [torch.randn(512, generator=gen).to(torch.bfloat16) for _ in range(3)]
+    for biases in (None, cbs):
+        (q, k, v), g, ab = lo.proj_conv(x.to(device), W.to(device), [w.to(device) for w in cws],
+                                        None if biases is None else [b.to(device) for b in biases], 512, 512, tokens_per_wg)
+        assert q.shape == (B, T, 512) and g.shape == (B, T, 512) and ab.shape == (B, T, 16) and q.is_contiguous()
+        pre = _f64(x) @ _f64(W).T                                             # [B, T, 2064]
+        pre_b = torch.from_numpy(pre).to(torch.bfloat16)                        # the rounding the kernel applies
+        for i, got in enumerate((q, k, v)):
+            want = ol.causal_conv1d(_f64(pre_b[..., 512 * i:512 * (i + 1)]), _f64(cws[i]).reshape(512, 4),
+                                    None if biases is None else _f64(biases[i]), None, "silu")
+            err = np.abs(_f64(got) - want)
+            # one bf16 rounding of the result plus the effect of last-bit differences of the rounded projections
+            assert np.all(err <= 2 ** -7 * np.abs(want) + 2e-2), float(err.max())
+            assert err.mean() < 2e-3
+        assert np.all(np.abs(_f64(g) - pre[..., 1536:2048]) <= 2 ** -8 * np.abs(pre[..., 1536:2048]) + 1e-6)
+        assert np.all(np.abs(_f64(ab) - pre[..., 2048:]) <= 2 ** -8 * np.abs(pre[..., 2048:]) + 1e-6)
+    # two-step route on the GPU
+    proj = torch.nn.functional.linear(x.to(device), W.to(device))
+    q2, k2, v2 = lo.causal_conv1d_split(proj[..., :1536], [w.to(device) for w in cws], [b.to(device) for b in cbs], "silu")
+    for a, b2 in ((q, q2), (k, k2), (v, v2)):
+        assert (a.float() - b2.float()).abs().max() < 0.1 and (a.float() - b2.float()).abs().mean() < 2e-3
+    assert (g.float() - proj[..., 1536:2048].float()).abs().max() < 0.05
+
+
 def test_short_convolution_module_cache_and_step(device):
     torch.manual_seed(4)
     D, W, T = 64, 4, 19
