@@ -176,6 +176,15 @@ int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_tokens, int64
                         const float* conv_w, const float* conv_b, int n_conv, int conv_split, void* conv_out,
                         int plain_cols, void* plain_out, int tail_cols, void* tail_out, int tokens_per_wg, void* stream);
 
+/* Gated RMS norm of every head fused with the output projection (bf16; 8 heads of 64 channels -> 128 columns).
+ * Replaces FusedRMSNormSwishGate followed by o_proj (models/hattention/fused_norm.py:40-111 with the swish gate;
+ * models/hattention/modeling_gated_deltaproduct.py:612-623): y[t] = W * vec(rmsnorm(o[t, h]) * norm_w * g[t, h] *
+ * sigmoid(g[t, h])), the normalised tensor rounded to bf16 as the unfused pair would store it but never written.
+ * o [n_tokens, heads, head_dim] contiguous; g the same shape with token stride g_stride elements; norm_w fp32
+ * [head_dim] or NULL; W [n_out, heads * head_dim] row-major; y [n_tokens, n_out]. */
+int lampa_norm_proj_fwd(const void* o, const void* g, int64_t g_stride, const float* norm_w, const void* W, int64_t n_tokens,
+                        int heads, int head_dim, int n_out, float eps, void* y, int tokens_per_wg, void* stream);
+
 /* RMS norm over the last dimension with optional residual add, weight, bias and output gate. Replaces
  * layer_norm_gated_fwd / layer_norm_fwd with is_rms_norm (models/hattention/fused_norm.py:40-111,456-531,1436-1506).
  * s = x + residual; residual_out = s; y = s / sqrt(mean(s^2) + eps) * weight + bias; with g: y *= g * sigmoid(g)

@@ -17,7 +17,7 @@ import torch.nn.functional as F
 from . import lsh
 from .gated_delta import chunk_gated_delta_rule
 from .layer_ops import (PROJ_CONV_HIDDEN, FusedRMSNormSwishGate, RMSNorm, ShortConvolution, causal_conv1d,
-                        causal_conv1d_split, gdr_gates, proj_conv)
+                        causal_conv1d_split, gdr_gates, norm_proj, norm_proj_supported, proj_conv)
 
 
 class GatedDeltaLayer(nn.Module):
@@ -81,7 +81,10 @@ class GatedDeltaLayer(nn.Module):
         o, state = chunk_gated_delta_rule(q.view(B, T, H, dk), k.view(B, T, H, dk), v.view(B, T, H, dv), g, beta,
                                           initial_state=initial_state, output_final_state=output_final_state,
                                           cu_seqlens=cu_seqlens, use_qk_l2norm_in_kernel=True)
-        o = self.o_norm(o, xg.unflatten(-1, (H, dv)))
+        gate = xg.unflatten(-1, (H, dv))
+        if norm_proj_supported(o, self.hidden_size) and self.o_proj.weight.dtype == torch.bfloat16:
+            return norm_proj(o, gate, self.o_norm.weight, self.o_proj.weight, self.o_norm.eps), state  # norm + gate + GEMM
+        o = self.o_norm(o, gate)
         return self.o_proj(o.reshape(B, T, vd)), state
 
 

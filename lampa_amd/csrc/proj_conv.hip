@@ -247,3 +247,118 @@ extern "C" int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_to
   LAMPA_PROF(s, "pc_proj_conv_kernel");
   return lampa_launch_status();
 }
+
+// ------------------------------------------------------------------------------- gated RMS norm + output projection
+// y[t, :] = W_o * vec_h( rmsnorm(o[t, h, :]) * weight * swish(g[t, h, :]) ): the gated norm of every head
+// (models/hattention/fused_norm.py:40-111 with IS_RMS_NORM and the swish gate) feeding the bias-free output projection
+// (modeling_gated_deltaproduct.py:612-623) without writing the normalised tensor. One workgroup = 4 waves walks a run
+// of 32-token tiles: all threads normalise and gate the tile into LDS (bf16, the A operand; 8 lanes share a head's 64
+// channels), then every wave multiplies it with its 32 rows of W_o, which it keeps in registers as B-operand fragments.
+#define NP_D 64        // channels per head
+#define NP_KMAX 512    // heads * channels this kernel is built for (32 contraction steps of 16)
+#define NP_OUT 128     // output columns (4 waves x 32)
+#define NP_LDA (NP_KMAX + 8)
+
+__global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restrict__ o, const __bf16* __restrict__ g,
+                                                          int64_t g_stride, const float* __restrict__ norm_w,
+                                                          const __bf16* __restrict__ W, int64_t n_tokens, float eps,
+                                                          __bf16* __restrict__ y, int tokens_per_wg) {
+  constexpr int NKS = NP_KMAX / 16;
+  __shared__ __align__(16) __bf16 s_a[2][PC_ROWS * NP_LDA];
+  __shared__ __align__(16) __bf16 s_out[4][PC_ROWS * (32 + 8)];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int64_t T0 = (int64_t)blockIdx.x * tokens_per_wg;
+  const int64_t T1 = T0 + tokens_per_wg < n_tokens ? T0 + tokens_per_wg : n_tokens;
+
+  bf16x8 bfrag[NKS];  // rows 32 wave + ln of W_o
+  {
+    const __bf16* wp = W + (int64_t)(32 * wave + ln) * NP_KMAX + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) bfrag[ks] = *reinterpret_cast<const bf16x8*>(wp + 16 * ks);
+  }
+  // norm role: 8 lanes per (token, head) row, 8 channels each; 32 rows per pass, 8 passes per tile
+  const int sub = tid & 7, rrow = tid >> 3;
+  float nw[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) nw[c] = norm_w ? norm_w[8 * sub + c] : 1.0f;
+
+  auto stage = [&](int64_t t0, int buf) {
+#pragma unroll 2
+    for (int pass = 0; pass < 8; ++pass) {
+      const int r = 32 * pass + rrow;           // (token, head) row of the tile: token r / 8, head r % 8
+      const int tok = r >> 3, head = r & 7;
+      int64_t t = t0 + tok;
+      t = t < n_tokens ? t : n_tokens - 1;
+      const bf16x8 ov = *reinterpret_cast<const bf16x8*>(o + t * NP_KMAX + head * NP_D + 8 * sub);
+      const bf16x8 gv = *reinterpret_cast<const bf16x8*>(g + t * g_stride + head * NP_D + 8 * sub);
+      float x[8], ss = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) { x[c] = (float)ov[c]; ss = __builtin_fmaf(x[c], x[c], ss); }
+      ss += __shfl_xor(ss, 1);
+      ss += __shfl_xor(ss, 2);
+      ss += __shfl_xor(ss, 4);
+      const float rstd = 1.0f / sqrtf(ss * (1.0f / NP_D) + eps);
+      bf16x8 out;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const float gc = (float)gv[c];
+        out[c] = (__bf16)(x[c] * rstd * nw[c] * gc * pc_sigmoid(gc));
+      }
+      *reinterpret_cast<bf16x8*>(&s_a[buf][tok * NP_LDA + head * NP_D + 8 * sub]) = out;
+    }
+  };
+
+  const int cg = lane & 3, tq = lane >> 2;  // output role: row 2 tq + i (i < 2), columns 8 cg .. 8 cg + 7 of the wave's 32
+  int buf = 0;
+  if (T0 < T1) stage(T0, 0);
+  __syncthreads();
+  for (int64_t t0 = T0; t0 < T1; t0 += PC_ROWS, buf ^= 1) {
+    if (t0 + PC_ROWS < T1) stage(t0 + PC_ROWS, buf ^ 1);   // next tile while this one is multiplied
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    const __bf16* ap = &s_a[buf][ln * NP_LDA + 8 * hh];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) acc = mfma32(*reinterpret_cast<const bf16x8*>(ap + 16 * ks), bfrag[ks], acc);
+    __bf16* so = s_out[wave];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) so[(8 * (r / 4) + 4 * hh + (r % 4)) * 40 + ln] = (__bf16)acc[r];
+    lds_fence();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int tr = 2 * tq + i;
+      const int64_t t = t0 + tr;
+      if (t < T1)
+        *reinterpret_cast<bf16x8*>(y + t * NP_OUT + 32 * wave + 8 * cg) = *reinterpret_cast<const bf16x8*>(&so[tr * 40 + 8 * cg]);
+    }
+    __syncthreads();  // the next tile is staged, this tile's A operand is free again
+  }
+}
+
+// o [n_tokens, 8, 64] bf16 contiguous; g the same shape with token stride g_stride elements; norm_w fp32 [64] or NULL;
+// W [128, 512] bf16 row-major (the output projection); y [n_tokens, 128] bf16.
+extern "C" int lampa_norm_proj_fwd(const void* o, const void* g, int64_t g_stride, const float* norm_w, const void* W,
+                                   int64_t n_tokens, int heads, int head_dim, int n_out, float eps, void* y, int tokens_per_wg,
+                                   void* stream) {
+  if (!o || !g || !W || !y || n_tokens < 0) return LAMPA_ERR_INVALID;
+  if (heads * head_dim != NP_KMAX || head_dim != NP_D || n_out != NP_OUT) return LAMPA_ERR_UNSUPPORTED;
+  if (g_stride < NP_KMAX || g_stride % 8 || ((uintptr_t)o | (uintptr_t)g | (uintptr_t)W | (uintptr_t)y) % 16)
+    return LAMPA_ERR_UNSUPPORTED;
+  if (n_tokens == 0) return LAMPA_OK;
+  if (tokens_per_wg <= 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+      cus = 256;
+    tokens_per_wg = (int)((n_tokens + 2 * cus - 1) / (2 * cus));
+    if (tokens_per_wg < 2 * PC_ROWS) tokens_per_wg = 2 * PC_ROWS;
+  }
+  tokens_per_wg = (tokens_per_wg + PC_ROWS - 1) / PC_ROWS * PC_ROWS;
+  hipStream_t s = (hipStream_t)stream;
+  LAMPA_PROF(s, "start");
+  hipLaunchKernelGGL(pc_norm_proj_kernel, dim3((unsigned)((n_tokens + tokens_per_wg - 1) / tokens_per_wg)), dim3(256), 0, s,
+                     (const __bf16*)o, (const __bf16*)g, g_stride, norm_w, (const __bf16*)W, n_tokens, eps, (__bf16*)y,
+                     tokens_per_wg);
+  LAMPA_PROF(s, "pc_norm_proj_kernel");
+  return lampa_launch_status();
+}

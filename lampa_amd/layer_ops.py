@@ -193,6 +193,34 @@ def proj_conv(x: torch.Tensor, weight: torch.Tensor, conv_weights, conv_biases, 
             y_tail.view(B, T, tail))
 
 
+def norm_proj_supported(o: torch.Tensor, n_out: int) -> bool:
+    """Shapes the fused gated-norm + output-projection kernel is built for."""
+    return o.dtype == torch.bfloat16 and o.dim() == 4 and o.shape[2] * o.shape[3] == 512 and o.shape[3] == 64 and n_out == 128
+
+
+@torch.no_grad()
+def norm_proj(o: torch.Tensor, g: torch.Tensor, norm_weight: Optional[torch.Tensor], weight: torch.Tensor,
+              eps: float = 1e-5, tokens_per_wg: int = 0) -> torch.Tensor:
+    """``o_proj(FusedRMSNormSwishGate(o, g))`` in one kernel: o, g [B, T, 8, 64] bf16 (g may be a view with a token
+    stride), norm_weight [64] or None, weight [128, 512] bf16 -> [B, T, 128]. The normalised tensor is rounded to bf16
+    as the two-step route stores it, but never written."""
+    require_cuda(o, g, norm_weight, weight)
+    if not norm_proj_supported(o, weight.shape[0]) or weight.dtype != torch.bfloat16 or weight.shape[1] != 512:
+        raise ValueError("norm_proj: bf16 o [B, T, 8, 64] and weight [128, 512] expected")
+    B, T, H, D = o.shape
+    o = o.contiguous()
+    g = g.to(o.dtype)
+    if not (g.stride(-1) == 1 and g.stride(-2) == D and g.stride(1) % 8 == 0 and g.data_ptr() % 16 == 0
+            and (B == 1 or g.stride(0) == T * g.stride(1))):
+        g = g.contiguous()
+    w32 = _f32(norm_weight, o.device)
+    weight = weight.detach().contiguous()
+    y = torch.empty((B, T, weight.shape[0]), dtype=o.dtype, device=o.device)
+    check(_capi.lib().lampa_norm_proj_fwd(ptr(o), ptr(g), g.stride(1), ptr(w32), ptr(weight), B * T, H, D, weight.shape[0],
+                                          float(eps), ptr(y), tokens_per_wg, stream_of(o)), "lampa_norm_proj_fwd")
+    return y
+
+
 class ShortConvolution(nn.Conv1d):
     """``short_convolution.py:528-721``: depthwise causal convolution over the time axis of a [B, T, D] tensor with
     an optional SiLU, a cache of the last W inputs per sequence ([N, D, W]) and a one-token ``step``."""

@@ -112,6 +112,28 @@ def test_fused_projection_convolution(device, B, T, tokens_per_wg):
     assert (g.float() - proj[..., 1536:2048].float()).abs().max() < 0.05
 
 
+@pytest.mark.parametrize("B,T,tokens_per_wg", [(1, 1, 0), (2, 333, 64), (1, 6000, 0), (1, 100, 32)])
+def test_fused_gated_norm_output_projection(device, B, T, tokens_per_wg):
+    gen = torch.Generator().manual_seed(T)
+    o = torch.randn(B, T, 8, 64, generator=gen).to(torch.bfloat16)
+    wide = torch.randn(B, T, 1024, generator=gen).to(torch.bfloat16).to(device)
+    g = wide[..., 256:768].unflatten(-1, (8, 64))                               # a strided view, read in place
+    nw = (torch.rand(64, generator=gen) + 0.5).to(torch.bfloat16)
+    W = (torch.randn(128, 512, generator=gen) * 0.05).to(torch.bfloat16)
+    y = lo.norm_proj(o.to(device), g, nw.to(device), W.to(device), 1e-6, tokens_per_wg)
+    assert y.shape == (B, T, 128) and y.dtype == torch.bfloat16
+    normed, _ = ol.rms_norm(_f64(o), _f64(g), _f64(nw), eps=1e-6, activation="swish")
+    normed_b = torch.from_numpy(normed).to(torch.bfloat16)                     # the rounding the kernel applies
+    want = _f64(normed_b).reshape(B, T, 512) @ _f64(W).T
+    err = np.abs(_f64(y) - want)
+    # one bf16 rounding of the result plus last-bit differences of the rounded normalised tensor (512 terms)
+    assert np.all(err <= 2 ** -7 * np.abs(want) + 2e-2), float(err.max())
+    assert err.mean() < 3e-3
+    two_step = torch.nn.functional.linear(lo.rms_norm_gated(o.to(device), g, nw.to(device), None, "swish", eps=1e-6)
+                                          .reshape(B, T, 512), W.to(device))
+    assert (y.float() - two_step.float()).abs().max() < 0.06 and (y.float() - two_step.float()).abs().mean() < 3e-3
+
+
 def test_short_convolution_module_cache_and_step(device):
     torch.manual_seed(4)
     D, W, T = 64, 4, 19
