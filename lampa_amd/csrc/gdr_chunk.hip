@@ -512,7 +512,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     // per-token factors of chunk c (gate, beta, norms) into tile set par
     auto stage_factors = [&](int c, int par) {
       const GdrTiles tl = tiles(par);
-      const int len = chunk_len[uniform(c)];
+      (void)c;
       // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction) and beta, lane = token; both
       // come ready from the chunk's record (zero decay increment and zero beta past the end of a partial chunk)
       const float bv = rb, gv = rg;

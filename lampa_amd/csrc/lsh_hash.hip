@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
     if (c < n_cols && part == 0) { s_lo[c] = n_valid == 0 ? 0 : lo; s_hi[c] = n_valid == 0 ? 0 : hi; }
   }
   __syncthreads();
-  if (threadIdx.x < n_tables) {
+  if ((int)threadIdx.x < n_tables) {
     const int table = threadIdx.x;
     uint64_t total = 1;
     int overflow = 0;
