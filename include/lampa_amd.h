@@ -181,9 +181,13 @@ int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_tokens, int64
  * models/hattention/modeling_gated_deltaproduct.py:612-623): y[t] = W * vec(rmsnorm(o[t, h]) * norm_w * g[t, h] *
  * sigmoid(g[t, h])), the normalised tensor rounded to bf16 as the unfused pair would store it but never written.
  * o [n_tokens, heads, head_dim] contiguous; g the same shape with token stride g_stride elements; norm_w fp32
- * [head_dim] or NULL; W [n_out, heads * head_dim] row-major; y [n_tokens, n_out]. */
+ * [head_dim] or NULL; W [n_out, heads * head_dim] row-major; y [n_tokens, n_out].
+ * With residual [n_tokens, n_out] (bf16) the residual add and the next layer's pre-norm (RMSNorm with residual,
+ * models/hattention/fused_norm.py:2307-2354, as GatedDeltaProductBlock.forward uses it) are applied too:
+ * res_out = residual + projection, y = rmsnorm(res_out) * next_w (fp32 [n_out] or NULL) with next_eps. */
 int lampa_norm_proj_fwd(const void* o, const void* g, int64_t g_stride, const float* norm_w, const void* W, int64_t n_tokens,
-                        int heads, int head_dim, int n_out, float eps, void* y, int tokens_per_wg, void* stream);
+                        int heads, int head_dim, int n_out, float eps, void* y, const void* residual, const float* next_w,
+                        float next_eps, void* res_out, int tokens_per_wg, void* stream);
 
 /* RMS norm over the last dimension with optional residual add, weight, bias and output gate. Replaces
  * layer_norm_gated_fwd / layer_norm_fwd with is_rms_norm (models/hattention/fused_norm.py:40-111,456-531,1436-1506).

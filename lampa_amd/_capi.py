@@ -45,7 +45,8 @@ _SIGNATURES = {
                                        _i64, _i32, _i64, _vp]),
     "lampa_proj_conv_fwd": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _i32, _vp, _i32,
                                    _vp]),
-    "lampa_norm_proj_fwd": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _i32, _vp]),
+    "lampa_norm_proj_fwd": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _vp, _vp, _f32, _vp, _i32,
+                                   _vp]),
     "lampa_rms_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _f32, _i32, _i32, _i32, _i32, _i64,
                                   _vp]),
     "lampa_gdr_gates_fwd": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i32, _f32, _i32, _vp, _vp, _vp]),

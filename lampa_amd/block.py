@@ -56,8 +56,12 @@ class GatedDeltaLayer(nn.Module):
         return self._fused[1]
 
     @torch.no_grad()
-    def forward(self, hidden_states: torch.Tensor, cu_seqlens=None, initial_state=None, output_final_state=False):
-        """hidden_states [B, T, hidden] -> (o [B, T, hidden], final_state or None)."""
+    def forward(self, hidden_states: torch.Tensor, cu_seqlens=None, initial_state=None, output_final_state=False,
+                residual=None, next_norm=None):
+        """hidden_states [B, T, hidden] -> (o [B, T, hidden], final_state or None). With ``residual`` and ``next_norm``
+        (an ``RMSNorm``) the layer also applies the residual add and that norm and returns
+        ((next_norm(o + residual), o + residual), final_state): the pre-norm wiring of a stack of layers, fused into
+        the output projection kernel when the shapes allow it."""
         B, T, _ = hidden_states.shape
         H, dk, dv, kd, vd = self.num_heads, self.head_dim, self.head_v_dim, self.key_dim, self.value_dim
         convs = (self.q_conv1d, self.k_conv1d, self.v_conv1d)
@@ -82,10 +86,14 @@ class GatedDeltaLayer(nn.Module):
                                           initial_state=initial_state, output_final_state=output_final_state,
                                           cu_seqlens=cu_seqlens, use_qk_l2norm_in_kernel=True)
         gate = xg.unflatten(-1, (H, dv))
-        if norm_proj_supported(o, self.hidden_size) and self.o_proj.weight.dtype == torch.bfloat16:
-            return norm_proj(o, gate, self.o_norm.weight, self.o_proj.weight, self.o_norm.eps), state  # norm + gate + GEMM
-        o = self.o_norm(o, gate)
-        return self.o_proj(o.reshape(B, T, vd)), state
+        if norm_proj_supported(o, self.hidden_size) and self.o_proj.weight.dtype == torch.bfloat16:  # norm + gate + GEMM
+            if residual is not None and residual.dtype == torch.bfloat16 and next_norm.bias is None:
+                return norm_proj(o, gate, self.o_norm.weight, self.o_proj.weight, self.o_norm.eps, residual=residual,
+                                 next_norm_weight=next_norm.weight, next_eps=next_norm.eps), state
+            out = norm_proj(o, gate, self.o_norm.weight, self.o_proj.weight, self.o_norm.eps)
+        else:
+            out = self.o_proj(self.o_norm(o, gate).reshape(B, T, vd))
+        return (out if residual is None else next_norm(out, residual, True)), state
 
 
 class LshgdBlock(nn.Module):
@@ -132,10 +140,9 @@ class LshgdBlock(nn.Module):
         perm = self.order(coords)
         x = self.input(feats.to(dtype))
         x = lsh.gather_rows(x[None], perm[None])                                 # [1, N, hidden], LSH order
-        residual = None
-        for norm, layer in zip(self.norms, self.layers):
-            h, residual = norm(x, residual, True)                                # residual <- x + residual; h = norm(residual)
-            x, _ = layer(h)
-        h, _ = self.norm_f(x, residual, True)
+        h, residual = self.norms[0](x, None, True)                               # residual = x, h = norm(x)
+        for i, layer in enumerate(self.layers):                                  # residual <- out + residual; h = next norm
+            next_norm = self.norms[i + 1] if i + 1 < len(self.layers) else self.norm_f
+            (h, residual), _ = layer(h, residual=residual, next_norm=next_norm)
         h = lsh.scatter_rows(h, perm[None])[0]                                   # back to the input order
         return self.head(h)

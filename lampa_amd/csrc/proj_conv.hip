@@ -262,10 +262,13 @@ extern "C" int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_to
 __global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restrict__ o, const __bf16* __restrict__ g,
                                                           int64_t g_stride, const float* __restrict__ norm_w,
                                                           const __bf16* __restrict__ W, int64_t n_tokens, float eps,
-                                                          __bf16* __restrict__ y, int tokens_per_wg) {
+                                                          __bf16* __restrict__ y, const __bf16* __restrict__ residual,
+                                                          const float* __restrict__ next_w, float next_eps,
+                                                          __bf16* __restrict__ res_out, int tokens_per_wg) {
   constexpr int NKS = NP_KMAX / 16;
   __shared__ __align__(16) __bf16 s_a[2][PC_ROWS * NP_LDA];
   __shared__ __align__(16) __bf16 s_out[4][PC_ROWS * (32 + 8)];
+  __shared__ float s_ss[4][PC_ROWS];  // with a residual: every wave's share of the rows' sums of squares
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   const int64_t T0 = (int64_t)blockIdx.x * tokens_per_wg;
   const int64_t T1 = T0 + tokens_per_wg < n_tokens ? T0 + tokens_per_wg : n_tokens;
@@ -309,10 +312,22 @@ __global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restr
   };
 
   const int cg = lane & 3, tq = lane >> 2;  // output role: row 2 tq + i (i < 2), columns 8 cg .. 8 cg + 7 of the wave's 32
+  float nxw[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) nxw[c] = (residual && next_w) ? next_w[32 * wave + 8 * cg + c] : 1.0f;
   int buf = 0;
   if (T0 < T1) stage(T0, 0);
   __syncthreads();
   for (int64_t t0 = T0; t0 < T1; t0 += PC_ROWS, buf ^= 1) {
+    // the residual rows of this tile are requested first: their latency hides behind the staging and the MFMAs
+    bf16x8 rv[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) rv[i][c] = (__bf16)0.0f;
+      const int64_t t = t0 + 2 * tq + i;
+      if (residual && t < T1) rv[i] = *reinterpret_cast<const bf16x8*>(residual + t * NP_OUT + 32 * wave + 8 * cg);
+    }
     if (t0 + PC_ROWS < T1) stage(t0 + PC_ROWS, buf ^ 1);   // next tile while this one is multiplied
     f32x16 acc;
 #pragma unroll
@@ -324,23 +339,65 @@ __global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restr
 #pragma unroll
     for (int r = 0; r < 16; ++r) so[(8 * (r / 4) + 4 * hh + (r % 4)) * 40 + ln] = (__bf16)acc[r];
     lds_fence();
+    if (!residual) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int tr = 2 * tq + i;
-      const int64_t t = t0 + tr;
-      if (t < T1)
-        *reinterpret_cast<bf16x8*>(y + t * NP_OUT + 32 * wave + 8 * cg) = *reinterpret_cast<const bf16x8*>(&so[tr * 40 + 8 * cg]);
+      for (int i = 0; i < 2; ++i) {
+        const int tr = 2 * tq + i;
+        const int64_t t = t0 + tr;
+        if (t < T1)
+          *reinterpret_cast<bf16x8*>(y + t * NP_OUT + 32 * wave + 8 * cg) = *reinterpret_cast<const bf16x8*>(&so[tr * 40 + 8 * cg]);
+      }
+    } else {
+      // residual add and the next layer's RMS norm over the 128 output columns (fused_norm.py:1436-1506 with a
+      // residual): res_out = residual + y, y = rmsnorm(res_out) * next_w, the sum of squares taken before rounding
+      float sres[2][8];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int tr = 2 * tq + i;
+        const bf16x8 yv = *reinterpret_cast<const bf16x8*>(&so[tr * 40 + 8 * cg]);
+        float ss = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          sres[i][c] = (float)yv[c] + (float)rv[i][c];
+          ss = __builtin_fmaf(sres[i][c], sres[i][c], ss);
+        }
+        ss += __shfl_xor(ss, 1);
+        ss += __shfl_xor(ss, 2);
+        if (cg == 0) s_ss[wave][tr] = ss;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int tr = 2 * tq + i;
+        const int64_t t = t0 + tr;
+        const float tot = s_ss[0][tr] + s_ss[1][tr] + s_ss[2][tr] + s_ss[3][tr];
+        const float rstd = 1.0f / sqrtf(tot * (1.0f / NP_OUT) + next_eps);
+        bf16x8 ro, ho;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          ro[c] = (__bf16)sres[i][c];
+          ho[c] = (__bf16)(sres[i][c] * rstd * nxw[c]);
+        }
+        if (t < T1) {
+          *reinterpret_cast<bf16x8*>(res_out + t * NP_OUT + 32 * wave + 8 * cg) = ro;
+          *reinterpret_cast<bf16x8*>(y + t * NP_OUT + 32 * wave + 8 * cg) = ho;
+        }
+      }
     }
-    __syncthreads();  // the next tile is staged, this tile's A operand is free again
+    __syncthreads();  // the next tile is staged, this tile's A operand and the row sums are free again
   }
 }
 
 // o [n_tokens, 8, 64] bf16 contiguous; g the same shape with token stride g_stride elements; norm_w fp32 [64] or NULL;
 // W [128, 512] bf16 row-major (the output projection); y [n_tokens, 128] bf16.
+// With residual [n_tokens, 128] bf16: res_out = residual + projection (bf16) and y = rmsnorm(res_out) * next_w
+// (next_w fp32 [128] or NULL, next_eps), i.e. the residual add and the next layer's pre-norm are applied as well.
 extern "C" int lampa_norm_proj_fwd(const void* o, const void* g, int64_t g_stride, const float* norm_w, const void* W,
-                                   int64_t n_tokens, int heads, int head_dim, int n_out, float eps, void* y, int tokens_per_wg,
-                                   void* stream) {
+                                   int64_t n_tokens, int heads, int head_dim, int n_out, float eps, void* y,
+                                   const void* residual, const float* next_w, float next_eps, void* res_out,
+                                   int tokens_per_wg, void* stream) {
   if (!o || !g || !W || !y || n_tokens < 0) return LAMPA_ERR_INVALID;
+  if (residual && (!res_out || ((uintptr_t)residual | (uintptr_t)res_out) % 16)) return LAMPA_ERR_INVALID;
   if (heads * head_dim != NP_KMAX || head_dim != NP_D || n_out != NP_OUT) return LAMPA_ERR_UNSUPPORTED;
   if (g_stride < NP_KMAX || g_stride % 8 || ((uintptr_t)o | (uintptr_t)g | (uintptr_t)W | (uintptr_t)y) % 16)
     return LAMPA_ERR_UNSUPPORTED;
@@ -358,7 +415,7 @@ extern "C" int lampa_norm_proj_fwd(const void* o, const void* g, int64_t g_strid
   LAMPA_PROF(s, "start");
   hipLaunchKernelGGL(pc_norm_proj_kernel, dim3((unsigned)((n_tokens + tokens_per_wg - 1) / tokens_per_wg)), dim3(256), 0, s,
                      (const __bf16*)o, (const __bf16*)g, g_stride, norm_w, (const __bf16*)W, n_tokens, eps, (__bf16*)y,
-                     tokens_per_wg);
+                     (const __bf16*)residual, next_w, next_eps, (__bf16*)res_out, tokens_per_wg);
   LAMPA_PROF(s, "pc_norm_proj_kernel");
   return lampa_launch_status();
 }

@@ -200,10 +200,13 @@ def norm_proj_supported(o: torch.Tensor, n_out: int) -> bool:
 
 @torch.no_grad()
 def norm_proj(o: torch.Tensor, g: torch.Tensor, norm_weight: Optional[torch.Tensor], weight: torch.Tensor,
-              eps: float = 1e-5, tokens_per_wg: int = 0) -> torch.Tensor:
+              eps: float = 1e-5, tokens_per_wg: int = 0, residual: Optional[torch.Tensor] = None,
+              next_norm_weight: Optional[torch.Tensor] = None, next_eps: float = 1e-5):
     """``o_proj(FusedRMSNormSwishGate(o, g))`` in one kernel: o, g [B, T, 8, 64] bf16 (g may be a view with a token
     stride), norm_weight [64] or None, weight [128, 512] bf16 -> [B, T, 128]. The normalised tensor is rounded to bf16
-    as the two-step route stores it, but never written."""
+    as the two-step route stores it, but never written. With ``residual`` [B, T, 128] (bf16) the kernel also applies the
+    residual add and the next pre-norm, ``RMSNorm(next_norm_weight, next_eps)(y, residual, prenorm=True)``, and returns
+    (normalised [B, T, 128], residual + y [B, T, 128])."""
     require_cuda(o, g, norm_weight, weight)
     if not norm_proj_supported(o, weight.shape[0]) or weight.dtype != torch.bfloat16 or weight.shape[1] != 512:
         raise ValueError("norm_proj: bf16 o [B, T, 8, 64] and weight [128, 512] expected")
@@ -216,9 +219,18 @@ def norm_proj(o: torch.Tensor, g: torch.Tensor, norm_weight: Optional[torch.Tens
     w32 = _f32(norm_weight, o.device)
     weight = weight.detach().contiguous()
     y = torch.empty((B, T, weight.shape[0]), dtype=o.dtype, device=o.device)
+    res_out, nw32 = None, None
+    if residual is not None:
+        require_cuda(residual, next_norm_weight)
+        if residual.shape != y.shape or residual.dtype != o.dtype:
+            raise ValueError("norm_proj: residual must be bf16 [B, T, 128]")
+        residual = residual.contiguous()
+        res_out = torch.empty_like(y)
+        nw32 = _f32(next_norm_weight, o.device)
     check(_capi.lib().lampa_norm_proj_fwd(ptr(o), ptr(g), g.stride(1), ptr(w32), ptr(weight), B * T, H, D, weight.shape[0],
-                                          float(eps), ptr(y), tokens_per_wg, stream_of(o)), "lampa_norm_proj_fwd")
-    return y
+                                          float(eps), ptr(y), ptr(residual), ptr(nw32), float(next_eps), ptr(res_out),
+                                          tokens_per_wg, stream_of(o)), "lampa_norm_proj_fwd")
+    return y if residual is None else (y, res_out)
 
 
 class ShortConvolution(nn.Conv1d):

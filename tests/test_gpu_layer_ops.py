@@ -132,6 +132,19 @@ def test_fused_gated_norm_output_projection(device, B, T, tokens_per_wg):
     two_step = torch.nn.functional.linear(lo.rms_norm_gated(o.to(device), g, nw.to(device), None, "swish", eps=1e-6)
                                           .reshape(B, T, 512), W.to(device))
     assert (y.float() - two_step.float()).abs().max() < 0.06 and (y.float() - two_step.float()).abs().mean() < 3e-3
+    # with the residual add and the next pre-norm applied in the same kernel
+    res = torch.randn(B, T, 128, generator=gen).to(torch.bfloat16)
+    nxt = (torch.rand(128, generator=gen) + 0.5).to(torch.bfloat16)
+    h, r = lo.norm_proj(o.to(device), g, nw.to(device), W.to(device), 1e-6, tokens_per_wg, residual=res.to(device),
+                        next_norm_weight=nxt.to(device), next_eps=1e-6)
+    y_b = _f64(torch.from_numpy(want).to(torch.bfloat16))                        # the projection as the kernel rounds it
+    want_h, want_r = ol.rms_norm(y_b, None, _f64(nxt), residual=_f64(res), eps=1e-6)
+    assert h.shape == (B, T, 128) and r.dtype == torch.bfloat16
+    err_r, err_h = np.abs(_f64(r) - want_r), np.abs(_f64(h) - want_h)
+    assert np.all(err_r <= 2 ** -7 * np.abs(want_r) + 3e-2) and err_r.mean() < 4e-3
+    assert np.all(err_h <= 2 ** -6 * np.abs(want_h) + 3e-2) and err_h.mean() < 4e-3
+    h2, r2 = lo.rms_norm(y, nxt.to(device), None, residual=res.to(device), eps=1e-6, prenorm=True)   # two-step route
+    assert (r.float() - r2.float()).abs().max() < 0.04 and (h.float() - h2.float()).abs().max() < 0.06
 
 
 def test_short_convolution_module_cache_and_step(device):
