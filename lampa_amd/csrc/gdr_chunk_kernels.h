@@ -1,0 +1,1081 @@
+// Chunkwise gated-delta-rule forward on gfx950 (bf16 MFMA 32x32x16, fp32 accumulate, fp32 state).
+//
+// Replaces the forward pipeline of chunk_gated_delta_rule (reference chengjiang123/Lampa,
+// models/hattention/gated_delta_rule_ori.py:29-80): chunk_local_cumsum (cumsum.py:27-62), l2norm_fwd
+// (l2norm.py:87-103), chunk_scaled_dot_kkt_fwd (chunk_scaled_dot_kkt.py:27-71), solve_tril (solve_tril.py),
+// recompute_w_u_fwd (wy_fast.py:140-189), chunk_gated_delta_rule_fwd_h (chunk_delta_h.py:34-189) and
+// chunk_fwd_o (chunk_o.py:33-111).
+//
+// Per chunk of C = 64 tokens of one head, with gamma the in-chunk cumulative log-decay, rk / rq the l2-norm
+// factors of the raw k / q rows and S the K x V state entering the chunk:
+//   A     = strict_lower( beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j} ),   T = (I + A)^-1
+//   R     = beta_i ( v_i - e^{gamma_i} rk_i (K S)_i )                v_new = T R
+//   o_i   = scale e^{gamma_i} rq_i (Q S)_i + (P v_new)_i,    P_ij = scale rq_i rk_j (q_i . k_j) e^{gamma_i - gamma_j}, j <= i
+//   S'    = e^{gamma_last} S + K^T ( e^{gamma_last - gamma_j} rk_j v_new_j )
+// All per-token factors are applied to accumulator rows in fp32, so the MFMA operands are the RAW bf16 k, q, v
+// tiles and the only intermediate that goes through HBM is T (6 KiB per chunk and head).
+//
+// Kernels:
+//   tinv     wave per (chunk, head): K K^T on MFMA with operand fragments loaded straight from HBM, gating, blocked
+//            inverse (two 32x32 forward substitutions in fp32 + an MFMA merge with bf16 high/remainder splits);
+//            T goes to HBM as three 32x32 bf16 blocks.
+//   segment  workgroup per (segment of chunks, head), one "chain" wave per 32 columns plus two "stager" waves. Each
+//            chunk's k, v, q, T tiles are staged once in LDS (row-major only), the coming chunks' global loads are
+//            in flight meanwhile, and every chain wave runs the recurrence on its columns with the state in
+//            accumulator registers. PASS_A: columns of [M | N] of the segment's affine map S -> M S + N (start
+//            identity / zero). PASS_B: value columns, from the segment's true initial state, writing o (and the
+//            final state).
+//   scan     S_{p+1} = M_p S_p + N_p over the segments of a sequence, storing each segment's initial state.
+// The state tile is fed back as the next MFMA's B operand straight from the accumulator registers: register r of
+// lane l is row 8*(r/4) + 4*(l/32) + r%4, and since a contraction may visit its index in any order as long as
+// both operands agree, every A operand is read from LDS in that slot order (ld_kappa).
+#pragma once
+#include "gdr_common.h"
+#include "gdr_plan.h"
+
+// Device pointers to the tables of the plan (resolved on the host, so that a kernel reaches an entry with one
+// load instead of a dependent pair).
+struct GdrPlanView {
+  const int32_t *chunk_tok0, *chunk_len, *seg_chunk0, *seg_nchunks, *seg_seq, *seg_flags, *seq_seg0, *seq_nseg;
+};
+static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_dev) {
+  GdrPlanView pv;
+  pv.chunk_tok0 = plan_dev + plan_host[PLAN_OFF_CHUNK_TOK0];
+  pv.chunk_len = plan_dev + plan_host[PLAN_OFF_CHUNK_LEN];
+  pv.seg_chunk0 = plan_dev + plan_host[PLAN_OFF_SEG_CHUNK0];
+  pv.seg_nchunks = plan_dev + plan_host[PLAN_OFF_SEG_NCHUNKS];
+  pv.seg_seq = plan_dev + plan_host[PLAN_OFF_SEG_SEQ];
+  pv.seg_flags = plan_dev + plan_host[PLAN_OFF_SEG_FLAGS];
+  pv.seq_seg0 = plan_dev + plan_host[PLAN_OFF_SEQ_SEG0];
+  pv.seq_nseg = plan_dev + plan_host[PLAN_OFF_SEQ_NSEG];
+  return pv;
+}
+
+#define T_BYTES (3 * 32 * 32 * 2)  // T of one chunk and head in HBM: bf16 blocks T11 | T21 | T22, 32x32 row-major each
+// Record of one chunk and head: T, then the chunk's cumulative log-decay (units of log 2) and beta per token, fp32
+// [64] each. The segment kernels take the two factor rows from here: in g and beta themselves a head's 64 values sit
+// 4 bytes apart in rows that interleave all heads, so every workgroup would fetch the sectors of all of them.
+#define REC_BYTES (T_BYTES + 2 * 64 * 4)
+
+__device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
+  return *reinterpret_cast<const bf16x8*>(base + (size_t)frag * 1024 + lane * 16);
+}
+__device__ __forceinline__ void frag_store(unsigned char* base, int frag, int lane, bf16x8 v) {
+  *reinterpret_cast<bf16x8*>(base + (size_t)frag * 1024 + lane * 16) = v;
+}
+
+// A-operand fragment (rows row0..row0+31 of a row-major bf16 array with `stride` elements per row, contraction
+// step starting at column col0) in accumulator slot order: slots 0-3 = columns col0 + 4hh + 0..3,
+// slots 4-7 = columns col0 + 8 + 4hh + 0..3.
+__device__ __forceinline__ bf16x8 ld_kappa(const __bf16* arr, int stride, int row, int col0, int hh) {
+  const bf16x4 lo = *reinterpret_cast<const bf16x4*>(arr + row * stride + col0 + 4 * hh);
+  const bf16x4 hi = *reinterpret_cast<const bf16x4*>(arr + row * stride + col0 + 8 + 4 * hh);
+  bf16x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
+__device__ __forceinline__ f32x16 zero16() {
+  f32x16 z;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+  return z;
+}
+
+// Tells the compiler that x is the same in every lane, so that a table lookup with it becomes a scalar load: a
+// vector load would join the queue of the prefetches and its wait would drain all of them.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+__device__ __forceinline__ int acc_row(int r, int hh) { return 8 * (r / 4) + 4 * hh + (r % 4); }
+
+__device__ __forceinline__ float l2_factor(float ss, int l2norm) {
+  if (l2norm == GDR_L2_CHUNK) return 1.0f / __fsqrt_rn(ss + 1e-6f);
+  if (l2norm == GDR_L2_RECURRENT) return 1.0f / (__fsqrt_rn(ss) + 1e-6f);
+  return 1.0f;
+}
+
+// 16-byte vector of the input element type
+template <typename T>
+struct Raw8 {
+  typedef T type __attribute__((ext_vector_type(8)));
+};
+
+// Raw input piece -> bf16 operand piece (+ its sum of squares when the rows get l2-normalised). bf16 inputs are
+// passed through bit for bit; fp16 inputs are rounded to bf16 here.
+template <typename T>
+__device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& ss, bool want_ss) {
+  bf16x8 out;
+  if constexpr (sizeof(T) == 2 && !__is_same(T, _Float16)) {
+    out = __builtin_bit_cast(bf16x8, v);
+    if (want_ss) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)out[e];
+        ss = __builtin_fmaf(f, f, ss);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)v[e];
+      if (want_ss) ss = __builtin_fmaf(f, f, ss);
+      out[e] = (__bf16)f;
+    }
+  }
+  return out;
+}
+
+// ---- T = (I + A)^-1 ------------------------------------------------------------------------------------------
+// One WAVE per (chunk, head), one wave per workgroup: the forward substitution is a single-wave job, so many small
+// workgroups per CU keep every SIMD busy. The k tile never touches LDS: the MFMA operand fragments of K K^T are
+// 16-byte global loads (lane = row, its half of each 16-wide contraction step). LDS holds only the two diagonal
+// blocks (fp32) and the per-token factors, all wave-private (LDS operations of one wave complete in order).
+// T is stored as three row-major 32x32 bf16 blocks: T11 | T21 | T22 (the upper-right block is zero and not kept).
+template <typename T, int KT>
+__global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
+                                                         const float* __restrict__ beta, const GdrPlanView pv,
+                                                         unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
+  constexpr int SB = 36, NK = KT / 16;
+  // diagonal blocks of A, later of T. ONE array: the forward substitution indexes it with the lane's block, and
+  // two separate arrays would make the compiler read both and select per value.
+  __shared__ __align__(16) float s_Ad[2 * 32 * SB];
+  __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64];
+  float* s_A11 = s_Ad;
+  float* s_A22 = s_Ad + 32 * SB;
+
+  const int chunk = blockIdx.x, hv = blockIdx.y;
+  const int h = hv / (HV / H);
+  const int tok0 = pv.chunk_tok0[chunk];
+  const int len = pv.chunk_len[chunk];
+  const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+
+  // operand fragments of the k tile: f[tm][ks] = k[32 tm + ln][16 ks + 8 hh .. + 7]; rows past the end of a
+  // partial chunk behave as k = 0, g = 0, beta = 0
+  typename Raw8<T>::type raw[2][NK];
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm) {
+    const T* kp = k + ((size_t)(tok0 + min(32 * tm + ln, len - 1)) * H + h) * KT + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) raw[tm][ks] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 16 * ks);
+  }
+  {  // gamma is kept in units of log 2 (exp2 is one instruction)
+    const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
+    const float gv = g[gi], bv = beta[gi];
+    const float gcum = 1.44269504f * wave_inclusive_scan(lane < len ? gv : 0.0f), bz = lane < len ? bv : 0.0f;
+    s_gamma[lane] = gcum;
+    s_beta[lane] = bz;
+    float* fact = reinterpret_cast<float*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES + T_BYTES);
+    fact[lane] = gcum;
+    fact[64 + lane] = bz;
+  }
+  bf16x8 f[2][NK];
+  {
+    typename Raw8<T>::type zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+      float ss = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        f[tm][ks] = raw_to_bf16<T>(32 * tm + ln < len ? raw[tm][ks] : zero, ss, l2norm != GDR_L2_NONE);
+      ss += __shfl_xor(ss, 32);
+      s_rk[32 * tm + ln] = l2_factor(ss, l2norm);
+    }
+  }
+  lds_fence();
+
+  // A = strict_lower(beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j}). The diagonal blocks go to LDS; the
+  // off-diagonal block is computed transposed (rows j < 32, columns i >= 32) and stays in registers, because an
+  // accumulator that holds A21^T is, rounded to bf16, the A operand of A21 X.
+  f32x16 a21t;
+#pragma unroll
+  for (int t = 0; t < 3; ++t) {
+    const int tr = t == 2 ? 1 : 0, tc = t == 0 ? 0 : 1;  // accumulator rows / columns: (0,0), (0,1) = A21^T, (1,1)
+    f32x4 gr4[4], rr4[4], br4[4];
+#pragma unroll
+    for (int b4 = 0; b4 < 4; ++b4) {
+      gr4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tr + 8 * b4 + 4 * hh]);
+      rr4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tr + 8 * b4 + 4 * hh]);
+      br4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tr + 8 * b4 + 4 * hh]);
+    }
+    const int cidx = 32 * tc + ln;
+    const float gc = s_gamma[cidx], rc = s_rk[cidx], bc = s_beta[cidx];
+    lds_fence();
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) acc = mfma32(f[tr][ks], f[tc][ks], acc);
+    if (t == 1) {  // rows j (tile 0), columns i (tile 1): i > j always
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * __builtin_amdgcn_exp2f(gc - gr4[r / 4][r % 4]);
+    } else {       // rows i, columns j of a diagonal block; the mask goes on the exponent (branch-free)
+      float* blk = t == 0 ? s_A11 : s_A22;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int il = acc_row(r, hh);
+        blk[il * SB + ln] = acc[r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
+                            __builtin_amdgcn_exp2f(il > ln ? gr4[r / 4][r % 4] - gc : -1e30f);
+      }
+    }
+  }
+  lds_fence();
+
+  // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
+  // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
+  // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
+  const int b = hh, c = ln;
+  float* Ab = s_Ad + b * (32 * SB);
+  {
+    float x[32];
+    f32x4 rowbuf[2][8];  // rows i and i+1: the next row loads while this one is reduced
+    rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SB);
+    x[0] = (c == 0) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int i = 1; i < 32; ++i) {
+      if (i + 1 < 32) {
+#pragma unroll
+        for (int q = 0; q < (i + 1 + 3) / 4; ++q)
+          rowbuf[(i + 1) & 1][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 1) * SB + 4 * q);
+      }
+      float acc0 = (i == c) ? 1.0f : 0.0f, acc1 = 0.0f;
+#pragma unroll
+      for (int j = 0; j < i; ++j) {
+        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc1);
+        else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
+      }
+      x[i] = acc0 + acc1;
+      // pins the order "loads of row i+1, arithmetic of row i": without it the compiler either serialises every
+      // load behind a wait or hoists all the loads to the top and spills
+      asm volatile("" : "+v"(x[i]) : : "memory");
+    }
+    lds_fence();  // every lane is done reading A11 / A22 before they are overwritten
+#pragma unroll
+    for (int i = 0; i < 32; ++i) Ab[i * SB + c] = x[i];  // fp32 T11 / T22 in place of A11 / A22
+  }
+  lds_fence();
+
+  f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11: A from the A21^T accumulator, T11 rows in the same slot order
+    bf16x8 ahi, alo, bhi, blo;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float av = a21t[8 * ks + q];
+      const float bv = s_A11[(16 * ks + kappa(hh, q)) * SB + ln];
+      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    }
+    y0 = mfma32(ahi, bhi, y0);
+    y1 = mfma32(alo, bhi, y1);
+    y2 = mfma32(ahi, blo, y2);
+  }
+  f32x16 t0 = zero16(), t1 = zero16(), t2 = zero16();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) y0[r] += y1[r] + y2[r];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
+    bf16x8 ahi, alo, bhi, blo;
+    const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
+    const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float av = q < 4 ? a0[q % 4] : a1[q % 4];
+      const float bv = y0[8 * ks + q];
+      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
+      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
+      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    }
+    t0 = mfma32(ahi, bhi, t0);
+    t1 = mfma32(alo, bhi, t1);
+    t2 = mfma32(ahi, blo, t2);
+  }
+
+  // T -> HBM: the diagonal blocks from LDS in 16-byte pieces; T21 from the accumulator, two columns per store
+  // (lanes 2j and 2j+1 swap one value of every adjacent row pair, as in the segment kernel's output)
+  __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES);
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const float* src = blk == 0 ? s_A11 : s_A22;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int piece = lane + 64 * j, row = piece >> 2, part = piece & 3;
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part]);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part + 4]);
+      bf16x8 pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { pk[e] = (__bf16)lo[e]; pk[4 + e] = (__bf16)hi[e]; }
+      *reinterpret_cast<bf16x8*>(out + (blk == 0 ? 0 : 2048) + row * 32 + 8 * part) = pk;
+    }
+  }
+  {
+    const bool odd = ln & 1;
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int pr = 0; pr < 8; ++pr) {
+      const int r0 = 2 * pr, r1 = r0 + 1;
+      const float x0 = -(t0[r0] + (t1[r0] + t2[r0])), x1 = -(t0[r1] + (t1[r1] + t2[r1]));
+      const float keep = odd ? x1 : x0;
+      const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
+      bf16x2 pk;
+      pk[0] = (__bf16)(odd ? got : keep);
+      pk[1] = (__bf16)(odd ? keep : got);
+      const int row = acc_row(r0, hh) + (odd ? 1 : 0);
+      *reinterpret_cast<bf16x2*>(out + 1024 + row * 32 + (ln & ~1)) = pk;
+    }
+  }
+}
+
+// ---- segment kernel --------------------------------------------------------------------------------------------
+// Workgroup per (segment, head). Waves 0 .. SLABS-1 ("chain" waves) each own 32 columns of the state and run the
+// recurrence; the last two waves ("stagers") load the coming chunks' tiles from HBM, stage them ROW-MAJOR in LDS
+// (16-byte writes only), derive the per-token factors and (PASS_B) build the P fragments. Operands that contract
+// over the tokens (K^T, and v in accumulator layout) are read from the row-major tiles with the transposing LDS
+// load (ds_read_b64_tr_b16), so no transposed copy is ever written.
+//
+// The k, v, T tiles and the per-token factors are DOUBLE-buffered in LDS, so the stagers fill the tiles of chunk c+1
+// while the chain waves work on chunk c; q, P and the o tile exist once. LDS-only barriers per chunk (every barrier is
+// a rendezvous of all waves, so the stagers' work is spread such that they are never the slower side):
+//   Qb(c) (PASS_B) q(c) is staged                         -> the stagers build P(c)
+//   B(c)  the chain waves hold every k / v / T operand of chunk c in registers, and tiles (c+1) [PASS_A: also its
+//         factors] and P(c) are complete                   -> buffer c%2 is free for chunk c+2
+//   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
+//                                                          -> the stagers may write q(c+1)
+// Global loads are issued about one chunk period before their data is staged.
+template <int KT, int VT, bool PASS_B>
+struct GdrSegSmem {
+  static constexpr int SK = KT + 8;  // row stride of the k / q tiles (bf16 elements)
+  static constexpr int SV = VT + 8;  // row stride of the v and o tiles
+  static constexpr int ST = 40;      // row stride of a 32x32 block of T (blocks T11, T21, T22)
+  // one set of tiles (two of them)
+  static constexpr int T_OFF_K = 0;
+  static constexpr int T_OFF_V = T_OFF_K + 64 * SK * 2;
+  static constexpr int T_OFF_T = T_OFF_V + 64 * SV * 2;
+  static constexpr int T_OFF_F = T_OFF_T + 3 * 32 * ST * 2;
+  static constexpr int N_FACT = 6;  // beta, ek, dk, gamma, rk, misc
+  static constexpr int TILE_BYTES = T_OFF_F + N_FACT * 64 * 4;
+  static constexpr int OFF_Q = 2 * TILE_BYTES;
+  static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
+  static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
+  static constexpr int OFF_QF = OFF_O + (PASS_B ? 64 * SV * 2 : 0);  // qs, rq
+  static constexpr int BYTES = OFF_QF + (PASS_B ? 2 * 64 * 4 : 0);
+};
+
+// pointers into one of the two tile sets
+struct GdrTiles {
+  __bf16 *k, *v, *t;
+  float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
+};
+
+template <int KT, int VT, bool PASS_B>
+struct GdrSegShape {
+  static constexpr int SLABS = PASS_B ? VT / 32 : (KT + VT) / 32;  // chain waves
+  static constexpr int WAVES = SLABS + 2;                          // + two stager waves
+};
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: lane i of every block of 16 lanes receives element (i % 4) of the four 8-byte rows that
+// lanes i/4, i/4 + 4, i/4 + 8 and i/4 + 12 of its block point at.
+__device__ __forceinline__ bf16x4 lds_read_tr4(const __bf16* p) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p));
+}
+
+// Four consecutive rows row0 + 4hh .. +3 of column col0 + (lane % 32) of a row-major bf16 tile: lane L of a block
+// points at row L / 4, column group L % 4 of the block's 16 columns.
+__device__ __forceinline__ bf16x4 ld_col4(const __bf16* arr, int stride, int col0, int row0, int lane) {
+  const int L = lane & 15, blk = (lane >> 4) & 1, hh = lane >> 5;
+  return lds_read_tr4(arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * (L & 3));
+}
+
+// A-operand fragment of the TRANSPOSE of a row-major tile: operand row = tile column col0 + (lane % 32),
+// contraction over the tile rows row0 .. row0 + 15 in accumulator slot order.
+__device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int col0, int row0, int lane) {
+  const bf16x4 lo = ld_col4(arr, stride, col0, row0, lane), hi = ld_col4(arr, stride, col0, row0 + 8, lane);
+  bf16x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
+template <typename T, int KT, int VT, bool PASS_B>
+__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
+    gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                       const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
+                       const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
+                       const unsigned char* __restrict__ tmat,
+                       const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
+                       unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o,
+                       float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
+  using SM = GdrSegSmem<KT, VT, PASS_B>;
+  constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
+  constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
+  extern __shared__ __align__(16) unsigned char smem[];
+  auto tiles = [&](int par) {
+    unsigned char* base = smem + par * SM::TILE_BYTES;
+    GdrTiles t;
+    t.k = reinterpret_cast<__bf16*>(base + SM::T_OFF_K);
+    t.v = reinterpret_cast<__bf16*>(base + SM::T_OFF_V);
+    t.t = reinterpret_cast<__bf16*>(base + SM::T_OFF_T);
+    t.beta = reinterpret_cast<float*>(base + SM::T_OFF_F);
+    t.ek = t.beta + 64;
+    t.dk = t.beta + 128;
+    t.gamma = t.beta + 192;
+    t.rk = t.beta + 256;
+    t.misc = t.beta + 320;
+    return t;
+  };
+  __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
+  unsigned char* s_P = smem + SM::OFF_P;
+  T* s_o = reinterpret_cast<T*>(smem + SM::OFF_O);
+  float* s_qs = reinterpret_cast<float*>(smem + SM::OFF_QF);  // scale e^{gamma_i} rq_i
+  float* s_rq = s_qs + 64;
+
+  const int seg = blockIdx.x, hv = blockIdx.y;
+  const int h = hv / (HV / H);
+  const int flags = pv.seg_flags[seg];
+  if (!PASS_B && (flags & SEG_LAST)) return;  // nothing follows the last segment of a sequence
+  const int c0 = pv.seg_chunk0[seg], nc = pv.seg_nchunks[seg];
+  const int c1 = c0 + nc;
+  // (the per-chunk tables are separate restrict parameters: read through the view they could alias the kernel's
+  // stores, would be fetched with vector loads and would sit in the same queue as the stagers' prefetches)
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+
+  if (wave >= NSLAB) {
+    // ================================================ stager ================================================
+    constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
+    const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
+    const int srow = stid >> 1, spart = stid & 1;
+    typename Raw8<T>::type rk_[KU], rv_[VU];
+    typename Raw8<T>::type rq0_[PASS_B ? KU : 1], rq1_[PASS_B ? KU : 1];  // q of even / odd chunks of the segment
+    bf16x8 rt_[3];
+    float rg = 0.0f, rb = 0.0f;
+    float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
+    // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
+    // a select on a freshly loaded value would make the wave wait for the load at once.
+    auto issue_tiles = [&](int c) {  // k, v, T
+      c = uniform(c);
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+      const T* kb = k + ((size_t)tok0 * H + h) * KT;
+      const T* vb = v + ((size_t)tok0 * HV + hv) * VT;
+      const int r = min(srow, len - 1);
+      const int koff = r * H * KT + spart * (KT / 2), voff = r * HV * VT + spart * (VT / 2);
+#pragma unroll
+      for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
+#pragma unroll
+      for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
+      const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * REC_BYTES);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
+    };
+    auto issue_gb = [&](int c) {  // cumulative log-decay and beta of the chunk's tokens (lane = token)
+      c = uniform(c);
+      const float* fact = reinterpret_cast<const float*>(tmat + ((size_t)c * HV + hv) * REC_BYTES + T_BYTES);
+      rg = fact[lane];
+      rb = fact[64 + lane];
+    };
+    auto issue_q = [&](int c, typename Raw8<T>::type* rq_) {
+      c = uniform(c);
+      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+      const T* qb = q + ((size_t)tok0 * H + h) * KT;
+      const int koff = min(srow, len - 1) * H * KT + spart * (KT / 2);
+#pragma unroll
+      for (int u = 0; u < KU; ++u) rq_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(qb + koff + 8 * u);
+    };
+    typename Raw8<T>::type zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+    const bool want_ss = l2norm != GDR_L2_NONE;
+
+    float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
+    // k, v and T of chunk c from the registers to tile set par
+    auto stage_data = [&](int c, int par) {
+      const GdrTiles tl = tiles(par);
+      const bool live = srow < chunk_len[uniform(c)];
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        *reinterpret_cast<bf16x8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
+      kss = 0.0f;
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+        *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+#pragma unroll
+      for (int u = 0; u < VU; ++u) {
+        float unused = 0.0f;
+        *reinterpret_cast<bf16x8*>(&tl.v[srow * SV + spart * (VT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
+      }
+    };
+    // per-token factors of chunk c (gate, beta, norms) into tile set par
+    auto stage_factors = [&](int c, int par) {
+      const GdrTiles tl = tiles(par);
+      (void)c;
+      // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction) and beta, lane = token; both
+      // come ready from the chunk's record (zero decay increment and zero beta past the end of a partial chunk)
+      const float bv = rb, gv = rg;
+      const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gv), 63));
+      const float kss2 = kss + dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
+      // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
+      grow = __shfl(gv, srow);
+      const float brow = __shfl(bv, srow);
+      if (spart == 0) {
+        const float rk = l2_factor(kss2, l2norm);
+        tl.beta[srow] = brow;
+        tl.ek[srow] = __builtin_amdgcn_exp2f(grow) * rk;
+        tl.dk[srow] = __builtin_amdgcn_exp2f(g_last - grow) * rk;
+        tl.gamma[srow] = grow;
+        tl.rk[srow] = rk;
+        if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
+      }
+    };
+    auto stage_q = [&](int c, const typename Raw8<T>::type* rq_) {
+      const bool live = srow < chunk_len[uniform(c)];
+      float qss = 0.0f;
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+        *reinterpret_cast<bf16x8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
+            raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
+      qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
+      if (spart == 0) {
+        const float rq = l2_factor(qss, l2norm);
+        s_qs[srow] = scale * __builtin_amdgcn_exp2f(grow) * rq;
+        s_rq[srow] = rq;
+      }
+    };
+
+    auto build_p = [&](int par) {
+      if constexpr (PASS_B) {
+        const GdrTiles tl = tiles(par);
+        // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tile 0, stager 1 tile 2,
+        // and they share tile 1: both run its four MFMAs, each finishes and stores one of its two fragments.
+        auto p_tile = [&](int t, int half) {  // half: -1 = whole tile, 0 / 1 = accumulator registers 0-7 / 8-15
+          const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
+          bf16x8 fa[KT / 16], fb[KT / 16];
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) {
+            fa[ks] = *reinterpret_cast<const bf16x8*>(&tl.k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
+            fb[ks] = *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
+          }
+          f32x4 gj[4], rj[4];  // gamma_j, rk_j of this lane's 16 accumulator rows
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4) {
+            gj[b4] = *reinterpret_cast<const f32x4*>(&tl.gamma[32 * jm + 8 * b4 + 4 * hh]);
+            rj[b4] = *reinterpret_cast<const f32x4*>(&tl.rk[32 * jm + 8 * b4 + 4 * hh]);
+          }
+          const int i = 32 * tn + ln;
+          const float gi = tl.gamma[i], fi = scale * s_rq[i];
+          lds_fence();
+          f32x16 acc = zero16();
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
+          const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
+#pragma unroll
+          for (int part = 0; part < 2; ++part) {
+            if (half >= 0 && half != part) continue;
+#pragma unroll
+            for (int r = 8 * part; r < 8 * part + 8; ++r) {  // the mask goes on the exponent: branch-free
+              const int j = 32 * jm + acc_row(r, hh);
+              acc[r] *= fi * rj[r / 4][r % 4] * __builtin_amdgcn_exp2f(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
+            }
+            frag_store(s_P, f0 + part, lane, acc_to_operand(acc, 8 * part));
+          }
+        };
+        p_tile(sw == 0 ? 0 : 2, -1);
+        p_tile(1, sw);
+      }
+    };
+    // Chunk indices past the end of the segment are clamped (the last chunk is fetched again for nothing), so that
+    // every iteration issues the same loads: with conditional issues the compiler could not count the loads in
+    // flight any more and would drain the queue at every wait. q(c) / q(c+2) share a register set.
+    const int cl = c1 - 1;
+    if (nc > 0) {
+      issue_tiles(c0);
+      issue_gb(c0);
+      if constexpr (PASS_B) { issue_q(c0, rq0_); issue_q(min(c0 + 1, cl), rq1_); }
+      stage_data(c0, 0);
+      stage_factors(c0, 0);
+      issue_tiles(min(c0 + 1, cl));
+      issue_gb(min(c0 + 1, cl));
+      lds_barrier();  // tiles (c0) are ready
+      auto one_chunk = [&](int c, int par, typename Raw8<T>::type* rq_) {
+        if (c + 1 < c1) stage_data(c + 1, par ^ 1);
+        issue_tiles(min(c + 2, cl));
+        if constexpr (PASS_B) {
+          stage_q(c, rq_);
+          issue_q(min(c + 2, cl), rq_);
+          lds_barrier();  // Qb(c)
+          build_p(par);
+          lds_barrier();  // B(c)
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          issue_gb(min(c + 2, cl));
+          lds_barrier();  // C(c)
+        } else {
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          issue_gb(min(c + 2, cl));
+          lds_barrier();  // B(c)
+        }
+      };
+      for (int c = c0; c < c1; c += 2) {
+        one_chunk(c, 0, rq0_);
+        if (c + 1 < c1) one_chunk(c + 1, 1, rq1_);
+      }
+    }
+    return;
+  }
+
+  // ================================================== chain ==================================================
+  // this wave's 32 columns: PASS_B value columns; PASS_A columns of [M | N]
+  const bool is_m = !PASS_B && wave < KT / 32;
+  const int vslab = PASS_B ? wave : (is_m ? 0 : wave - KT / 32);
+  const int col = 32 * vslab + ln;  // value column (unused for M slabs)
+  const float vmask = is_m ? 0.0f : 1.0f;
+
+  f32x16 S[KT / 32];
+  if (PASS_B) {  // the scan leaves every segment's initial state as 32-column slabs in accumulator order
+    const f32x4* si = reinterpret_cast<const f32x4*>(Sinit + (((size_t)seg * HV + hv) * (VT / 32) + vslab) * (KT * 32));
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const f32x4 t = si[(km * 4 + q4) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[km][4 * q4 + e] = t[e];
+      }
+  } else {
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[km][r] = (is_m && 32 * km + acc_row(r, hh) == 32 * wave + ln) ? 1.0f : 0.0f;
+  }
+
+  float dtot = 1.0f;  // product of the chunks' decays over the segment (PASS_A)
+  // The LDS operand reads of a stage are issued as one batch one stage ahead of the MFMAs that use them
+  // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
+  // pays the LDS latency once per MFMA.
+  if (nc > 0) lds_barrier();  // tiles (c0) are ready
+  for (int c = c0; c < c1; ++c) {
+    const GdrTiles tl = tiles((c - c0) & 1);
+    if constexpr (PASS_B) lds_barrier();  // Qb(c) (the chain waves only take part)
+    bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+    bf16x8 ft[6];              // T (stage 2), P (output)
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
+    bf16x8 Sb[KT / 16];
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+    lds_fence();
+    // batch for stage 2: T fragments and the per-token factors / v tile of stage 1's epilogue
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks)  // blocks T11 | T21, T22
+        ft[2 * tm + ks] = ld_kappa(tl.t + (tm == 0 ? 0 : (ks < 2 ? 1 : 2)) * 32 * ST, ST, ln, 16 * (ks & 1), hh);
+    f32x4 be[8], ek[8];
+    bf16x4 vv[8];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+      const int i0 = 8 * t8 + 4 * hh;
+      be[t8] = *reinterpret_cast<const f32x4*>(&tl.beta[i0]);
+      ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
+      // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
+      // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
+      vv[t8] = ld_col4(tl.v, SV, 32 * vslab, 8 * t8, lane);
+    }
+    bf16x8 Rb[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {  // R = beta (v - ek (K S))
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], acc);
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc[4 * b4 + e] =
+              be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ek[4 * tm + b4][e] * acc[4 * b4 + e]);
+      Rb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Rb[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    lds_fence();
+    // batch for stage 3: K^T fragments (transposing reads of the row-major k tile) and the decay factors
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.k, SK, 32 * km, 16 * ks, lane);
+    f32x4 dk[8];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
+    const float dec = tl.misc[0];
+    bf16x8 Vb[4], Vsb[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {  // v_new = T R (T is lower triangular: tile tm needs 2 (tm + 1) steps)
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ft[2 * tm + ks], Rb[ks], acc);
+      Vb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Vb[2 * tm + 1] = acc_to_operand(acc, 8);
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[4 * b4 + e] *= dk[4 * tm + b4][e];
+      Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
+      Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    lds_fence();
+    lds_barrier();  // B(c): every operand that comes from the k, v and T tiles of chunk c is in registers
+    dtot *= dec;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) {  // S <- dec S + K^T (dk v_new)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[km][r] *= dec;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(fk[km * 4 + ks], Vsb[ks], S[km]);
+    }
+    if constexpr (PASS_B) {
+      // batch: Q rows, P fragments, output factors
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+#pragma unroll
+      for (int f = 0; f < 6; ++f) ft[f] = frag_load(s_P, f, lane);
+      f32x4 qs[8];
+#pragma unroll
+      for (int t8 = 0; t8 < 8; ++t8) qs[t8] = *reinterpret_cast<const f32x4*>(&s_qs[8 * t8 + 4 * hh]);
+      lds_fence();
+      lds_barrier();  // C(c): the q and P operands of chunk c are in registers
+      // o = qs (Q S_old) + P v_new, packed to the output type two columns at a time: lanes 2j and 2j+1 swap one
+      // value of every adjacent row pair, so the even lane holds both columns of the even row and the odd lane
+      // both columns of the odd row. The slab goes to this wave's own part of the o tile and from there to HBM
+      // in 16-byte pieces.
+      const bool odd = ln & 1;
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm) {
+        f32x16 a1 = zero16(), a2 = zero16();
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], a1);
+#pragma unroll
+        for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(ft[2 * tm + ks], Vb[ks], a2);
+#pragma unroll
+        for (int pr = 0; pr < 8; ++pr) {
+          const int r0 = 2 * pr, r1 = r0 + 1;
+          const float x0 = qs[4 * tm + r0 / 4][r0 % 4] * a1[r0] + a2[r0];
+          const float x1 = qs[4 * tm + r1 / 4][r1 % 4] * a1[r1] + a2[r1];
+          const float keep = odd ? x1 : x0;
+          const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
+          typedef T T2 __attribute__((ext_vector_type(2)));
+          T2 pk;
+          pk[0] = GdrElem<T>::from_float(odd ? got : keep);
+          pk[1] = GdrElem<T>::from_float(odd ? keep : got);
+          const int row = 32 * tm + acc_row(r0, hh) + (odd ? 1 : 0);
+          *reinterpret_cast<T2*>(&s_o[row * SV + 32 * vslab + (ln & ~1)]) = pk;
+        }
+      }
+      lds_fence();
+      {
+        const int cu = uniform(c), tok0 = chunk_tok0[cu], len = chunk_len[cu];
+        T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
+        const int rs = HV * VT;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int piece = lane + 64 * j, row = piece >> 2, part = piece & 3;
+          const uint4 val = *reinterpret_cast<const uint4*>(&s_o[row * SV + 32 * vslab + 8 * part]);
+          if (row < len) *reinterpret_cast<uint4*>(ob + row * rs + 32 * vslab + 8 * part) = val;
+        }
+      }
+    }
+  }
+
+  // epilogue; the opaque zero keeps the compiler from computing all these addresses before the loop
+  int late = 0;
+  asm volatile("" : "+v"(late));
+  if constexpr (PASS_B) {
+    if (ht && (flags & SEG_LAST)) {
+      const int seq = pv.seg_seq[seg];
+      float* out = ht + ((size_t)seq * HV + hv) * KT * VT + late;
+#pragma unroll
+      for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[(32 * km + acc_row(r, hh)) * VT + col] = S[km][r];
+    }
+  } else if (is_m) {
+    // M = dtot I + M': M' as bf16 A-operand fragments (rows = state rows, contraction over the columns in
+    // accumulator slot order), element (row, col) -> fragment (row/32, col/16), lane 32*hh' + row%32, slot s
+    unsigned char* out = Mcomp + ((size_t)seg * HV + hv) * (KT * KT * 2) + late;
+    const int mcol = 32 * wave + ln, ks = mcol >> 4, c16 = mcol & 15;
+    const int hs = (c16 >> 2) & 1, slot = 4 * (c16 >> 3) + (c16 & 3);
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * km + acc_row(r, hh);
+        const float val = S[km][r] - (row == mcol ? dtot : 0.0f);
+        *reinterpret_cast<__bf16*>(out + ((size_t)((km * (KT / 16) + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) =
+            (__bf16)val;
+      }
+    if (wave == 0 && lane == 0) Dcomp[(size_t)seg * HV + hv] = dtot;
+  } else {
+    // N slab in accumulator order: tile (vslab, km), plane q (registers 4q..4q+3), lane -> 16 bytes
+    unsigned char* out = Ncomp + (((size_t)seg * HV + hv) * (VT / 32) + vslab) * (KT * 32 * 4) + late;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
+        reinterpret_cast<f32x4*>(out)[(km * 4 + q4) * 64 + lane] = t;
+      }
+  }
+}
+
+// ---- scan ---------------------------------------------------------------------------------------------------------
+// grid (VT/32, n_seq, HV), KT/32 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column
+// slab of the state; Sinit receives the state every segment starts from, as 32-column slabs in accumulator order
+// (the layout the output pass loads with 16-byte reads).
+// The composite pass stores M_p as d_p I + M'_p (d_p = the segment's total decay, exact in fp32) with M' in bf16
+// MFMA A-operand fragment order and N_p in accumulator order, so a step is
+//   S <- d S + N + M' S      (one MFMA per fragment; the state feeds the B operand straight from the accumulator).
+// The chain is serial in p, so nothing else may sit on it. Wave w owns rows 32w .. 32w+31 of the slab: it loads
+// only its own row tile of M' and N (DEPTH steps ahead, straight into registers in operand order: no staging) and
+// needs the other waves' rows of the state only as B operand: every wave publishes its two operand fragments in
+// LDS (double-buffered by step parity, one LDS-only barrier per step) and starts the step's MFMAs with its own
+// fragments while the others' are on their way.
+template <int KT, int VT, int DEPTH>
+__global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanView pv,
+                                                                 const unsigned char* __restrict__ Mcomp,
+                                                                 const unsigned char* __restrict__ Ncomp,
+                                                                 const float* __restrict__ Dcomp,
+                                                                 const float* __restrict__ h0,
+                                                                 float* __restrict__ Sinit, int HV, int n_segments) {
+  constexpr int NKS = KT / 16;
+  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
+  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
+  const int nsteps = nseg - 1;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int col = 32 * vn + ln;
+
+  f32x16 S = zero16();
+  if (h0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + col];
+  }
+
+  bf16x8 rm[DEPTH][NKS];
+  f32x4 rn[DEPTH][4];
+  float rd[DEPTH];
+  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+    const size_t sh = (size_t)(seg0 + p) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * N_BYTES);
+#pragma unroll
+    for (int j = 0; j < NKS; ++j) m[j] = M[(wave * NKS + (2 * wave + j) % NKS) * 64 + lane];  // own fragments first
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) n[q4] = N[(wave * 4 + q4) * 64 + lane];
+    d = Dcomp[sh];
+  };
+  // (every step issues the same loads, clamped at the end, so that the waits can leave younger loads in flight)
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
+
+  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+    {  // the state segment seg0 + p starts from; steps past the end write to the spare slot behind the last segment
+      const size_t slot = p <= nsteps ? (size_t)(seg0 + p) : (size_t)n_segments;
+      f32x4* si = reinterpret_cast<f32x4*>(Sinit + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        si[(wave * 4 + q4) * 64 + lane] = t;
+      }
+    }
+    const float dec = dd;
+    unsigned char* xbuf = s_x[p & 1];
+    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
+    frag_store(xbuf, 2 * wave + 0, lane, own0);
+    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    f32x16 acc;
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[4 * q4 + e], n[q4][e]);
+    acc = mfma32(m[0], own0, acc);
+    acc = mfma32(m[1], own1, acc);
+    lds_barrier();
+#pragma unroll
+    for (int j = 2; j < NKS; ++j) acc = mfma32(m[j], frag_load(xbuf, (2 * wave + j) % NKS, lane), acc);
+    S = acc;
+    issue(max(0, min(p + DEPTH, nsteps - 1)), m, n, dd);
+  };
+  // The step loops have NO early exit: they run in whole groups, and the steps past the last segment work on clamped
+  // operands and store to the spare slot. With a branch around a step the compiler can no longer count the loads in
+  // flight and waits for all of them at every step; and since it drains the queue at every loop header anyway (the
+  // ring registers are loaded in one iteration and used in the next), the main loop covers LONG groups of steps.
+  constexpr int LONG = 4 * DEPTH;
+  int p0 = 0;
+  for (; p0 + LONG <= nsteps + 1; p0 += LONG) {
+#pragma unroll
+    for (int u = 0; u < LONG; ++u) step(p0 + u, rm[u % DEPTH], rn[u % DEPTH], rd[u % DEPTH]);
+  }
+  for (; p0 <= nsteps; p0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) step(p0 + d, rm[d], rn[d], rd[d]);
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------
+// ---- two-level scan ------------------------------------------------------------------------------------------------
+// A long sequence has many segments and the scan above walks them one after the other (0.45 us per step, a chain of
+// dependent MFMA / LDS-exchange stages with 16 workgroups on the whole chip). With groups of G segments the serial
+// depth drops from n to about n / G + 2 G:
+//   GROUP  every group but the last of a sequence, in parallel: the composite of its G segments, i.e. the scan step
+//          applied to the KT + VT columns [P_M | P_N] starting from [I | 0]; written as a segment composite is
+//          (D = product of the decays, M' = P_M - D I as bf16 A-operand fragments, N = P_N in accumulator order);
+//   LEAF   every group in parallel: the workgroup of group j first walks the composites of groups 0 .. j-1 from the
+//          sequence's initial state (at most gmax - 1 redundant steps; a separate serial pass over the groups would
+//          cost a launch more), then its own segments, writing the state every segment starts from (what the
+//          single-level scan writes).
+// Same step code in both modes; loops are branch free with clamped operands and a spare store slot as above.
+enum { SCAN_GROUP = 1, SCAN_LEAF = 2 };
+#define GDR_SCAN_GROUP 8  // segments per group; a multiple of the ring depth
+
+template <int KT, int VT, int DEPTH, int MODE>
+__global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlanView pv,
+                                                                  const unsigned char* __restrict__ Msrc,
+                                                                  const unsigned char* __restrict__ Nsrc,
+                                                                  const float* __restrict__ Dsrc,
+                                                                  const float* __restrict__ h0,
+                                                                  float* __restrict__ dst, unsigned char* __restrict__ Mout,
+                                                                  unsigned char* __restrict__ Nout, float* __restrict__ Dout,
+                                                                  int HV, int spare_slot, int gmax) {
+  constexpr int G = GDR_SCAN_GROUP;
+  static_assert(G % DEPTH == 0, "a group must be a whole number of ring rounds");
+  constexpr int NKS = KT / 16;
+  constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  constexpr int NCB = MODE == SCAN_GROUP ? (KT + VT) / 32 : VT / 32;  // 32-column blocks per item of the grid
+  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
+  const int vn = blockIdx.x % NCB, j = blockIdx.x / NCB, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
+  const int ngroups = (nseg + G - 1) / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  // items = the maps this workgroup applies, slots = where it stores the running state before each of them
+  int item0, nsteps, slot0, lead = 0;  // lead: group-level maps walked before the workgroup's own items (LEAF)
+  if (MODE == SCAN_GROUP) {
+    if (j >= ngroups - 1) return;  // the composite of a sequence's last group is never needed
+    item0 = seg0 + j * G; nsteps = G - 1; slot0 = 0;
+  } else {
+    if (j >= ngroups) return;
+    item0 = seg0 + j * G; lead = j; nsteps = lead + min(G, nseg - j * G) - 1; slot0 = item0;
+  }
+  const int last = MODE == SCAN_GROUP ? nsteps : nsteps - 1;   // last map that is really applied (prefetches are clamped to it)
+  const bool is_pm = MODE == SCAN_GROUP && vn < KT / 32;       // a block of P_M: no additive term, starts from I
+  const int nblk = MODE == SCAN_GROUP ? max(vn - KT / 32, 0) : vn;  // 32-column block of N / of the state
+
+  f32x16 S = zero16();
+  if (MODE == SCAN_GROUP) {
+    if (is_pm) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[r] = (32 * wave + acc_row(r, hh) == 32 * vn + ln) ? 1.0f : 0.0f;
+    }
+  } else if (h0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + 32 * vn + ln];
+  }
+
+  bf16x8 rm[DEPTH][NKS];
+  f32x4 rn[DEPTH][4];
+  float rd[DEPTH];
+  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+    const bool top = MODE == SCAN_LEAF && p < lead;  // a group composite (read through the *out pointers)
+    const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mout : Msrc) + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>((top ? Nout : Nsrc) + (sh * (VT / 32) + nblk) * N_BYTES);
+#pragma unroll
+    for (int f = 0; f < NKS; ++f) m[f] = M[(wave * NKS + (2 * wave + f) % NKS) * 64 + lane];  // own fragments first
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) n[q4] = N[(wave * 4 + q4) * 64 + lane];
+    d = (top ? Dout : Dsrc)[sh];
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, last)), rm[d], rn[d], rd[d]);
+
+  float dprod = 1.0f;
+  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+    if (MODE != SCAN_GROUP) {
+      const size_t slot = (p >= lead && p <= nsteps) ? (size_t)(slot0 + (p - lead)) : (size_t)spare_slot;
+      f32x4* si = reinterpret_cast<f32x4*>(dst + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        si[(wave * 4 + q4) * 64 + lane] = t;
+      }
+    }
+    const float dec = dd;
+    dprod *= dec;
+    unsigned char* xbuf = s_x[p & 1];
+    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
+    frag_store(xbuf, 2 * wave + 0, lane, own0);
+    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    f32x16 acc;
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(dec, S[4 * q4 + e], is_pm ? 0.0f : n[q4][e]);
+    acc = mfma32(m[0], own0, acc);
+    acc = mfma32(m[1], own1, acc);
+    lds_barrier();
+#pragma unroll
+    for (int f = 2; f < NKS; ++f) acc = mfma32(m[f], frag_load(xbuf, (2 * wave + f) % NKS, lane), acc);
+    S = acc;
+    issue(max(0, min(p + DEPTH, last)), m, n, dd);
+  };
+  constexpr int LONG = 4 * DEPTH;
+  int p0 = 0;
+  if (MODE != SCAN_GROUP) {
+    for (; p0 + LONG <= nsteps + 1; p0 += LONG) {
+#pragma unroll
+      for (int u = 0; u < LONG; ++u) step(p0 + u, rm[u % DEPTH], rn[u % DEPTH], rd[u % DEPTH]);
+    }
+  }
+  for (; p0 <= nsteps; p0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) step(p0 + d, rm[d], rn[d], rd[d]);
+  }
+
+  if (MODE == SCAN_GROUP) {  // exactly G maps were applied (G is a multiple of DEPTH): store the composite
+    const size_t gh = (size_t)(seq * gmax + j) * HV + hv;
+    if (is_pm) {
+      unsigned char* out = Mout + gh * M_BYTES;
+      const int mcol = 32 * vn + ln, ks = mcol >> 4, c16 = mcol & 15;
+      const int hs = (c16 >> 2) & 1, slot = 4 * (c16 >> 3) + (c16 & 3);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * wave + acc_row(r, hh);
+        const float val = S[r] - (row == mcol ? dprod : 0.0f);
+        *reinterpret_cast<__bf16*>(out + ((size_t)((wave * NKS + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) = (__bf16)val;
+      }
+      if (vn == 0 && tid == 0) Dout[gh] = dprod;
+    } else {
+      f32x4* out = reinterpret_cast<f32x4*>(Nout + (gh * (VT / 32) + nblk) * N_BYTES);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = S[4 * q4 + e];
+        out[(wave * 4 + q4) * 64 + lane] = t;
+      }
+    }
+  }
+}
