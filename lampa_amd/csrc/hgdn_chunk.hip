@@ -1,0 +1,733 @@
+// Hierarchical (level-weighted) chunkwise gated-delta-rule forward on gfx950.
+//
+// Replaces chunk_h_gated_delta_rule -> hattention_kernel -> chunkwise_fwd (reference chengjiang123/Lampa,
+// models/hattention/gated_delta_rule_apis.py:21-91, kernel.py:338-374, chunkwise_hgdn.py:565-791), whose
+// specification is the token loop of recurrent.py:134-216: the sources s <= t of a target token t are split into
+// buckets ("levels": 0 = the token itself, otherwise 1 + the position of the highest bit in which t and s differ,
+// base.py:41-46), every bucket keeps a state of its own that the same gated-delta transition acts on, and
+//   o_t = sum_l lambda_t[l] q_t^T S_t^(l).
+//
+// With chunks of 64 tokens the levels 0..6 stay inside a chunk and level 7 + j collects the earlier chunks c' of the
+// sequence with highest differing chunk-index bit j. Per chunk (T, gamma, beta, rk, rq, P as in gdr_chunk_kernels.h):
+//   W   = T diag(beta e^{gamma} rk) K          (the state's share of v_new is -W S)
+//   Q~  = diag(scale e^{gamma} rq) Q - P W     (a state S entering the chunk adds Q~ S to the outputs)
+//   S'  = e^{gamma_last} S - K^T diag(e^{gamma_last - gamma} rk) (W S)
+//   N   = K^T diag(e^{gamma_last - gamma} rk) T diag(beta) V          (the chunk's own sources, at its end)
+//   o_intra = ((P T diag(beta)) . Lambda) V,   Lambda_ij = lambda_i[level(i, j)]
+// Kernels:
+//   prep   workgroup per (chunk, head), fully parallel: W, Q~ and K^T as MFMA operand fragments, the decay factors,
+//          the inter-chunk lambdas (transposed), N and o_intra go to HBM.
+//   walk   workgroup per (segment of chunks, head, 32 value columns): four "chain" waves hold up to three level
+//          states each in accumulator registers (level j -> wave j % 4) and walk the chunks: for every level whose
+//          chunk-index bit is set, o += lambda . (Q~ S), S <- S'; after the chunk the levels below the lowest clear
+//          bit and N are summed into that bit's level (the carry chain of a binary counter) through LDS. Two loader
+//          waves stage the chunks' operand records, add the chain waves' partial outputs to o_intra and store o.
+//   scan   (sequences cut into segments of 2^p chunks) the same walk over whole segments with the segment
+//          composites (M, N) of the plain rule: leaves every segment's entering level states.
+#include "gdr_chunk_kernels.h"
+
+#define HG_CW 4                  // chain waves
+#define HG_LPW 3                 // levels per chain wave
+#define HG_NLV (HG_CW * HG_LPW)  // inter-chunk levels: sequences of up to 2^12 chunks
+#define HG_INTRA 7               // levels 0..6 live inside a chunk
+
+// Record of one chunk and head for the walk kernel
+template <int KT>
+struct HgRec {
+  static constexpr int NKS = KT / 16;
+  static constexpr int WF = 0;                          // W fragments   [2][NKS] KiB
+  static constexpr int QF = WF + 2 * NKS * 1024;        // Q~ fragments  [2][NKS] KiB
+  static constexpr int KF = QF + 2 * NKS * 1024;        // K^T fragments [KT/32][4] KiB
+  static constexpr int DK = KF + (KT / 32) * 4 * 1024;  // e^{gamma_last - gamma_i} rk_i, fp32 [64]
+  static constexpr int LT = DK + 256;                   // lambda_i[7 + j], fp32 [HG_NLV][64]
+  static constexpr int MISC = LT + HG_NLV * 256;        // e^{gamma_last}
+  static constexpr int BYTES = MISC + 256;
+  static constexpr int PIECES = BYTES / 16;
+};
+
+// ---- prep ---------------------------------------------------------------------------------------------------------
+template <int KT, int VT>
+struct HgPrepSmem {
+  static constexpr int SK = KT + 8, SV = VT + 8, ST = 40, LMAX = HG_INTRA + HG_NLV + 1;
+  static constexpr int OFF_K = 0;
+  static constexpr int OFF_Q = OFF_K + 64 * SK * 2;
+  static constexpr int OFF_KB = OFF_Q + 64 * SK * 2;  // beta e^{gamma} rk k; later Q~
+  static constexpr int OFF_W = OFF_KB + 64 * SK * 2;
+  static constexpr int OFF_V = OFF_W + 64 * SK * 2;
+  static constexpr int OFF_VB = OFF_V + 64 * SV * 2;  // beta v
+  static constexpr int OFF_T = OFF_VB + 64 * SV * 2;
+  static constexpr int OFF_P = OFF_T + 3 * 32 * ST * 2;
+  static constexpr int OFF_PL = OFF_P + 6 * 1024;
+  static constexpr int OFF_LAM = OFF_PL + 6 * 1024;
+  static constexpr int OFF_F = OFF_LAM + LMAX * 64 * 4;  // gamma, beta, rk, qsc, qs, dk
+  static constexpr int BYTES = OFF_F + 6 * 64 * 4;
+};
+
+template <typename T, int KT, int VT>
+__global__ void __launch_bounds__(256)
+    hgdn_prep_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                     const float* __restrict__ lam, const int32_t* __restrict__ chunk_tok0,
+                     const int32_t* __restrict__ chunk_len, const unsigned char* __restrict__ tmat,
+                     unsigned char* __restrict__ wrec, float* __restrict__ Nc, float* __restrict__ Oi, int H, int HV,
+                     int L, float scale, int l2norm) {
+  using SM = HgPrepSmem<KT, VT>;
+  using REC = HgRec<KT>;
+  constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST, NKS = KT / 16;
+  extern __shared__ __align__(16) unsigned char smem[];
+  __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
+  __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
+  __bf16* s_kb = reinterpret_cast<__bf16*>(smem + SM::OFF_KB);
+  __bf16* s_qt = s_kb;
+  __bf16* s_w = reinterpret_cast<__bf16*>(smem + SM::OFF_W);
+  __bf16* s_v = reinterpret_cast<__bf16*>(smem + SM::OFF_V);
+  __bf16* s_vb = reinterpret_cast<__bf16*>(smem + SM::OFF_VB);
+  __bf16* s_t = reinterpret_cast<__bf16*>(smem + SM::OFF_T);
+  unsigned char* s_P = smem + SM::OFF_P;
+  unsigned char* s_PL = smem + SM::OFF_PL;
+  float* s_lam = reinterpret_cast<float*>(smem + SM::OFF_LAM);
+  float* s_gamma = reinterpret_cast<float*>(smem + SM::OFF_F);
+  float* s_beta = s_gamma + 64;
+  float* s_rk = s_gamma + 128;
+  float* s_qsc = s_gamma + 192;  // scale rq_i
+  float* s_qs = s_gamma + 256;   // scale e^{gamma_i} rq_i
+  float* s_dk = s_gamma + 320;   // e^{gamma_last - gamma_i} rk_i
+
+  const int chunk = blockIdx.x, hv = blockIdx.y;
+  const int h = hv / (HV / H);
+  const int tok0 = chunk_tok0[chunk], len = chunk_len[chunk];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const size_t ch = (size_t)chunk * HV + hv;
+  const unsigned char* rec_in = tmat + ch * REC_BYTES;
+  unsigned char* rec = wrec + ch * REC::BYTES;
+
+  {  // ---- stage the tiles: thread = (row, quarter of the row)
+    const int row = tid >> 2, part = tid & 3;
+    const bool live = row < len;
+    const int rr = min(row, len - 1);
+    constexpr int KU = KT / 32, VU = VT / 32;  // 16-byte pieces per thread
+    typename Raw8<T>::type rk_[KU], rq_[KU], rv_[VU], zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+    const T* kp = k + ((size_t)(tok0 + rr) * H + h) * KT + part * (KT / 4);
+    const T* qp = q + ((size_t)(tok0 + rr) * H + h) * KT + part * (KT / 4);
+    const T* vp = v + ((size_t)(tok0 + rr) * HV + hv) * VT + part * (VT / 4);
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * u);
+      rq_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(qp + 8 * u);
+    }
+#pragma unroll
+    for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vp + 8 * u);
+    const float* fact = reinterpret_cast<const float*>(rec_in + T_BYTES);
+    const float gv = fact[row], g_last = fact[63], bv = fact[64 + row];
+    {  // T blocks
+      const bf16x8* tp = reinterpret_cast<const bf16x8*>(rec_in);
+      for (int p = tid; p < 384; p += 256)
+        *reinterpret_cast<bf16x8*>(&s_t[((p >> 7) * 32 + ((p & 127) >> 2)) * ST + 8 * (p & 3)]) = tp[p];
+    }
+    const bool want_ss = l2norm != GDR_L2_NONE;
+    bf16x8 kb[KU], qb[KU];
+    float kss = 0.0f, qss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      kb[u] = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+      qb[u] = raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
+      *reinterpret_cast<bf16x8*>(&s_k[row * SK + part * (KT / 4) + 8 * u]) = kb[u];
+      *reinterpret_cast<bf16x8*>(&s_q[row * SK + part * (KT / 4) + 8 * u]) = qb[u];
+    }
+    kss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, kss);
+    kss += dpp_f32<GDR_DPP_QUAD_XOR2, 0xF>(0.0f, kss);
+    qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
+    qss += dpp_f32<GDR_DPP_QUAD_XOR2, 0xF>(0.0f, qss);
+    const float rk = l2_factor(kss, l2norm), rq = l2_factor(qss, l2norm);
+    const float eg = __builtin_amdgcn_exp2f(gv);
+    const float bek = bv * eg * rk;
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      bf16x8 t;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[e] = (__bf16)(bek * (float)kb[u][e]);
+      *reinterpret_cast<bf16x8*>(&s_kb[row * SK + part * (KT / 4) + 8 * u]) = t;
+    }
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      float unused = 0.0f;
+      const bf16x8 vb = raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
+      bf16x8 t;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[e] = (__bf16)(bv * (float)vb[e]);
+      *reinterpret_cast<bf16x8*>(&s_v[row * SV + part * (VT / 4) + 8 * u]) = vb;
+      *reinterpret_cast<bf16x8*>(&s_vb[row * SV + part * (VT / 4) + 8 * u]) = t;
+    }
+    if (part == 0) {
+      const float dk = __builtin_amdgcn_exp2f(g_last - gv) * rk;
+      s_gamma[row] = gv;
+      s_beta[row] = bv;
+      s_rk[row] = rk;
+      s_qsc[row] = scale * rq;
+      s_qs[row] = scale * eg * rq;
+      s_dk[row] = dk;
+      reinterpret_cast<float*>(rec + REC::DK)[row] = dk;
+      if (row == 0) reinterpret_cast<float*>(rec + REC::MISC)[0] = __builtin_amdgcn_exp2f(g_last);
+    }
+    // lambda, transposed: s_lam[level][row]; the inter-chunk levels also go to the record
+    float* lt = reinterpret_cast<float*>(rec + REC::LT);
+    for (int idx = tid; idx < 64 * L; idx += 256) {
+      const int r = idx / L, lvl = idx - r * L;
+      const float x = lam[((size_t)(tok0 + min(r, len - 1)) * HV + hv) * L + lvl];
+      if (lvl < SM::LMAX) s_lam[lvl * 64 + r] = x;
+      if (lvl >= HG_INTRA && lvl < HG_INTRA + HG_NLV) lt[(lvl - HG_INTRA) * 64 + r] = x;
+    }
+    for (int idx = tid; idx < HG_NLV * 64; idx += 256)
+      if (HG_INTRA + idx / 64 >= L) lt[idx] = 0.0f;
+  }
+  __syncthreads();
+
+  auto t_frag = [&](int tm, int ks) {  // A operand of T: rows 32 tm + ln, contraction step ks (tokens 16 ks ..)
+    const int blk = tm == 0 ? 0 : (ks < 2 ? 1 : 2);
+    return ld_kappa(s_t + blk * 32 * ST, ST, ln, 16 * (ks & 1), hh);
+  };
+  auto w_tile = [&](int tm, int ct) {  // W rows 32 tm .., columns 32 ct ..
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+      if (ks < 2 * (tm + 1)) acc = mfma32(t_frag(tm, ks), ld_kappa_tr(s_kb, SK, 32 * ct, 16 * ks, lane), acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_w[(32 * tm + acc_row(r, hh)) * SK + 32 * ct + ln] = (__bf16)acc[r];
+  };
+  auto p_tile = [&](int t) {  // P^T tile: rows j (k tile jm), columns i (q tile tn) -> P fragments
+    const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      acc = mfma32(*reinterpret_cast<const bf16x8*>(&s_k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]),
+                   *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]), acc);
+    const int i = 32 * tn + ln;
+    const float gi = s_gamma[i], fi = s_qsc[i];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 32 * jm + acc_row(r, hh);
+      acc[r] *= fi * s_rk[j] * __builtin_amdgcn_exp2f(i >= j ? gi - s_gamma[j] : -1e30f);
+    }
+    const int f0 = tn == 0 ? 0 : 2 + 2 * jm;
+    frag_store(s_P, f0, lane, acc_to_operand(acc, 0));
+    frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
+  };
+  auto un_tile = [&](int vt) {  // U = T (beta v) for 32 value columns, then N = K^T (dk U)
+    bf16x8 Ub[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        if (ks < 2 * (tm + 1)) acc = mfma32(t_frag(tm, ks), ld_kappa_tr(s_vb, SV, 32 * vt, 16 * ks, lane), acc);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] *= s_dk[32 * tm + acc_row(r, hh)];
+      Ub[2 * tm] = acc_to_operand(acc, 0);
+      Ub[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    f32x4* out = reinterpret_cast<f32x4*>(Nc + (ch * (VT / 32) + vt) * (KT * 32));
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) {
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) acc = mfma32(ld_kappa_tr(s_k, SK, 32 * km, 16 * ks, lane), Ub[ks], acc);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = acc[4 * q4 + e];
+        out[(km * 4 + q4) * 64 + lane] = t;
+      }
+    }
+  };
+  // ---- W, P, the chunk's own state N, the K^T fragments (tasks spread over the four waves)
+  constexpr int NW = 2 * (KT / 32), NU = VT / 32, NKF = (KT / 32) * 4;
+  for (int task = wave; task < NW + 3 + NU + NKF; task += 4) {
+    if (task < NW) w_tile(task / (KT / 32), task % (KT / 32));
+    else if (task < NW + 3) p_tile(task - NW);
+    else if (task < NW + 3 + NU) un_tile(task - NW - 3);
+    else {
+      const int f = task - NW - 3 - NU;
+      frag_store(rec + REC::KF, f, lane, ld_kappa_tr(s_k, SK, 32 * (f / 4), 16 * (f % 4), lane));
+    }
+  }
+  __syncthreads();
+
+  auto q_tile = [&](int tm, int ct) {  // Q~ = qs Q - P W
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+      if (ks < 2 * (tm + 1))
+        acc = mfma32(frag_load(s_P, 2 * tm + ks, lane), ld_kappa_tr(s_w, SK, 32 * ct, 16 * ks, lane), acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 32 * tm + acc_row(r, hh);
+      s_qt[row * SK + 32 * ct + ln] = (__bf16)(s_qs[row] * (float)s_q[row * SK + 32 * ct + ln] - acc[r]);
+    }
+  };
+  auto a_tile = [&](int t) {  // ((P T diag(beta)) . Lambda)^T tile: rows j' (tile tj), columns i (tile ti)
+    const int tj = t == 2 ? 1 : 0, ti = t == 0 ? 0 : 1;
+    f32x16 acc = zero16();
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks / 2 < tj || ks / 2 > ti) continue;  // T[j][j'] = 0 for j < j', P[i][j] = 0 for j > i
+      const int blk = ks < 2 ? 0 : (tj == 0 ? 1 : 2);
+      acc = mfma32(ld_kappa_tr(s_t + blk * 32 * ST, ST, 0, 16 * (ks & 1), lane), frag_load(s_P, 2 * ti + ks, lane), acc);
+    }
+    const int i = 32 * ti + ln;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 32 * tj + acc_row(r, hh);
+      const int lvl = i == j ? 0 : 32 - __builtin_clz(i ^ j);
+      acc[r] = j <= i ? acc[r] * s_beta[j] * s_lam[lvl * 64 + i] : 0.0f;
+    }
+    const int f0 = ti == 0 ? 0 : 2 + 2 * tj;
+    frag_store(s_PL, f0, lane, acc_to_operand(acc, 0));
+    frag_store(s_PL, f0 + 1, lane, acc_to_operand(acc, 8));
+  };
+  for (int task = wave; task < NW + 3; task += 4) {
+    if (task < NW) q_tile(task / (KT / 32), task % (KT / 32));
+    else a_tile(task - NW);
+  }
+  __syncthreads();
+
+  // ---- o_intra and the W / Q~ fragments
+  for (int task = wave; task < 2 * NU + 4 * NKS; task += 4) {
+    if (task < 2 * NU) {
+      const int tm = task / NU, vt = task % NU;
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        if (ks < 2 * (tm + 1))
+          acc = mfma32(frag_load(s_PL, 2 * tm + ks, lane), ld_kappa_tr(s_v, SV, 32 * vt, 16 * ks, lane), acc);
+      float* out = Oi + ch * (64 * VT) + 32 * vt + ln;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) out[(32 * tm + acc_row(r, hh)) * VT] = acc[r];
+    } else {
+      const int f = task - 2 * NU, which = f / (2 * NKS), g = f % (2 * NKS);  // fragment (tm, ks) = (g / NKS, g % NKS)
+      const bf16x8 fr = ld_kappa(which == 0 ? s_w : s_qt, SK, 32 * (g / NKS) + ln, 16 * (g % NKS), hh);
+      frag_store(rec + (which == 0 ? REC::WF : REC::QF), g, lane, fr);
+    }
+  }
+}
+
+// ---- walk ---------------------------------------------------------------------------------------------------------
+template <int KT>
+struct HgWalkSmem {
+  static constexpr int SP = 36;  // row stride of a partial output tile (fp32)
+  static constexpr int OFF_REC = 0;
+  static constexpr int OFF_PART = 2 * HgRec<KT>::BYTES;
+  static constexpr int OFF_ACC = OFF_PART + HG_CW * 64 * SP * 4;
+  static constexpr int BYTES = OFF_ACC + KT * 32 * 4;
+};
+
+// accumulator-order slab (KT x 32 fp32) <-> registers
+template <int KT>
+__device__ __forceinline__ void slab_load(const float* p, int lane, f32x16* S) {
+  const f32x4* s = reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 t = s[(km * 4 + q4) * 64 + lane];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) S[km][4 * q4 + e] = t[e];
+    }
+}
+template <int KT>
+__device__ __forceinline__ void slab_store(float* p, int lane, const f32x16* S) {
+  f32x4* s = reinterpret_cast<f32x4*>(p);
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f32x4 t;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) t[e] = S[km][4 * q4 + e];
+      s[(km * 4 + q4) * 64 + lane] = t;
+    }
+}
+template <int KT>
+__device__ __forceinline__ void slab_add(float* p, int lane, const f32x16* S) {
+  f32x4* s = reinterpret_cast<f32x4*>(p);
+#pragma unroll
+  for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f32x4 t = s[(km * 4 + q4) * 64 + lane];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) t[e] += S[km][4 * q4 + e];
+      s[(km * 4 + q4) * 64 + lane] = t;
+    }
+}
+
+// The carry chain after chunk cs (index in its sequence): the levels below the lowest clear bit z of cs are all
+// occupied; they and the new state already in s_acc are summed, in level order, and become level z. One barrier
+// per level (uniform over the workgroup); a wave that owns none of the levels only takes part in the barriers.
+template <int KT>
+__device__ __forceinline__ void hg_merge(int cs, int lvl0, int wave, bool chain, int lane, float* s_acc,
+                                         f32x16 (*S)[KT / 32]) {
+  const int z = __builtin_ctz(~cs);
+  for (int j = lvl0; j < z; ++j) {
+    if (chain) {
+#pragma unroll
+      for (int slot = 0; slot < HG_LPW; ++slot)
+        if (slot * HG_CW + wave == j) {
+          slab_add<KT>(s_acc, lane, S[slot]);
+#pragma unroll
+          for (int km = 0; km < KT / 32; ++km) S[slot][km] = zero16();
+        }
+    }
+    lds_barrier();
+  }
+  if (chain) {
+#pragma unroll
+    for (int slot = 0; slot < HG_LPW; ++slot)
+      if (slot * HG_CW + wave == z) slab_load<KT>(s_acc, lane, S[slot]);
+  }
+}
+
+template <typename T, int KT, int VT>
+__global__ void __launch_bounds__(64 * (HG_CW + 2))
+    hgdn_walk_kernel(const GdrPlanView pv, const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
+                     const unsigned char* __restrict__ wrec, const float* __restrict__ Nc,
+                     const float* __restrict__ Oi, const float* __restrict__ Xinit, T* __restrict__ o, int HV) {
+  using REC = HgRec<KT>;
+  using SM = HgWalkSmem<KT>;
+  constexpr int NKS = KT / 16, SP = SM::SP;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_part = reinterpret_cast<float*>(smem + SM::OFF_PART);
+  float* s_acc = reinterpret_cast<float*>(smem + SM::OFF_ACC);
+
+  const int seg = blockIdx.x, hv = blockIdx.y, vslab = blockIdx.z;
+  const int c0 = pv.seg_chunk0[seg], nc = pv.seg_nchunks[seg], c1 = c0 + nc;
+  if (nc <= 0) return;
+  const int cs0 = c0 - pv.seg_chunk0[pv.seq_seg0[pv.seg_seq[seg]]];  // index of the first chunk in its sequence
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+
+  if (wave >= HG_CW) {
+    // ================================================ loader ================================================
+    const int ltid = tid - 64 * HG_CW;
+    constexpr int NP = (REC::PIECES + 127) / 128;
+    const int row = ltid >> 1, half = ltid & 1;
+    uint4 recA[NP], recB[NP];
+    f32x4 nA[KT / 16], nB[KT / 16], oA[4], oB[4];  // N slab: KT * 32 * 4 bytes = KT * 8 pieces over 128 threads
+    auto load_rec = [&](int c, uint4* r) {
+      const uint4* src = reinterpret_cast<const uint4*>(wrec + ((size_t)uniform(c) * HV + hv) * REC::BYTES);
+#pragma unroll
+      for (int j = 0; j < NP; ++j) r[j] = src[min(ltid + 128 * j, REC::PIECES - 1)];
+    };
+    auto store_rec = [&](int par, const uint4* r) {
+      uint4* dst = reinterpret_cast<uint4*>(smem + SM::OFF_REC + par * REC::BYTES);
+#pragma unroll
+      for (int j = 0; j < NP; ++j)
+        if (ltid + 128 * j < REC::PIECES) dst[ltid + 128 * j] = r[j];
+    };
+    auto load_no = [&](int c, f32x4* n, f32x4* oo) {
+      const size_t ch = (size_t)uniform(c) * HV + hv;
+      const f32x4* ns = reinterpret_cast<const f32x4*>(Nc + (ch * (VT / 32) + vslab) * (KT * 32));
+#pragma unroll
+      for (int j = 0; j < KT / 16; ++j) n[j] = ns[ltid + 128 * j];
+      const f32x4* os = reinterpret_cast<const f32x4*>(Oi + ch * (64 * VT) + row * VT + 32 * vslab + 16 * half);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) oo[e] = os[e];
+    };
+    load_rec(c0, recA);
+    store_rec(0, recA);
+    const int cl = c1 - 1;
+    load_rec(min(c0 + 1, cl), recA);
+    load_no(c0, nA, oA);
+    auto one_chunk = [&](int c, uint4* rHeld, f32x4* nHeld, f32x4* oHeld, uint4* rNext, f32x4* nNext, f32x4* oNext) {
+      lds_barrier();  // T(c): record (c) is staged; record buffer (c+1)&1, s_acc and the partial tiles are free
+      store_rec((c - c0 + 1) & 1, rHeld);
+#pragma unroll
+      for (int j = 0; j < KT / 16; ++j) reinterpret_cast<f32x4*>(s_acc)[ltid + 128 * j] = nHeld[j];
+      load_rec(min(c + 2, cl), rNext);
+      load_no(min(c + 1, cl), nNext, oNext);
+      lds_barrier();  // M0(c): the chain waves' partial tiles are complete
+      {
+        const int cu = uniform(c), tok0 = chunk_tok0[cu], len = chunk_len[cu];
+        float x[16];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          f32x4 a = oHeld[e];
+#pragma unroll
+          for (int w = 0; w < HG_CW; ++w) {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(&s_part[w * 64 * SP + row * SP + 16 * half + 4 * e]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] += t[i];
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[4 * e + i] = a[i];
+        }
+        typedef T T8 __attribute__((ext_vector_type(8)));
+        T8 lo, hi;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { lo[i] = GdrElem<T>::from_float(x[i]); hi[i] = GdrElem<T>::from_float(x[8 + i]); }
+        if (row < len) {
+          T* op = o + ((size_t)(tok0 + row) * HV + hv) * VT + 32 * vslab + 16 * half;
+          *reinterpret_cast<T8*>(op) = lo;
+          *reinterpret_cast<T8*>(op + 8) = hi;
+        }
+      }
+      if (c + 1 < c1) hg_merge<KT>(cs0 + (c - c0), 0, wave, false, lane, s_acc, nullptr);
+    };
+    for (int c = c0; c < c1; c += 2) {
+      one_chunk(c, recA, nA, oA, recB, nB, oB);
+      if (c + 1 < c1) one_chunk(c + 1, recB, nB, oB, recA, nA, oA);
+    }
+    return;
+  }
+
+  // ================================================== chain ==================================================
+  f32x16 S[HG_LPW][KT / 32];
+#pragma unroll
+  for (int slot = 0; slot < HG_LPW; ++slot) {
+    const int lvl = slot * HG_CW + wave;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) S[slot][km] = zero16();
+    if (Xinit && ((cs0 >> lvl) & 1))
+      slab_load<KT>(Xinit + ((((size_t)seg * HG_NLV + lvl) * HV + hv) * (VT / 32) + vslab) * (KT * 32), lane, S[slot]);
+  }
+  for (int c = c0; c < c1; ++c) {
+    const int cs = cs0 + (c - c0);
+    lds_barrier();  // T(c)
+    const unsigned char* rec = smem + SM::OFF_REC + ((c - c0) & 1) * REC::BYTES;
+    const float* s_dk = reinterpret_cast<const float*>(rec + REC::DK);
+    const float* s_lt = reinterpret_cast<const float*>(rec + REC::LT);
+    const float dec = reinterpret_cast<const float*>(rec + REC::MISC)[0];
+    f32x16 O[2] = {zero16(), zero16()};
+#pragma unroll
+    for (int slot = 0; slot < HG_LPW; ++slot) {
+      const int lvl = slot * HG_CW + wave;
+      if (!((cs >> lvl) & 1)) continue;
+      bf16x8 Sb[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_operand(S[slot][ks / 2], 8 * (ks % 2));
+      bf16x8 Zb[4];
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm) {
+        f32x16 z = zero16(), a = zero16();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) z = mfma32(frag_load(rec + REC::WF, tm * NKS + ks, lane), Sb[ks], z);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) a = mfma32(frag_load(rec + REC::QF, tm * NKS + ks, lane), Sb[ks], a);
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const f32x4 dk = *reinterpret_cast<const f32x4*>(&s_dk[32 * tm + 8 * b4 + 4 * hh]);
+          const f32x4 lm = *reinterpret_cast<const f32x4*>(&s_lt[lvl * 64 + 32 * tm + 8 * b4 + 4 * hh]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            z[4 * b4 + e] *= -dk[e];
+            O[tm][4 * b4 + e] = __builtin_fmaf(lm[e], a[4 * b4 + e], O[tm][4 * b4 + e]);
+          }
+        }
+        Zb[2 * tm] = acc_to_operand(z, 0);
+        Zb[2 * tm + 1] = acc_to_operand(z, 8);
+      }
+#pragma unroll
+      for (int km = 0; km < KT / 32; ++km) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[slot][km][r] *= dec;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) S[slot][km] = mfma32(frag_load(rec + REC::KF, km * 4 + ks, lane), Zb[ks], S[slot][km]);
+      }
+    }
+    {
+      float* part = s_part + wave * 64 * SP;
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[(32 * tm + acc_row(r, hh)) * SP + ln] = O[tm][r];
+    }
+    lds_barrier();  // M0(c)
+    if (c + 1 < c1) hg_merge<KT>(cs, 0, wave, true, lane, s_acc, S);
+  }
+}
+
+// ---- scan over the segments --------------------------------------------------------------------------------------
+// grid (VT/32, n_seq, HV), HG_CW waves. Segments hold G = 2^p chunks, so at a segment's first chunk only levels >= p
+// can be occupied; they are carried from segment to segment with the segment's composite map of the plain rule
+// (S -> d S + M' S; its N is the sum of everything the segment's own chunks contribute) and merged by the same carry
+// chain. Xinit[seg][level] receives every occupied level's state at the segment's first chunk.
+template <int KT, int VT>
+__global__ void __launch_bounds__(64 * HG_CW)
+    hgdn_scan_kernel(const GdrPlanView pv, const unsigned char* __restrict__ Mcomp, const unsigned char* __restrict__ Ncomp,
+                     const float* __restrict__ Dcomp, float* __restrict__ Xinit, int HV, int p) {
+  constexpr int NKS = KT / 16, M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+  __shared__ __align__(16) float s_acc[KT * 32];
+  const int vslab = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  f32x16 S[HG_LPW][KT / 32];
+#pragma unroll
+  for (int slot = 0; slot < HG_LPW; ++slot)
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) S[slot][km] = zero16();
+  for (int i = 0; i < nseg; ++i) {
+    const int seg = seg0 + i, cs = i << p;
+#pragma unroll
+    for (int slot = 0; slot < HG_LPW; ++slot) {
+      const int lvl = slot * HG_CW + wave;
+      if ((cs >> lvl) & 1)
+        slab_store<KT>(Xinit + ((((size_t)seg * HG_NLV + lvl) * HV + hv) * (VT / 32) + vslab) * (KT * 32), lane, S[slot]);
+    }
+    if (i == nseg - 1) break;
+    const size_t sh = (size_t)seg * HV + hv;
+    const float d = Dcomp[sh];
+    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+#pragma unroll
+    for (int slot = 0; slot < HG_LPW; ++slot) {
+      const int lvl = slot * HG_CW + wave;
+      if (!((cs >> lvl) & 1)) continue;
+      bf16x8 Sb[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_operand(S[slot][ks / 2], 8 * (ks % 2));
+#pragma unroll
+      for (int km = 0; km < KT / 32; ++km) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[slot][km][r] *= d;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) S[slot][km] = mfma32(M[(km * NKS + ks) * 64 + lane], Sb[ks], S[slot][km]);
+      }
+    }
+    lds_barrier();  // the level that took the last carry has read s_acc
+    {
+      const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vslab) * N_BYTES);
+      for (int j = tid; j < KT * 8; j += 64 * HG_CW) reinterpret_cast<f32x4*>(s_acc)[j] = N[j];
+    }
+    lds_barrier();
+    hg_merge<KT>(cs + (1 << p) - 1, p, wave, true, lane, s_acc, S);
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------
+struct HgWorkspace {
+  int64_t off_t, off_m, off_n, off_d, off_rec, off_nc, off_oi, off_x, bytes;
+};
+
+static HgWorkspace hg_workspace(int64_t chunks, int64_t segs, int HV, int K, int V) {
+  HgWorkspace w;
+  const int64_t rec_bytes = K == 64 ? HgRec<64>::BYTES : HgRec<128>::BYTES;
+  int64_t off = 0;
+  w.off_t = off;   off += lampa_align_up(chunks * HV * (int64_t)REC_BYTES, 256);
+  w.off_m = off;   off += lampa_align_up(segs * HV * (int64_t)K * K * 2, 256);
+  w.off_n = off;   off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
+  w.off_d = off;   off += lampa_align_up(segs * HV * 4, 256);
+  w.off_rec = off; off += lampa_align_up(chunks * HV * rec_bytes, 256);
+  w.off_nc = off;  off += lampa_align_up(chunks * HV * (int64_t)K * V * 4, 256);
+  w.off_oi = off;  off += lampa_align_up(chunks * HV * (int64_t)64 * V * 4, 256);
+  w.off_x = off;   off += lampa_align_up(segs * HG_NLV * HV * (int64_t)K * V * 4, 256);
+  w.bytes = off > 0 ? off : 256;
+  return w;
+}
+
+static bool hg_supported(int K, int V) { return K == 64 && (V == 64 || V == 128); }
+
+extern "C" int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V) {
+  if (total_chunks < 0 || n_segments < 0 || HV < 1) return LAMPA_ERR_INVALID;
+  if (!hg_supported(K, V)) return LAMPA_ERR_UNSUPPORTED;
+  return hg_workspace(total_chunks, n_segments, HV, K, V).bytes;
+}
+
+template <typename T, int KT, int VT>
+static int hg_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* lam,
+                     void* o, const GdrPlanView pv, int n_seq, int chunks, int segs, int p, int H, int HV, int L,
+                     float scale, int l2norm, unsigned char* ws, hipStream_t s) {
+  const HgWorkspace w = hg_workspace(chunks, segs, HV, KT, VT);
+  unsigned char* tf = ws + w.off_t;
+  unsigned char* Mc = ws + w.off_m;
+  unsigned char* Nm = ws + w.off_n;
+  float* Dc = (float*)(ws + w.off_d);
+  unsigned char* rec = ws + w.off_rec;
+  float* Nc = (float*)(ws + w.off_nc);
+  float* Oi = (float*)(ws + w.off_oi);
+  float* Xi = (float*)(ws + w.off_x);
+  constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_p = HgPrepSmem<KT, VT>::BYTES,
+                smem_w = HgWalkSmem<KT>::BYTES;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
+        hipFuncSetAttribute((const void*)hgdn_prep_kernel<T, KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            smem_p) != hipSuccess ||
+        hipFuncSetAttribute((const void*)hgdn_walk_kernel<T, KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            smem_w) != hipSuccess)
+      return LAMPA_ERR_LAUNCH;
+    attr_set = true;
+  }
+  LAMPA_PROF(s, "start");
+  if (chunks == 0) return LAMPA_OK;
+  hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv, tf, H, HV,
+                     l2norm);
+  LAMPA_PROF(s, "gdr_tinv_kernel");
+  hipLaunchKernelGGL((hgdn_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem_p, s, (const T*)q, (const T*)k,
+                     (const T*)v, lam, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, H, HV, L, scale, l2norm);
+  LAMPA_PROF(s, "hgdn_prep_kernel");
+  const bool split = segs > n_seq;
+  if (split) {
+    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV),
+                       dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s, (const T*)q, (const T*)k, (const T*)v, g,
+                       beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nm, Dc, (T*)nullptr,
+                       (float*)nullptr, H, HV, scale, l2norm);
+    LAMPA_PROF(s, "gdr_segment_kernel<composite>");
+    hipLaunchKernelGGL((hgdn_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64 * HG_CW), 0, s, pv, Mc, Nm, Dc, Xi,
+                       HV, p);
+    LAMPA_PROF(s, "hgdn_scan_kernel");
+  }
+  hipLaunchKernelGGL((hgdn_walk_kernel<T, KT, VT>), dim3(segs, HV, VT / 32), dim3(64 * (HG_CW + 2)), smem_w, s, pv,
+                     pv.chunk_tok0, pv.chunk_len, rec, Nc, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
+                     HV);
+  LAMPA_PROF(s, "hgdn_walk_kernel");
+  return lampa_launch_status();
+}
+
+// Hierarchical chunkwise forward. q, k [total_tokens, H, K]; v, o [total_tokens, HV, V] (dtype 0 bf16 / 1 fp16);
+// g, beta fp32 [total_tokens, HV]; lam fp32 [total_tokens, HV, L] (level weights as they enter the kernel: the
+// caller has divided them by `scale`, which multiplies q). The plan's chunks_per_segment must be a power of two
+// (or at least the longest sequence's chunk count: one segment per sequence); every sequence may hold at most
+// 2^12 chunks and L must cover 7 + the number of chunk-index bits of the longest sequence.
+extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                    const float* lam, void* o, const int32_t* plan_host, const int32_t* plan_dev,
+                                    int H, int HV, int K, int V, int L, int dtype, float scale, int l2norm,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!q || !k || !v || !g || !beta || !lam || !o || !plan_host || !plan_dev) return LAMPA_ERR_INVALID;
+  if (H < 1 || HV < H || HV % H != 0 || l2norm < 0 || l2norm > 2 || L < HG_INTRA) return LAMPA_ERR_INVALID;
+  if (!hg_supported(K, V) || (dtype != GDR_BF16 && dtype != GDR_FP16)) return LAMPA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) return LAMPA_ERR_INVALID;
+  const int n_seq = plan_host[PLAN_N_SEQ], chunks = plan_host[PLAN_TOTAL_CHUNKS], segs = plan_host[PLAN_N_SEGMENTS];
+  const int cps = plan_host[PLAN_CHUNKS_PER_SEGMENT];
+  if (n_seq < 1 || segs < n_seq) return LAMPA_ERR_INVALID;
+  int p = 0;
+  if (segs > n_seq) {
+    if (cps & (cps - 1)) return LAMPA_ERR_INVALID;
+    while ((1 << p) < cps) ++p;
+  }
+  int max_nc = 0;
+  for (int i = 0; i < n_seq; ++i) {
+    const int s0 = plan_host[plan_host[PLAN_OFF_SEQ_SEG0] + i], ns = plan_host[plan_host[PLAN_OFF_SEQ_NSEG] + i];
+    int nc = 0;
+    for (int j = 0; j < ns; ++j) nc += plan_host[plan_host[PLAN_OFF_SEG_NCHUNKS] + s0 + j];
+    max_nc = nc > max_nc ? nc : max_nc;
+  }
+  if (max_nc > (1 << HG_NLV)) return LAMPA_ERR_UNSUPPORTED;
+  int bits = 0;
+  while ((1 << bits) < max_nc) ++bits;
+  if (HG_INTRA + bits > L) return LAMPA_ERR_INVALID;
+  if (!workspace || workspace_bytes < hg_workspace(chunks, segs, HV, K, V).bytes) return LAMPA_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  unsigned char* ws = (unsigned char*)workspace;
+  const GdrPlanView pv = gdr_plan_view(plan_host, plan_dev);
+#define HG_CASE(TT, KK, VV) \
+  return hg_launch<TT, KK, VV>(q, k, v, g, beta, lam, o, pv, n_seq, chunks, segs, p, H, HV, L, scale, l2norm, ws, s)
+  if (dtype == GDR_BF16) {
+    if (V == 64) HG_CASE(__bf16, 64, 64);
+    if (V == 128) HG_CASE(__bf16, 64, 128);
+  } else {
+    if (V == 64) HG_CASE(_Float16, 64, 64);
+    if (V == 128) HG_CASE(_Float16, 64, 128);
+  }
+#undef HG_CASE
+  return LAMPA_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,109 @@
+"""GPU parity of the hierarchical gated-delta forward against the CPU oracle (fp64 token loop with level states).
+
+Tolerances as for the plain chunk forward: bf16 / fp16 inputs with fp32 accumulation -- max-abs 2e-2 and
+mean-relative 5e-3 on the outputs.
+"""
+import pytest
+import torch
+
+from lampa_amd import gated_delta as gd
+from lampa_amd import hgdn
+from lampa_amd import synth
+from oracle import hgdn as oh
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_REL = 2e-2, 5e-3
+
+
+def _errors(got, want):
+    got, want = got.detach().float().cpu(), want.float()
+    diff = (got - want).abs()
+    return diff.max().item(), (diff.mean() / want.abs().mean().clamp_min(1e-12)).item()
+
+
+def _inputs(B, T, H, K, V, dtype, seed, HV=None, g_scale=1.0, L=None):
+    q, k, v, g, beta = synth.gdr_inputs(B, T, H, K, V, dtype, seed, g_scale)
+    gen = torch.Generator().manual_seed(seed + 11)
+    if HV is not None and HV != H:
+        v = torch.randn(B, T, HV, V, generator=gen).to(dtype)
+        beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
+        g = -g_scale * torch.nn.functional.softplus(torch.randn(B, T, HV, generator=gen))
+    L = L or hgdn.num_levels(T)
+    lam = (torch.rand(B, T, v.shape[2], L, generator=gen) + 0.25).to(dtype)
+    return q, k, v, g, beta, lam
+
+
+def _run(device, q, k, v, g, beta, lam, cps=None):
+    old = hgdn.CHUNKS_PER_SEGMENT
+    hgdn.CHUNKS_PER_SEGMENT = cps
+    try:
+        o, state = hgdn.chunk_h_gated_delta_rule(*(x.to(device) for x in (q, k, v, g, lam, beta)),
+                                                 use_qk_l2norm_in_kernel=True)
+    finally:
+        hgdn.CHUNKS_PER_SEGMENT = old
+    assert state is None and o.dtype == v.dtype and o.shape == v.shape
+    return o
+
+
+def _want(q, k, v, g, beta, lam):
+    # what reaches the kernel of the reference: lambda / scale in lambda's dtype, q * scale
+    scale = q.shape[-1] ** -0.5
+    return oh.recurrent_c(q, k, v, g, beta, lam / scale, scale=scale)
+
+
+@pytest.mark.parametrize("T,cps", [(64, None), (256, None), (1024, None), (1024, 4), (4096, 8), (4096, 16), (2560, 8)])
+def test_matches_oracle(device, T, cps):
+    q, k, v, g, beta, lam = _inputs(1, T, 2, 64, 64, torch.bfloat16, seed=T)
+    o = _run(device, q, k, v, g, beta, lam, cps)
+    max_abs, mean_rel = _errors(o, _want(q, k, v, g, beta, lam))
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"T={T} cps={cps}: {max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_batch_grouped_heads_wide_values_fp16(device):
+    q, k, v, g, beta, lam = _inputs(2, 1536, 2, 64, 128, torch.float16, seed=5, HV=4, g_scale=0.3, L=14)
+    for cps in (None, 8):
+        o = _run(device, q, k, v, g, beta, lam, cps)
+        max_abs, mean_rel = _errors(o, _want(q, k, v, g, beta, lam))
+        assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"cps={cps}: {max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_unit_weights_equal_plain_chunk_forward(device):
+    # every level weighted by `scale` (lambda / scale = 1): the plain gated delta rule, at a size only the GPU walks
+    T = 60032
+    q, k, v, g, beta, _ = _inputs(1, T, 8, 64, 64, torch.bfloat16, seed=1, g_scale=0.1)
+    lam = torch.full((1, T, 8, hgdn.num_levels(T)), 1.0, dtype=torch.bfloat16)
+    o = _run(device, q, k, v, g, beta, lam)
+    ref, _ = gd.chunk_gated_delta_rule(*(x.to(device) for x in (q, k, v, g, beta)), scale=1.0,
+                                       use_qk_l2norm_in_kernel=True)
+    max_abs, mean_rel = _errors(o, ref.cpu())
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"{max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_levels_are_linear_at_full_size(device):
+    # o is linear in lambda: two disjoint level masks add up to the run with both
+    T = 16384
+    q, k, v, g, beta, lam = _inputs(1, T, 4, 64, 64, torch.bfloat16, seed=2, g_scale=0.1)
+    lam = lam.float()
+    low, high = lam.clone(), lam.clone()
+    low[..., 9:] = 0
+    high[..., :9] = 0
+    o_all = _run(device, q, k, v, g, beta, lam.bfloat16()).float()
+    o_sum = _run(device, q, k, v, g, beta, low.bfloat16()).float() + _run(device, q, k, v, g, beta, high.bfloat16()).float()
+    max_abs, mean_rel = _errors(o_sum, o_all.cpu())
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"{max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_argument_checks(device):
+    q, k, v, g, beta, lam = (x.to(device) for x in _inputs(1, 128, 2, 64, 64, torch.bfloat16, seed=0))
+    with pytest.raises(AssertionError):
+        hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta)  # the reference insists on the in-kernel l2norm
+    with pytest.raises(AssertionError):
+        hgdn.chunk_h_gated_delta_rule(q.float(), k.float(), v.float(), g, lam, beta, use_qk_l2norm_in_kernel=True)
+    with pytest.raises(ValueError):
+        hgdn.chunk_h_gated_delta_rule(q[:, :100], k[:, :100], v[:, :100], g[:, :100], lam[:, :100], beta[:, :100],
+                                      use_qk_l2norm_in_kernel=True)
+    with pytest.raises(ValueError):
+        hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam[..., :7], beta, use_qk_l2norm_in_kernel=True)
+    with pytest.raises(NotImplementedError):
+        hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, output_final_state=True, use_qk_l2norm_in_kernel=True)
