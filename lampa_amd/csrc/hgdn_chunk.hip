@@ -26,6 +26,8 @@
 //          composites (M, N) of the plain rule: leaves every segment's entering level states.
 #include "gdr_chunk_kernels.h"
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 #define HG_CW 4                  // chain waves
 #define HG_LPW 3                 // levels per chain wave
 #define HG_NLV (HG_CW * HG_LPW)  // inter-chunk levels: sequences of up to 2^12 chunks
@@ -95,7 +97,7 @@ __global__ void __launch_bounds__(256)
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
   const int tok0 = chunk_tok0[chunk], len = chunk_len[chunk];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   const size_t ch = (size_t)chunk * HV + hv;
   const unsigned char* rec_in = tmat + ch * REC_BYTES;
   unsigned char* rec = wrec + ch * REC::BYTES;
@@ -404,27 +406,27 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
   const int c0 = pv.seg_chunk0[seg], nc = pv.seg_nchunks[seg], c1 = c0 + nc;
   if (nc <= 0) return;
   const int cs0 = c0 - pv.seg_chunk0[pv.seq_seg0[pv.seg_seq[seg]]];  // index of the first chunk in its sequence
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63, hh = lane >> 5, ln = lane & 31;
 
   if (wave >= HG_CW) {
     // ================================================ loader ================================================
     const int ltid = tid - 64 * HG_CW;
     constexpr int NP = (REC::PIECES + 127) / 128;
     const int row = ltid >> 1, half = ltid & 1;
-    uint4 recA[NP], recB[NP];
+    u32x4 recA[NP], recB[NP];
     f32x4 nA[KT / 16], nB[KT / 16], oA[4], oB[4];  // N slab: KT * 32 * 4 bytes = KT * 8 pieces over 128 threads
-    auto load_rec = [&](int c, uint4* r) {
-      const uint4* src = reinterpret_cast<const uint4*>(wrec + ((size_t)uniform(c) * HV + hv) * REC::BYTES);
+    auto load_rec = [&](int c, u32x4* r) __attribute__((always_inline)) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(wrec + ((size_t)uniform(c) * HV + hv) * REC::BYTES);
 #pragma unroll
       for (int j = 0; j < NP; ++j) r[j] = src[min(ltid + 128 * j, REC::PIECES - 1)];
     };
-    auto store_rec = [&](int par, const uint4* r) {
-      uint4* dst = reinterpret_cast<uint4*>(smem + SM::OFF_REC + par * REC::BYTES);
+    auto store_rec = [&](int par, const u32x4* r) __attribute__((always_inline)) {
+      u32x4* dst = reinterpret_cast<u32x4*>(smem + SM::OFF_REC + par * REC::BYTES);
 #pragma unroll
       for (int j = 0; j < NP; ++j)
         if (ltid + 128 * j < REC::PIECES) dst[ltid + 128 * j] = r[j];
     };
-    auto load_no = [&](int c, f32x4* n, f32x4* oo) {
+    auto load_no = [&](int c, f32x4* n, f32x4* oo) __attribute__((always_inline)) {
       const size_t ch = (size_t)uniform(c) * HV + hv;
       const f32x4* ns = reinterpret_cast<const f32x4*>(Nc + (ch * (VT / 32) + vslab) * (KT * 32));
 #pragma unroll
@@ -438,7 +440,7 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
     const int cl = c1 - 1;
     load_rec(min(c0 + 1, cl), recA);
     load_no(c0, nA, oA);
-    auto one_chunk = [&](int c, uint4* rHeld, f32x4* nHeld, f32x4* oHeld, uint4* rNext, f32x4* nNext, f32x4* oNext) {
+    auto one_chunk = [&](int c, u32x4* rHeld, f32x4* nHeld, f32x4* oHeld, u32x4* rNext, f32x4* nNext, f32x4* oNext) __attribute__((always_inline)) {
       lds_barrier();  // T(c): record (c) is staged; record buffer (c+1)&1, s_acc and the partial tiles are free
       store_rec((c - c0 + 1) & 1, rHeld);
 #pragma unroll
@@ -559,7 +561,7 @@ __global__ void __launch_bounds__(64 * HG_CW)
   __shared__ __align__(16) float s_acc[KT * 32];
   const int vslab = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
   const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
   f32x16 S[HG_LPW][KT / 32];
 #pragma unroll
   for (int slot = 0; slot < HG_LPW; ++slot)
