@@ -5,8 +5,8 @@ A step is one chunkwise gated-delta layer forward (B=1, H=8, T=60000, d_k=d_v=64
 tokens in the LSH-sorted order of a 60000-hit event) with every input resident in HBM.
 Prints one JSON line: `value` = hits/s over the timed steps (wall clock), `roofline` = the slowest kernel of the layer
 against the HBM peak on its algorithmic bytes (duration from HIP events on the launch stream), `cpu_baseline` = the
-pure-PyTorch token loop on this box's host cores, `layer` / `lsh` / `block` = per-kernel times, the LSH stage on one
-event and on a batch, and the 4-layer block.
+pure-PyTorch token loop on this box's host cores, `layer` / `lsh` / `block` / `hgdn` = per-kernel times, the LSH stage on one
+event and on a batch, the 4-layer block, and the hierarchical (level-weighted) forward.
 """
 import argparse
 import json
@@ -255,6 +255,43 @@ def main():
     }
     del blk
 
+    # ---- hierarchical (level-weighted) forward on the config-2 shape padded to whole chunks ----
+    from lampa_amd import hgdn
+    T_H = (T + 63) // 64 * 64
+    pad = T_H - T
+    qh, kh, vh = (torch.nn.functional.pad(x, (0, 0, 0, 0, 0, pad)) for x in (qd, kd, vd))
+    gh, bh = (torch.nn.functional.pad(x, (0, 0, 0, pad)) for x in (gd_, bd))
+    L_H = hgdn.num_levels(T_H)
+    lam = (torch.rand(1, T_H, H, L_H, generator=torch.Generator().manual_seed(3)) + 0.25).to(torch.bfloat16).to(dev)
+    for _ in range(5):
+        hgdn.chunk_h_gated_delta_rule(qh, kh, vh, gh, lam, bh, use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        hgdn.chunk_h_gated_delta_rule(qh, kh, vh, gh, lam, bh, use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    hgdn_us = 1e6 * (time.perf_counter() - t0) / 20
+    _capi.profile_begin()
+    for _ in range(10):
+        hgdn.chunk_h_gated_delta_rule(qh, kh, vh, gh, lam, bh, use_qk_l2norm_in_kernel=True)
+    hstage = {}
+    for name, ms in _capi.profile_end(max_entries=512):
+        if name != "start":
+            hstage[name] = hstage.get(name, 0.0) + 1e3 * ms / 10
+    live = sum(bin(c).count("1") for c in range(T_H // 64)) * H  # (chunk, head, level) triples that hold a state
+    hgdn_flop = (T_H // 64) * H * 2 * 64 * 64 * (3 * K + 2 * V + 42) + live * 6 * 64 * K * V
+    hgdn_info = {
+        "workload": f"hierarchical gated-delta forward, B=1 H={H} T={T_H} K=V={K}, L={L_H} levels, bf16, weak "
+                    "hierarchy base 2",
+        "us": round(hgdn_us, 1), "hits_per_s": round(T / (hgdn_us * 1e-6), 1),
+        "kernel_us": {n: round(v_, 1) for n, v_ in hstage.items()},
+        "mfma_frac": round(hgdn_flop / (hgdn_us * 1e-6) / 2.5e15, 4),
+        "note": "includes the wrapper's lambda / scale and fp32 conversion of lambda; mfma_frac = algorithmic flops "
+                "(per chunk and head 2*64*64*(3K+2V+42) for the chunk-local products with triangular factors counted as such, 6*64*K*V per occupied level) "
+                "over the bf16 dense peak",
+    }
+    del qh, kh, vh, gh, bh, lam
+
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
     if not args.no_cpu:
@@ -275,7 +312,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info,
     }
     print(json.dumps(out))
 

@@ -61,7 +61,7 @@ struct HgPrepSmem {
   static constexpr int OFF_P = OFF_T + 3 * 32 * ST * 2;
   static constexpr int OFF_PL = OFF_P + 6 * 1024;
   static constexpr int OFF_LAM = OFF_PL + 6 * 1024;
-  static constexpr int OFF_F = OFF_LAM + LMAX * 64 * 4;  // gamma, beta, rk, qsc, qs, dk
+  static constexpr int OFF_F = OFF_LAM + HG_INTRA * 64 * 4;  // gamma, beta, rk, qsc, qs, dk
   static constexpr int BYTES = OFF_F + 6 * 64 * 4;
 };
 
@@ -122,10 +122,26 @@ __global__ void __launch_bounds__(256)
     for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vp + 8 * u);
     const float* fact = reinterpret_cast<const float*>(rec_in + T_BYTES);
     const float gv = fact[row], g_last = fact[63], bv = fact[64 + row];
-    {  // T blocks
+    // every global load of the stage is issued before the first use: T blocks and the lambda rows (at most
+    // LMAX levels: five values per thread), indices clamped instead of branches
+    constexpr int NLAM = (64 * SM::LMAX + 255) / 256;
+    const int Lc = min(L, SM::LMAX);
+    float lv[NLAM];
+    bf16x8 tp0, tp1;
+    {
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(rec_in);
-      for (int p = tid; p < 384; p += 256)
-        *reinterpret_cast<bf16x8*>(&s_t[((p >> 7) * 32 + ((p & 127) >> 2)) * ST + 8 * (p & 3)]) = tp[p];
+      tp0 = tp[tid];
+      tp1 = tp[256 + (tid & 127)];
+#pragma unroll
+      for (int j = 0; j < NLAM; ++j) {
+        const int idx = min(tid + 256 * j, 64 * Lc - 1), r = idx / Lc, lvl = idx - r * Lc;
+        lv[j] = lam[((size_t)(tok0 + min(r, len - 1)) * HV + hv) * L + lvl];
+      }
+    }
+    {
+      const int p0 = tid, p1 = 256 + tid;
+      *reinterpret_cast<bf16x8*>(&s_t[((p0 >> 7) * 32 + ((p0 & 127) >> 2)) * ST + 8 * (p0 & 3)]) = tp0;
+      if (tid < 128) *reinterpret_cast<bf16x8*>(&s_t[((p1 >> 7) * 32 + ((p1 & 127) >> 2)) * ST + 8 * (p1 & 3)]) = tp1;
     }
     const bool want_ss = l2norm != GDR_L2_NONE;
     bf16x8 kb[KU], qb[KU];
@@ -174,11 +190,13 @@ __global__ void __launch_bounds__(256)
     }
     // lambda, transposed: s_lam[level][row]; the inter-chunk levels also go to the record
     float* lt = reinterpret_cast<float*>(rec + REC::LT);
-    for (int idx = tid; idx < 64 * L; idx += 256) {
-      const int r = idx / L, lvl = idx - r * L;
-      const float x = lam[((size_t)(tok0 + min(r, len - 1)) * HV + hv) * L + lvl];
-      if (lvl < SM::LMAX) s_lam[lvl * 64 + r] = x;
-      if (lvl >= HG_INTRA && lvl < HG_INTRA + HG_NLV) lt[(lvl - HG_INTRA) * 64 + r] = x;
+#pragma unroll
+    for (int j = 0; j < NLAM; ++j) {
+      const int idx = tid + 256 * j, r = idx / Lc, lvl = idx - r * Lc;
+      if (idx < 64 * Lc) {
+        if (lvl < HG_INTRA) s_lam[lvl * 64 + r] = lv[j];
+        else if (lvl < HG_INTRA + HG_NLV) lt[(lvl - HG_INTRA) * 64 + r] = lv[j];
+      }
     }
     for (int idx = tid; idx < HG_NLV * 64; idx += 256)
       if (HG_INTRA + idx / 64 >= L) lt[idx] = 0.0f;
@@ -567,7 +585,23 @@ __global__ void __launch_bounds__(64 * HG_CW)
   for (int slot = 0; slot < HG_LPW; ++slot)
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km) S[slot][km] = zero16();
-  for (int i = 0; i < nseg; ++i) {
+  // composite of the coming segment: loaded one step ahead (two register sets that swap roles)
+  constexpr int NM = (KT / 32) * NKS, NPT = KT / 32;
+  bf16x8 mA[NM], mB[NM];
+  f32x4 nA[NPT], nB[NPT];
+  float dA = 0.0f, dB = 0.0f;
+  auto issue = [&](int i, bf16x8* m, f32x4* n, float& d) __attribute__((always_inline)) {
+    const size_t sh = (size_t)(seg0 + max(0, min(i, nseg - 2))) * HV + hv;
+    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+    const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vslab) * N_BYTES);
+#pragma unroll
+    for (int f = 0; f < NM; ++f) m[f] = M[f * 64 + lane];
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) n[j] = N[tid + 64 * HG_CW * j];
+    d = Dcomp[sh];
+  };
+  auto step = [&](int i, const bf16x8* m, const f32x4* n, float d, bf16x8* m2, f32x4* n2, float& d2)
+                  __attribute__((always_inline)) {
     const int seg = seg0 + i, cs = i << p;
 #pragma unroll
     for (int slot = 0; slot < HG_LPW; ++slot) {
@@ -575,10 +609,8 @@ __global__ void __launch_bounds__(64 * HG_CW)
       if ((cs >> lvl) & 1)
         slab_store<KT>(Xinit + ((((size_t)seg * HG_NLV + lvl) * HV + hv) * (VT / 32) + vslab) * (KT * 32), lane, S[slot]);
     }
-    if (i == nseg - 1) break;
-    const size_t sh = (size_t)seg * HV + hv;
-    const float d = Dcomp[sh];
-    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+    if (i == nseg - 1) return;
+    issue(i + 1, m2, n2, d2);
 #pragma unroll
     for (int slot = 0; slot < HG_LPW; ++slot) {
       const int lvl = slot * HG_CW + wave;
@@ -591,16 +623,19 @@ __global__ void __launch_bounds__(64 * HG_CW)
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[slot][km][r] *= d;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) S[slot][km] = mfma32(M[(km * NKS + ks) * 64 + lane], Sb[ks], S[slot][km]);
+        for (int ks = 0; ks < NKS; ++ks) S[slot][km] = mfma32(m[km * NKS + ks], Sb[ks], S[slot][km]);
       }
     }
     lds_barrier();  // the level that took the last carry has read s_acc
-    {
-      const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vslab) * N_BYTES);
-      for (int j = tid; j < KT * 8; j += 64 * HG_CW) reinterpret_cast<f32x4*>(s_acc)[j] = N[j];
-    }
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) reinterpret_cast<f32x4*>(s_acc)[tid + 64 * HG_CW * j] = n[j];
     lds_barrier();
     hg_merge<KT>(cs + (1 << p) - 1, p, wave, true, lane, s_acc, S);
+  };
+  if (nseg > 1) issue(0, mA, nA, dA);
+  for (int i = 0; i < nseg; i += 2) {
+    step(i, mA, nA, dA, mB, nB, dB);
+    if (i + 1 < nseg) step(i + 1, mB, nB, dB, mA, nA, dA);
   }
 }
 
