@@ -28,8 +28,8 @@
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-#define HG_CW 4                  // chain waves
-#define HG_LPW 3                 // levels per chain wave
+#define HG_CW 6                  // chain waves
+#define HG_LPW 2                 // levels per chain wave
 #define HG_NLV (HG_CW * HG_LPW)  // inter-chunk levels: sequences of up to 2^12 chunks
 #define HG_INTRA 7               // levels 0..6 live inside a chunk
 
@@ -426,13 +426,33 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
   const int cs0 = c0 - pv.seg_chunk0[pv.seq_seg0[pv.seg_seq[seg]]];  // index of the first chunk in its sequence
   const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63, hh = lane >> 5, ln = lane & 31;
 
+  // Output of a chunk: every wave of the workgroup sums eight rows of the chain waves' partial tiles and the intra-chunk
+  // part (read one chunk ahead), rounds and stores them -- lane = (row, four columns).
+  const int orow = 8 * wave + (lane >> 3), ocol = 4 * (lane & 7);
+  auto oi_load = [&](int c) __attribute__((always_inline)) {
+    return *reinterpret_cast<const f32x4*>(Oi + ((size_t)uniform(c) * HV + hv) * (64 * VT) + orow * VT + 32 * vslab + ocol);
+  };
+  auto out_rows = [&](int tok0, int len, f32x4 a) __attribute__((always_inline)) {
+#pragma unroll
+    for (int w = 0; w < HG_CW; ++w) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(&s_part[w * 64 * SP + orow * SP + ocol]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] += t[i];
+    }
+    typedef T T4 __attribute__((ext_vector_type(4)));
+    T4 pk;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pk[i] = GdrElem<T>::from_float(a[i]);
+    if (orow < len) *reinterpret_cast<T4*>(o + ((size_t)(tok0 + orow) * HV + hv) * VT + 32 * vslab + ocol) = pk;
+  };
+  static_assert(HG_CW + 2 == 8, "eight waves share the 64 output rows");
+
   if (wave >= HG_CW) {
     // ================================================ loader ================================================
     const int ltid = tid - 64 * HG_CW;
     constexpr int NP = (REC::PIECES + 127) / 128;
-    const int row = ltid >> 1, half = ltid & 1;
     u32x4 recA[NP], recB[NP];
-    f32x4 nA[KT / 16], nB[KT / 16], oA[4], oB[4];  // N slab: KT * 32 * 4 bytes = KT * 8 pieces over 128 threads
+    f32x4 nA[KT / 16], nB[KT / 16];  // N slab: KT * 32 * 4 bytes = KT * 8 pieces over 128 threads
     auto load_rec = [&](int c, u32x4* r) __attribute__((always_inline)) {
       const u32x4* src = reinterpret_cast<const u32x4*>(wrec + ((size_t)uniform(c) * HV + hv) * REC::BYTES);
 #pragma unroll
@@ -444,58 +464,34 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
       for (int j = 0; j < NP; ++j)
         if (ltid + 128 * j < REC::PIECES) dst[ltid + 128 * j] = r[j];
     };
-    auto load_no = [&](int c, f32x4* n, f32x4* oo) __attribute__((always_inline)) {
-      const size_t ch = (size_t)uniform(c) * HV + hv;
-      const f32x4* ns = reinterpret_cast<const f32x4*>(Nc + (ch * (VT / 32) + vslab) * (KT * 32));
+    auto load_set = [&](int c, u32x4* r, f32x4* n) __attribute__((always_inline)) {  // what chunk c issues
+      const int cr = min(c + 2, c1 - 1), cn = min(c + 1, c1 - 1);
+      load_rec(cr, r);
+      const f32x4* ns = reinterpret_cast<const f32x4*>(Nc + (((size_t)uniform(cn) * HV + hv) * (VT / 32) + vslab) * (KT * 32));
 #pragma unroll
       for (int j = 0; j < KT / 16; ++j) n[j] = ns[ltid + 128 * j];
-      const f32x4* os = reinterpret_cast<const f32x4*>(Oi + ch * (64 * VT) + row * VT + 32 * vslab + 16 * half);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) oo[e] = os[e];
     };
     load_rec(c0, recA);
     store_rec(0, recA);
-    const int cl = c1 - 1;
-    load_rec(min(c0 + 1, cl), recA);
-    load_no(c0, nA, oA);
-    auto one_chunk = [&](int c, u32x4* rHeld, f32x4* nHeld, f32x4* oHeld, u32x4* rNext, f32x4* nNext, f32x4* oNext) __attribute__((always_inline)) {
+    load_set(c0 - 1, recA, nA);  // record (c0 + 1), own state (c0)
+    f32x4 oi_cur = oi_load(c0);
+    auto one_chunk = [&](int c, const u32x4* rHeld, const f32x4* nHeld, u32x4* rNext, f32x4* nNext)
+                         __attribute__((always_inline)) {
       lds_barrier();  // T(c): record (c) is staged; record buffer (c+1)&1, s_acc and the partial tiles are free
+      const int tok0 = chunk_tok0[uniform(c)], len = chunk_len[uniform(c)];  // (scalar loads: early, so that they land)
       store_rec((c - c0 + 1) & 1, rHeld);
 #pragma unroll
       for (int j = 0; j < KT / 16; ++j) reinterpret_cast<f32x4*>(s_acc)[ltid + 128 * j] = nHeld[j];
-      load_rec(min(c + 2, cl), rNext);
-      load_no(min(c + 1, cl), nNext, oNext);
+      load_set(c, rNext, nNext);
+      const f32x4 oi_next = oi_load(min(c + 1, c1 - 1));
       lds_barrier();  // M0(c): the chain waves' partial tiles are complete
-      {
-        const int cu = uniform(c), tok0 = chunk_tok0[cu], len = chunk_len[cu];
-        float x[16];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          f32x4 a = oHeld[e];
-#pragma unroll
-          for (int w = 0; w < HG_CW; ++w) {
-            const f32x4 t = *reinterpret_cast<const f32x4*>(&s_part[w * 64 * SP + row * SP + 16 * half + 4 * e]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] += t[i];
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) x[4 * e + i] = a[i];
-        }
-        typedef T T8 __attribute__((ext_vector_type(8)));
-        T8 lo, hi;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { lo[i] = GdrElem<T>::from_float(x[i]); hi[i] = GdrElem<T>::from_float(x[8 + i]); }
-        if (row < len) {
-          T* op = o + ((size_t)(tok0 + row) * HV + hv) * VT + 32 * vslab + 16 * half;
-          *reinterpret_cast<T8*>(op) = lo;
-          *reinterpret_cast<T8*>(op + 8) = hi;
-        }
-      }
-      if (c + 1 < c1) hg_merge<KT>(cs0 + (c - c0), 0, wave, false, lane, s_acc, nullptr);
+      out_rows(tok0, len, oi_cur);
+      if (c + 1 < c1) hg_merge<KT>(cs0 + (c - c0), 0, wave, false, lane, nullptr, nullptr);
+      oi_cur = oi_next;
     };
     for (int c = c0; c < c1; c += 2) {
-      one_chunk(c, recA, nA, oA, recB, nB, oB);
-      if (c + 1 < c1) one_chunk(c + 1, recB, nB, oB, recA, nA, oA);
+      one_chunk(c, recA, nA, recB, nB);
+      if (c + 1 < c1) one_chunk(c + 1, recB, nB, recA, nA);
     }
     return;
   }
@@ -510,9 +506,12 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
     if (Xinit && ((cs0 >> lvl) & 1))
       slab_load<KT>(Xinit + ((((size_t)seg * HG_NLV + lvl) * HV + hv) * (VT / 32) + vslab) * (KT * 32), lane, S[slot]);
   }
+  f32x4 oi_cur = oi_load(c0);
   for (int c = c0; c < c1; ++c) {
     const int cs = cs0 + (c - c0);
     lds_barrier();  // T(c)
+    const int tok0 = chunk_tok0[uniform(c)], len = chunk_len[uniform(c)];
+    const f32x4 oi_next = oi_load(min(c + 1, c1 - 1));
     const unsigned char* rec = smem + SM::OFF_REC + ((c - c0) & 1) * REC::BYTES;
     const float* s_dk = reinterpret_cast<const float*>(rec + REC::DK);
     const float* s_lt = reinterpret_cast<const float*>(rec + REC::LT);
@@ -562,7 +561,9 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
         for (int r = 0; r < 16; ++r) part[(32 * tm + acc_row(r, hh)) * SP + ln] = O[tm][r];
     }
     lds_barrier();  // M0(c)
+    out_rows(tok0, len, oi_cur);
     if (c + 1 < c1) hg_merge<KT>(cs, 0, wave, true, lane, s_acc, S);
+    oi_cur = oi_next;
   }
 }
 
