@@ -51,18 +51,16 @@ struct HgRec {
 template <int KT, int VT>
 struct HgPrepSmem {
   static constexpr int SK = KT + 8, SV = VT + 8, ST = 40, LMAX = HG_INTRA + HG_NLV + 1;
-  static constexpr int OFF_K = 0;
-  static constexpr int OFF_Q = OFF_K + 64 * SK * 2;
-  static constexpr int OFF_KB = OFF_Q + 64 * SK * 2;  // beta e^{gamma} rk k; later Q~
-  static constexpr int OFF_W = OFF_KB + 64 * SK * 2;
+  static constexpr int OFF_K = 0;                     // raw k; later the (P T beta . Lambda) fragments and lambda
+  static constexpr int OFF_Q = OFF_K + 64 * SK * 2;   // raw q; Q~ is written over it in place
+  static constexpr int OFF_W = OFF_Q + 64 * SK * 2;
   static constexpr int OFF_V = OFF_W + 64 * SK * 2;
-  static constexpr int OFF_VB = OFF_V + 64 * SV * 2;  // beta v
-  static constexpr int OFF_T = OFF_VB + 64 * SV * 2;
+  static constexpr int OFF_T = OFF_V + 64 * SV * 2;
   static constexpr int OFF_P = OFF_T + 3 * 32 * ST * 2;
-  static constexpr int OFF_PL = OFF_P + 6 * 1024;
-  static constexpr int OFF_LAM = OFF_PL + 6 * 1024;
-  static constexpr int OFF_F = OFF_LAM + HG_INTRA * 64 * 4;  // gamma, beta, rk, qsc, qs, dk
-  static constexpr int BYTES = OFF_F + 6 * 64 * 4;
+  static constexpr int OFF_LAM = OFF_K + 6 * 1024;           // levels 0..6, written once the k tile is done with
+  static constexpr int OFF_F = OFF_P + 6 * 1024;             // gamma, beta, rk, qsc, qs, dk, bek
+  static constexpr int BYTES = OFF_F + 7 * 64 * 4;           // 51.25 KiB at K = V = 64: three workgroups per CU
+  static_assert(6 * 1024 + HG_INTRA * 64 * 4 <= 64 * SK * 2, "fragments + lambda fit in the k tile");
 };
 
 template <typename T, int KT, int VT>
@@ -78,14 +76,12 @@ __global__ void __launch_bounds__(256)
   extern __shared__ __align__(16) unsigned char smem[];
   __bf16* s_k = reinterpret_cast<__bf16*>(smem + SM::OFF_K);
   __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
-  __bf16* s_kb = reinterpret_cast<__bf16*>(smem + SM::OFF_KB);
-  __bf16* s_qt = s_kb;
+  __bf16* s_qt = s_q;
   __bf16* s_w = reinterpret_cast<__bf16*>(smem + SM::OFF_W);
   __bf16* s_v = reinterpret_cast<__bf16*>(smem + SM::OFF_V);
-  __bf16* s_vb = reinterpret_cast<__bf16*>(smem + SM::OFF_VB);
   __bf16* s_t = reinterpret_cast<__bf16*>(smem + SM::OFF_T);
   unsigned char* s_P = smem + SM::OFF_P;
-  unsigned char* s_PL = smem + SM::OFF_PL;
+  unsigned char* s_PL = smem + SM::OFF_K;
   float* s_lam = reinterpret_cast<float*>(smem + SM::OFF_LAM);
   float* s_gamma = reinterpret_cast<float*>(smem + SM::OFF_F);
   float* s_beta = s_gamma + 64;
@@ -93,6 +89,7 @@ __global__ void __launch_bounds__(256)
   float* s_qsc = s_gamma + 192;  // scale rq_i
   float* s_qs = s_gamma + 256;   // scale e^{gamma_i} rq_i
   float* s_dk = s_gamma + 320;   // e^{gamma_last - gamma_i} rk_i
+  float* s_bek = s_gamma + 384;  // beta_i e^{gamma_i} rk_i
 
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
@@ -102,6 +99,11 @@ __global__ void __launch_bounds__(256)
   const unsigned char* rec_in = tmat + ch * REC_BYTES;
   unsigned char* rec = wrec + ch * REC::BYTES;
 
+  // lambda rows (at most LMAX levels: five values per thread); the intra-chunk levels wait in registers until the
+  // k tile's space is free
+  constexpr int NLAM = (64 * SM::LMAX + 255) / 256;
+  const int Lc = min(L, SM::LMAX);
+  float lv[NLAM];
   {  // ---- stage the tiles: thread = (row, quarter of the row)
     const int row = tid >> 2, part = tid & 3;
     const bool live = row < len;
@@ -122,11 +124,8 @@ __global__ void __launch_bounds__(256)
     for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vp + 8 * u);
     const float* fact = reinterpret_cast<const float*>(rec_in + T_BYTES);
     const float gv = fact[row], g_last = fact[63], bv = fact[64 + row];
-    // every global load of the stage is issued before the first use: T blocks and the lambda rows (at most
-    // LMAX levels: five values per thread), indices clamped instead of branches
-    constexpr int NLAM = (64 * SM::LMAX + 255) / 256;
-    const int Lc = min(L, SM::LMAX);
-    float lv[NLAM];
+    // every global load of the stage is issued before the first use: T blocks and the lambda rows, indices
+    // clamped instead of branches
     bf16x8 tp0, tp1;
     {
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(rec_in);
@@ -161,21 +160,10 @@ __global__ void __launch_bounds__(256)
     const float eg = __builtin_amdgcn_exp2f(gv);
     const float bek = bv * eg * rk;
 #pragma unroll
-    for (int u = 0; u < KU; ++u) {
-      bf16x8 t;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) t[e] = (__bf16)(bek * (float)kb[u][e]);
-      *reinterpret_cast<bf16x8*>(&s_kb[row * SK + part * (KT / 4) + 8 * u]) = t;
-    }
-#pragma unroll
     for (int u = 0; u < VU; ++u) {
       float unused = 0.0f;
-      const bf16x8 vb = raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
-      bf16x8 t;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) t[e] = (__bf16)(bv * (float)vb[e]);
-      *reinterpret_cast<bf16x8*>(&s_v[row * SV + part * (VT / 4) + 8 * u]) = vb;
-      *reinterpret_cast<bf16x8*>(&s_vb[row * SV + part * (VT / 4) + 8 * u]) = t;
+      *reinterpret_cast<bf16x8*>(&s_v[row * SV + part * (VT / 4) + 8 * u]) =
+          raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
     }
     if (part == 0) {
       const float dk = __builtin_amdgcn_exp2f(g_last - gv) * rk;
@@ -185,17 +173,17 @@ __global__ void __launch_bounds__(256)
       s_qsc[row] = scale * rq;
       s_qs[row] = scale * eg * rq;
       s_dk[row] = dk;
+      s_bek[row] = bek;
       reinterpret_cast<float*>(rec + REC::DK)[row] = dk;
       if (row == 0) reinterpret_cast<float*>(rec + REC::MISC)[0] = __builtin_amdgcn_exp2f(g_last);
     }
-    // lambda, transposed: s_lam[level][row]; the inter-chunk levels also go to the record
+    // lambda, transposed ([level][row]): the inter-chunk levels go to the record
     float* lt = reinterpret_cast<float*>(rec + REC::LT);
 #pragma unroll
     for (int j = 0; j < NLAM; ++j) {
       const int idx = tid + 256 * j, r = idx / Lc, lvl = idx - r * Lc;
       if (idx < 64 * Lc) {
-        if (lvl < HG_INTRA) s_lam[lvl * 64 + r] = lv[j];
-        else if (lvl < HG_INTRA + HG_NLV) lt[(lvl - HG_INTRA) * 64 + r] = lv[j];
+        if (lvl >= HG_INTRA && lvl < HG_INTRA + HG_NLV) lt[(lvl - HG_INTRA) * 64 + r] = lv[j];
       }
     }
     for (int idx = tid; idx < HG_NLV * 64; idx += 256)
@@ -207,11 +195,25 @@ __global__ void __launch_bounds__(256)
     const int blk = tm == 0 ? 0 : (ks < 2 ? 1 : 2);
     return ld_kappa(s_t + blk * 32 * ST, ST, ln, 16 * (ks & 1), hh);
   };
+  // the same with column j scaled by fac[j] (T diag(fac)): the per-token factor of a product's right-hand rows goes
+  // onto T, so that the right-hand operand is the raw tile
+  auto t_frag_scaled = [&](int tm, int ks, const float* fac) {
+    const bf16x8 t = t_frag(tm, ks);
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(&fac[16 * ks + 4 * hh]);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(&fac[16 * ks + 8 + 4 * hh]);
+    bf16x8 out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      out[e] = (__bf16)((float)t[e] * lo[e]);
+      out[4 + e] = (__bf16)((float)t[4 + e] * hi[e]);
+    }
+    return out;
+  };
   auto w_tile = [&](int tm, int ct) {  // W rows 32 tm .., columns 32 ct ..
     f32x16 acc = zero16();
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
-      if (ks < 2 * (tm + 1)) acc = mfma32(t_frag(tm, ks), ld_kappa_tr(s_kb, SK, 32 * ct, 16 * ks, lane), acc);
+      if (ks < 2 * (tm + 1)) acc = mfma32(t_frag_scaled(tm, ks, s_bek), ld_kappa_tr(s_k, SK, 32 * ct, 16 * ks, lane), acc);
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_w[(32 * tm + acc_row(r, hh)) * SK + 32 * ct + ln] = (__bf16)acc[r];
   };
@@ -233,14 +235,14 @@ __global__ void __launch_bounds__(256)
     frag_store(s_P, f0, lane, acc_to_operand(acc, 0));
     frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
   };
-  auto un_tile = [&](int vt) {  // U = T (beta v) for 32 value columns, then N = K^T (dk U)
+  auto un_tile = [&](int vt) {  // U = (T diag(beta)) V for 32 value columns, then N = K^T (dk U)
     bf16x8 Ub[4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {
       f32x16 acc = zero16();
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
-        if (ks < 2 * (tm + 1)) acc = mfma32(t_frag(tm, ks), ld_kappa_tr(s_vb, SV, 32 * vt, 16 * ks, lane), acc);
+        if (ks < 2 * (tm + 1)) acc = mfma32(t_frag_scaled(tm, ks, s_beta), ld_kappa_tr(s_v, SV, 32 * vt, 16 * ks, lane), acc);
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] *= s_dk[32 * tm + acc_row(r, hh)];
       Ub[2 * tm] = acc_to_operand(acc, 0);
@@ -271,6 +273,12 @@ __global__ void __launch_bounds__(256)
       const int f = task - NW - 3 - NU;
       frag_store(rec + REC::KF, f, lane, ld_kappa_tr(s_k, SK, 32 * (f / 4), 16 * (f % 4), lane));
     }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NLAM; ++j) {
+    const int idx = tid + 256 * j, r = idx / Lc, lvl = idx - r * Lc;
+    if (idx < 64 * Lc && lvl < HG_INTRA) s_lam[lvl * 64 + r] = lv[j];
   }
   __syncthreads();
 
