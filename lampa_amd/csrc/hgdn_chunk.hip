@@ -529,37 +529,64 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
     for (int slot = 0; slot < HG_LPW; ++slot) {
       const int lvl = slot * HG_CW + wave;
       if (!((cs >> lvl) & 1)) continue;
+      // The fragments of a stage are read from LDS as one batch ahead of its MFMAs (lds_fence() pins that order; left
+      // alone the compiler fetches each fragment right before its MFMA and pays the LDS latency every time), and the
+      // two accumulation chains of a stage are interleaved.
+      bf16x8 fr[2 * NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        fr[ks] = frag_load(rec + REC::WF, ks, lane);
+        fr[NKS + ks] = frag_load(rec + REC::QF, ks, lane);
+      }
       bf16x8 Sb[NKS];
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_operand(S[slot][ks / 2], 8 * (ks % 2));
       bf16x8 Zb[4];
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm) {
-        f32x16 z = zero16(), a = zero16();
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) z = mfma32(frag_load(rec + REC::WF, tm * NKS + ks, lane), Sb[ks], z);
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) a = mfma32(frag_load(rec + REC::QF, tm * NKS + ks, lane), Sb[ks], a);
+        f32x4 dk[4], lm[4];
 #pragma unroll
         for (int b4 = 0; b4 < 4; ++b4) {
-          const f32x4 dk = *reinterpret_cast<const f32x4*>(&s_dk[32 * tm + 8 * b4 + 4 * hh]);
-          const f32x4 lm = *reinterpret_cast<const f32x4*>(&s_lt[lvl * 64 + 32 * tm + 8 * b4 + 4 * hh]);
+          dk[b4] = *reinterpret_cast<const f32x4*>(&s_dk[32 * tm + 8 * b4 + 4 * hh]);
+          lm[b4] = *reinterpret_cast<const f32x4*>(&s_lt[lvl * 64 + 32 * tm + 8 * b4 + 4 * hh]);
+        }
+        lds_fence();
+        f32x16 z = zero16(), a = zero16();
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            z[4 * b4 + e] *= -dk[e];
-            O[tm][4 * b4 + e] = __builtin_fmaf(lm[e], a[4 * b4 + e], O[tm][4 * b4 + e]);
+        for (int ks = 0; ks < NKS; ++ks) {
+          z = mfma32(fr[ks], Sb[ks], z);
+          a = mfma32(fr[NKS + ks], Sb[ks], a);
+        }
+        // the next stage's fragments: row tile 1 of W and Q~, then K^T
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          if (tm == 0) {
+            fr[ks] = frag_load(rec + REC::WF, NKS + ks, lane);
+            fr[NKS + ks] = frag_load(rec + REC::QF, NKS + ks, lane);
+          } else if (ks < 4) {
+#pragma unroll
+            for (int km = 0; km < KT / 32; ++km) fr[km * 4 + ks] = frag_load(rec + REC::KF, km * 4 + ks, lane);
           }
         }
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            z[4 * b4 + e] *= -dk[b4][e];
+            O[tm][4 * b4 + e] = __builtin_fmaf(lm[b4][e], a[4 * b4 + e], O[tm][4 * b4 + e]);
+          }
         Zb[2 * tm] = acc_to_operand(z, 0);
         Zb[2 * tm + 1] = acc_to_operand(z, 8);
       }
 #pragma unroll
-      for (int km = 0; km < KT / 32; ++km) {
+      for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[slot][km][r] *= dec;
+      lds_fence();
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) S[slot][km] = mfma32(frag_load(rec + REC::KF, km * 4 + ks, lane), Zb[ks], S[slot][km]);
-      }
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int km = 0; km < KT / 32; ++km) S[slot][km] = mfma32(fr[km * 4 + ks], Zb[ks], S[slot][km]);
     }
     {
       float* part = s_part + wave * 64 * SP;

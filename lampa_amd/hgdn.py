@@ -39,11 +39,11 @@ def _plan(B: int, T: int, device, n_value_heads: int, n_slabs: int):
     nt = (T + 63) // 64
     cps = CHUNKS_PER_SEGMENT
     if not cps:
-        # one workgroup per (segment, head, 32 value columns) and compute unit; the scan in between is serial in the
-        # segments of a sequence
+        # a compute unit holds one workgroup of the walk (segment, head, 32 value columns): the shortest segments that
+        # still run in one round; the scan in between is serial in the segments of a sequence
         cus = torch.cuda.get_device_properties(device).multi_processor_count
         cps = 1 << max(nt - 1, 1).bit_length()  # one segment per sequence
-        while cps > 8 and B * ((nt + cps // 2 - 1) // (cps // 2)) * n_value_heads * n_slabs <= 2 * cus:
+        while cps > 8 and B * ((nt + cps // 2 - 1) // (cps // 2)) * n_value_heads * n_slabs <= cus:
             cps //= 2
     key = (B, T, cps, str(device))
     hit = _plan_cache.get(key)
