@@ -94,6 +94,34 @@ def test_plan_rejects_bad_input(lib):
     assert lib.lampa_gdr_plan_size(ok, 1, 0) == -1
 
 
+def test_hierarchical_forward_argument_checks(lib):
+    """Every check of lampa_hgdn_chunk_fwd runs on the host before the first launch (dummy, never dereferenced
+    device addresses; the plan is real)."""
+    assert lib.lampa_hgdn_chunk_workspace_bytes(938, 30, 8, 64, 64) > 938 * 8 * (24 * 1024 + 2 * 64 * 64 * 4)
+    assert lib.lampa_hgdn_chunk_workspace_bytes(938, 30, 8, 128, 128) == -4
+    assert lib.lampa_hgdn_chunk_workspace_bytes(-1, 30, 8, 64, 64) == -1
+    d = ctypes.c_void_p(0x1000)  # 16-byte aligned dummy
+
+    def call(cu, cps, L=20, K=64, V=64, q=d, ws=None, dtype=0):
+        arr = (ctypes.c_int64 * len(cu))(*cu)
+        size = lib.lampa_gdr_plan_size(arr, len(cu) - 1, cps)
+        plan = torch.zeros(size, dtype=torch.int32)
+        assert lib.lampa_gdr_plan_fill(arr, len(cu) - 1, cps, ctypes.c_void_p(plan.data_ptr())) == 0
+        return lib.lampa_hgdn_chunk_fwd(q, d, d, d, d, d, d, ctypes.c_void_p(plan.data_ptr()), d, 2, 2, K, V, L, dtype,
+                                        0.125, 1, ws, 0, None)
+
+    assert call([0, 4096], 8, q=None) == -1                      # null pointer
+    assert call([0, 4096], 8, q=ctypes.c_void_p(0x1008)) == -1   # misaligned
+    assert call([0, 4096], 8, K=128) == -4                       # head size
+    assert call([0, 4096], 8, dtype=2) == -4                     # fp32 inputs
+    assert call([0, 4096], 12) == -1                             # split sequences need a power-of-two segment length
+    assert call([0, 4096], 8, L=12) == -1                        # 64 chunks need 7 + 6 levels
+    assert call([0, 4096], 8, L=13) == -2                        # all checks passed: the workspace is missing
+    assert call([0, 4096], 100, L=13) == -2                      # one segment per sequence: any segment length
+    assert call([0, 64 * 4097], 4096, L=32) == -4                # more than 4096 chunks in a sequence
+    assert call([0, 64 * 4096], 4096, L=19) == -2
+
+
 def test_operators_refuse_cpu_tensors():
     from lampa_amd import gated_delta as gd
     from lampa_amd import lsh
