@@ -286,7 +286,7 @@ def main():
         "us": round(hgdn_us, 1), "hits_per_s": round(T / (hgdn_us * 1e-6), 1),
         "kernel_us": {n: round(v_, 1) for n, v_ in hstage.items()},
         "mfma_frac": round(hgdn_flop / (hgdn_us * 1e-6) / 2.5e15, 4),
-        "note": "includes the wrapper's lambda / scale and fp32 conversion of lambda; mfma_frac = algorithmic flops "
+        "note": "wall clock of chunk_h_gated_delta_rule; mfma_frac = algorithmic flops "
                 "(per chunk and head 2*64*64*(3K+2V+42) for the chunk-local products with triangular factors counted as such, 6*64*K*V per occupied level) "
                 "over the bf16 dense peak",
     }

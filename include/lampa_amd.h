@@ -237,16 +237,18 @@ int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float
 /* Hierarchical (level-weighted) chunkwise forward. Replaces chunk_h_gated_delta_rule -> hattention_kernel ->
  * chunkwise_fwd (models/hattention/gated_delta_rule_apis.py:21-91, kernel.py:338-374, chunkwise_hgdn.py:565-791;
  * specification: hattention_recurrent, recurrent.py:169-216, with HType.WEAK, HStruct.GDELTA, base 2).
- * lam: fp32 [total_tokens, HV, L], the level weights as they enter hattention_kernel (already divided by `scale`);
- * level 0 = the token itself, level l > 0 = sources whose highest differing position bit is l-1 (base.py:41-46).
+ * lam: [total_tokens, HV, L] of type lam_dtype (LAMPA_BF16 / LAMPA_FP16 / LAMPA_FP32), the level weights; the kernel
+ * uses lam / lam_div rounded to lam's type, which is what gated_delta_rule_apis.py:68-70 does with lam_div = scale
+ * (lam_div = 1: as given). Level 0 = the token itself, level l > 0 = sources whose highest differing position bit is
+ * l-1 (base.py:41-46).
  * K = 64, V in {64, 128}; l2norm as for the chunk forward (the reference requires the chunk-path l2norm);
  * the plan's chunks_per_segment must be a power of two unless every sequence is one segment; sequences of at most
  * 4096 chunks; L >= 7 + number of bits of the largest chunk index. Zero initial state, no final state. */
 int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V);
 int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                         const float* lam, void* o, const int32_t* plan_host, const int32_t* plan_dev, int H, int HV,
-                         int K, int V, int L, int dtype, float scale, int l2norm, void* workspace,
-                         int64_t workspace_bytes, void* stream);
+                         const void* lam, int lam_dtype, float lam_div, void* o, const int32_t* plan_host,
+                         const int32_t* plan_dev, int H, int HV, int K, int V, int L, int dtype, float scale, int l2norm,
+                         void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------- profiling */
 

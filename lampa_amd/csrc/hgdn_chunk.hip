@@ -66,7 +66,8 @@ struct HgPrepSmem {
 template <typename T, int KT, int VT>
 __global__ void __launch_bounds__(256)
     hgdn_prep_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-                     const float* __restrict__ lam, const int32_t* __restrict__ chunk_tok0,
+                     const void* __restrict__ lam, int lam_dtype, float lam_div,
+                     const int32_t* __restrict__ chunk_tok0,
                      const int32_t* __restrict__ chunk_len, const unsigned char* __restrict__ tmat,
                      unsigned char* __restrict__ wrec, float* __restrict__ Nc, float* __restrict__ Oi, int H, int HV,
                      int L, float scale, int l2norm) {
@@ -131,10 +132,28 @@ __global__ void __launch_bounds__(256)
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(rec_in);
       tp0 = tp[tid];
       tp1 = tp[256 + (tid & 127)];
+      size_t li[NLAM];
 #pragma unroll
       for (int j = 0; j < NLAM; ++j) {
         const int idx = min(tid + 256 * j, 64 * Lc - 1), r = idx / Lc, lvl = idx - r * Lc;
-        lv[j] = lam[((size_t)(tok0 + min(r, len - 1)) * HV + hv) * L + lvl];
+        li[j] = ((size_t)(tok0 + min(r, len - 1)) * HV + hv) * L + lvl;
+      }
+      // (one branch around all the loads of a type, so that they are in flight together)
+      if (lam_dtype == GDR_FP32) {
+#pragma unroll
+        for (int j = 0; j < NLAM; ++j) lv[j] = reinterpret_cast<const float*>(lam)[li[j]];
+      } else if (lam_dtype == GDR_BF16) {
+        __bf16 t[NLAM];
+#pragma unroll
+        for (int j = 0; j < NLAM; ++j) t[j] = reinterpret_cast<const __bf16*>(lam)[li[j]];
+#pragma unroll
+        for (int j = 0; j < NLAM; ++j) lv[j] = (float)t[j];
+      } else {
+        _Float16 t[NLAM];
+#pragma unroll
+        for (int j = 0; j < NLAM; ++j) t[j] = reinterpret_cast<const _Float16*>(lam)[li[j]];
+#pragma unroll
+        for (int j = 0; j < NLAM; ++j) lv[j] = (float)t[j];
       }
     }
     {
@@ -178,6 +197,13 @@ __global__ void __launch_bounds__(256)
       if (row == 0) reinterpret_cast<float*>(rec + REC::MISC)[0] = __builtin_amdgcn_exp2f(g_last);
     }
     // lambda, transposed ([level][row]): the inter-chunk levels go to the record
+    if (lam_div != 1.0f) {  // lambda / scale, rounded to lambda's own type as the element-wise division would
+#pragma unroll
+      for (int j = 0; j < NLAM; ++j) {
+        const float x = __fdiv_rn(lv[j], lam_div);
+        lv[j] = lam_dtype == GDR_FP32 ? x : lam_dtype == GDR_BF16 ? (float)(__bf16)x : (float)(_Float16)x;
+      }
+    }
     float* lt = reinterpret_cast<float*>(rec + REC::LT);
 #pragma unroll
     for (int j = 0; j < NLAM; ++j) {
@@ -705,8 +731,8 @@ extern "C" int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_
 }
 
 template <typename T, int KT, int VT>
-static int hg_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* lam,
-                     void* o, const GdrPlanView pv, int n_seq, int chunks, int segs, int p, int H, int HV, int L,
+static int hg_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, const void* lam,
+                     int lam_dtype, float lam_div, void* o, const GdrPlanView pv, int n_seq, int chunks, int segs, int p, int H, int HV, int L,
                      float scale, int l2norm, unsigned char* ws, hipStream_t s) {
   const HgWorkspace w = hg_workspace(chunks, segs, HV, KT, VT);
   unsigned char* tf = ws + w.off_t;
@@ -736,7 +762,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
                      l2norm);
   LAMPA_PROF(s, "gdr_tinv_kernel");
   hipLaunchKernelGGL((hgdn_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem_p, s, (const T*)q, (const T*)k,
-                     (const T*)v, lam, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, H, HV, L, scale, l2norm);
+                     (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, H, HV, L, scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
   const bool split = segs > n_seq;
   if (split) {
@@ -757,16 +783,18 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
 }
 
 // Hierarchical chunkwise forward. q, k [total_tokens, H, K]; v, o [total_tokens, HV, V] (dtype 0 bf16 / 1 fp16);
-// g, beta fp32 [total_tokens, HV]; lam fp32 [total_tokens, HV, L] (level weights as they enter the kernel: the
-// caller has divided them by `scale`, which multiplies q). The plan's chunks_per_segment must be a power of two
-// (or at least the longest sequence's chunk count: one segment per sequence); every sequence may hold at most
-// 2^12 chunks and L must cover 7 + the number of chunk-index bits of the longest sequence.
+// g, beta fp32 [total_tokens, HV]; lam [total_tokens, HV, L] of type lam_dtype (0 bf16 / 1 fp16 / 2 fp32): the level
+// weights; the kernel uses lam / lam_div rounded to lam's type (the reference divides the weights by `scale`, which
+// multiplies q, before its kernel; lam_div = 1 takes them as they are). The plan's chunks_per_segment must be a
+// power of two (or at least the longest sequence's chunk count: one segment per sequence); every sequence may hold at
+// most 2^12 chunks and L must cover 7 + the number of chunk-index bits of the longest sequence.
 extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                                    const float* lam, void* o, const int32_t* plan_host, const int32_t* plan_dev,
-                                    int H, int HV, int K, int V, int L, int dtype, float scale, int l2norm,
-                                    void* workspace, int64_t workspace_bytes, void* stream) {
+                                    const void* lam, int lam_dtype, float lam_div, void* o, const int32_t* plan_host,
+                                    const int32_t* plan_dev, int H, int HV, int K, int V, int L, int dtype, float scale,
+                                    int l2norm, void* workspace, int64_t workspace_bytes, void* stream) {
   if (!q || !k || !v || !g || !beta || !lam || !o || !plan_host || !plan_dev) return LAMPA_ERR_INVALID;
   if (H < 1 || HV < H || HV % H != 0 || l2norm < 0 || l2norm > 2 || L < HG_INTRA) return LAMPA_ERR_INVALID;
+  if (lam_dtype < 0 || lam_dtype > 2 || !(lam_div > 0.0f)) return LAMPA_ERR_INVALID;
   if (!hg_supported(K, V) || (dtype != GDR_BF16 && dtype != GDR_FP16)) return LAMPA_ERR_UNSUPPORTED;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) return LAMPA_ERR_INVALID;
   const int n_seq = plan_host[PLAN_N_SEQ], chunks = plan_host[PLAN_TOTAL_CHUNKS], segs = plan_host[PLAN_N_SEGMENTS];
@@ -793,7 +821,7 @@ extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v,
   unsigned char* ws = (unsigned char*)workspace;
   const GdrPlanView pv = gdr_plan_view(plan_host, plan_dev);
 #define HG_CASE(TT, KK, VV) \
-  return hg_launch<TT, KK, VV>(q, k, v, g, beta, lam, o, pv, n_seq, chunks, segs, p, H, HV, L, scale, l2norm, ws, s)
+  return hg_launch<TT, KK, VV>(q, k, v, g, beta, lam, lam_dtype, lam_div, o, pv, n_seq, chunks, segs, p, H, HV, L, scale, l2norm, ws, s)
   if (dtype == GDR_BF16) {
     if (V == 64) HG_CASE(__bf16, 64, 64);
     if (V == 128) HG_CASE(__bf16, 64, 128);

@@ -5,7 +5,8 @@ order, defaults and checks. The reference's own chunk pipeline for this operator
 (``chunkwise_hgdn.py:661`` unpacks the single tensor ``chunk_scaled_dot_kkt_fwd`` returns into two), so the function
 implemented is its specification, ``hattention_recurrent`` (``recurrent.py:169-216``), reached the way the operator
 reaches it: q l2-normalised and scaled, k l2-normalised (``kernel.py:100-101``), lambda divided by ``scale``
-(``gated_delta_rule_apis.py:68-70``), weak hierarchy, base 2.
+(``gated_delta_rule_apis.py:68-70``; the kernel does it, with the rounding of a division in lambda's dtype), weak
+hierarchy, base 2.
 
 Differences a caller can observe: forward only; ``output_final_state=True`` (the prefill and single-step branches,
 ``gated_delta_rule_apis.py:92-128``) raises ``NotImplementedError``; head sizes K = 64 and V in {64, 128} only.
@@ -64,11 +65,13 @@ def _plan(B: int, T: int, device, n_value_heads: int, n_slabs: int):
 
 class _ForwardOnly(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, g, lam, beta, scale):
+    def forward(ctx, q, k, v, g, lam, beta, scale, lam_div):
         require_cuda(q, k, v, g, lam, beta)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
-        lam = lam.to(torch.float32).contiguous()
+        if lam.dtype not in _gd._DTYPES:
+            lam = lam.to(torch.float32)
+        lam = lam.contiguous()
         B, T, H, K = q.shape
         HV, V, L = v.shape[2], v.shape[3], lam.shape[-1]
         plan_host, plan_dev = _plan(B, T, q.device, HV, V // 32)
@@ -77,7 +80,8 @@ class _ForwardOnly(torch.autograd.Function):
         ws_bytes = check(lib.lampa_hgdn_chunk_workspace_bytes(chunks, segs, HV, K, V), "lampa_hgdn_chunk_workspace_bytes")
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         o = torch.empty_like(v)
-        check(lib.lampa_hgdn_chunk_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(lam), ptr(o),
+        check(lib.lampa_hgdn_chunk_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(lam), _gd._DTYPES[lam.dtype],
+                                       float(lam_div), ptr(o),
                                        ctypes.c_void_p(plan_host.data_ptr()), ptr(plan_dev), H, HV, K, V, L,
                                        _gd._DTYPES[q.dtype], float(scale), _gd.L2_CHUNK, ptr(ws), ws_bytes, stream_of(q)),
               "lampa_hgdn_chunk_fwd")
@@ -111,8 +115,7 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
             "Please verify your input tensor format matches the expected shape [B, T, H, ...].")
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    if SCALE_LAMBDA:
-        l = l / scale
+    lam_div = scale if SCALE_LAMBDA else 1.0  # l = l / scale (gated_delta_rule_apis.py:68-70), done by the kernel
     if output_final_state or initial_state is not None:
         raise NotImplementedError("hierarchical final / initial states are not built")
     B, T, H, K = q.shape
@@ -124,5 +127,5 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
         raise ValueError
     if (T // 64) > 4096:
         raise NotImplementedError("hierarchical forward: at most 4096 chunks per sequence")
-    o = _ForwardOnly.apply(q, k, v, g, l, beta, scale)
+    o = _ForwardOnly.apply(q, k, v, g, l, beta, scale, lam_div)
     return o, None

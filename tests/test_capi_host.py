@@ -102,18 +102,19 @@ def test_hierarchical_forward_argument_checks(lib):
     assert lib.lampa_hgdn_chunk_workspace_bytes(-1, 30, 8, 64, 64) == -1
     d = ctypes.c_void_p(0x1000)  # 16-byte aligned dummy
 
-    def call(cu, cps, L=20, K=64, V=64, q=d, ws=None, dtype=0):
+    def call(cu, cps, L=20, K=64, V=64, q=d, ws=None, dtype=0, lam_dtype=0):
         arr = (ctypes.c_int64 * len(cu))(*cu)
         size = lib.lampa_gdr_plan_size(arr, len(cu) - 1, cps)
         plan = torch.zeros(size, dtype=torch.int32)
         assert lib.lampa_gdr_plan_fill(arr, len(cu) - 1, cps, ctypes.c_void_p(plan.data_ptr())) == 0
-        return lib.lampa_hgdn_chunk_fwd(q, d, d, d, d, d, d, ctypes.c_void_p(plan.data_ptr()), d, 2, 2, K, V, L, dtype,
+        return lib.lampa_hgdn_chunk_fwd(q, d, d, d, d, d, lam_dtype, 0.125, d, ctypes.c_void_p(plan.data_ptr()), d, 2, 2, K, V, L, dtype,
                                         0.125, 1, ws, 0, None)
 
     assert call([0, 4096], 8, q=None) == -1                      # null pointer
     assert call([0, 4096], 8, q=ctypes.c_void_p(0x1008)) == -1   # misaligned
     assert call([0, 4096], 8, K=128) == -4                       # head size
     assert call([0, 4096], 8, dtype=2) == -4                     # fp32 inputs
+    assert call([0, 4096], 8, lam_dtype=3) == -1                 # unknown type of the level weights
     assert call([0, 4096], 12) == -1                             # split sequences need a power-of-two segment length
     assert call([0, 4096], 8, L=12) == -1                        # 64 chunks need 7 + 6 levels
     assert call([0, 4096], 8, L=13) == -2                        # all checks passed: the workspace is missing
