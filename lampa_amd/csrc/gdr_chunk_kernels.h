@@ -932,7 +932,6 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
   }
 }
 
-// ---- host side ------------------------------------------------------------------------------------------------
 // ---- two-level scan ------------------------------------------------------------------------------------------------
 // A long sequence has many segments and the scan above walks them one after the other (0.45 us per step, a chain of
 // dependent MFMA / LDS-exchange stages with 16 workgroups on the whole chip). With groups of G segments the serial

@@ -17,11 +17,12 @@
 // Kernels:
 //   prep   workgroup per (chunk, head), fully parallel: W, Q~ and K^T as MFMA operand fragments, the decay factors,
 //          the inter-chunk lambdas (transposed), N and o_intra go to HBM.
-//   walk   workgroup per (segment of chunks, head, 32 value columns): four "chain" waves hold up to three level
-//          states each in accumulator registers (level j -> wave j % 4) and walk the chunks: for every level whose
+//   walk   workgroup per (segment of chunks, head, 32 value columns): six "chain" waves hold up to two level
+//          states each in accumulator registers (level j -> wave j % 6) and walk the chunks: for every level whose
 //          chunk-index bit is set, o += lambda . (Q~ S), S <- S'; after the chunk the levels below the lowest clear
 //          bit and N are summed into that bit's level (the carry chain of a binary counter) through LDS. Two loader
-//          waves stage the chunks' operand records, add the chain waves' partial outputs to o_intra and store o.
+//          waves stage the chunks' operand records and N; all eight waves add the chain waves' partial outputs to
+//          o_intra, eight rows each, and store o.
 //   scan   (sequences cut into segments of 2^p chunks) the same walk over whole segments with the segment
 //          composites (M, N) of the plain rule: leaves every segment's entering level states.
 #include "gdr_chunk_kernels.h"
