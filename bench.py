@@ -161,8 +161,36 @@ def main():
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "kernel_us": round(stage_us[dominant], 2), "algorithmic_bytes_per_launch": dom_bytes}
+    # ---- per-step distribution (HIP events on the launch stream, one pair per step) and a cold variant that rotates
+    #      among input sets totalling more than 512 MB, so that no step finds its inputs in the memory-side cache ----
+    def event_times(fn, n):
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for i, (a, b) in enumerate(evs):
+            a.record()
+            fn(i)
+            b.record()
+        torch.cuda.synchronize()
+        return sorted(1e3 * a.elapsed_time(b) for a, b in evs)
+
+    def pct(xs, p):
+        return round(xs[min(len(xs) - 1, int(p * len(xs)))], 2)
+
+    n_dist = max(100, args.steps)
+    warm = event_times(lambda i: step(), n_dist)
+    sets = [(qd, kd, vd, gd_, bd)] + [tuple(x.clone() for x in (qd, kd, vd, gd_, bd)) for _ in range(2)]
+    set_mb = sum(x.numel() * x.element_size() for x in sets[0]) / 1e6
+    for i in range(6):
+        gd.chunk_gated_delta_rule(*sets[i % 3], output_final_state=True)
+    cold = event_times(lambda i: gd.chunk_gated_delta_rule(*sets[i % 3], output_final_state=True), n_dist)
+    del sets
+    timing = {
+        "steps": n_dist, "unit": "us per layer, HIP events around each step",
+        "warm": {"median": pct(warm, 0.5), "p10": pct(warm, 0.1), "p90": pct(warm, 0.9)},
+        "cold": {"median": pct(cold, 0.5), "p10": pct(cold, 0.1), "p90": pct(cold, 0.9),
+                 "input_sets": 3, "mb_per_set": round(set_mb, 1)},
+    }
     layer = {
-        "us_per_layer": round(layer_us, 2),
+        "us_per_layer": round(layer_us, 2), "timing": timing,
         "hbm_frac": round(LAYER_BYTES_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "mfma_frac": round(LAYER_FLOP_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "kernel_us": {n: round(u, 2) for n, u in stage_us.items()},
