@@ -328,7 +328,20 @@ def main():
         cpu_hits_per_s, cpu_dt = cpu_baseline_gdr(q, k, v, g, beta, n_cpu)
         lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha)
         lsh_info["cpu_baseline_us"] = round(lsh_cpu_s * 1e6, 1)
+        # the same loop on one thread, on a shorter prefix (the loop is serial in the tokens: time scales linearly)
+        n_one = min(n_cpu, 8192)
+        torch.set_num_threads(1)
+        one_hits_per_s, one_dt = cpu_baseline_gdr(q, k, v, g, beta, n_one)
+        torch.set_num_threads(cores)
+        cpu_model = ""
+        try:
+            with open("/proc/cpuinfo") as fh:
+                cpu_model = next((ln.split(":", 1)[1].strip() for ln in fh if ln.startswith("model name")), "")
+        except OSError:
+            pass
         cpu = {"value": round(cpu_hits_per_s, 1), "unit": "hits/s", "cores": cores, "kind": "port",
+               "cpu_model": cpu_model,
+               "one_thread": {"value": round(one_hits_per_s, 1), "sample": f"first {n_one} tokens ({one_dt:.2f} s)"},
                "sample": f"first {n_cpu} of {T} tokens, all {H} heads, fp32 token loop in PyTorch ({cpu_dt:.2f} s)"
                          + ("" if n_cpu == T else ", scaled linearly"),
                "cpu_count": os.cpu_count()}

@@ -17,6 +17,7 @@ sys.path.insert(0, ROOT)
 
 from lampa_amd import synth  # noqa: E402  (seeded input generators only; no GPU code runs here)
 from oracle import gated_delta as og  # noqa: E402
+from oracle import hgdn as oh  # noqa: E402
 from oracle import lsh as ol  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -40,7 +41,18 @@ def gdr_fixture():
                         final_state=s.numpy())
 
 
+def hgdn_fixture():
+    # three chunks, two heads: levels 0..8 (the 7 inside a chunk and two chunk-index bits); lambda as it enters the
+    # operator (the operator divides it by scale = 1/8)
+    q, k, v, g, beta = synth.gdr_inputs(1, 192, 2, 64, 64, torch.bfloat16, seed=8, g_scale=0.2)
+    lam = (torch.rand(1, 192, 2, 9, generator=torch.Generator().manual_seed(9)) + 0.25).bfloat16()
+    o = oh.recurrent_c(q, k, v, g, beta, lam / 0.125, scale=0.125)
+    np.savez_compressed(os.path.join(HERE, "hgdn_t192_h2_d64.npz"), q=q.float().numpy(), k=k.float().numpy(),
+                        v=v.float().numpy(), g=g.numpy(), beta=beta.numpy(), lam=lam.float().numpy(), o=o.numpy())
+
+
 if __name__ == "__main__":
     lsh_fixture()
     gdr_fixture()
+    hgdn_fixture()
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
