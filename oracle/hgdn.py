@@ -111,3 +111,24 @@ def recurrent_c(q, k, v, g, beta, lam, scale=None, l2=L2_CHUNK):
     lib().oracle_hgdn_recurrent_f64(ptr(qa), ptr(ka), ptr(va), ptr(ga), ptr(ba), ptr(la), ptr(cu), B, H, HV, K, V, L,
                                     ctypes.c_float(scale), l2, ptr(o))
     return torch.from_numpy(o)
+
+
+def recurrent_c_state(q, k, v, g, beta, lam, scale=None, l2=L2_CHUNK, states=None, counts=None):
+    """As ``recurrent_c``, carrying the level states: ``states`` [B,HV,K,V,L] and ``counts`` [L] (the ``HState`` of
+    ``recurrent.py:9-40``) enter when given (zero otherwise); returns ``(o, states, counts)`` after the last token."""
+    B, T, H, K = q.shape
+    HV, V, L = v.shape[2], v.shape[3], lam.shape[-1]
+    f = lambda x: np.ascontiguousarray(x.detach().to("cpu", torch.float32).numpy())
+    qa, ka, va, ga, ba, la = f(q), f(k), f(v), f(g), f(beta), f(lam)
+    if scale is None:
+        scale = K ** -0.5
+    cu = np.arange(B + 1, dtype=np.int64) * T
+    o = np.empty((B, T, HV, V), np.float32)
+    s_in = None if states is None else f(states)
+    c_in = None if counts is None else np.ascontiguousarray(np.asarray(counts, dtype=np.int32))
+    s_out = np.empty((B, HV, K, V, L), np.float32)
+    c_out = np.empty((L,), np.int32)
+    lib().oracle_hgdn_recurrent_state_f64(ptr(qa), ptr(ka), ptr(va), ptr(ga), ptr(ba), ptr(la), ptr(cu), B, H, HV, K, V,
+                                          L, ctypes.c_float(scale), l2, ptr(s_in), ptr(c_in), ptr(o), ptr(s_out),
+                                          ptr(c_out))
+    return torch.from_numpy(o), torch.from_numpy(s_out), torch.from_numpy(c_out)

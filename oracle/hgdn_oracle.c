@@ -21,9 +21,13 @@
 #include <stdlib.h>
 #include <string.h>
 
-void oracle_hgdn_recurrent_f64(const float* q, const float* k, const float* v, const float* g, const float* beta,
-                               const float* lam, const int64_t* cu_seqlens, int n_seq, int H, int HV, int K, int V,
-                               int L, float scale, int l2norm, float* o) {
+/* states_in / states_out: optional level states [n_seq, HV, K, V, L] (L fastest, the reference's HState.states layout,
+ * recurrent.py:33-36); counts_in / counts_out: optional token counts per level [L] (shared by all sequences and heads,
+ * recurrent.py:37-40). */
+void oracle_hgdn_recurrent_state_f64(const float* q, const float* k, const float* v, const float* g, const float* beta,
+                                     const float* lam, const int64_t* cu_seqlens, int n_seq, int H, int HV, int K, int V,
+                                     int L, float scale, int l2norm, const float* states_in, const int32_t* counts_in,
+                                     float* o, float* states_out, int32_t* counts_out) {
   const size_t KV = (size_t)K * V;
   double* S = (double*)malloc(sizeof(double) * KV * L);
   int64_t* cnt = (int64_t*)malloc(sizeof(int64_t) * L);
@@ -36,6 +40,11 @@ void oracle_hgdn_recurrent_f64(const float* q, const float* k, const float* v, c
       const int h = hv / rep;
       memset(S, 0, sizeof(double) * KV * L);
       memset(cnt, 0, sizeof(int64_t) * L);
+      if (states_in)
+        for (int l = 0; l < L; ++l)
+          for (size_t i = 0; i < KV; ++i) S[(size_t)l * KV + i] = states_in[(((size_t)s * HV + hv) * KV + i) * L + l];
+      if (counts_in)
+        for (int l = 0; l < L; ++l) cnt[l] = counts_in[l];
       for (int64_t t = cu_seqlens[s]; t < cu_seqlens[s + 1]; ++t) {
         const float* qt = q + (t * H + h) * K;
         const float* kt = k + (t * H + h) * K;
@@ -86,6 +95,17 @@ void oracle_hgdn_recurrent_f64(const float* q, const float* k, const float* v, c
         }
         for (int j = 0; j < V; ++j) ot[j] = (float)d[j];
       }
+      if (states_out)
+        for (int l = 0; l < L; ++l)
+          for (size_t i = 0; i < KV; ++i) states_out[(((size_t)s * HV + hv) * KV + i) * L + l] = (float)S[(size_t)l * KV + i];
+      if (counts_out)
+        for (int l = 0; l < L; ++l) counts_out[l] = (int32_t)cnt[l];
     }
   free(S); free(cnt); free(qn); free(kn); free(d);
+}
+
+void oracle_hgdn_recurrent_f64(const float* q, const float* k, const float* v, const float* g, const float* beta,
+                               const float* lam, const int64_t* cu_seqlens, int n_seq, int H, int HV, int K, int V,
+                               int L, float scale, int l2norm, float* o) {
+  oracle_hgdn_recurrent_state_f64(q, k, v, g, beta, lam, cu_seqlens, n_seq, H, HV, K, V, L, scale, l2norm, 0, 0, o, 0, 0);
 }

@@ -89,3 +89,23 @@ def test_one_hot_weights_select_one_bucket():
         total += part
     want, _ = og.recurrent_c(q, k, v, g, beta, l2=og.L2_CHUNK)
     assert torch.allclose(total, want, atol=1e-5)
+
+
+def test_states_split_the_plain_state_and_continue_exactly():
+    q, k, v, g, beta, lam = _inputs(B=2, T=77, H=2, L=9)
+    o, S, counts = oh.recurrent_c_state(q, k, v, g, beta, lam)
+    # token counts: level 0 holds the last token, level l > 0 is occupied (2^(l-1) tokens) iff bit l-1 of T-1 is set
+    want = [1] + [(1 << (l - 1)) if ((76 >> (l - 1)) & 1) else 0 for l in range(1, 9)]
+    assert counts.tolist() == want and sum(want) == 77
+    assert all(S[..., l].abs().max() == 0 for l in range(9) if want[l] == 0)
+    # the level states sum to the plain rule's state (recurrent.py:96-100)
+    _, plain = og.recurrent_c(q, k, v, g, beta, l2=og.L2_CHUNK)
+    assert torch.allclose(S.sum(-1), plain, atol=1e-5)
+    # against the token loop with explicit level states of the first statement
+    assert torch.allclose(o.double(), oh.recurrent_states(q, k, v, g, beta, lam), atol=2e-6)
+    # stopping after 40 tokens and continuing from the returned state is the same as one run
+    cut = lambda x, a, b: x[:, a:b]
+    o1, S1, c1 = oh.recurrent_c_state(*(cut(x, 0, 40) for x in (q, k, v, g, beta, lam)))
+    o2, S2, c2 = oh.recurrent_c_state(*(cut(x, 40, 77) for x in (q, k, v, g, beta, lam)), states=S1, counts=c1)
+    assert torch.allclose(torch.cat([o1, o2], 1), o, atol=1e-5) and torch.allclose(S2, S, atol=1e-5)
+    assert c2.tolist() == counts.tolist()
