@@ -243,12 +243,24 @@ int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float
  * l-1 (base.py:41-46).
  * K = 64, V in {64, 128}; l2norm as for the chunk forward (the reference requires the chunk-path l2norm);
  * the plan's chunks_per_segment must be a power of two unless every sequence is one segment; sequences of at most
- * 4096 chunks; L >= 7 + number of bits of the largest chunk index. Zero initial state, no final state. */
+ * 4096 chunks; L >= 7 + number of bits of the largest chunk index. Zero initial state. level_states (nullable): fp32
+ * [n_seq, HV, K, V, L] zeroed by the caller, receives HState.states (recurrent.py:33-36) after the last token of every
+ * sequence -- what hattention_prefill returns (kernel.py:467-575); needs equal sequence lengths, multiples of 64. */
 int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V);
 int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                         const void* lam, int lam_dtype, float lam_div, void* o, const int32_t* plan_host,
-                         const int32_t* plan_dev, int H, int HV, int K, int V, int L, int dtype, float scale, int l2norm,
-                         void* workspace, int64_t workspace_bytes, void* stream);
+                         const void* lam, int lam_dtype, float lam_div, void* o, float* level_states,
+                         const int32_t* plan_host, const int32_t* plan_dev, int H, int HV, int K, int V, int L, int dtype,
+                         float scale, int l2norm, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* One token of the hierarchical rule on explicit level states. Replaces hattention_step (models/hattention/
+ * kernel.py:577-633; step_state / step_output, recurrent.py:134-166; HState.cascade_weak / insert, recurrent.py:44-97).
+ * q, k [B, H, K]; v, o [B, HV, V] (dtype LAMPA_BF16/FP16/FP32); g, beta fp32 [B, HV]; lam [B, HV, L] as above;
+ * states fp32 [B, HV, K, V, L] (HState.states), updated in place; z: the levels 0 .. z-1 are full and cascade into
+ * level z before the token is inserted (0 for an empty state; otherwise 1 + the number of trailing one bits of
+ * tokens_seen - 1). V <= 256, L <= 32. */
+int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g, const float* beta, const void* lam,
+                    int lam_dtype, float lam_div, float* states, void* o, int B, int H, int HV, int K, int V, int L, int z,
+                    int dtype, float scale, int l2norm, void* stream);
 
 /* ------------------------------------------------------------------------------------------------- profiling */
 

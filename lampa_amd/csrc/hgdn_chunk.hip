@@ -70,8 +70,8 @@ __global__ void __launch_bounds__(256)
                      const void* __restrict__ lam, int lam_dtype, float lam_div,
                      const int32_t* __restrict__ chunk_tok0,
                      const int32_t* __restrict__ chunk_len, const unsigned char* __restrict__ tmat,
-                     unsigned char* __restrict__ wrec, float* __restrict__ Nc, float* __restrict__ Oi, int H, int HV,
-                     int L, float scale, int l2norm) {
+                     unsigned char* __restrict__ wrec, float* __restrict__ Nc, float* __restrict__ Oi,
+                     float* __restrict__ hstates, int chunks_per_seq, int H, int HV, int L, float scale, int l2norm) {
   using SM = HgPrepSmem<KT, VT>;
   using REC = HgRec<KT>;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST, NKS = KT / 16;
@@ -290,15 +290,56 @@ __global__ void __launch_bounds__(256)
       }
     }
   };
+  // The last chunk of a sequence, when the caller wants the level states after the last token (HState.states of
+  // the reference, [B, HV, K, V, L]): level l < 7 holds the chunk's own sources j with level(63, j) = l, carried to
+  // the end of the chunk -- N with beta masked to that bucket (the mask acts on the sources, i.e. on T's columns).
+  const bool want_tail = hstates != nullptr && (chunk % chunks_per_seq) == chunks_per_seq - 1;
+  auto tail_tile = [&](int vt, int lvl) {
+    bf16x8 Ub[4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        if (ks >= 2 * (tm + 1)) continue;
+        const bf16x8 t = t_frag(tm, ks);
+        bf16x8 ts;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = 16 * ks + kappa(hh, e);
+          const int lj = j == 63 ? 0 : 32 - __builtin_clz(63 ^ j);
+          ts[e] = (__bf16)(lj == lvl ? (float)t[e] * s_beta[j] : 0.0f);
+        }
+        acc = mfma32(ts, ld_kappa_tr(s_v, SV, 32 * vt, 16 * ks, lane), acc);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] *= s_dk[32 * tm + acc_row(r, hh)];
+      Ub[2 * tm] = acc_to_operand(acc, 0);
+      Ub[2 * tm + 1] = acc_to_operand(acc, 8);
+    }
+    float* out = hstates + ((size_t)(chunk / chunks_per_seq) * HV + hv) * KT * VT * L + lvl;
+#pragma unroll
+    for (int km = 0; km < KT / 32; ++km) {
+      f32x16 acc = zero16();
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) acc = mfma32(ld_kappa_tr(s_k, SK, 32 * km, 16 * ks, lane), Ub[ks], acc);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) out[((size_t)(32 * km + acc_row(r, hh)) * VT + 32 * vt + ln) * L] = acc[r];
+    }
+  };
   // ---- W, P, the chunk's own state N, the K^T fragments (tasks spread over the four waves)
   constexpr int NW = 2 * (KT / 32), NU = VT / 32, NKF = (KT / 32) * 4;
-  for (int task = wave; task < NW + 3 + NU + NKF; task += 4) {
+  const int n_tail = want_tail ? NU * HG_INTRA : 0;
+  for (int task = wave; task < NW + 3 + NU + NKF + n_tail; task += 4) {
     if (task < NW) w_tile(task / (KT / 32), task % (KT / 32));
     else if (task < NW + 3) p_tile(task - NW);
     else if (task < NW + 3 + NU) un_tile(task - NW - 3);
-    else {
+    else if (task < NW + 3 + NU + NKF) {
       const int f = task - NW - 3 - NU;
       frag_store(rec + REC::KF, f, lane, ld_kappa_tr(s_k, SK, 32 * (f / 4), 16 * (f % 4), lane));
+    } else {
+      const int f = task - NW - 3 - NU - NKF;
+      tail_tile(f / HG_INTRA, f % HG_INTRA);
     }
   }
   __syncthreads();
@@ -447,7 +488,8 @@ template <typename T, int KT, int VT>
 __global__ void __launch_bounds__(64 * (HG_CW + 2))
     hgdn_walk_kernel(const GdrPlanView pv, const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
                      const unsigned char* __restrict__ wrec, const float* __restrict__ Nc,
-                     const float* __restrict__ Oi, const float* __restrict__ Xinit, T* __restrict__ o, int HV) {
+                     const float* __restrict__ Oi, const float* __restrict__ Xinit, T* __restrict__ o,
+                     float* __restrict__ hstates, int L, int HV) {
   using REC = HgRec<KT>;
   using SM = HgWalkSmem<KT>;
   constexpr int NKS = KT / 16, SP = SM::SP;
@@ -627,6 +669,21 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
     if (c + 1 < c1) hg_merge<KT>(cs, 0, wave, true, lane, s_acc, S);
     oi_cur = oi_next;
   }
+  // the level states after the sequence's last token (before any carry): level 7 + j for the occupied inter-chunk levels
+  if (hstates && (pv.seg_flags[seg] & SEG_LAST)) {
+    const int cs = cs0 + nc - 1;
+    float* out = hstates + ((size_t)pv.seg_seq[seg] * HV + hv) * KT * VT * L;
+#pragma unroll
+    for (int slot = 0; slot < HG_LPW; ++slot) {
+      const int lvl = slot * HG_CW + wave;
+      if (!((cs >> lvl) & 1) || HG_INTRA + lvl >= L) continue;
+#pragma unroll
+      for (int km = 0; km < KT / 32; ++km)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          out[((size_t)(32 * km + acc_row(r, hh)) * VT + 32 * vslab + ln) * L + HG_INTRA + lvl] = S[slot][km][r];
+    }
+  }
 }
 
 // ---- scan over the segments --------------------------------------------------------------------------------------
@@ -733,7 +790,7 @@ extern "C" int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_
 
 template <typename T, int KT, int VT>
 static int hg_launch(const void* q, const void* k, const void* v, const float* g, const float* beta, const void* lam,
-                     int lam_dtype, float lam_div, void* o, const GdrPlanView pv, int n_seq, int chunks, int segs, int p, int H, int HV, int L,
+                     int lam_dtype, float lam_div, void* o, float* hstates, int chunks_per_seq, const GdrPlanView pv, int n_seq, int chunks, int segs, int p, int H, int HV, int L,
                      float scale, int l2norm, unsigned char* ws, hipStream_t s) {
   const HgWorkspace w = hg_workspace(chunks, segs, HV, KT, VT);
   unsigned char* tf = ws + w.off_t;
@@ -763,7 +820,8 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
                      l2norm);
   LAMPA_PROF(s, "gdr_tinv_kernel");
   hipLaunchKernelGGL((hgdn_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem_p, s, (const T*)q, (const T*)k,
-                     (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, H, HV, L, scale, l2norm);
+                     (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, hstates, chunks_per_seq, H, HV, L,
+                     scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
   const bool split = segs > n_seq;
   if (split) {
@@ -778,7 +836,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   }
   hipLaunchKernelGGL((hgdn_walk_kernel<T, KT, VT>), dim3(segs, HV, VT / 32), dim3(64 * (HG_CW + 2)), smem_w, s, pv,
                      pv.chunk_tok0, pv.chunk_len, rec, Nc, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
-                     HV);
+                     hstates, L, HV);
   LAMPA_PROF(s, "hgdn_walk_kernel");
   return lampa_launch_status();
 }
@@ -789,10 +847,13 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
 // multiplies q, before its kernel; lam_div = 1 takes them as they are). The plan's chunks_per_segment must be a
 // power of two (or at least the longest sequence's chunk count: one segment per sequence); every sequence may hold at
 // most 2^12 chunks and L must cover 7 + the number of chunk-index bits of the longest sequence.
+// level_states (nullable): fp32 [n_seq, HV, K, V, L], ZEROED by the caller; receives the occupied levels' states after
+// the last token of every sequence (the reference's HState.states); needs sequences of equal length, a multiple of 64.
 extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                                    const void* lam, int lam_dtype, float lam_div, void* o, const int32_t* plan_host,
-                                    const int32_t* plan_dev, int H, int HV, int K, int V, int L, int dtype, float scale,
-                                    int l2norm, void* workspace, int64_t workspace_bytes, void* stream) {
+                                    const void* lam, int lam_dtype, float lam_div, void* o, float* level_states,
+                                    const int32_t* plan_host, const int32_t* plan_dev, int H, int HV, int K, int V, int L,
+                                    int dtype, float scale, int l2norm, void* workspace, int64_t workspace_bytes,
+                                    void* stream) {
   if (!q || !k || !v || !g || !beta || !lam || !o || !plan_host || !plan_dev) return LAMPA_ERR_INVALID;
   if (H < 1 || HV < H || HV % H != 0 || l2norm < 0 || l2norm > 2 || L < HG_INTRA) return LAMPA_ERR_INVALID;
   if (lam_dtype < 0 || lam_dtype > 2 || !(lam_div > 0.0f)) return LAMPA_ERR_INVALID;
@@ -814,6 +875,10 @@ extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v,
     max_nc = nc > max_nc ? nc : max_nc;
   }
   if (max_nc > (1 << HG_NLV)) return LAMPA_ERR_UNSUPPORTED;
+  if (level_states) {  // every sequence: the same whole number of chunks
+    const int total = plan_host[PLAN_TOTAL_TOKENS];
+    if (max_nc < 1 || (int64_t)max_nc * n_seq != chunks || (int64_t)chunks * GDR_C != total) return LAMPA_ERR_INVALID;
+  }
   int bits = 0;
   while ((1 << bits) < max_nc) ++bits;
   if (HG_INTRA + bits > L) return LAMPA_ERR_INVALID;
@@ -822,7 +887,7 @@ extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v,
   unsigned char* ws = (unsigned char*)workspace;
   const GdrPlanView pv = gdr_plan_view(plan_host, plan_dev);
 #define HG_CASE(TT, KK, VV) \
-  return hg_launch<TT, KK, VV>(q, k, v, g, beta, lam, lam_dtype, lam_div, o, pv, n_seq, chunks, segs, p, H, HV, L, scale, l2norm, ws, s)
+  return hg_launch<TT, KK, VV>(q, k, v, g, beta, lam, lam_dtype, lam_div, o, level_states, max_nc, pv, n_seq, chunks, segs, p, H, HV, L, scale, l2norm, ws, s)
   if (dtype == GDR_BF16) {
     if (V == 64) HG_CASE(__bf16, 64, 64);
     if (V == 128) HG_CASE(__bf16, 64, 128);

@@ -1,0 +1,150 @@
+// One token of the hierarchical (level-weighted) gated delta rule on explicit level states.
+//
+// Replaces hattention_step (reference chengjiang123/Lampa, models/hattention/kernel.py:577-633) with
+// step_state / step_output (recurrent.py:134-166) and HState.cascade_weak / insert (recurrent.py:44-97):
+//   cascade   the full levels 0 .. z-1 are added into level z and emptied (lowest first);
+//   gate      S_l <- a (S_l - b k (k^T S_l)) for every level, a = e^g;
+//   insert    S_0 <- b k v^T;
+//   output    o = q^T sum_l lambda_l S_l      (q l2-normalised and scaled, k l2-normalised, kernel.py:613-616).
+// The level states are the reference's HState.states: fp32 [B, HV, K, V, L] with the level index fastest. Which levels
+// are full depends only on the number of tokens seen, so the caller passes z (0 = nothing to merge).
+// One workgroup per (sequence, value head), one thread per value column: two passes over the K rows of its column
+// (k^T S_l first, then the update), every row's L level values being contiguous.
+#include "gdr_common.h"
+
+#define HGS_LMAX 32
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    hgdn_step_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                     const float* __restrict__ g, const float* __restrict__ beta, const void* __restrict__ lam,
+                     int lam_dtype, float lam_div, float* __restrict__ states, T* __restrict__ o, int H, int HV, int K,
+                     int V, int L, int z, float scale, int l2norm) {
+  extern __shared__ float s_qk[];  // qn [K], kn [K], lambda [HGS_LMAX], reduction scratch [8]
+  float* s_q = s_qk;
+  float* s_k = s_qk + K;
+  float* s_l = s_qk + 2 * K;
+  float* s_red = s_l + HGS_LMAX;
+  const int b = blockIdx.x / HV, hv = blockIdx.x % HV, h = hv / (HV / H);
+  const int tid = threadIdx.x;
+  const T* qp = q + ((size_t)b * H + h) * K;
+  const T* kp = k + ((size_t)b * H + h) * K;
+  float qs = 0.0f, ks = 0.0f;
+  for (int i = tid; i < K; i += blockDim.x) {
+    const float qi = GdrElem<T>::to_float(qp[i]), ki = GdrElem<T>::to_float(kp[i]);
+    s_q[i] = qi;
+    s_k[i] = ki;
+    qs = __builtin_fmaf(qi, qi, qs);
+    ks = __builtin_fmaf(ki, ki, ks);
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    qs += __shfl_xor(qs, off);
+    ks += __shfl_xor(ks, off);
+  }
+  if ((tid & 63) == 0) {
+    s_red[2 * (tid >> 6)] = qs;
+    s_red[2 * (tid >> 6) + 1] = ks;
+  }
+  if (tid < L) {
+    const size_t li = ((size_t)b * HV + hv) * L + tid;
+    float x = lam_dtype == GDR_FP32   ? reinterpret_cast<const float*>(lam)[li]
+              : lam_dtype == GDR_BF16 ? (float)reinterpret_cast<const __bf16*>(lam)[li]
+                                      : (float)reinterpret_cast<const _Float16*>(lam)[li];
+    if (lam_div != 1.0f) {  // lambda / scale, rounded to lambda's own type as the element-wise division would
+      x = __fdiv_rn(x, lam_div);
+      x = lam_dtype == GDR_FP32 ? x : lam_dtype == GDR_BF16 ? (float)(__bf16)x : (float)(_Float16)x;
+    }
+    s_l[tid] = x;
+  }
+  __syncthreads();
+  qs = 0.0f;
+  ks = 0.0f;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
+    qs += s_red[2 * w];
+    ks += s_red[2 * w + 1];
+  }
+  float rq = scale, rk = 1.0f;
+  if (l2norm == GDR_L2_CHUNK) {
+    rq = scale / __fsqrt_rn(qs + 1e-6f);
+    rk = 1.0f / __fsqrt_rn(ks + 1e-6f);
+  } else if (l2norm == GDR_L2_RECURRENT) {
+    rq = scale / (__fsqrt_rn(qs) + 1e-6f);
+    rk = 1.0f / (__fsqrt_rn(ks) + 1e-6f);
+  }
+  const int j = tid;
+  if (j >= V) return;
+  const float a = __expf(g[(size_t)b * HV + hv]), bt = beta[(size_t)b * HV + hv];
+  const float vj = GdrElem<T>::to_float(v[((size_t)b * HV + hv) * V + j]);
+  float* col = states + (((size_t)b * HV + hv) * K * V + j) * L;  // row i of this column: col + i * V * L
+  const size_t rs = (size_t)V * L;
+
+  auto load_cascaded = [&](const float* p, float* S) {
+#pragma unroll
+    for (int l = 0; l < HGS_LMAX; ++l) S[l] = l < L ? p[l] : 0.0f;
+    if (z > 0) {
+      float acc = S[0];
+#pragma unroll
+      for (int l = 1; l < HGS_LMAX; ++l) {
+        if (l < z) acc = S[l] + acc;
+        else if (l == z) S[l] = S[l] + acc;
+      }
+#pragma unroll
+      for (int l = 0; l < HGS_LMAX; ++l)
+        if (l < z) S[l] = 0.0f;
+    }
+  };
+  float d[HGS_LMAX];
+#pragma unroll
+  for (int l = 0; l < HGS_LMAX; ++l) d[l] = 0.0f;
+  for (int i = 0; i < K; ++i) {
+    float S[HGS_LMAX];
+    load_cascaded(col + i * rs, S);
+    const float ki = s_k[i] * rk;
+#pragma unroll
+    for (int l = 1; l < HGS_LMAX; ++l) d[l] = __builtin_fmaf(ki, S[l], d[l]);
+  }
+  float acc_o = 0.0f;
+  for (int i = 0; i < K; ++i) {
+    float S[HGS_LMAX];
+    load_cascaded(col + i * rs, S);
+    const float ki = s_k[i] * rk, qi = s_q[i] * rq;
+    float sl = 0.0f;
+    S[0] = bt * ki * vj;
+#pragma unroll
+    for (int l = 1; l < HGS_LMAX; ++l) S[l] = a * (S[l] - bt * ki * d[l]);
+#pragma unroll
+    for (int l = 0; l < HGS_LMAX; ++l)
+      if (l < L) {
+        col[i * rs + l] = S[l];
+        sl = __builtin_fmaf(s_l[l], S[l], sl);
+      }
+    acc_o = __builtin_fmaf(qi, sl, acc_o);
+  }
+  o[((size_t)b * HV + hv) * V + j] = GdrElem<T>::from_float(acc_o);
+}
+
+// q, k [B, H, K]; v, o [B, HV, V] (dtype 0 bf16 / 1 fp16 / 2 fp32); g (log decay), beta fp32 [B, HV]; lam [B, HV, L] of
+// lam_dtype, used as lam / lam_div rounded to its type; states fp32 [B, HV, K, V, L], updated in place;
+// z: the levels 0 .. z-1 are full and cascade into level z (0: the state is empty). V <= 256, L <= 32.
+extern "C" int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                               const void* lam, int lam_dtype, float lam_div, float* states, void* o, int B, int H, int HV,
+                               int K, int V, int L, int z, int dtype, float scale, int l2norm, void* stream) {
+  if (!q || !k || !v || !g || !beta || !lam || !states || !o) return LAMPA_ERR_INVALID;
+  if (B < 0 || H < 1 || HV < H || HV % H != 0 || K < 1 || V < 1 || L < 1 || z < 0 || z >= L) return LAMPA_ERR_INVALID;
+  if (l2norm < 0 || l2norm > 2 || lam_dtype < 0 || lam_dtype > 2 || !(lam_div > 0.0f)) return LAMPA_ERR_INVALID;
+  if (V > 256 || L > HGS_LMAX || K > 4096 || dtype < 0 || dtype > 2) return LAMPA_ERR_UNSUPPORTED;
+  if (B == 0) return LAMPA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = V <= 64 ? 64 : (V <= 128 ? 128 : 256);
+  const size_t smem = (2 * (size_t)K + HGS_LMAX + 8) * sizeof(float);
+  LAMPA_PROF(s, "start");
+#define HGS_CASE(TT)                                                                                                \
+  hipLaunchKernelGGL((hgdn_step_kernel<TT>), dim3(B * HV), dim3(threads), smem, s, (const TT*)q, (const TT*)k,      \
+                     (const TT*)v, g, beta, lam, lam_dtype, lam_div, states, (TT*)o, H, HV, K, V, L, z, scale, l2norm)
+  if (dtype == GDR_BF16) HGS_CASE(__bf16);
+  else if (dtype == GDR_FP16) HGS_CASE(_Float16);
+  else HGS_CASE(float);
+#undef HGS_CASE
+  LAMPA_PROF(s, "hgdn_step_kernel");
+  return lampa_launch_status();
+}

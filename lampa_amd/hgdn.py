@@ -8,12 +8,19 @@ reaches it: q l2-normalised and scaled, k l2-normalised (``kernel.py:100-101``),
 (``gated_delta_rule_apis.py:68-70``; the kernel does it, with the rounding of a division in lambda's dtype), weak
 hierarchy, base 2.
 
-Differences a caller can observe: forward only; ``output_final_state=True`` (the prefill and single-step branches,
-``gated_delta_rule_apis.py:92-128``) raises ``NotImplementedError``; head sizes K = 64 and V in {64, 128} only.
+All three branches of the operator are here: outputs only (``hattention_kernel``), prefill returning the level
+states (``hattention_prefill``, ``kernel.py:467-575``: the whole chunks through the chunk kernels, the remaining
+tokens one by one) and the single-token step on an ``HState`` (``hattention_step``, ``kernel.py:577-633``).
+
+Differences a caller can observe: forward only; the chunk kernels take K = 64 and V in {64, 128} (the single-token step
+takes any K and V <= 256); ``HState.counts`` lives on the host (the reference keeps it on the device and synchronises
+on every comparison, ``recurrent.py:44-56``); the step computes its output from the fp32 states, the reference rounds
+them to the output type first (``kernel.py:628-631``).
 """
 import ctypes
+import enum
 import warnings
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -27,6 +34,68 @@ SCALE_LAMBDA = True  # gated_delta_rule_apis.py:17
 CHUNKS_PER_SEGMENT: Optional[int] = None
 
 _plan_cache = {}
+
+
+class HType(enum.Enum):  # base.py:12-14
+    WEAK = 0
+    STRONG = 1
+
+
+class HStruct(enum.Enum):  # base.py:17-19
+    MAMBA2 = 0
+    GDELTA = 1
+
+
+class HState(object):
+    """Level states of one batch: ``recurrent.py:9-132``. ``states`` fp32 ``[B, HV, K, V, L]``, ``counts`` int32
+    ``[L]`` (tokens per level). The cascade, the gate and the insert run inside the step kernel; the bookkeeping of
+    the counts (``cascade_weak``, ``recurrent.py:44-56``) is replayed on host integers."""
+
+    def __init__(self, base: int, htype: HType, hstruct: HStruct, shape: Tuple[int, ...], dtype: torch.dtype,
+                 device: torch.device) -> None:
+        if htype != HType.WEAK or base != 2 or hstruct != HStruct.GDELTA:
+            raise NotImplementedError
+        self.base, self.htype, self.hstruct = base, htype, hstruct
+        self.shape, self.dtype, self.device = tuple(shape), dtype, device
+        self.max_num_levels = self.shape[-1]
+        self.states = torch.zeros(self.shape, dtype=self.dtype, device=self.device)
+        self.counts = torch.zeros(self.max_num_levels, dtype=torch.int32)
+
+    @property
+    def tokens_seen(self) -> int:
+        return int(self.counts.sum())
+
+    def cascade_weak(self) -> int:
+        """Replays ``recurrent.py:44-56`` on the counts; returns the level that received the full ones (0: none)."""
+        z = 0
+        for level in range(self.max_num_levels):
+            capacity = self.base ** level
+            if int(self.counts[level]) == capacity:
+                if level + 1 >= self.max_num_levels:
+                    raise ValueError("the state has no level left for this many tokens")
+                self.counts[level + 1] += self.counts[level]
+                self.counts[level] = 0
+                z = level + 1
+            elif int(self.counts[level]) < capacity:
+                break
+            else:
+                raise ValueError
+        return z
+
+    def reset_states(self) -> None:
+        self.states = torch.zeros_like(self.states)
+
+    def replace(self, other: "HState") -> None:
+        if not all([tuple(self.shape) == tuple(other.shape), self.base == other.base, self.htype == other.htype,
+                    self.dtype == other.dtype, self.device == other.device]):
+            raise ValueError("Shape, dtype or device mismatch")
+        self.states = other.states
+
+    def to(self, dtype: Optional[torch.dtype] = None, device: Optional[torch.device] = None) -> "HState":
+        new_state = HState(self.base, self.htype, self.hstruct, self.shape, dtype or self.dtype, device or self.device)
+        new_state.states = self.states.to(dtype=new_state.dtype, device=new_state.device)
+        new_state.counts = self.counts.clone()
+        return new_state
 
 
 def num_levels(length: int, chunk: int = 64) -> int:
@@ -65,7 +134,7 @@ def _plan(B: int, T: int, device, n_value_heads: int, n_slabs: int):
 
 class _ForwardOnly(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, g, lam, beta, scale, lam_div):
+    def forward(ctx, q, k, v, g, lam, beta, scale, lam_div, level_states=None):
         require_cuda(q, k, v, g, lam, beta)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
@@ -81,7 +150,7 @@ class _ForwardOnly(torch.autograd.Function):
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         o = torch.empty_like(v)
         check(lib.lampa_hgdn_chunk_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(lam), _gd._DTYPES[lam.dtype],
-                                       float(lam_div), ptr(o),
+                                       float(lam_div), ptr(o), ptr(level_states),
                                        ctypes.c_void_p(plan_host.data_ptr()), ptr(plan_dev), H, HV, K, V, L,
                                        _gd._DTYPES[q.dtype], float(scale), _gd.L2_CHUNK, ptr(ws), ws_bytes, stream_of(q)),
               "lampa_hgdn_chunk_fwd")
@@ -97,7 +166,9 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
                              output_final_state: bool = False, cu_seqlens: Optional[torch.LongTensor] = None,
                              head_first: bool = False, use_qk_l2norm_in_kernel: bool = False):
     """``gated_delta_rule_apis.py:21-134``. q, k ``[B,T,H,K]``, v ``[B,T,HV,V]``, g, beta ``[B,T,HV]``, l
-    ``[B,T,HV,L]`` with ``L >= num_levels(T)``; T a multiple of 64. Returns ``(o, None)``."""
+    ``[B,T,HV,L]`` with ``L >= num_levels(T)``. ``output_final_state=False``: T a multiple of 64, returns ``(o, None)``;
+    ``output_final_state=True``: any T, returns ``(o, HState)``; with ``initial_state`` (an ``HState``) and T = 1: one
+    step, returns ``(o, initial_state)`` updated in place."""
     assert q.dtype == k.dtype == v.dtype
     assert q.dtype != torch.float32, "ChunkGatedDeltaRuleFunction does not support float32. Please use bfloat16."
     assert len(beta.shape) == 3, "beta must be of shape [B, T, H] if head_first=False, or [B, H, T] otherwise."
@@ -116,16 +187,72 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
     if scale is None:
         scale = k.shape[-1] ** -0.5
     lam_div = scale if SCALE_LAMBDA else 1.0  # l = l / scale (gated_delta_rule_apis.py:68-70), done by the kernel
-    if output_final_state or initial_state is not None:
-        raise NotImplementedError("hierarchical final / initial states are not built")
     B, T, H, K = q.shape
-    if T % 64 != 0:  # chunkwise_hgdn.py:598-601
-        raise ValueError(f"T={T} and BT=64")
-    if K != 64 or v.shape[-1] not in (64, 128):
-        raise NotImplementedError("hierarchical forward: K = 64 and V in {64, 128} only")
-    if num_levels(T) > l.shape[-1]:  # chunkwise_hgdn.py:718-721
+    HV, V, L = v.shape[2], v.shape[3], l.shape[-1]
+    if output_final_state is False:
+        if initial_state is not None:
+            raise NotImplementedError
+        _check_chunk_shapes(T, K, V, L)
+        if T % 64 != 0:  # chunkwise_hgdn.py:598-601
+            raise ValueError(f"T={T} and BT=64")
+        return _ForwardOnly.apply(q, k, v, g, l, beta, scale, lam_div), None
+    if initial_state is None:  # hattention_prefill, kernel.py:467-575
+        require_cuda(q, k, v, g, l, beta)
+        hstate = HState(2, HType.WEAK, HStruct.GDELTA, (B, HV, K, V, L), torch.float32, q.device)
+        T0 = T - T % 64
+        o = torch.empty_like(v)
+        if T0:
+            _check_chunk_shapes(T0, K, V, L)
+            cut = lambda x: x[:, :T0]
+            o[:, :T0] = _ForwardOnly.apply(cut(q), cut(k), cut(v), cut(g), cut(l), cut(beta), scale, lam_div,
+                                           hstate.states)
+            # counts after T0 tokens (kernel.py:451-462): the last token alone in level 0, level l > 0 holds 2^(l-1)
+            # tokens iff that bit of T0 - 1 is set
+            hstate.counts[0] = 1
+            for level in range(1, L):
+                hstate.counts[level] = (1 << (level - 1)) if ((T0 - 1) >> (level - 1)) & 1 else 0
+        for t in range(T0, T):
+            o[:, t] = _step(hstate, q[:, t], k[:, t], v[:, t], g[:, t], l[:, t], beta[:, t], scale, lam_div)
+        return o, hstate
+    if not all([q.ndim == 4, q.shape[1] == 1, k.ndim == 4, k.shape[1] == 1, v.ndim == 4, v.shape[1] == 1,
+                beta.ndim == 3, beta.shape[1] == 1, g.ndim == 3, g.shape[1] == 1, l.ndim == 4, l.shape[1] == 1]):
+        raise ValueError
+    o = _step(initial_state, q[:, 0], k[:, 0], v[:, 0], g[:, 0], l[:, 0], beta[:, 0], scale, lam_div)
+    return o.unsqueeze(1), initial_state
+
+
+def _check_chunk_shapes(T: int, K: int, V: int, L: int) -> None:
+    if K != 64 or V not in (64, 128):
+        raise NotImplementedError("hierarchical chunk kernels: K = 64 and V in {64, 128} only")
+    if num_levels(T) > L:  # chunkwise_hgdn.py:718-721
         raise ValueError
     if (T // 64) > 4096:
-        raise NotImplementedError("hierarchical forward: at most 4096 chunks per sequence")
-    o = _ForwardOnly.apply(q, k, v, g, l, beta, scale, lam_div)
-    return o, None
+        raise NotImplementedError("hierarchical chunk kernels: at most 4096 chunks per sequence")
+
+
+def _step(hstate: HState, q, k, v, g, l, beta, scale, lam_div) -> torch.Tensor:
+    """``hattention_step`` (``kernel.py:577-633``) on ``[B, H, K]`` / ``[B, HV, V]`` / ``[B, HV]`` / ``[B, HV, L]``
+    slices; updates ``hstate`` in place and returns ``o [B, HV, V]``."""
+    if not all([q.ndim == 3, k.ndim == 3, v.ndim == 3, beta.ndim == 2, g.ndim == 2, l.ndim == 3,
+                hstate.dtype == torch.float32, q.dtype == k.dtype == v.dtype, hstate.base == 2,
+                hstate.htype == HType.WEAK, hstate.hstruct == HStruct.GDELTA]):
+        raise TypeError
+    require_cuda(q, k, v, g, l, beta, hstate.states)
+    B, H, K = q.shape
+    HV, V, L = v.shape[1], v.shape[2], l.shape[-1]
+    if tuple(hstate.shape) != (B, HV, K, V, L):
+        raise ValueError("Shape, dtype or device mismatch")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
+    if l.dtype not in _gd._DTYPES:
+        l = l.to(torch.float32)
+    l = l.contiguous()
+    if not hstate.states.is_contiguous():
+        hstate.states = hstate.states.contiguous()
+    z = hstate.cascade_weak()
+    o = torch.empty_like(v)
+    check(_capi.lib().lampa_hgdn_step(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(l), _gd._DTYPES[l.dtype],
+                                      float(lam_div), ptr(hstate.states), ptr(o), B, H, HV, K, V, L, z,
+                                      _gd._DTYPES[q.dtype], float(scale), _gd.L2_CHUNK, stream_of(q)), "lampa_hgdn_step")
+    hstate.counts[0] += 1
+    return o

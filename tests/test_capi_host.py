@@ -102,12 +102,12 @@ def test_hierarchical_forward_argument_checks(lib):
     assert lib.lampa_hgdn_chunk_workspace_bytes(-1, 30, 8, 64, 64) == -1
     d = ctypes.c_void_p(0x1000)  # 16-byte aligned dummy
 
-    def call(cu, cps, L=20, K=64, V=64, q=d, ws=None, dtype=0, lam_dtype=0):
+    def call(cu, cps, L=20, K=64, V=64, q=d, ws=None, dtype=0, lam_dtype=0, states=None):
         arr = (ctypes.c_int64 * len(cu))(*cu)
         size = lib.lampa_gdr_plan_size(arr, len(cu) - 1, cps)
         plan = torch.zeros(size, dtype=torch.int32)
         assert lib.lampa_gdr_plan_fill(arr, len(cu) - 1, cps, ctypes.c_void_p(plan.data_ptr())) == 0
-        return lib.lampa_hgdn_chunk_fwd(q, d, d, d, d, d, lam_dtype, 0.125, d, ctypes.c_void_p(plan.data_ptr()), d, 2, 2, K, V, L, dtype,
+        return lib.lampa_hgdn_chunk_fwd(q, d, d, d, d, d, lam_dtype, 0.125, d, states, ctypes.c_void_p(plan.data_ptr()), d, 2, 2, K, V, L, dtype,
                                         0.125, 1, ws, 0, None)
 
     assert call([0, 4096], 8, q=None) == -1                      # null pointer
@@ -121,6 +121,13 @@ def test_hierarchical_forward_argument_checks(lib):
     assert call([0, 4096], 100, L=13) == -2                      # one segment per sequence: any segment length
     assert call([0, 64 * 4097], 4096, L=32) == -4                # more than 4096 chunks in a sequence
     assert call([0, 64 * 4096], 4096, L=19) == -2
+    assert call([0, 4096, 8192], 8, L=13, states=d) == -2         # level states: equal whole-chunk sequences
+    assert call([0, 4096, 8000], 8, L=13, states=d) == -1
+    assert call([0, 4096, 12288], 8, L=14, states=d) == -1
+    # the single-token step
+    assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 64, 13, 13, 0, 0.125, 1, None) == -1  # z < L
+    assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 512, 13, 1, 0, 0.125, 1, None) == -4
+    assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 0, 2, 2, 64, 64, 13, 0, 0, 0.125, 1, None) == 0     # empty batch
 
 
 def test_operators_refuse_cpu_tensors():

@@ -105,5 +105,67 @@ def test_argument_checks(device):
                                       use_qk_l2norm_in_kernel=True)
     with pytest.raises(ValueError):
         hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam[..., :7], beta, use_qk_l2norm_in_kernel=True)
-    with pytest.raises(NotImplementedError):
-        hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, output_final_state=True, use_qk_l2norm_in_kernel=True)
+    with pytest.raises(NotImplementedError):  # an initial state without output_final_state (gated_delta_rule_apis.py:73-74)
+        hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, initial_state=object(), use_qk_l2norm_in_kernel=True)
+
+
+# ------------------------------------------------------------------------------------ level states: prefill and step
+def _state_errors(got: "hgdn.HState", want_states, want_counts):
+    assert got.counts.tolist() == want_counts.tolist()
+    return _errors(got.states, want_states)
+
+
+@pytest.mark.parametrize("T,cps", [(64, None), (1024, None), (2560, 8), (1000, None), (4096 + 37, 16)])
+def test_prefill_returns_the_level_states(device, T, cps):
+    q, k, v, g, beta, lam = _inputs(2, T, 2, 64, 64, torch.bfloat16, seed=T + 1, g_scale=0.3, L=hgdn.num_levels(T) + 1)
+    old = hgdn.CHUNKS_PER_SEGMENT
+    hgdn.CHUNKS_PER_SEGMENT = cps
+    try:
+        o, st = hgdn.chunk_h_gated_delta_rule(*(x.to(device) for x in (q, k, v, g, lam, beta)), output_final_state=True,
+                                              use_qk_l2norm_in_kernel=True)
+    finally:
+        hgdn.CHUNKS_PER_SEGMENT = old
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, lam / 0.125, scale=0.125)
+    max_abs, mean_rel = _errors(o, want_o)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"o: {max_abs:.3e} {mean_rel:.3e}"
+    max_abs, mean_rel = _state_errors(st, want_s, want_c)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"states: {max_abs:.3e} {mean_rel:.3e}"
+    assert st.states.shape == (2, 2, 64, 64, lam.shape[-1]) and st.states.dtype == torch.float32
+
+
+def test_steps_continue_a_prefill(device):
+    # 256 tokens through the chunk kernels, then 70 single-token calls with the returned state: one run of 326 tokens
+    T0, T1 = 256, 70
+    q, k, v, g, beta, lam = _inputs(1, T0 + T1, 2, 64, 128, torch.bfloat16, seed=3, HV=4, g_scale=0.3, L=11)
+    d = [x.to(device) for x in (q, k, v, g, lam, beta)]
+    o0, st = hgdn.chunk_h_gated_delta_rule(*(x[:, :T0] for x in d), output_final_state=True, use_qk_l2norm_in_kernel=True)
+    outs = [o0]
+    for t in range(T0, T0 + T1):
+        o_t, st2 = hgdn.chunk_h_gated_delta_rule(*(x[:, t:t + 1] for x in d), initial_state=st, output_final_state=True,
+                                                 use_qk_l2norm_in_kernel=True)
+        assert st2 is st and o_t.shape == (1, 1, 4, 128)
+        outs.append(o_t)
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, lam / 0.125, scale=0.125)
+    max_abs, mean_rel = _errors(torch.cat(outs, 1), want_o)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"o: {max_abs:.3e} {mean_rel:.3e}"
+    max_abs, mean_rel = _state_errors(st, want_s, want_c)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"states: {max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_steps_from_an_empty_state_any_head_size(device):
+    # fewer than 64 tokens: the prefill is the token-serial kernel alone (fp32 arithmetic on bf16 inputs)
+    gen = torch.Generator().manual_seed(4)
+    T, H, K, V, L = 45, 3, 32, 48, 8
+    q, k, v = (torch.randn(2, T, H, d, generator=gen).bfloat16() for d in (K, K, V))
+    g = -0.3 * torch.rand(2, T, H, generator=gen)
+    beta = torch.rand(2, T, H, generator=gen)
+    lam = torch.randn(2, T, H, L, generator=gen).bfloat16()
+    o, st = hgdn.chunk_h_gated_delta_rule(*(x.to(device) for x in (q, k, v, g, lam, beta)), scale=0.25,
+                                          output_final_state=True, use_qk_l2norm_in_kernel=True)
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, (lam / 0.25), scale=0.25)
+    assert st.counts.tolist() == want_c.tolist()
+    assert _errors(o, want_o)[0] <= 2e-2 and _errors(st.states, want_s)[0] <= 1e-4
+    with pytest.raises(ValueError):  # one more level than the state has
+        for _ in range(100):
+            hgdn.chunk_h_gated_delta_rule(*(x[:, :1].to(device) for x in (q, k, v, g, lam, beta)), scale=0.25,
+                                          initial_state=st, output_final_state=True, use_qk_l2norm_in_kernel=True)
