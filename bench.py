@@ -308,12 +308,40 @@ def main():
             hstage[name] = hstage.get(name, 0.0) + 1e3 * ms / 10
     live = sum(bin(c).count("1") for c in range(T_H // 64)) * H  # (chunk, head, level) triples that hold a state
     hgdn_flop = (T_H // 64) * H * 2 * 64 * 64 * (3 * K + 2 * V + 42) + live * 6 * 64 * K * V
+    # prefill (outputs + level states) and the single-token step that continues it
+    for _ in range(3):
+        _, hst = hgdn.chunk_h_gated_delta_rule(qh, kh, vh, gh, lam, bh, output_final_state=True,
+                                               use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        _, hst = hgdn.chunk_h_gated_delta_rule(qh, kh, vh, gh, lam, bh, output_final_state=True,
+                                               use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    prefill_us = 1e6 * (time.perf_counter() - t0) / 10
+    one = [x[:, :1].contiguous() for x in (qh, kh, vh, gh, lam, bh)]
+    import warnings as _w
+    with _w.catch_warnings():
+        _w.simplefilter("ignore")  # the operator warns when seq_len (1) < num_heads, as the reference does
+        for _ in range(5):
+            hgdn.chunk_h_gated_delta_rule(*one, initial_state=hst, output_final_state=True, use_qk_l2norm_in_kernel=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(50):
+            hgdn.chunk_h_gated_delta_rule(*one, initial_state=hst, output_final_state=True, use_qk_l2norm_in_kernel=True)
+        torch.cuda.synchronize()
+    step_us = 1e6 * (time.perf_counter() - t0) / 50
+    step_bytes = 2 * hst.states.numel() * 4
+    del hst, one
     hgdn_info = {
         "workload": f"hierarchical gated-delta forward, B=1 H={H} T={T_H} K=V={K}, L={L_H} levels, bf16, weak "
                     "hierarchy base 2",
         "us": round(hgdn_us, 1), "hits_per_s": round(T / (hgdn_us * 1e-6), 1),
         "kernel_us": {n: round(v_, 1) for n, v_ in hstage.items()},
         "mfma_frac": round(hgdn_flop / (hgdn_us * 1e-6) / 2.5e15, 4),
+        "prefill_us": round(prefill_us, 1),
+        "step": {"us": round(step_us, 1), "state_bytes_read_and_written": step_bytes,
+                 "hbm_frac": round(step_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
         "note": "wall clock of chunk_h_gated_delta_rule; mfma_frac = algorithmic flops "
                 "(per chunk and head 2*64*64*(3K+2V+42) for the chunk-local products with triangular factors counted as such, 6*64*K*V per occupied level) "
                 "over the bf16 dense peak",

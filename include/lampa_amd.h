@@ -257,7 +257,7 @@ int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const floa
  * q, k [B, H, K]; v, o [B, HV, V] (dtype LAMPA_BF16/FP16/FP32); g, beta fp32 [B, HV]; lam [B, HV, L] as above;
  * states fp32 [B, HV, K, V, L] (HState.states), updated in place; z: the levels 0 .. z-1 are full and cascade into
  * level z before the token is inserted (0 for an empty state; otherwise 1 + the number of trailing one bits of
- * tokens_seen - 1). V <= 256, L <= 32. */
+ * tokens_seen - 1). L <= 32. */
 int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g, const float* beta, const void* lam,
                     int lam_dtype, float lam_div, float* states, void* o, int B, int H, int HV, int K, int V, int L, int z,
                     int dtype, float scale, int l2norm, void* stream);

@@ -8,11 +8,15 @@
 //   output    o = q^T sum_l lambda_l S_l      (q l2-normalised and scaled, k l2-normalised, kernel.py:613-616).
 // The level states are the reference's HState.states: fp32 [B, HV, K, V, L] with the level index fastest. Which levels
 // are full depends only on the number of tokens seen, so the caller passes z (0 = nothing to merge).
-// One workgroup per (sequence, value head), one thread per value column: two passes over the K rows of its column
-// (k^T S_l first, then the update), every row's L level values being contiguous.
+// Workgroup per (sequence, value head, 16 value columns), 256 threads = 16 row groups x 16 columns: every thread walks
+// the rows i = group, group + 16, ... of its column twice (k^T S_l first, summed over the groups through LDS, then the
+// update); a row's L level values are contiguous, 16 columns of a row are one contiguous piece.
 #include "gdr_common.h"
 
 #define HGS_LMAX 32
+
+#define HGS_COLS 16
+#define HGS_GROUPS 16
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -20,11 +24,12 @@ __global__ void __launch_bounds__(256)
                      const float* __restrict__ g, const float* __restrict__ beta, const void* __restrict__ lam,
                      int lam_dtype, float lam_div, float* __restrict__ states, T* __restrict__ o, int H, int HV, int K,
                      int V, int L, int z, float scale, int l2norm) {
-  extern __shared__ float s_qk[];  // qn [K], kn [K], lambda [HGS_LMAX], reduction scratch [8]
+  extern __shared__ float s_qk[];  // q [K], k [K], lambda [HGS_LMAX], norm scratch [8], partial sums
   float* s_q = s_qk;
   float* s_k = s_qk + K;
   float* s_l = s_qk + 2 * K;
   float* s_red = s_l + HGS_LMAX;
+  float* s_part = s_red + 8;  // [HGS_GROUPS][HGS_COLS][HGS_LMAX + 1]
   const int b = blockIdx.x / HV, hv = blockIdx.x % HV, h = hv / (HV / H);
   const int tid = threadIdx.x;
   const T* qp = q + ((size_t)b * H + h) * K;
@@ -59,7 +64,7 @@ __global__ void __launch_bounds__(256)
   __syncthreads();
   qs = 0.0f;
   ks = 0.0f;
-  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
+  for (int w = 0; w < 4; ++w) {
     qs += s_red[2 * w];
     ks += s_red[2 * w + 1];
   }
@@ -71,11 +76,13 @@ __global__ void __launch_bounds__(256)
     rq = scale / (__fsqrt_rn(qs) + 1e-6f);
     rk = 1.0f / (__fsqrt_rn(ks) + 1e-6f);
   }
-  const int j = tid;
-  if (j >= V) return;
+  const int grp = tid / HGS_COLS, jl = tid % HGS_COLS;
+  const int j = blockIdx.y * HGS_COLS + jl;
+  const bool live = j < V;
+  const int jc = live ? j : V - 1;  // (idle threads shadow the last column and store nothing)
   const float a = __expf(g[(size_t)b * HV + hv]), bt = beta[(size_t)b * HV + hv];
-  const float vj = GdrElem<T>::to_float(v[((size_t)b * HV + hv) * V + j]);
-  float* col = states + (((size_t)b * HV + hv) * K * V + j) * L;  // row i of this column: col + i * V * L
+  const float vj = GdrElem<T>::to_float(v[((size_t)b * HV + hv) * V + jc]);
+  float* col = states + (((size_t)b * HV + hv) * K * V + jc) * L;  // row i of this column: col + i * V * L
   const size_t rs = (size_t)V * L;
 
   auto load_cascaded = [&](const float* p, float* S) {
@@ -96,15 +103,27 @@ __global__ void __launch_bounds__(256)
   float d[HGS_LMAX];
 #pragma unroll
   for (int l = 0; l < HGS_LMAX; ++l) d[l] = 0.0f;
-  for (int i = 0; i < K; ++i) {
+  for (int i = grp; i < K; i += HGS_GROUPS) {
     float S[HGS_LMAX];
     load_cascaded(col + i * rs, S);
     const float ki = s_k[i] * rk;
 #pragma unroll
     for (int l = 1; l < HGS_LMAX; ++l) d[l] = __builtin_fmaf(ki, S[l], d[l]);
   }
+  float* mine = s_part + (grp * HGS_COLS + jl) * (HGS_LMAX + 1);
+#pragma unroll
+  for (int l = 1; l < HGS_LMAX; ++l)
+    if (l < L) mine[l] = d[l];
+  __syncthreads();
+#pragma unroll
+  for (int l = 1; l < HGS_LMAX; ++l) {
+    if (l >= L) continue;
+    float t = 0.0f;
+    for (int gq = 0; gq < HGS_GROUPS; ++gq) t += s_part[(gq * HGS_COLS + jl) * (HGS_LMAX + 1) + l];
+    d[l] = t;
+  }
   float acc_o = 0.0f;
-  for (int i = 0; i < K; ++i) {
+  for (int i = grp; i < K; i += HGS_GROUPS) {
     float S[HGS_LMAX];
     load_cascaded(col + i * rs, S);
     const float ki = s_k[i] * rk, qi = s_q[i] * rq;
@@ -115,31 +134,37 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int l = 0; l < HGS_LMAX; ++l)
       if (l < L) {
-        col[i * rs + l] = S[l];
+        if (live) col[i * rs + l] = S[l];
         sl = __builtin_fmaf(s_l[l], S[l], sl);
       }
     acc_o = __builtin_fmaf(qi, sl, acc_o);
   }
-  o[((size_t)b * HV + hv) * V + j] = GdrElem<T>::from_float(acc_o);
+  __syncthreads();  // every thread is done with the k^T S sums
+  mine[0] = acc_o;
+  __syncthreads();
+  if (grp == 0 && live) {
+    float t = 0.0f;
+    for (int gq = 0; gq < HGS_GROUPS; ++gq) t += s_part[(gq * HGS_COLS + jl) * (HGS_LMAX + 1)];
+    o[((size_t)b * HV + hv) * V + j] = GdrElem<T>::from_float(t);
+  }
 }
 
 // q, k [B, H, K]; v, o [B, HV, V] (dtype 0 bf16 / 1 fp16 / 2 fp32); g (log decay), beta fp32 [B, HV]; lam [B, HV, L] of
 // lam_dtype, used as lam / lam_div rounded to its type; states fp32 [B, HV, K, V, L], updated in place;
-// z: the levels 0 .. z-1 are full and cascade into level z (0: the state is empty). V <= 256, L <= 32.
+// z: the levels 0 .. z-1 are full and cascade into level z (0: the state is empty). L <= 32.
 extern "C" int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                const void* lam, int lam_dtype, float lam_div, float* states, void* o, int B, int H, int HV,
                                int K, int V, int L, int z, int dtype, float scale, int l2norm, void* stream) {
   if (!q || !k || !v || !g || !beta || !lam || !states || !o) return LAMPA_ERR_INVALID;
   if (B < 0 || H < 1 || HV < H || HV % H != 0 || K < 1 || V < 1 || L < 1 || z < 0 || z >= L) return LAMPA_ERR_INVALID;
   if (l2norm < 0 || l2norm > 2 || lam_dtype < 0 || lam_dtype > 2 || !(lam_div > 0.0f)) return LAMPA_ERR_INVALID;
-  if (V > 256 || L > HGS_LMAX || K > 4096 || dtype < 0 || dtype > 2) return LAMPA_ERR_UNSUPPORTED;
+  if (V > 1024 || L > HGS_LMAX || K > 4096 || dtype < 0 || dtype > 2) return LAMPA_ERR_UNSUPPORTED;
   if (B == 0) return LAMPA_OK;
   hipStream_t s = (hipStream_t)stream;
-  const int threads = V <= 64 ? 64 : (V <= 128 ? 128 : 256);
-  const size_t smem = (2 * (size_t)K + HGS_LMAX + 8) * sizeof(float);
+  const size_t smem = (2 * (size_t)K + HGS_LMAX + 8 + HGS_GROUPS * HGS_COLS * (HGS_LMAX + 1)) * sizeof(float);
   LAMPA_PROF(s, "start");
 #define HGS_CASE(TT)                                                                                                \
-  hipLaunchKernelGGL((hgdn_step_kernel<TT>), dim3(B * HV), dim3(threads), smem, s, (const TT*)q, (const TT*)k,      \
+  hipLaunchKernelGGL((hgdn_step_kernel<TT>), dim3(B * HV, (V + HGS_COLS - 1) / HGS_COLS), dim3(256), smem, s, (const TT*)q, (const TT*)k,      \
                      (const TT*)v, g, beta, lam, lam_dtype, lam_div, states, (TT*)o, H, HV, K, V, L, z, scale, l2norm)
   if (dtype == GDR_BF16) HGS_CASE(__bf16);
   else if (dtype == GDR_FP16) HGS_CASE(_Float16);

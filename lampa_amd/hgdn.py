@@ -13,7 +13,7 @@ states (``hattention_prefill``, ``kernel.py:467-575``: the whole chunks through 
 tokens one by one) and the single-token step on an ``HState`` (``hattention_step``, ``kernel.py:577-633``).
 
 Differences a caller can observe: forward only; the chunk kernels take K = 64 and V in {64, 128} (the single-token step
-takes any K and V <= 256); ``HState.counts`` lives on the host (the reference keeps it on the device and synchronises
+takes any K and V, up to 32 levels); ``HState.counts`` lives on the host (the reference keeps it on the device and synchronises
 on every comparison, ``recurrent.py:44-56``); the step computes its output from the fp32 states, the reference rounds
 them to the output type first (``kernel.py:628-631``).
 """

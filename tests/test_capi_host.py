@@ -126,7 +126,7 @@ def test_hierarchical_forward_argument_checks(lib):
     assert call([0, 4096, 12288], 8, L=14, states=d) == -1
     # the single-token step
     assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 64, 13, 13, 0, 0.125, 1, None) == -1  # z < L
-    assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 512, 13, 1, 0, 0.125, 1, None) == -4
+    assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 64, 40, 1, 0, 0.125, 1, None) == -4     # more than 32 levels
     assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 0, 2, 2, 64, 64, 13, 0, 0, 0.125, 1, None) == 0     # empty batch
 
 
