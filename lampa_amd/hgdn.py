@@ -59,24 +59,32 @@ class HState(object):
         self.shape, self.dtype, self.device = tuple(shape), dtype, device
         self.max_num_levels = self.shape[-1]
         self.states = torch.zeros(self.shape, dtype=self.dtype, device=self.device)
-        self.counts = torch.zeros(self.max_num_levels, dtype=torch.int32)
+        self._counts = [0] * self.max_num_levels  # host integers; ``counts`` shows them as the reference's tensor
+
+    @property
+    def counts(self) -> torch.Tensor:
+        return torch.tensor(self._counts, dtype=torch.int32)
+
+    @counts.setter
+    def counts(self, value) -> None:
+        self._counts = [int(c) for c in value]
 
     @property
     def tokens_seen(self) -> int:
-        return int(self.counts.sum())
+        return sum(self._counts)
 
     def cascade_weak(self) -> int:
         """Replays ``recurrent.py:44-56`` on the counts; returns the level that received the full ones (0: none)."""
-        z = 0
+        z, counts = 0, self._counts
         for level in range(self.max_num_levels):
             capacity = self.base ** level
-            if int(self.counts[level]) == capacity:
+            if counts[level] == capacity:
                 if level + 1 >= self.max_num_levels:
                     raise ValueError("the state has no level left for this many tokens")
-                self.counts[level + 1] += self.counts[level]
-                self.counts[level] = 0
+                counts[level + 1] += counts[level]
+                counts[level] = 0
                 z = level + 1
-            elif int(self.counts[level]) < capacity:
+            elif counts[level] < capacity:
                 break
             else:
                 raise ValueError
@@ -94,7 +102,7 @@ class HState(object):
     def to(self, dtype: Optional[torch.dtype] = None, device: Optional[torch.device] = None) -> "HState":
         new_state = HState(self.base, self.htype, self.hstruct, self.shape, dtype or self.dtype, device or self.device)
         new_state.states = self.states.to(dtype=new_state.dtype, device=new_state.device)
-        new_state.counts = self.counts.clone()
+        new_state._counts = list(self._counts)
         return new_state
 
 
@@ -208,9 +216,9 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
                                            hstate.states)
             # counts after T0 tokens (kernel.py:451-462): the last token alone in level 0, level l > 0 holds 2^(l-1)
             # tokens iff that bit of T0 - 1 is set
-            hstate.counts[0] = 1
+            hstate._counts[0] = 1
             for level in range(1, L):
-                hstate.counts[level] = (1 << (level - 1)) if ((T0 - 1) >> (level - 1)) & 1 else 0
+                hstate._counts[level] = (1 << (level - 1)) if ((T0 - 1) >> (level - 1)) & 1 else 0
         for t in range(T0, T):
             o[:, t] = _step(hstate, q[:, t], k[:, t], v[:, t], g[:, t], l[:, t], beta[:, t], scale, lam_div)
         return o, hstate
@@ -254,5 +262,5 @@ def _step(hstate: HState, q, k, v, g, l, beta, scale, lam_div) -> torch.Tensor:
     check(_capi.lib().lampa_hgdn_step(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(l), _gd._DTYPES[l.dtype],
                                       float(lam_div), ptr(hstate.states), ptr(o), B, H, HV, K, V, L, z,
                                       _gd._DTYPES[q.dtype], float(scale), _gd.L2_CHUNK, stream_of(q)), "lampa_hgdn_step")
-    hstate.counts[0] += 1
+    hstate._counts[0] += 1
     return o
