@@ -18,7 +18,7 @@
 #define HGS_COLS 16
 #define HGS_GROUPS 16
 
-template <typename T>
+template <typename T, int LM>
 __global__ void __launch_bounds__(256)
     hgdn_step_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                      const float* __restrict__ g, const float* __restrict__ beta, const void* __restrict__ lam,
@@ -30,6 +30,8 @@ __global__ void __launch_bounds__(256)
   float* s_l = s_qk + 2 * K;
   float* s_red = s_l + HGS_LMAX;
   float* s_part = s_red + 8;  // [HGS_GROUPS][HGS_COLS][HGS_LMAX + 1]
+  float* s_tot = s_part + HGS_GROUPS * HGS_COLS * (HGS_LMAX + 1);  // [HGS_COLS][HGS_LMAX + 1]
+  float* s_m = s_tot + HGS_COLS * (HGS_LMAX + 1);                  // cascade coefficients, 3 x [HGS_LMAX]
   const int b = blockIdx.x / HV, hv = blockIdx.x % HV, h = hv / (HV / H);
   const int tid = threadIdx.x;
   const T* qp = q + ((size_t)b * H + h) * K;
@@ -50,16 +52,24 @@ __global__ void __launch_bounds__(256)
     s_red[2 * (tid >> 6)] = qs;
     s_red[2 * (tid >> 6) + 1] = ks;
   }
-  if (tid < L) {
-    const size_t li = ((size_t)b * HV + hv) * L + tid;
-    float x = lam_dtype == GDR_FP32   ? reinterpret_cast<const float*>(lam)[li]
-              : lam_dtype == GDR_BF16 ? (float)reinterpret_cast<const __bf16*>(lam)[li]
-                                      : (float)reinterpret_cast<const _Float16*>(lam)[li];
-    if (lam_div != 1.0f) {  // lambda / scale, rounded to lambda's own type as the element-wise division would
-      x = __fdiv_rn(x, lam_div);
-      x = lam_dtype == GDR_FP32 ? x : lam_dtype == GDR_BF16 ? (float)(__bf16)x : (float)(_Float16)x;
+  if (tid < HGS_LMAX) {
+    float x = 0.0f;  // levels past L weigh nothing
+    if (tid < L) {
+      const size_t li = ((size_t)b * HV + hv) * L + tid;
+      x = lam_dtype == GDR_FP32   ? reinterpret_cast<const float*>(lam)[li]
+          : lam_dtype == GDR_BF16 ? (float)reinterpret_cast<const __bf16*>(lam)[li]
+                                  : (float)reinterpret_cast<const _Float16*>(lam)[li];
+      if (lam_div != 1.0f) {  // lambda / scale, rounded to lambda's own type as the element-wise division would
+        x = __fdiv_rn(x, lam_div);
+        x = lam_dtype == GDR_FP32 ? x : lam_dtype == GDR_BF16 ? (float)(__bf16)x : (float)(_Float16)x;
+      }
     }
     s_l[tid] = x;
+    // the cascade as arithmetic on 0 / 1 coefficients (no branches in the row loops): the full levels below z are
+    // summed, level z takes the sum, levels past L (loaded from a clamped index) are dropped
+    s_m[tid] = (tid < L && tid < z) ? 1.0f : 0.0f;                 // enters the sum
+    s_m[HGS_LMAX + tid] = (tid < L && tid >= z) ? 1.0f : 0.0f;     // keeps its value
+    s_m[2 * HGS_LMAX + tid] = (z > 0 && tid == z) ? 1.0f : 0.0f;   // receives the sum
   }
   __syncthreads();
   qs = 0.0f;
@@ -85,59 +95,83 @@ __global__ void __launch_bounds__(256)
   float* col = states + (((size_t)b * HV + hv) * K * V + jc) * L;  // row i of this column: col + i * V * L
   const size_t rs = (size_t)V * L;
 
-  auto load_cascaded = [&](const float* p, float* S) {
+  // A row's level values: LM unconditional loads (indices past L - 1 re-read the last level and are dropped), so that
+  // all of them -- and those of the second row of a pair -- are in flight together; then the cascade.
+  auto load_row = [&](const float* p, float* S) {
 #pragma unroll
-    for (int l = 0; l < HGS_LMAX; ++l) S[l] = l < L ? p[l] : 0.0f;
-    if (z > 0) {
-      float acc = S[0];
-#pragma unroll
-      for (int l = 1; l < HGS_LMAX; ++l) {
-        if (l < z) acc = S[l] + acc;
-        else if (l == z) S[l] = S[l] + acc;
-      }
-#pragma unroll
-      for (int l = 0; l < HGS_LMAX; ++l)
-        if (l < z) S[l] = 0.0f;
-    }
+    for (int l = 0; l < LM; ++l) S[l] = p[min(l, L - 1)];
   };
-  float d[HGS_LMAX];
+  float m_sum[LM], m_keep[LM], m_take[LM];
 #pragma unroll
-  for (int l = 0; l < HGS_LMAX; ++l) d[l] = 0.0f;
-  for (int i = grp; i < K; i += HGS_GROUPS) {
-    float S[HGS_LMAX];
-    load_cascaded(col + i * rs, S);
-    const float ki = s_k[i] * rk;
+  for (int l = 0; l < LM; ++l) {
+    m_sum[l] = s_m[l];
+    m_keep[l] = s_m[HGS_LMAX + l];
+    m_take[l] = s_m[2 * HGS_LMAX + l];
+  }
+  auto cascade = [&](float* S) {
+    float acc = m_sum[0] * S[0];
 #pragma unroll
-    for (int l = 1; l < HGS_LMAX; ++l) d[l] = __builtin_fmaf(ki, S[l], d[l]);
+    for (int l = 1; l < LM; ++l) acc = __builtin_fmaf(m_sum[l], S[l], acc);  // S_1 + S_0, then + S_2 ...: exact 0 / 1 factors
+#pragma unroll
+    for (int l = 0; l < LM; ++l) S[l] = __builtin_fmaf(m_take[l], acc, m_keep[l] * S[l]);
+  };
+  float d[LM];
+#pragma unroll
+  for (int l = 0; l < LM; ++l) d[l] = 0.0f;
+  for (int i = grp; i < K; i += 2 * HGS_GROUPS) {
+    const int i2 = i + HGS_GROUPS;
+    const bool two = i2 < K;
+    float S[LM], S2[LM];
+    load_row(col + i * rs, S);
+    load_row(col + (two ? i2 : i) * rs, S2);
+    cascade(S);
+    cascade(S2);
+    const float ki = s_k[i] * rk, ki2 = two ? s_k[i2] * rk : 0.0f;
+#pragma unroll
+    for (int l = 1; l < LM; ++l) d[l] = __builtin_fmaf(ki2, S2[l], __builtin_fmaf(ki, S[l], d[l]));
   }
   float* mine = s_part + (grp * HGS_COLS + jl) * (HGS_LMAX + 1);
+  mine[0] = 0.0f;
 #pragma unroll
-  for (int l = 1; l < HGS_LMAX; ++l)
-    if (l < L) mine[l] = d[l];
+  for (int l = 1; l < LM; ++l) mine[l] = d[l];
+  __syncthreads();
+  // sums over the row groups: one (column, level) pair per thread and round, then every thread takes its column's
+  for (int pair = tid; pair < HGS_COLS * LM; pair += 256) {
+    const int pc = pair / LM, pl = pair % LM;
+    float t = 0.0f;
+#pragma unroll
+    for (int gq = 0; gq < HGS_GROUPS; ++gq) t += s_part[(gq * HGS_COLS + pc) * (HGS_LMAX + 1) + pl];
+    s_tot[pc * (HGS_LMAX + 1) + pl] = t;
+  }
   __syncthreads();
 #pragma unroll
-  for (int l = 1; l < HGS_LMAX; ++l) {
-    if (l >= L) continue;
-    float t = 0.0f;
-    for (int gq = 0; gq < HGS_GROUPS; ++gq) t += s_part[(gq * HGS_COLS + jl) * (HGS_LMAX + 1) + l];
-    d[l] = t;
-  }
+  for (int l = 1; l < LM; ++l) d[l] = s_tot[jl * (HGS_LMAX + 1) + l];
   float acc_o = 0.0f;
-  for (int i = grp; i < K; i += HGS_GROUPS) {
-    float S[HGS_LMAX];
-    load_cascaded(col + i * rs, S);
+  auto update_row = [&](int i, float* S) {
     const float ki = s_k[i] * rk, qi = s_q[i] * rq;
     float sl = 0.0f;
     S[0] = bt * ki * vj;
 #pragma unroll
-    for (int l = 1; l < HGS_LMAX; ++l) S[l] = a * (S[l] - bt * ki * d[l]);
+    for (int l = 1; l < LM; ++l) S[l] = a * (S[l] - bt * ki * d[l]);
 #pragma unroll
-    for (int l = 0; l < HGS_LMAX; ++l)
-      if (l < L) {
-        if (live) col[i * rs + l] = S[l];
-        sl = __builtin_fmaf(s_l[l], S[l], sl);
-      }
+    for (int l = 0; l < LM; ++l) sl = __builtin_fmaf(s_l[l], S[l], sl);
+    if (live) {
+#pragma unroll
+      for (int l = 0; l < LM; ++l)
+        if (l < L) col[i * rs + l] = S[l];
+    }
     acc_o = __builtin_fmaf(qi, sl, acc_o);
+  };
+  for (int i = grp; i < K; i += 2 * HGS_GROUPS) {
+    const int i2 = i + HGS_GROUPS;
+    const bool two = i2 < K;
+    float S[LM], S2[LM];
+    load_row(col + i * rs, S);
+    load_row(col + (two ? i2 : i) * rs, S2);
+    cascade(S);
+    cascade(S2);
+    update_row(i, S);
+    if (two) update_row(i2, S2);
   }
   __syncthreads();  // every thread is done with the k^T S sums
   mine[0] = acc_o;
@@ -161,15 +195,23 @@ extern "C" int lampa_hgdn_step(const void* q, const void* k, const void* v, cons
   if (V > 1024 || L > HGS_LMAX || K > 4096 || dtype < 0 || dtype > 2) return LAMPA_ERR_UNSUPPORTED;
   if (B == 0) return LAMPA_OK;
   hipStream_t s = (hipStream_t)stream;
-  const size_t smem = (2 * (size_t)K + HGS_LMAX + 8 + HGS_GROUPS * HGS_COLS * (HGS_LMAX + 1)) * sizeof(float);
+  const size_t smem = (2 * (size_t)K + 4 * HGS_LMAX + 8 + (HGS_GROUPS + 1) * HGS_COLS * (HGS_LMAX + 1)) * sizeof(float);
   LAMPA_PROF(s, "start");
-#define HGS_CASE(TT)                                                                                                \
-  hipLaunchKernelGGL((hgdn_step_kernel<TT>), dim3(B * HV, (V + HGS_COLS - 1) / HGS_COLS), dim3(256), smem, s, (const TT*)q, (const TT*)k,      \
-                     (const TT*)v, g, beta, lam, lam_dtype, lam_div, states, (TT*)o, H, HV, K, V, L, z, scale, l2norm)
+#define HGS_LAUNCH(TT, LM)                                                                                         \
+  hipLaunchKernelGGL((hgdn_step_kernel<TT, LM>), dim3(B * HV, (V + HGS_COLS - 1) / HGS_COLS), dim3(256), smem, s,  \
+                     (const TT*)q, (const TT*)k, (const TT*)v, g, beta, lam, lam_dtype, lam_div, states, (TT*)o, H, \
+                     HV, K, V, L, z, scale, l2norm)
+#define HGS_CASE(TT)                    \
+  do {                                  \
+    if (L <= 16) HGS_LAUNCH(TT, 16);    \
+    else if (L <= 24) HGS_LAUNCH(TT, 24); \
+    else HGS_LAUNCH(TT, 32);            \
+  } while (0)
   if (dtype == GDR_BF16) HGS_CASE(__bf16);
   else if (dtype == GDR_FP16) HGS_CASE(_Float16);
   else HGS_CASE(float);
 #undef HGS_CASE
+#undef HGS_LAUNCH
   LAMPA_PROF(s, "hgdn_step_kernel");
   return lampa_launch_status();
 }
