@@ -242,8 +242,8 @@ int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float
  * (lam_div = 1: as given). Level 0 = the token itself, level l > 0 = sources whose highest differing position bit is
  * l-1 (base.py:41-46).
  * K = 64, V in {64, 128}; l2norm as for the chunk forward (the reference requires the chunk-path l2norm);
- * the plan's chunks_per_segment must be a power of two unless every sequence is one segment; sequences of at most
- * 4096 chunks; L >= 7 + number of bits of the largest chunk index. Zero initial state. level_states (nullable): fp32
+ * the plan's chunks_per_segment must be a power of two unless every sequence is one segment; sequence lengths are
+ * multiples of 64 (chunkwise_hgdn.py:598-601), at most 4096 chunks each; L >= 7 + number of bits of the largest chunk index. Zero initial state. level_states (nullable): fp32
  * [n_seq, HV, K, V, L] zeroed by the caller, receives HState.states (recurrent.py:33-36) after the last token of every
  * sequence -- what hattention_prefill returns (kernel.py:467-575); needs equal sequence lengths, multiples of 64. */
 int64_t lampa_hgdn_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V);

@@ -846,7 +846,8 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
 // weights; the kernel uses lam / lam_div rounded to lam's type (the reference divides the weights by `scale`, which
 // multiplies q, before its kernel; lam_div = 1 takes them as they are). The plan's chunks_per_segment must be a
 // power of two (or at least the longest sequence's chunk count: one segment per sequence); every sequence may hold at
-// most 2^12 chunks and L must cover 7 + the number of chunk-index bits of the longest sequence.
+// most 2^12 chunks, every sequence length must be a multiple of 64 and L must cover 7 + the number of chunk-index bits
+// of the longest sequence.
 // level_states (nullable): fp32 [n_seq, HV, K, V, L], ZEROED by the caller; receives the occupied levels' states after
 // the last token of every sequence (the reference's HState.states); needs sequences of equal length, a multiple of 64.
 extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
@@ -875,9 +876,10 @@ extern "C" int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v,
     max_nc = nc > max_nc ? nc : max_nc;
   }
   if (max_nc > (1 << HG_NLV)) return LAMPA_ERR_UNSUPPORTED;
+  // whole chunks only, as the reference demands (chunkwise_hgdn.py:598-601)
+  if ((int64_t)chunks * GDR_C != plan_host[PLAN_TOTAL_TOKENS]) return LAMPA_ERR_INVALID;
   if (level_states) {  // every sequence: the same whole number of chunks
-    const int total = plan_host[PLAN_TOTAL_TOKENS];
-    if (max_nc < 1 || (int64_t)max_nc * n_seq != chunks || (int64_t)chunks * GDR_C != total) return LAMPA_ERR_INVALID;
+    if (max_nc < 1 || (int64_t)max_nc * n_seq != chunks) return LAMPA_ERR_INVALID;
   }
   int bits = 0;
   while ((1 << bits) < max_nc) ++bits;

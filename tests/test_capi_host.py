@@ -123,6 +123,7 @@ def test_hierarchical_forward_argument_checks(lib):
     assert call([0, 64 * 4096], 4096, L=19) == -2
     assert call([0, 4096, 8192], 8, L=13, states=d) == -2         # level states: equal whole-chunk sequences
     assert call([0, 4096, 8000], 8, L=13, states=d) == -1
+    assert call([0, 4000], 8, L=13) == -1                        # a ragged last chunk
     assert call([0, 4096, 12288], 8, L=14, states=d) == -1
     # the single-token step
     assert lib.lampa_hgdn_step(d, d, d, d, d, d, 0, 0.125, d, d, 2, 2, 2, 64, 64, 13, 13, 0, 0.125, 1, None) == -1  # z < L
