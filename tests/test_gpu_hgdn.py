@@ -169,3 +169,37 @@ def test_steps_from_an_empty_state_any_head_size(device):
         for _ in range(100):
             hgdn.chunk_h_gated_delta_rule(*(x[:, :1].to(device) for x in (q, k, v, g, lam, beta)), scale=0.25,
                                           initial_state=st, output_final_state=True, use_qk_l2norm_in_kernel=True)
+
+
+def test_step_entry_point_fp32_and_odd_sizes(device):
+    # the C entry point itself: fp32 tokens, K = 24, V = 40 (not a multiple of the 16-column tiles), 9 levels, weights
+    # taken as given (lam_div = 1), recurrent-style l2norm off; ten tokens from an empty state
+    import ctypes
+    from lampa_amd import _capi
+    from lampa_amd._capi import ptr
+    gen = torch.Generator().manual_seed(11)
+    B, T, H, HV, K, V, L = 2, 10, 2, 4, 24, 40, 9
+    q, k = (torch.randn(B, T, H, K, generator=gen) for _ in range(2))
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g = -0.2 * torch.rand(B, T, HV, generator=gen)
+    beta = torch.rand(B, T, HV, generator=gen)
+    lam = torch.randn(B, T, HV, L, generator=gen)
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, lam, scale=0.3, l2=0)
+    states = torch.zeros(B, HV, K, V, L, device=device)
+    st = hgdn.HState(2, hgdn.HType.WEAK, hgdn.HStruct.GDELTA, (B, HV, K, V, L), torch.float32, device)
+    outs = []
+    lib = _capi.lib()
+    for t in range(T):
+        z = st.cascade_weak()
+        args = [x[:, t].contiguous().to(device) for x in (q, k, v, g, beta, lam)]
+        o = torch.empty(B, HV, V, device=device)
+        rc = lib.lampa_hgdn_step(ptr(args[0]), ptr(args[1]), ptr(args[2]), ptr(args[3]), ptr(args[4]), ptr(args[5]), 2,
+                                 1.0, ptr(states), ptr(o), B, H, HV, K, V, L, z, 2, 0.3, 0,
+                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        st._counts[0] += 1
+        outs.append(o.cpu())
+    assert st.counts.tolist() == want_c.tolist()
+    # fp32 arithmetic against fp64: relative to the size of the values (the keys are not normalised here, so they grow)
+    assert (torch.stack(outs, 1) - want_o).abs().max() <= 2e-5 * want_o.abs().max()
+    assert (states.cpu() - want_s).abs().max() <= 2e-5 * want_s.abs().max()
