@@ -15,13 +15,15 @@
 //   N   = K^T diag(e^{gamma_last - gamma} rk) T diag(beta) V          (the chunk's own sources, at its end)
 //   o_intra = ((P T diag(beta)) . Lambda) V,   Lambda_ij = lambda_i[level(i, j)]
 // Kernels:
-//   prep   workgroup per (chunk, head), fully parallel: W, Q~ and K^T as MFMA operand fragments, the decay factors,
-//          the inter-chunk lambdas (transposed), N and o_intra go to HBM.
+//   prep   workgroup per (chunk, head), fully parallel: W and Q~ as MFMA operand fragments, the decay factors, the
+//          inter-chunk lambdas (transposed), diag(e^{gamma_last - gamma} rk) T diag(beta) V as B-operand fragments (the
+//          walk multiplies it by K^T: the chunk's own state N) and o_intra go to HBM.
 //   walk   workgroup per (segment of chunks, head, 32 value columns): six "chain" waves hold up to two level
 //          states each in accumulator registers (level j -> wave j % 6) and walk the chunks: for every level whose
 //          chunk-index bit is set, o += lambda . (Q~ S), S <- S'; after the chunk the levels below the lowest clear
 //          bit and N are summed into that bit's level (the carry chain of a binary counter) through LDS. Two loader
-//          waves stage the chunks' operand records and N; all eight waves add the chain waves' partial outputs to
+//          waves stage the chunks' operand records and raw k tiles (K^T operands come from the tile with the
+//          transposing LDS read) and one of them forms N; all eight waves add the chain waves' partial outputs to
 //          o_intra, eight rows each, and store o.
 //   scan   (sequences cut into segments of 2^p chunks) the same walk over whole segments with the segment
 //          composites (M, N) of the plain rule: leaves every segment's entering level states.
@@ -40,8 +42,7 @@ struct HgRec {
   static constexpr int NKS = KT / 16;
   static constexpr int WF = 0;                          // W fragments   [2][NKS] KiB
   static constexpr int QF = WF + 2 * NKS * 1024;        // Q~ fragments  [2][NKS] KiB
-  static constexpr int KF = QF + 2 * NKS * 1024;        // K^T fragments [KT/32][4] KiB
-  static constexpr int DK = KF + (KT / 32) * 4 * 1024;  // e^{gamma_last - gamma_i} rk_i, fp32 [64]
+  static constexpr int DK = QF + 2 * NKS * 1024;        // e^{gamma_last - gamma_i} rk_i, fp32 [64]
   static constexpr int LT = DK + 256;                   // lambda_i[7 + j], fp32 [HG_NLV][64]
   static constexpr int MISC = LT + HG_NLV * 256;        // e^{gamma_last}
   static constexpr int BYTES = MISC + 256;
@@ -70,7 +71,7 @@ __global__ void __launch_bounds__(256)
                      const void* __restrict__ lam, int lam_dtype, float lam_div,
                      const int32_t* __restrict__ chunk_tok0,
                      const int32_t* __restrict__ chunk_len, const unsigned char* __restrict__ tmat,
-                     unsigned char* __restrict__ wrec, float* __restrict__ Nc, float* __restrict__ Oi,
+                     unsigned char* __restrict__ wrec, unsigned char* __restrict__ Ub_out, float* __restrict__ Oi,
                      float* __restrict__ hstates, int chunks_per_seq, int H, int HV, int L, float scale, int l2norm) {
   using SM = HgPrepSmem<KT, VT>;
   using REC = HgRec<KT>;
@@ -262,8 +263,7 @@ __global__ void __launch_bounds__(256)
     frag_store(s_P, f0, lane, acc_to_operand(acc, 0));
     frag_store(s_P, f0 + 1, lane, acc_to_operand(acc, 8));
   };
-  auto un_tile = [&](int vt) {  // U = (T diag(beta)) V for 32 value columns, then N = K^T (dk U)
-    bf16x8 Ub[4];
+  auto un_tile = [&](int vt) {  // dk . U with U = (T diag(beta)) V for 32 value columns, as B-operand fragments
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {
       f32x16 acc = zero16();
@@ -272,22 +272,9 @@ __global__ void __launch_bounds__(256)
         if (ks < 2 * (tm + 1)) acc = mfma32(t_frag_scaled(tm, ks, s_beta), ld_kappa_tr(s_v, SV, 32 * vt, 16 * ks, lane), acc);
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] *= s_dk[32 * tm + acc_row(r, hh)];
-      Ub[2 * tm] = acc_to_operand(acc, 0);
-      Ub[2 * tm + 1] = acc_to_operand(acc, 8);
-    }
-    f32x4* out = reinterpret_cast<f32x4*>(Nc + (ch * (VT / 32) + vt) * (KT * 32));
-#pragma unroll
-    for (int km = 0; km < KT / 32; ++km) {
-      f32x16 acc = zero16();
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) acc = mfma32(ld_kappa_tr(s_k, SK, 32 * km, 16 * ks, lane), Ub[ks], acc);
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        f32x4 t;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) t[e] = acc[4 * q4 + e];
-        out[(km * 4 + q4) * 64 + lane] = t;
-      }
+      unsigned char* out = Ub_out + (ch * (VT / 32) + vt) * 4096;
+      frag_store(out, 2 * tm, lane, acc_to_operand(acc, 0));
+      frag_store(out, 2 * tm + 1, lane, acc_to_operand(acc, 8));
     }
   };
   // The last chunk of a sequence, when the caller wants the level states after the last token (HState.states of
@@ -327,18 +314,15 @@ __global__ void __launch_bounds__(256)
       for (int r = 0; r < 16; ++r) out[((size_t)(32 * km + acc_row(r, hh)) * VT + 32 * vt + ln) * L] = acc[r];
     }
   };
-  // ---- W, P, the chunk's own state N, the K^T fragments (tasks spread over the four waves)
-  constexpr int NW = 2 * (KT / 32), NU = VT / 32, NKF = (KT / 32) * 4;
+  // ---- W, P, the scaled U of the chunk's own state (tasks spread over the four waves)
+  constexpr int NW = 2 * (KT / 32), NU = VT / 32;
   const int n_tail = want_tail ? NU * HG_INTRA : 0;
-  for (int task = wave; task < NW + 3 + NU + NKF + n_tail; task += 4) {
+  for (int task = wave; task < NW + 3 + NU + n_tail; task += 4) {
     if (task < NW) w_tile(task / (KT / 32), task % (KT / 32));
     else if (task < NW + 3) p_tile(task - NW);
     else if (task < NW + 3 + NU) un_tile(task - NW - 3);
-    else if (task < NW + 3 + NU + NKF) {
+    else {
       const int f = task - NW - 3 - NU;
-      frag_store(rec + REC::KF, f, lane, ld_kappa_tr(s_k, SK, 32 * (f / 4), 16 * (f % 4), lane));
-    } else {
-      const int f = task - NW - 3 - NU - NKF;
       tail_tile(f / HG_INTRA, f % HG_INTRA);
     }
   }
@@ -412,8 +396,10 @@ __global__ void __launch_bounds__(256)
 template <int KT>
 struct HgWalkSmem {
   static constexpr int SP = 36;  // row stride of a partial output tile (fp32)
+  static constexpr int SK = KT + 8;  // row stride of the k tile
   static constexpr int OFF_REC = 0;
-  static constexpr int OFF_PART = 2 * HgRec<KT>::BYTES;
+  static constexpr int OFF_KT = 2 * HgRec<KT>::BYTES;          // raw k tile (row-major), double-buffered
+  static constexpr int OFF_PART = OFF_KT + 2 * 64 * SK * 2;
   static constexpr int OFF_ACC = OFF_PART + HG_CW * 64 * SP * 4;
   static constexpr int BYTES = OFF_ACC + KT * 32 * 4;
 };
@@ -487,7 +473,7 @@ __device__ __forceinline__ void hg_merge(int cs, int lvl0, int wave, bool chain,
 template <typename T, int KT, int VT>
 __global__ void __launch_bounds__(64 * (HG_CW + 2))
     hgdn_walk_kernel(const GdrPlanView pv, const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
-                     const unsigned char* __restrict__ wrec, const float* __restrict__ Nc,
+                     const T* __restrict__ k, int H, const unsigned char* __restrict__ wrec, const unsigned char* __restrict__ Ub_in,
                      const float* __restrict__ Oi, const float* __restrict__ Xinit, T* __restrict__ o,
                      float* __restrict__ hstates, int L, int HV) {
   using REC = HgRec<KT>;
@@ -527,39 +513,67 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
   if (wave >= HG_CW) {
     // ================================================ loader ================================================
     const int ltid = tid - 64 * HG_CW;
-    constexpr int NP = (REC::PIECES + 127) / 128;
-    u32x4 recA[NP], recB[NP];
-    f32x4 nA[KT / 16], nB[KT / 16];  // N slab: KT * 32 * 4 bytes = KT * 8 pieces over 128 threads
-    auto load_rec = [&](int c, u32x4* r) __attribute__((always_inline)) {
+    constexpr int NP = (REC::PIECES + 127) / 128, KU = KT / 16;  // 16-byte pieces per thread: record; half a k row
+    const int h = hv / (HV / H);
+    const int krow = ltid >> 1, khalf = ltid & 1;
+    const bool nwave = wave == HG_CW;  // the loader wave that also turns (dk U) into the chunk's own state
+    struct Set {
+      u32x4 rec[NP];
+      typename Raw8<T>::type kk[KU];
+      bf16x8 ub[4];
+    };
+    Set sA, sB;
+    auto load_rec = [&](int c, Set& st) __attribute__((always_inline)) {  // record and k tile of chunk c
       const u32x4* src = reinterpret_cast<const u32x4*>(wrec + ((size_t)uniform(c) * HV + hv) * REC::BYTES);
 #pragma unroll
-      for (int j = 0; j < NP; ++j) r[j] = src[min(ltid + 128 * j, REC::PIECES - 1)];
+      for (int j = 0; j < NP; ++j) st.rec[j] = src[min(ltid + 128 * j, REC::PIECES - 1)];
+      const T* kp = k + ((size_t)(chunk_tok0[uniform(c)] + krow) * H + h) * KT + khalf * (KT / 2);
+#pragma unroll
+      for (int u = 0; u < KU; ++u) st.kk[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 8 * u);
     };
-    auto store_rec = [&](int par, const u32x4* r) __attribute__((always_inline)) {
+    auto store_rec = [&](int par, const Set& st) __attribute__((always_inline)) {
       u32x4* dst = reinterpret_cast<u32x4*>(smem + SM::OFF_REC + par * REC::BYTES);
 #pragma unroll
       for (int j = 0; j < NP; ++j)
-        if (ltid + 128 * j < REC::PIECES) dst[ltid + 128 * j] = r[j];
-    };
-    auto load_set = [&](int c, u32x4* r, f32x4* n) __attribute__((always_inline)) {  // what chunk c issues
-      const int cr = min(c + 2, c1 - 1), cn = min(c + 1, c1 - 1);
-      load_rec(cr, r);
-      const f32x4* ns = reinterpret_cast<const f32x4*>(Nc + (((size_t)uniform(cn) * HV + hv) * (VT / 32) + vslab) * (KT * 32));
+        if (ltid + 128 * j < REC::PIECES) dst[ltid + 128 * j] = st.rec[j];
+      __bf16* kt = reinterpret_cast<__bf16*>(smem + SM::OFF_KT) + par * (64 * SM::SK);
 #pragma unroll
-      for (int j = 0; j < KT / 16; ++j) n[j] = ns[ltid + 128 * j];
+      for (int u = 0; u < KU; ++u) {
+        float unused = 0.0f;
+        *reinterpret_cast<bf16x8*>(&kt[krow * SM::SK + khalf * (KT / 2) + 8 * u]) = raw_to_bf16<T>(st.kk[u], unused, false);
+      }
     };
-    load_rec(c0, recA);
-    store_rec(0, recA);
-    load_set(c0 - 1, recA, nA);  // record (c0 + 1), own state (c0)
+    auto load_set = [&](int c, Set& st) __attribute__((always_inline)) {  // what chunk c issues
+      load_rec(min(c + 2, c1 - 1), st);
+      const unsigned char* ub = Ub_in + (((size_t)uniform(min(c + 1, c1 - 1)) * HV + hv) * (VT / 32) + vslab) * 4096;
+#pragma unroll
+      for (int f = 0; f < 4; ++f) st.ub[f] = frag_load(ub, f, lane);  // (used by one wave; the other's copy is dropped)
+    };
+    load_rec(c0, sA);
+    store_rec(0, sA);
+    load_set(c0 - 1, sA);  // record and k (c0 + 1), scaled U (c0)
     f32x4 oi_cur = oi_load(c0);
-    auto one_chunk = [&](int c, const u32x4* rHeld, const f32x4* nHeld, u32x4* rNext, f32x4* nNext)
-                         __attribute__((always_inline)) {
-      lds_barrier();  // T(c): record (c) is staged; record buffer (c+1)&1, s_acc and the partial tiles are free
+    auto one_chunk = [&](int c, const Set& held, Set& next) __attribute__((always_inline)) {
+      lds_barrier();  // T(c): record and k (c) are staged; their buffers (c+1)&1, s_acc and the partial tiles are free
       const int tok0 = chunk_tok0[uniform(c)], len = chunk_len[uniform(c)];  // (scalar loads: early, so that they land)
-      store_rec((c - c0 + 1) & 1, rHeld);
+      store_rec((c - c0 + 1) & 1, held);
+      if (nwave) {  // N = K^T (dk U): the chunk's own sources at its end, into s_acc in accumulator order
+        const __bf16* kt = reinterpret_cast<const __bf16*>(smem + SM::OFF_KT) + ((c - c0) & 1) * (64 * SM::SK);
 #pragma unroll
-      for (int j = 0; j < KT / 16; ++j) reinterpret_cast<f32x4*>(s_acc)[ltid + 128 * j] = nHeld[j];
-      load_set(c, rNext, nNext);
+        for (int km = 0; km < KT / 32; ++km) {
+          f32x16 acc = zero16();
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) acc = mfma32(ld_kappa_tr(kt, SM::SK, 32 * km, 16 * ks, lane), held.ub[ks], acc);
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = acc[4 * q4 + e];
+            reinterpret_cast<f32x4*>(s_acc)[(km * 4 + q4) * 64 + lane] = t;
+          }
+        }
+      }
+      load_set(c, next);
       const f32x4 oi_next = oi_load(min(c + 1, c1 - 1));
       lds_barrier();  // M0(c): the chain waves' partial tiles are complete
       out_rows(tok0, len, oi_cur);
@@ -567,8 +581,8 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
       oi_cur = oi_next;
     };
     for (int c = c0; c < c1; c += 2) {
-      one_chunk(c, recA, nA, recB, nB);
-      if (c + 1 < c1) one_chunk(c + 1, recB, nB, recA, nA);
+      one_chunk(c, sA, sB);
+      if (c + 1 < c1) one_chunk(c + 1, sB, sA);
     }
     return;
   }
@@ -590,6 +604,7 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
     const int tok0 = chunk_tok0[uniform(c)], len = chunk_len[uniform(c)];
     const f32x4 oi_next = oi_load(min(c + 1, c1 - 1));
     const unsigned char* rec = smem + SM::OFF_REC + ((c - c0) & 1) * REC::BYTES;
+    const __bf16* s_kt = reinterpret_cast<const __bf16*>(smem + SM::OFF_KT) + ((c - c0) & 1) * (64 * SM::SK);
     const float* s_dk = reinterpret_cast<const float*>(rec + REC::DK);
     const float* s_lt = reinterpret_cast<const float*>(rec + REC::LT);
     const float dec = reinterpret_cast<const float*>(rec + REC::MISC)[0];
@@ -634,7 +649,7 @@ __global__ void __launch_bounds__(64 * (HG_CW + 2))
             fr[NKS + ks] = frag_load(rec + REC::QF, NKS + ks, lane);
           } else if (ks < 4) {
 #pragma unroll
-            for (int km = 0; km < KT / 32; ++km) fr[km * 4 + ks] = frag_load(rec + REC::KF, km * 4 + ks, lane);
+            for (int km = 0; km < KT / 32; ++km) fr[km * 4 + ks] = ld_kappa_tr(s_kt, SM::SK, 32 * km, 16 * ks, lane);
           }
         }
 #pragma unroll
@@ -773,7 +788,7 @@ static HgWorkspace hg_workspace(int64_t chunks, int64_t segs, int HV, int K, int
   w.off_n = off;   off += lampa_align_up(segs * HV * (int64_t)K * V * 4, 256);
   w.off_d = off;   off += lampa_align_up(segs * HV * 4, 256);
   w.off_rec = off; off += lampa_align_up(chunks * HV * rec_bytes, 256);
-  w.off_nc = off;  off += lampa_align_up(chunks * HV * (int64_t)K * V * 4, 256);
+  w.off_nc = off;  off += lampa_align_up(chunks * HV * (int64_t)(V / 32) * 4096, 256);  // dk . U fragments
   w.off_oi = off;  off += lampa_align_up(chunks * HV * (int64_t)64 * V * 4, 256);
   w.off_x = off;   off += lampa_align_up(segs * HG_NLV * HV * (int64_t)K * V * 4, 256);
   w.bytes = off > 0 ? off : 256;
@@ -798,7 +813,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   unsigned char* Nm = ws + w.off_n;
   float* Dc = (float*)(ws + w.off_d);
   unsigned char* rec = ws + w.off_rec;
-  float* Nc = (float*)(ws + w.off_nc);
+  unsigned char* Ubw = ws + w.off_nc;
   float* Oi = (float*)(ws + w.off_oi);
   float* Xi = (float*)(ws + w.off_x);
   constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_p = HgPrepSmem<KT, VT>::BYTES,
@@ -820,7 +835,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
                      l2norm);
   LAMPA_PROF(s, "gdr_tinv_kernel");
   hipLaunchKernelGGL((hgdn_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem_p, s, (const T*)q, (const T*)k,
-                     (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Nc, Oi, hstates, chunks_per_seq, H, HV, L,
+                     (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Ubw, Oi, hstates, chunks_per_seq, H, HV, L,
                      scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
   const bool split = segs > n_seq;
@@ -835,7 +850,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
     LAMPA_PROF(s, "hgdn_scan_kernel");
   }
   hipLaunchKernelGGL((hgdn_walk_kernel<T, KT, VT>), dim3(segs, HV, VT / 32), dim3(64 * (HG_CW + 2)), smem_w, s, pv,
-                     pv.chunk_tok0, pv.chunk_len, rec, Nc, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
+                     pv.chunk_tok0, pv.chunk_len, (const T*)k, H, rec, Ubw, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
                      hstates, L, HV);
   LAMPA_PROF(s, "hgdn_walk_kernel");
   return lampa_launch_status();
