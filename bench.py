@@ -348,6 +348,29 @@ def main():
     }
     del qh, kh, vh, gh, bh, lam
 
+    # ---- config 0: the reference's own CPU-runnable case (B=1, H=4, T=8192, d_k=d_v=32, fp32, seed 0) on the fp32 paths ----
+    q0, k0, v0, g0, b0 = synth.gdr_inputs(1, 8192, 4, 32, 32, torch.float32, seed=0)
+    d0 = [x.to(dev) for x in (q0, k0, v0, g0, b0)]
+
+    def time_us(fn, n=20, w=3):
+        for _ in range(w):
+            fn()
+        torch.cuda.synchronize()
+        t_ = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return 1e6 * (time.perf_counter() - t_) / n
+
+    c0_us = time_us(lambda: gd.fused_recurrent_gated_delta_rule(*d0, output_final_state=True))
+    config0 = {"workload": "config0: token-serial gated delta, B=1 H=4 T=8192 d_k=d_v=32, fp32, zero initial state",
+               "us": round(c0_us, 1), "hits_per_s": round(8192 / (c0_us * 1e-6), 1)}
+    if not args.no_cpu:
+        c0_cpu_hps, c0_cpu_dt = cpu_baseline_gdr(q0, k0, v0, g0, b0, 8192)
+        config0["cpu_baseline"] = {"value": round(c0_cpu_hps, 1), "unit": "hits/s", "seconds": round(c0_cpu_dt, 3),
+                                   "cores": torch.get_num_threads(), "kind": "port"}
+    del d0
+
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
     if not args.no_cpu:
@@ -381,7 +404,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0,
     }
     print(json.dumps(out))
 
