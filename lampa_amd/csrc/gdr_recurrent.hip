@@ -10,6 +10,11 @@
 // fp32 mode of the chunk operator and the on-GPU cross-check of the chunk kernels.
 #include "gdr_common.h"
 
+// value of lane `src` (a compile-time constant) in every lane: one v_readlane into a scalar register
+__device__ __forceinline__ float bcast(float x, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
+}
+
 template <typename T, int KT>
 __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                           const T* __restrict__ v, const float* __restrict__ g,
@@ -31,14 +36,33 @@ __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__
   for (int i = 0; i < KT; ++i)
     S[i] = (h0 && active && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + col] : 0.0f;
 
-  for (int64_t t = bos; t < eos; ++t) {
+  // The inputs of the coming tokens are loaded PF tokens ahead into a ring of registers (a step depends on the
+  // previous one through the state only, so without this every token pays a full memory latency). Loads past the end
+  // of the sequence re-read its last token and are dropped.
+  constexpr int PF = 8;
+  struct Tok {
+    float kv[KR], qv[KR], g, b, v;
+  };
+  Tok ring[PF];
+  auto issue = [&](int64_t t, Tok& x) __attribute__((always_inline)) {
+    t = t < eos ? t : eos - 1;
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+      const int i = r * 64 + lane;
+      x.kv[r] = i < K ? GdrElem<T>::to_float(k[(t * H + h) * K + i]) : 0.0f;
+      x.qv[r] = i < K ? GdrElem<T>::to_float(q[(t * H + h) * K + i]) : 0.0f;
+    }
+    x.g = g[t * HV + hv];
+    x.b = beta[t * HV + hv];
+    x.v = active ? GdrElem<T>::to_float(v[(t * HV + hv) * V + col]) : 0.0f;
+  };
+  auto step = [&](int64_t t, const Tok& x) __attribute__((always_inline)) {
     float kv[KR], qv[KR];
     float kss = 0.0f, qss = 0.0f;
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
-      const int i = r * 64 + lane;
-      kv[r] = i < K ? GdrElem<T>::to_float(k[(t * H + h) * K + i]) : 0.0f;
-      qv[r] = i < K ? GdrElem<T>::to_float(q[(t * H + h) * K + i]) : 0.0f;
+      kv[r] = x.kv[r];
+      qv[r] = x.qv[r];
       kss += kv[r] * kv[r];
       qss += qv[r] * qv[r];
     }
@@ -59,27 +83,40 @@ __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__
     }
 #pragma unroll
     for (int r = 0; r < KR; ++r) { kv[r] *= kinv; qv[r] *= qinv * scale; }
-    const float decay = expf(g[t * HV + hv]);
-    const float b = beta[t * HV + hv];
-    const float vt = active ? GdrElem<T>::to_float(v[(t * HV + hv) * V + col]) : 0.0f;
+    const float decay = expf(x.g);
+    const float b = x.b;
+    const float vt = x.v;
 
-    float dot = 0.0f;
-#pragma unroll
+    float dot4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // four interleaved partial sums: a single chain of KT dependent FMAs
+#pragma unroll                                  // would be the step's critical path
     for (int i = 0; i < KT; ++i) {
-      const float ki = __shfl(kv[i / 64], i % 64);
+      const float ki = bcast(kv[i / 64], i % 64);
       S[i] *= decay;
-      dot = __builtin_fmaf(S[i], ki, dot);
+      dot4[i & 3] = __builtin_fmaf(S[i], ki, dot4[i & 3]);
     }
-    const float d = b * (vt - dot);
-    float out = 0.0f;
+    const float d = b * (vt - ((dot4[0] + dot4[1]) + (dot4[2] + dot4[3])));
+    float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int i = 0; i < KT; ++i) {
-      const float ki = __shfl(kv[i / 64], i % 64);
-      const float qi = __shfl(qv[i / 64], i % 64);
+      const float ki = bcast(kv[i / 64], i % 64);
+      const float qi = bcast(qv[i / 64], i % 64);
       S[i] = __builtin_fmaf(ki, d, S[i]);
-      out = __builtin_fmaf(S[i], qi, out);
+      out4[i & 3] = __builtin_fmaf(S[i], qi, out4[i & 3]);
     }
+    const float out = (out4[0] + out4[1]) + (out4[2] + out4[3]);
     if (active) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out);
+  };
+  if (bos < eos) {
+#pragma unroll
+    for (int p = 0; p < PF; ++p) issue(bos + p, ring[p]);
+    for (int64_t t0 = bos; t0 < eos; t0 += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) {
+        const Tok cur = ring[p];
+        issue(t0 + p + PF, ring[p]);
+        if (t0 + p < eos) step(t0 + p, cur);
+      }
+    }
   }
   if (ht && active) {
 #pragma unroll
