@@ -203,3 +203,18 @@ def test_step_entry_point_fp32_and_odd_sizes(device):
     # fp32 arithmetic against fp64: relative to the size of the values (the keys are not normalised here, so they grow)
     assert (torch.stack(outs, 1) - want_o).abs().max() <= 2e-5 * want_o.abs().max()
     assert (states.cpu() - want_s).abs().max() <= 2e-5 * want_s.abs().max()
+
+
+@pytest.mark.parametrize("g_scale", [1.0, 0.003])
+def test_full_length_prefill_matches_oracle(device, g_scale):
+    # the benchmark's sequence length (938 chunks, 17 levels, split into segments by the default rule), two heads:
+    # outputs, level states and counts against the fp64 token loop (a few seconds on one core)
+    T = 60032
+    q, k, v, g, beta, lam = _inputs(1, T, 2, 64, 64, torch.bfloat16, seed=3, g_scale=g_scale)
+    o, st = hgdn.chunk_h_gated_delta_rule(*(x.to(device) for x in (q, k, v, g, lam, beta)), output_final_state=True,
+                                          use_qk_l2norm_in_kernel=True)
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, lam / 0.125, scale=0.125)
+    max_abs, mean_rel = _errors(o, want_o)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"o: {max_abs:.3e} {mean_rel:.3e}"
+    max_abs, mean_rel = _state_errors(st, want_s, want_c)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"states: {max_abs:.3e} {mean_rel:.3e}"
