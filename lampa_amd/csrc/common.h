@@ -22,4 +22,5 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 // recording is open; the launchers call LAMPA_PROF(stream, "start") first and LAMPA_PROF(stream, "<kernel>") after
 // each launch.
 void lampa_prof_mark(hipStream_t stream, const char* name);
+bool lampa_prof_recording();  // a recording is open: launchers keep everything on the caller's stream then
 #define LAMPA_PROF(stream, name) lampa_prof_mark((stream), (name))

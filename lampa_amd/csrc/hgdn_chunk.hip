@@ -834,21 +834,43 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv, tf, H, HV,
                      l2norm);
   LAMPA_PROF(s, "gdr_tinv_kernel");
+  const bool split = segs > n_seq;
+  // The segment composites and their scan depend on T only, like the prep kernel, and are latency bound on a few
+  // workgroups: they run on a second stream (default priority) beside the prep kernel (launched first, which
+  // measured slightly better than the other order) and join before the walk.
+  // With a profile recording open everything stays on the caller's stream, so that the intervals mean one kernel each.
+  static hipStream_t side = nullptr;
+  static hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  bool overlap = split && !lampa_prof_recording();
+  if (overlap && !side) {
+    if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&ev_join, hipEventDisableTiming) != hipSuccess) {
+      side = nullptr;
+      overlap = false;
+    }
+  }
+  hipStream_t cs = s;  // the stream of the composites
+  if (overlap) {
+    if (hipEventRecord(ev_fork, s) != hipSuccess || hipStreamWaitEvent(side, ev_fork, 0) != hipSuccess) return LAMPA_ERR_LAUNCH;
+    cs = side;
+  }
   hipLaunchKernelGGL((hgdn_prep_kernel<T, KT, VT>), dim3(chunks, HV), dim3(256), smem_p, s, (const T*)q, (const T*)k,
                      (const T*)v, lam, lam_dtype, lam_div, pv.chunk_tok0, pv.chunk_len, tf, rec, Ubw, Oi, hstates, chunks_per_seq, H, HV, L,
                      scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
-  const bool split = segs > n_seq;
   if (split) {
     hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV),
-                       dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s, (const T*)q, (const T*)k, (const T*)v, g,
+                       dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, cs, (const T*)q, (const T*)k, (const T*)v, g,
                        beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nm, Dc, (T*)nullptr,
                        (float*)nullptr, H, HV, scale, l2norm);
     LAMPA_PROF(s, "gdr_segment_kernel<composite>");
-    hipLaunchKernelGGL((hgdn_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64 * HG_CW), 0, s, pv, Mc, Nm, Dc, Xi,
+    hipLaunchKernelGGL((hgdn_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64 * HG_CW), 0, cs, pv, Mc, Nm, Dc, Xi,
                        HV, p);
     LAMPA_PROF(s, "hgdn_scan_kernel");
+    if (overlap && hipEventRecord(ev_join, side) != hipSuccess) return LAMPA_ERR_LAUNCH;
   }
+  if (overlap && hipStreamWaitEvent(s, ev_join, 0) != hipSuccess) return LAMPA_ERR_LAUNCH;
   hipLaunchKernelGGL((hgdn_walk_kernel<T, KT, VT>), dim3(segs, HV, VT / 32), dim3(64 * (HG_CW + 2)), smem_w, s, pv,
                      pv.chunk_tok0, pv.chunk_len, (const T*)k, H, rec, Ubw, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
                      hstates, L, HV);

@@ -11,6 +11,8 @@ static int g_count = 0;
 static hipEvent_t g_events[PROF_MAX];
 static const char* g_names[PROF_MAX];
 
+bool lampa_prof_recording() { return g_recording; }
+
 void lampa_prof_mark(hipStream_t stream, const char* name) {
   if (!g_recording || g_count >= PROF_MAX) return;
   if (hipEventCreate(&g_events[g_count]) != hipSuccess) return;
