@@ -355,7 +355,8 @@ struct GdrSegSmem {
   static constexpr int T_OFF_T = T_OFF_V + 64 * SV * 2;
   static constexpr int T_OFF_F = T_OFF_T + 3 * 32 * ST * 2;
   static constexpr int N_FACT = 6;  // beta, ek, dk, gamma, rk, misc
-  static constexpr int TILE_BYTES = T_OFF_F + N_FACT * 64 * 4;
+  static constexpr int T_OFF_KD = T_OFF_F + N_FACT * 64 * 4;  // PASS_A: second scaled copy of the k tile
+  static constexpr int TILE_BYTES = T_OFF_KD + (PASS_B ? 0 : 64 * SK * 2);
   static constexpr int OFF_Q = 2 * TILE_BYTES;
   static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
   static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
@@ -365,7 +366,9 @@ struct GdrSegSmem {
 
 // pointers into one of the two tile sets
 struct GdrTiles {
-  __bf16 *k, *v, *t;
+  // PASS_B: k = the raw k tile. PASS_A: k = diag(ek) K and kd = diag(dk) K, rounded to bf16 once (the stagers fold
+  // the per-token gate and norm factors into the tiles, so the chain waves neither read nor apply them)
+  __bf16 *k, *kd, *v, *t;
   float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
 };
 
@@ -418,6 +421,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     unsigned char* base = smem + par * SM::TILE_BYTES;
     GdrTiles t;
     t.k = reinterpret_cast<__bf16*>(base + SM::T_OFF_K);
+    t.kd = reinterpret_cast<__bf16*>(base + (PASS_B ? SM::T_OFF_K : SM::T_OFF_KD));
     t.v = reinterpret_cast<__bf16*>(base + SM::T_OFF_V);
     t.t = reinterpret_cast<__bf16*>(base + SM::T_OFF_T);
     t.beta = reinterpret_cast<float*>(base + SM::T_OFF_F);
@@ -449,14 +453,16 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
     const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
     const int srow = stid >> 1, spart = stid & 1;
-    typename Raw8<T>::type rk_[KU], rv_[VU];
+    // PASS_A keeps the raw k rows of two chunks (sets by chunk parity): the scaled tiles are written from the
+    // registers after the row norms are known, and the next k loads must already be on their way by then
+    typename Raw8<T>::type rk0_[KU], rk1_[PASS_B ? 1 : KU], rv_[VU];
     typename Raw8<T>::type rq0_[PASS_B ? KU : 1], rq1_[PASS_B ? KU : 1];  // q of even / odd chunks of the segment
     bf16x8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
-    auto issue_tiles = [&](int c) {  // k, v, T
+    auto issue_tiles = [&](int c, typename Raw8<T>::type* rk_) {  // k, v, T
       c = uniform(c);
       const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* kb = k + ((size_t)tok0 * H + h) * KT;
@@ -492,7 +498,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 
     float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
     // k, v and T of chunk c from the registers to tile set par
-    auto stage_data = [&](int c, int par) {
+    auto stage_data = [&](int c, int par, const typename Raw8<T>::type* rk_) {
       const GdrTiles tl = tiles(par);
       const bool live = srow < chunk_len[uniform(c)];
 #pragma unroll
@@ -500,9 +506,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         *reinterpret_cast<bf16x8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
       kss = 0.0f;
 #pragma unroll
-      for (int u = 0; u < KU; ++u)
-        *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) =
-            raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+      for (int u = 0; u < KU; ++u) {
+        const bf16x8 piece = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+        if constexpr (PASS_B) *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
+      }
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         float unused = 0.0f;
@@ -511,9 +518,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       }
     };
     // per-token factors of chunk c (gate, beta, norms) into tile set par
-    auto stage_factors = [&](int c, int par) {
+    auto stage_factors = [&](int c, int par, const typename Raw8<T>::type* rk_) {
       const GdrTiles tl = tiles(par);
-      (void)c;
       // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction) and beta, lane = token; both
       // come ready from the chunk's record (zero decay increment and zero beta past the end of a partial chunk)
       const float bv = rb, gv = rg;
@@ -522,14 +528,31 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       // the thread that owns row srow derives that token's factors (gamma / beta of the row sit in lane srow)
       grow = __shfl(gv, srow);
       const float brow = __shfl(bv, srow);
+      const float rk = l2_factor(kss2, l2norm);
+      const float ekr = __builtin_amdgcn_exp2f(grow) * rk, dkr = __builtin_amdgcn_exp2f(g_last - grow) * rk;
       if (spart == 0) {
-        const float rk = l2_factor(kss2, l2norm);
         tl.beta[srow] = brow;
-        tl.ek[srow] = __builtin_amdgcn_exp2f(grow) * rk;
-        tl.dk[srow] = __builtin_amdgcn_exp2f(g_last - grow) * rk;
+        tl.ek[srow] = ekr;
+        tl.dk[srow] = dkr;
         tl.gamma[srow] = grow;
         tl.rk[srow] = rk;
         if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
+      }
+      if constexpr (!PASS_B) {  // the two scaled k tiles, from the raw row that is still in registers
+        const bool live = srow < chunk_len[uniform(c)];
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+          const typename Raw8<T>::type piece = live ? rk_[u] : zero;
+          bf16x8 pe, pd;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float f = (float)piece[e];
+            pe[e] = (__bf16)(f * ekr);
+            pd[e] = (__bf16)(f * dkr);
+          }
+          *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = pe;
+          *reinterpret_cast<bf16x8*>(&tl.kd[srow * SK + spart * (KT / 2) + 8 * u]) = pd;
+        }
       }
     };
     auto stage_q = [&](int c, const typename Raw8<T>::type* rq_) {
@@ -593,35 +616,39 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     // flight any more and would drain the queue at every wait. q(c) / q(c+2) share a register set.
     const int cl = c1 - 1;
     if (nc > 0) {
-      issue_tiles(c0);
+      typename Raw8<T>::type* const rkA = rk0_;
+      typename Raw8<T>::type* const rkB = PASS_B ? rk0_ : rk1_;
+      issue_tiles(c0, rkA);
       issue_gb(c0);
       if constexpr (PASS_B) { issue_q(c0, rq0_); issue_q(min(c0 + 1, cl), rq1_); }
-      stage_data(c0, 0);
-      stage_factors(c0, 0);
-      issue_tiles(min(c0 + 1, cl));
+      stage_data(c0, 0, rkA);
+      stage_factors(c0, 0, rkA);
+      issue_tiles(min(c0 + 1, cl), rkB);
       issue_gb(min(c0 + 1, cl));
       lds_barrier();  // tiles (c0) are ready
-      auto one_chunk = [&](int c, int par, typename Raw8<T>::type* rq_) {
-        if (c + 1 < c1) stage_data(c + 1, par ^ 1);
-        issue_tiles(min(c + 2, cl));
+      // rk_next holds the raw k rows of chunk c + 1, rk_free is loaded with those of chunk c + 2
+      auto one_chunk = [&](int c, int par, typename Raw8<T>::type* rq_, typename Raw8<T>::type* rk_next,
+                           typename Raw8<T>::type* rk_free) {
+        if (c + 1 < c1) stage_data(c + 1, par ^ 1, rk_next);
+        issue_tiles(min(c + 2, cl), rk_free);
         if constexpr (PASS_B) {
           stage_q(c, rq_);
           issue_q(min(c + 2, cl), rq_);
           lds_barrier();  // Qb(c)
           build_p(par);
           lds_barrier();  // B(c)
-          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1, rk_next);
           issue_gb(min(c + 2, cl));
           lds_barrier();  // C(c)
         } else {
-          if (c + 1 < c1) stage_factors(c + 1, par ^ 1);
+          if (c + 1 < c1) stage_factors(c + 1, par ^ 1, rk_next);
           issue_gb(min(c + 2, cl));
           lds_barrier();  // B(c)
         }
       };
       for (int c = c0; c < c1; c += 2) {
-        one_chunk(c, 0, rq0_);
-        if (c + 1 < c1) one_chunk(c + 1, 1, rq1_);
+        one_chunk(c, 0, rq0_, rkB, rkA);
+        if (c + 1 < c1) one_chunk(c + 1, 1, rq1_, rkA, rkB);
       }
     }
     return;
@@ -682,7 +709,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     for (int t8 = 0; t8 < 8; ++t8) {
       const int i0 = 8 * t8 + 4 * hh;
       be[t8] = *reinterpret_cast<const f32x4*>(&tl.beta[i0]);
-      ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
+      if constexpr (PASS_B) ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
       // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
       // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
       vv[t8] = ld_col4(tl.v, SV, 32 * vslab, 8 * t8, lane);
@@ -696,9 +723,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          acc[4 * b4 + e] =
-              be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ek[4 * tm + b4][e] * acc[4 * b4 + e]);
+        for (int e = 0; e < 4; ++e) {
+          const float ks_ = PASS_B ? ek[4 * tm + b4][e] * acc[4 * b4 + e] : acc[4 * b4 + e];
+          acc[4 * b4 + e] = be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ks_);
+        }
       Rb[2 * tm + 0] = acc_to_operand(acc, 0);
       Rb[2 * tm + 1] = acc_to_operand(acc, 8);
     }
@@ -707,10 +735,12 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.k, SK, 32 * km, 16 * ks, lane);
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.kd, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
+    if constexpr (PASS_B) {
 #pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
+      for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
+    }
     const float dec = tl.misc[0];
     bf16x8 Vb[4], Vsb[4];
 #pragma unroll
@@ -720,12 +750,17 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ft[2 * tm + ks], Rb[ks], acc);
       Vb[2 * tm + 0] = acc_to_operand(acc, 0);
       Vb[2 * tm + 1] = acc_to_operand(acc, 8);
+      if constexpr (PASS_B) {
 #pragma unroll
-      for (int b4 = 0; b4 < 4; ++b4)
+        for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[4 * b4 + e] *= dk[4 * tm + b4][e];
-      Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
-      Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
+          for (int e = 0; e < 4; ++e) acc[4 * b4 + e] *= dk[4 * tm + b4][e];
+        Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
+        Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
+      } else {  // (the decay factors are in the kd tile)
+        Vsb[2 * tm + 0] = Vb[2 * tm + 0];
+        Vsb[2 * tm + 1] = Vb[2 * tm + 1];
+      }
     }
     lds_fence();
     lds_barrier();  // B(c): every operand that comes from the k, v and T tiles of chunk c is in registers
