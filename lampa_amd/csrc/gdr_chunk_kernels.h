@@ -344,7 +344,7 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
 //   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
 //                                                          -> the stagers may write q(c+1)
 // Global loads are issued about one chunk period before their data is staged.
-template <int KT, int VT, bool PASS_B>
+template <int KT, int VT, bool PASS_B, bool SCALED = !PASS_B>
 struct GdrSegSmem {
   static constexpr int SK = KT + 8;  // row stride of the k / q tiles (bf16 elements)
   static constexpr int SV = VT + 8;  // row stride of the v and o tiles
@@ -356,7 +356,7 @@ struct GdrSegSmem {
   static constexpr int T_OFF_F = T_OFF_T + 3 * 32 * ST * 2;
   static constexpr int N_FACT = 6;  // beta, ek, dk, gamma, rk, misc
   static constexpr int T_OFF_KD = T_OFF_F + N_FACT * 64 * 4;  // PASS_A: second scaled copy of the k tile
-  static constexpr int TILE_BYTES = T_OFF_KD + (PASS_B ? 0 : 64 * SK * 2);
+  static constexpr int TILE_BYTES = T_OFF_KD + (SCALED ? 64 * SK * 2 : 0);
   static constexpr int OFF_Q = 2 * TILE_BYTES;
   static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
   static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
@@ -366,8 +366,11 @@ struct GdrSegSmem {
 
 // pointers into one of the two tile sets
 struct GdrTiles {
-  // PASS_B: k = the raw k tile. PASS_A: k = diag(ek) K and kd = diag(dk) K, rounded to bf16 once (the stagers fold
-  // the per-token gate and norm factors into the tiles, so the chain waves neither read nor apply them)
+  // k = the raw k tile; or (composite pass with SCALED tiles) k = diag(ek) K and kd = diag(dk) K, rounded to bf16
+  // once: the stagers fold the per-token gate and norm factors into the tiles, so the chain waves neither read nor
+  // apply them. That takes a third of the chain waves' LDS traffic away and pays when many short segments share the
+  // CUs; with few long segments (one workgroup per CU) the stagers' extra work is the longer pole, so the
+  // hierarchical forward instantiates the composite pass with SCALED = false.
   __bf16 *k, *kd, *v, *t;
   float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
 };
@@ -404,7 +407,7 @@ __device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int
   return out;
 }
 
-template <typename T, int KT, int VT, bool PASS_B>
+template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B>
 __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
@@ -413,7 +416,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
                        const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
                        unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o,
                        float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
-  using SM = GdrSegSmem<KT, VT, PASS_B>;
+  constexpr bool SCALED = !PASS_B && SCALED_K;
+  using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -421,7 +425,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     unsigned char* base = smem + par * SM::TILE_BYTES;
     GdrTiles t;
     t.k = reinterpret_cast<__bf16*>(base + SM::T_OFF_K);
-    t.kd = reinterpret_cast<__bf16*>(base + (PASS_B ? SM::T_OFF_K : SM::T_OFF_KD));
+    t.kd = reinterpret_cast<__bf16*>(base + (SCALED ? SM::T_OFF_KD : SM::T_OFF_K));
     t.v = reinterpret_cast<__bf16*>(base + SM::T_OFF_V);
     t.t = reinterpret_cast<__bf16*>(base + SM::T_OFF_T);
     t.beta = reinterpret_cast<float*>(base + SM::T_OFF_F);
@@ -455,7 +459,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     const int srow = stid >> 1, spart = stid & 1;
     // PASS_A keeps the raw k rows of two chunks (sets by chunk parity): the scaled tiles are written from the
     // registers after the row norms are known, and the next k loads must already be on their way by then
-    typename Raw8<T>::type rk0_[KU], rk1_[PASS_B ? 1 : KU], rv_[VU];
+    typename Raw8<T>::type rk0_[KU], rk1_[SCALED ? KU : 1], rv_[VU];
     typename Raw8<T>::type rq0_[PASS_B ? KU : 1], rq1_[PASS_B ? KU : 1];  // q of even / odd chunks of the segment
     bf16x8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
@@ -508,7 +512,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int u = 0; u < KU; ++u) {
         const bf16x8 piece = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
-        if constexpr (PASS_B) *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
+        if constexpr (!SCALED) *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
       }
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
@@ -538,7 +542,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         tl.rk[srow] = rk;
         if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
       }
-      if constexpr (!PASS_B) {  // the two scaled k tiles, from the raw row that is still in registers
+      if constexpr (SCALED) {  // the two scaled k tiles, from the raw row that is still in registers
         const bool live = srow < chunk_len[uniform(c)];
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
@@ -617,7 +621,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     const int cl = c1 - 1;
     if (nc > 0) {
       typename Raw8<T>::type* const rkA = rk0_;
-      typename Raw8<T>::type* const rkB = PASS_B ? rk0_ : rk1_;
+      typename Raw8<T>::type* const rkB = SCALED ? rk1_ : rk0_;
       issue_tiles(c0, rkA);
       issue_gb(c0);
       if constexpr (PASS_B) { issue_q(c0, rq0_); issue_q(min(c0 + 1, cl), rq1_); }
@@ -709,7 +713,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     for (int t8 = 0; t8 < 8; ++t8) {
       const int i0 = 8 * t8 + 4 * hh;
       be[t8] = *reinterpret_cast<const f32x4*>(&tl.beta[i0]);
-      if constexpr (PASS_B) ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
+      if constexpr (!SCALED) ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
       // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
       // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
       vv[t8] = ld_col4(tl.v, SV, 32 * vslab, 8 * t8, lane);
@@ -724,7 +728,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float ks_ = PASS_B ? ek[4 * tm + b4][e] * acc[4 * b4 + e] : acc[4 * b4 + e];
+          const float ks_ = SCALED ? acc[4 * b4 + e] : ek[4 * tm + b4][e] * acc[4 * b4 + e];
           acc[4 * b4 + e] = be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ks_);
         }
       Rb[2 * tm + 0] = acc_to_operand(acc, 0);
@@ -737,7 +741,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.kd, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
-    if constexpr (PASS_B) {
+    if constexpr (!SCALED) {
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
     }
@@ -750,7 +754,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ft[2 * tm + ks], Rb[ks], acc);
       Vb[2 * tm + 0] = acc_to_operand(acc, 0);
       Vb[2 * tm + 1] = acc_to_operand(acc, 8);
-      if constexpr (PASS_B) {
+      if constexpr (!SCALED) {
 #pragma unroll
         for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll

@@ -816,11 +816,11 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   unsigned char* Ubw = ws + w.off_nc;
   float* Oi = (float*)(ws + w.off_oi);
   float* Xi = (float*)(ws + w.off_x);
-  constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_p = HgPrepSmem<KT, VT>::BYTES,
+  constexpr int smem_a = GdrSegSmem<KT, VT, false, false>::BYTES, smem_p = HgPrepSmem<KT, VT>::BYTES,
                 smem_w = HgWalkSmem<KT>::BYTES;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
+    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
         hipFuncSetAttribute((const void*)hgdn_prep_kernel<T, KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             smem_p) != hipSuccess ||
@@ -860,7 +860,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
                      scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
   if (split) {
-    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV),
+    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false, false>), dim3(segs, HV),
                        dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, cs, (const T*)q, (const T*)k, (const T*)v, g,
                        beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nm, Dc, (T*)nullptr,
                        (float*)nullptr, H, HV, scale, l2norm);
