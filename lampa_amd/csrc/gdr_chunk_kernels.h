@@ -502,23 +502,33 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 
     float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
     // k, v and T of chunk c from the registers to tile set par
-    auto stage_data = [&](int c, int par, const typename Raw8<T>::type* rk_) {
+    // rows past the end of a partial chunk become zero (a uniform branch: whole chunks pay nothing for it)
+    auto zero_dead_rows = [&](int c, typename Raw8<T>::type* regs, int n) __attribute__((always_inline)) {
+      const int len = chunk_len[uniform(c)];
+      if (len < 64) {
+        const bool live = srow < len;
+#pragma unroll
+        for (int u = 0; u < n; ++u) regs[u] = live ? regs[u] : zero;
+      }
+    };
+    auto stage_data = [&](int c, int par, typename Raw8<T>::type* rk_) {
       const GdrTiles tl = tiles(par);
-      const bool live = srow < chunk_len[uniform(c)];
+      zero_dead_rows(c, rk_, KU);
+      zero_dead_rows(c, rv_, VU);
 #pragma unroll
       for (int j = 0; j < 3; ++j)
         *reinterpret_cast<bf16x8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
       kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u) {
-        const bf16x8 piece = raw_to_bf16<T>(live ? rk_[u] : zero, kss, want_ss);
+        const bf16x8 piece = raw_to_bf16<T>(rk_[u], kss, want_ss);
         if constexpr (!SCALED) *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
       }
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         float unused = 0.0f;
         *reinterpret_cast<bf16x8*>(&tl.v[srow * SV + spart * (VT / 2) + 8 * u]) =
-            raw_to_bf16<T>(live ? rv_[u] : zero, unused, false);
+            raw_to_bf16<T>(rv_[u], unused, false);
       }
     };
     // per-token factors of chunk c (gate, beta, norms) into tile set par
@@ -543,10 +553,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
       }
       if constexpr (SCALED) {  // the two scaled k tiles, from the raw row that is still in registers
-        const bool live = srow < chunk_len[uniform(c)];
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
-          const typename Raw8<T>::type piece = live ? rk_[u] : zero;
+          const typename Raw8<T>::type piece = rk_[u];  // (dead rows were zeroed by stage_data)
           bf16x8 pe, pd;
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -559,13 +568,13 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         }
       }
     };
-    auto stage_q = [&](int c, const typename Raw8<T>::type* rq_) {
-      const bool live = srow < chunk_len[uniform(c)];
+    auto stage_q = [&](int c, typename Raw8<T>::type* rq_) {
+      zero_dead_rows(c, rq_, KU);
       float qss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
         *reinterpret_cast<bf16x8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
-            raw_to_bf16<T>(live ? rq_[u] : zero, qss, want_ss);
+            raw_to_bf16<T>(rq_[u], qss, want_ss);
       qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
       if (spart == 0) {
         const float rq = l2_factor(qss, l2norm);
