@@ -161,6 +161,33 @@ def main():
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "kernel_us": round(stage_us[dominant], 2), "algorithmic_bytes_per_launch": dom_bytes}
+    # ---- what the output pass's access pattern costs with no arithmetic (memory-only twin of that kernel: same rows
+    #      of q, k, v, the per-chunk records and the o rows per workgroup and chunk; whole chunks only) ----
+    n_chunks_probe = T // 64
+    rec = torch.zeros(n_chunks_probe * H * 6656, dtype=torch.uint8, device=dev)
+    o_probe = torch.empty_like(vd)
+    cps_probe = gd._default_chunks_per_segment([(T + 63) // 64], H, 2 * torch.cuda.get_device_properties(dev).multi_processor_count)
+
+    def probe():
+        _capi.check(_capi.lib().lampa_gdr_traffic_probe(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), rec.data_ptr(),
+                                                        o_probe.data_ptr(), n_chunks_probe, H, cps_probe,
+                                                        torch.cuda.current_stream().cuda_stream), "traffic probe")
+    for _ in range(20):
+        probe()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(100):
+        probe()
+    ev1.record()
+    torch.cuda.synchronize()
+    probe_us = 1e3 * ev0.elapsed_time(ev1) / 100
+    probe_bytes = n_chunks_probe * H * (4 * 64 * 64 * 2 + 6656)
+    roofline["memory_only_twin"] = {
+        "us": round(probe_us, 2), "bytes": probe_bytes, "GB/s": round(probe_bytes / (probe_us * 1e-6) / 1e9, 1),
+        "kernel_over_twin": round(stage_us.get("gdr_segment_kernel<output>", float("nan")) / probe_us, 3),
+        "note": "the output pass's loads and stores with no arithmetic (lampa_gdr_traffic_probe), 100 launches with "
+                "HIP events: the practical floor of that kernel on this memory system"}
+    del rec, o_probe
     # ---- per-step distribution (HIP events on the launch stream, one pair per step) and a cold variant that rotates
     #      among input sets totalling more than 512 MB, so that no step finds its inputs in the memory-side cache ----
     def event_times(fn, n):

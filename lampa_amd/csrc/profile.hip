@@ -50,3 +50,64 @@ extern "C" int lampa_profile_end(int max_entries, float* ms, const char** names)
   g_count = 0;
   return n;
 }
+
+// ---- memory-only twin of the output pass ----------------------------------------------------------------------------
+// The loads and stores of the chunk pipeline's output pass (K = V = 64, 2-byte elements, one dense sequence of whole
+// chunks) with no arithmetic at all: per (segment, head) workgroup and chunk, 128 threads fetch the chunk's k, v and q
+// rows (128 bytes per row and head, rows one token apart) and its 6.5 KiB record one chunk ahead, the other 128
+// threads store the o rows. Its duration is what this access pattern costs on the memory system alone, i.e. the
+// practical floor of the output pass (the algorithmic roofline assumes 8 TB/s for any pattern).
+typedef unsigned int prof_u32x4 __attribute__((ext_vector_type(4)));
+#define PROBE_REC_U4 416  // 6656-byte record of a chunk and head, in 16-byte units
+
+__global__ void __launch_bounds__(256, 2)
+    gdr_traffic_probe_kernel(const prof_u32x4* __restrict__ q, const prof_u32x4* __restrict__ k,
+                             const prof_u32x4* __restrict__ v, const prof_u32x4* __restrict__ rec,
+                             prof_u32x4* __restrict__ o, int n_chunks, int H, int cps) {
+  const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int c0 = seg * cps, c1 = min(c0 + cps, n_chunks);
+  if (tid < 128) {
+    const int row = tid >> 1, half = tid & 1;
+    prof_u32x4 buf[15], acc = {0, 0, 0, 0};
+    auto issue = [&](int c) __attribute__((always_inline)) {
+      c = min(c, c1 - 1);
+      const size_t base = ((size_t)(c * 64 + row) * H + h) * 8 + half * 4;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { buf[u] = k[base + u]; buf[4 + u] = v[base + u]; buf[8 + u] = q[base + u]; }
+      const prof_u32x4* rp = rec + ((size_t)c * H + h) * PROBE_REC_U4;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) buf[12 + j] = rp[tid + 128 * j];
+    };
+    issue(c0);
+    for (int c = c0; c < c1; ++c) {
+#pragma unroll
+      for (int u = 0; u < 15; ++u) acc += buf[u];
+      issue(c + 1);
+      __syncthreads();
+    }
+    if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) o[0] = acc;  // keeps the loads alive; never true in practice
+  } else {
+    const int t = tid - 128;
+    for (int c = c0; c < c1; ++c) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int piece = t + 128 * j, row = piece >> 3, part = piece & 7;
+        const prof_u32x4 val = {(unsigned)c, (unsigned)row, (unsigned)part, 0u};
+        o[((size_t)(c * 64 + row) * H + h) * 8 + part] = val;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// q, k, v, o: [n_chunks * 64, H, 64] 2-byte elements; records: n_chunks * H * 6656 bytes (any content). o is
+// overwritten with a pattern. One launch = one pass.
+extern "C" int lampa_gdr_traffic_probe(const void* q, const void* k, const void* v, const void* records, void* o,
+                                       int n_chunks, int H, int chunks_per_segment, void* stream) {
+  if (!q || !k || !v || !records || !o || n_chunks < 1 || H < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
+  const int segs = (n_chunks + chunks_per_segment - 1) / chunks_per_segment;
+  hipLaunchKernelGGL(gdr_traffic_probe_kernel, dim3(segs, H), dim3(256), 0, (hipStream_t)stream,
+                     (const prof_u32x4*)q, (const prof_u32x4*)k, (const prof_u32x4*)v, (const prof_u32x4*)records,
+                     (prof_u32x4*)o, n_chunks, H, chunks_per_segment);
+  return hipGetLastError() == hipSuccess ? LAMPA_OK : LAMPA_ERR_LAUNCH;
+}
