@@ -59,31 +59,38 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
     if (segs > n_seq) {
       hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
                          (const T*)q, (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nc, Dc,
-                         (T*)nullptr, (float*)nullptr, H, HV, scale, l2norm);
+                         (T*)nullptr, (float*)nullptr, H, HV, scale, l2norm, (const unsigned char*)nullptr,
+                         (const unsigned char*)nullptr, (const float*)nullptr, (const float*)nullptr, 0);
       LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     }
   }
   const int gmax = (max_nseg + GDR_SCAN_GROUP - 1) / GDR_SCAN_GROUP;
-  if (max_nseg >= 3 * GDR_SCAN_GROUP && (int64_t)n_seq * gmax <= w.max_groups) {
+  unsigned char* Gm = ws + w.off_gm;
+  unsigned char* Gn = ws + w.off_gn;
+  float* Gd = (float*)(ws + w.off_gd);
+  // The output pass can walk the composites before its segment itself (K = 64: its chain waves hold whole columns
+  // of the state in few enough registers); otherwise a leaf pass writes every segment's initial state.
+  const bool two_level = max_nseg >= 3 * GDR_SCAN_GROUP && (int64_t)n_seq * gmax <= w.max_groups;
+  const bool walk_in_output = two_level && KT == 64;
+  if (two_level) {
     // long sequences: group composites, then every group's scan (which walks the earlier groups' composites first)
-    unsigned char* Gm = ws + w.off_gm;
-    unsigned char* Gn = ws + w.off_gn;
-    float* Gd = (float*)(ws + w.off_gd);
     const dim3 block(64 * (KT / 32));
     hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
                        Nc, Dc, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<group>");
-    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc, Dc,
-                       h0, Si, Gm, Gn, Gd, HV, segs, gmax);
-    LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
+    if (!walk_in_output) {
+      hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc,
+                         Dc, h0, Si, Gm, Gn, Gd, HV, segs, gmax);
+      LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
+    }
   } else {
     hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
                        pv, Mc, Nc, Dc, h0, Si, HV, segs);
     LAMPA_PROF(s, "gdr_scan_kernel");
   }
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
-                     (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, (unsigned char*)nullptr, (unsigned char*)nullptr,
-                     (float*)nullptr, (T*)o, ht, H, HV, scale, l2norm);
+                     (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, Mc, Nc, Dc, (T*)o, ht, H, HV, scale,
+                     l2norm, (const unsigned char*)Gm, (const unsigned char*)Gn, (const float*)Gd, h0, walk_in_output ? gmax : 0);
   LAMPA_PROF(s, "gdr_segment_kernel<output>");
   return lampa_launch_status();
 }

@@ -56,6 +56,7 @@ static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_d
 // [64] each. The segment kernels take the two factor rows from here: in g and beta themselves a head's 64 values sit
 // 4 bytes apart in rows that interleave all heads, so every workgroup would fetch the sectors of all of them.
 #define REC_BYTES (T_BYTES + 2 * 64 * 4)
+#define GDR_SCAN_GROUP 8  // segments per group of the two-level scan; a multiple of its ring depth
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
   return *reinterpret_cast<const bf16x8*>(base + (size_t)frag * 1024 + lane * 16);
@@ -415,7 +416,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
                        const unsigned char* __restrict__ tmat,
                        const float* __restrict__ Sinit, unsigned char* __restrict__ Mcomp,
                        unsigned char* __restrict__ Ncomp, float* __restrict__ Dcomp, T* __restrict__ o,
-                       float* __restrict__ ht, int H, int HV, float scale, int l2norm) {
+                       float* __restrict__ ht, int H, int HV, float scale, int l2norm,
+                       const unsigned char* __restrict__ Mgrp, const unsigned char* __restrict__ Ngrp,
+                       const float* __restrict__ Dgrp, const float* __restrict__ h0, int gmax) {
   constexpr bool SCALED = !PASS_B && SCALED_K;
   using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
@@ -675,7 +678,68 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   const float vmask = is_m ? 0.0f : 1.0f;
 
   f32x16 S[KT / 32];
-  if (PASS_B) {  // the scan leaves every segment's initial state as 32-column slabs in accumulator order
+  bool walked = false;
+  if constexpr (PASS_B && KT == 64) if (gmax > 0) {
+    walked = true;
+    // Two-level scan, second level done here: the state this segment starts from = the sequence's initial state
+    // pushed through the composites of the groups before this segment's group (Mgrp / Ngrp / Dgrp, written by the
+    // group pass) and then through the composites of the segments before it inside its group (at most
+    // 2 (GDR_SCAN_GROUP - 1) steps S <- d S + N + M' S). This wave owns all rows of its 32 columns, so the state
+    // feeds the next step's B operand straight from the accumulators.
+    constexpr int NKS = KT / 16, NKM = KT / 32;
+    constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+    const int seq = pv.seg_seq[seg], local = seg - pv.seq_seg0[seq];
+    const int lead = local / GDR_SCAN_GROUP, nst = lead + local % GDR_SCAN_GROUP;
+    const int item0 = seg - local % GDR_SCAN_GROUP;
+#pragma unroll
+    for (int km = 0; km < NKM; ++km)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        S[km][r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col] : 0.0f;
+    bf16x8 rm[2][NKM * NKS];
+    f32x4 rn[2][NKM * 4];
+    float rd[2];
+    auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) __attribute__((always_inline)) {
+      p = uniform(max(0, min(p, nst - 1)));
+      const bool top = p < lead;
+      const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
+      const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mgrp : Mcomp) + sh * M_BYTES);
+      const f32x4* N = reinterpret_cast<const f32x4*>((top ? Ngrp : Ncomp) + (sh * (VT / 32) + vslab) * N_BYTES);
+#pragma unroll
+      for (int f = 0; f < NKM * NKS; ++f) m[f] = M[f * 64 + lane];
+#pragma unroll
+      for (int f = 0; f < NKM * 4; ++f) n[f] = N[f * 64 + lane];
+      d = (top ? Dgrp : Dcomp)[sh];
+    };
+    auto step = [&](const bf16x8* m, const f32x4* n, float d) __attribute__((always_inline)) {
+      bf16x8 Sb[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+#pragma unroll
+      for (int km = 0; km < NKM; ++km) {
+        f32x16 acc;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(d, S[km][4 * q4 + e], n[km * 4 + q4][e]);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) acc = mfma32(m[km * NKS + ks], Sb[ks], acc);
+        S[km] = acc;
+      }
+    };
+    if (nst > 0) {
+      issue(0, rm[0], rn[0], rd[0]);
+      issue(1, rm[1], rn[1], rd[1]);
+      for (int p = 0; p < nst; p += 2) {
+        step(rm[0], rn[0], rd[0]);
+        issue(p + 2, rm[0], rn[0], rd[0]);
+        if (p + 1 < nst) step(rm[1], rn[1], rd[1]);
+        issue(p + 3, rm[1], rn[1], rd[1]);
+      }
+    }
+  }
+  if (walked) {
+  } else if (PASS_B) {  // the scan leaves every segment's initial state as 32-column slabs in accumulator order
     const f32x4* si = reinterpret_cast<const f32x4*>(Sinit + (((size_t)seg * HV + hv) * (VT / 32) + vslab) * (KT * 32));
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
@@ -993,7 +1057,6 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 //          single-level scan writes).
 // Same step code in both modes; loops are branch free with clamped operands and a spare store slot as above.
 enum { SCAN_GROUP = 1, SCAN_LEAF = 2 };
-#define GDR_SCAN_GROUP 8  // segments per group; a multiple of the ring depth
 
 template <int KT, int VT, int DEPTH, int MODE>
 __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlanView pv,

@@ -863,7 +863,8 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
     hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false, false>), dim3(segs, HV),
                        dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, cs, (const T*)q, (const T*)k, (const T*)v, g,
                        beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nm, Dc, (T*)nullptr,
-                       (float*)nullptr, H, HV, scale, l2norm);
+                       (float*)nullptr, H, HV, scale, l2norm, (const unsigned char*)nullptr,
+                       (const unsigned char*)nullptr, (const float*)nullptr, (const float*)nullptr, 0);
     LAMPA_PROF(s, "gdr_segment_kernel<composite>");
     hipLaunchKernelGGL((hgdn_scan_kernel<KT, VT>), dim3(VT / 32, n_seq, HV), dim3(64 * HG_CW), 0, cs, pv, Mc, Nm, Dc, Xi,
                        HV, p);
