@@ -35,9 +35,9 @@ LSH_BYTES_PER_HIT_TABLE = 224
 # HBM bytes per launch at config 2 from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a plain
 # 256 MiB copy gives): profiles/bench_config1_config2_config3_hbm_traffic_pmc.md. Counters cannot be read from inside a run.
 MEASURED_TRAFFIC_BYTES = {
-    "gdr_segment_kernel<output>": 304.6e6,
-    "gdr_segment_kernel<composite>": 184.0e6,
-    "gdr_tinv_kernel": 142.2e6,
+    "gdr_segment_kernel<output>": 350.2e6,
+    "gdr_segment_kernel<composite>": 184.1e6,
+    "gdr_tinv_kernel": 141.8e6,
     "gdr_scan_kernel": 24.7e6,
     "gdr_scan2_kernel<group>": 30.9e6,
     "gdr_scan2_kernel<leaf>": 29.1e6,
