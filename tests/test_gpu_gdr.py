@@ -104,7 +104,8 @@ def test_chunk_segment_split_is_invisible(device, cps, monkeypatch):
 @pytest.mark.parametrize("K,V,n_chunks", [(64, 64, 24), (64, 64, 27), (64, 64, 63), (128, 128, 41), (64, 128, 33)])
 def test_two_level_scan_over_many_segments(device, K, V, n_chunks, monkeypatch):
     """One chunk per segment makes 24 or more segments per sequence: the scan then runs as group composites, a scan
-    over the groups and a scan inside the groups (groups of 8; 27 / 41 / 33 leave a ragged last group). Weak decay, so
+    over the groups and a scan inside the groups (groups of 8; 27 / 41 / 33 leave a ragged last group); at K = 64 the
+    output pass does the last two itself, at K = 128 a leaf launch does. Weak decay, so
     that the state really travels through all the levels; initial state and final state included."""
     monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", 1)
     T = 64 * n_chunks - 5
