@@ -233,3 +233,25 @@ def test_config4_varlen_batch_d128(device):
     o1, s1 = gd.chunk_gated_delta_rule(dq[:, a:b], dk[:, a:b], dv[:, a:b], dg[:, a:b], db[:, a:b], output_final_state=True)
     _assert_bf16_close(o[:, a:b], o1.float().cpu(), "o alone")
     _assert_bf16_close(s[i:i + 1], s1.cpu(), "state alone")
+
+
+def test_traffic_probe_writes_every_output_row(device):
+    """The memory-only twin of the output pass (a measurement aid): it must touch exactly the rows the real kernel
+    writes. Its stores carry (chunk, row, 16-byte piece) so that coverage can be checked; ragged last segment."""
+    from lampa_amd import _capi
+    n_chunks, H, cps = 11, 3, 4
+    T = 64 * n_chunks
+    q, k, v = (torch.zeros(T, H, 64, dtype=torch.bfloat16, device=device) for _ in range(3))
+    rec = torch.zeros(n_chunks * H * 6656, dtype=torch.uint8, device=device)
+    o = torch.full((T, H, 64), -1.0, dtype=torch.bfloat16, device=device)
+    _capi.check(_capi.lib().lampa_gdr_traffic_probe(q.data_ptr(), k.data_ptr(), v.data_ptr(), rec.data_ptr(), o.data_ptr(),
+                                                    n_chunks, H, cps, torch.cuda.current_stream().cuda_stream), "probe")
+    torch.cuda.synchronize()
+    words = o.view(torch.int32).reshape(n_chunks, 64, H, 8, 4).cpu()  # [chunk, row, head, piece, word]
+    want = torch.zeros_like(words)
+    want[..., 0] = torch.arange(n_chunks).view(-1, 1, 1, 1)
+    want[..., 1] = torch.arange(64).view(1, -1, 1, 1)
+    want[..., 2] = torch.arange(8).view(1, 1, 1, -1)
+    assert torch.equal(words, want)
+    assert _capi.lib().lampa_gdr_traffic_probe(None, k.data_ptr(), v.data_ptr(), rec.data_ptr(), o.data_ptr(), n_chunks, H,
+                                               cps, None) == -1
