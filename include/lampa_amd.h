@@ -8,7 +8,10 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all work is enqueued on it and the
  *     functions return without synchronising;
  *   - return value: 0 on success, negative on error (LAMPA_ERR_*). No C++ exception crosses the boundary;
- *   - the library keeps no state between calls apart from the optional profiling recorder.
+ *   - state the library keeps between calls: the optional profiling recorder; one helper stream with two events per
+ *     (device, caller stream) that lampa_hgdn_chunk_fwd creates on first use and keeps until the process ends (calls
+ *     on different streams or host threads never share them).
+ *     Everything else lives in caller-owned buffers, so calls on different streams do not interfere.
  * The reference (chengjiang123/Lampa) is Python over Triton/ATen, so each entry point names the Python operator or
  * kernel it replaces (file:line in the reference tree).
  */
@@ -107,11 +110,13 @@ int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, 
 
 /* dst[s, i, :] = src[s % src_segments, idx[s, i], :]. Replaces batched_index_select / sort_to_buckets /
  * unsort_from_buckets and the points.gather of LSHOrdering (hash_utils.py:83-93; hept.py:9-19;
- * full_mamba2.py:213-216,679-682). idx_bytes = 4 (int32) or 8 (int64); rows of row_bytes bytes. */
+ * full_mamba2.py:213-216,679-682). idx_bytes = 4 (int32) or 8 (int64); rows of row_bytes bytes. A row whose index
+ * is outside [0, n_src) is written as zeros (torch.gather would raise; no device-side error exists here). */
 int lampa_gather_rows(const void* src, int src_segments, int64_t n_src, const void* idx, int idx_bytes,
                       int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
 
-/* dst[s, idx[s, i], :] = src[s, i, :] (unsort by scatter, the O(n) alternative to full_mamba2.py:678-682). */
+/* dst[s, idx[s, i], :] = src[s, i, :] (unsort by scatter, the O(n) alternative to full_mamba2.py:678-682). Rows whose
+ * index is outside [0, n) are dropped. */
 int lampa_scatter_rows(const void* src, const void* idx, int idx_bytes, int n_segments, int64_t n,
                        int64_t row_bytes, void* dst, void* stream);
 

@@ -18,7 +18,7 @@ __device__ __forceinline__ int64_t gs_index(const void* idx, int64_t i) {
 template <typename VecT, typename IdxT, bool GATHER>
 __global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restrict__ src, int64_t src_seg_stride,
                                                           int src_segments, int group, const void* __restrict__ idx, int64_t n,
-                                                          int64_t n_src, int vec_per_row, char* __restrict__ dst, int* bad) {
+                                                          int64_t n_src, int vec_per_row, char* __restrict__ dst) {
   const int seg = blockIdx.y;
   const int64_t item = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
   const int64_t row = item / vec_per_row;
@@ -26,11 +26,13 @@ __global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restric
   if (row >= n) return;
   const int64_t other = gs_index<IdxT>(idx, (int64_t)seg * n + row);
   const int64_t limit = GATHER ? n_src : n;
+  const int64_t row_bytes = (int64_t)vec_per_row * (int64_t)sizeof(VecT);
   if (other < 0 || other >= limit) {
-    if (bad) *bad = 1;
+    // an index outside the source: a gathered row reads as zeros (never as whatever the output buffer held), a
+    // scattered row is dropped
+    if (GATHER) reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + row) * row_bytes)[piece] = VecT{};
     return;
   }
-  const int64_t row_bytes = (int64_t)vec_per_row * (int64_t)sizeof(VecT);
   const int64_t from = GATHER ? other : row, to = GATHER ? row : other;
   const VecT* s = reinterpret_cast<const VecT*>(src + ((seg / group) % src_segments) * src_seg_stride + from * row_bytes) + piece;
   VecT* d = reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + to) * row_bytes) + piece;
@@ -61,21 +63,21 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
   LAMPA_PROF(s, "start");
   if (vec == 16)
     hipLaunchKernelGGL((gs_rows_kernel<uint4, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride, src_segments,
-                       group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       group, idx, n, n_src, vec_per_row, (char*)dst);
   else if (vec == 4)
     hipLaunchKernelGGL((gs_rows_kernel<uint32_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
-                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst);
   else
     hipLaunchKernelGGL((gs_rows_kernel<uint8_t, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride,
-                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst, (int*)nullptr);
+                       src_segments, group, idx, n, n_src, vec_per_row, (char*)dst);
   LAMPA_PROF(s, "gs_rows_kernel");
   return lampa_launch_status();
 }
 
 // dst [S, n, row_bytes] = rows of src selected by idx [S, n]. src is [src_segments, n_src, row_bytes] and segment s
 // reads source segment s % src_segments (src_segments == S: one source per segment; a divisor of S: the sources
-// are shared round-robin, which is how a [1, batch, ...] tensor broadcasts over [n_hashes, batch, ...] indices). idx_bytes is 4 (int32) or 8 (int64). Out-of-range
-// indices are skipped (the destination row is left untouched).
+// are shared round-robin, which is how a [1, batch, ...] tensor broadcasts over [n_hashes, batch, ...] indices). idx_bytes is 4 (int32) or 8 (int64). A row whose
+// index lies outside the source is written as zeros.
 // Segment s reads source segment (s / group) % src_segments (group = 1: the exported behaviour; group = tables per
 // event: a batch of events whose tables share the event's rows).
 int lampa_gather_rows_grouped(const void* src, int src_segments, int group, int64_t n_src, const void* idx,

@@ -90,6 +90,11 @@ __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirs
 
 __device__ __forceinline__ int acc_row(int r, int hh) { return 8 * (r / 4) + 4 * hh + (r % 4); }
 
+// 2^x for x <= 0, otherwise 0 (also for NaN): the reference's safe_exp (models/hattention/fla_op.py:27-29), which it
+// applies to every DIFFERENCE of cumulative log-decays (chunk_scaled_dot_kkt.py:67, chunk_o.py:98, chunk_delta_h.py:152).
+// With g <= 0 those differences are never positive and this is a plain exp2.
+__device__ __forceinline__ float safe_exp2(float x) { return __builtin_amdgcn_exp2f(x <= 0.0f ? x : -1e30f); }
+
 __device__ __forceinline__ float l2_factor(float ss, int l2norm) {
   if (l2norm == GDR_L2_CHUNK) return 1.0f / __fsqrt_rn(ss + 1e-6f);
   if (l2norm == GDR_L2_RECURRENT) return 1.0f / (__fsqrt_rn(ss) + 1e-6f);
@@ -163,7 +168,7 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
   {  // gamma is kept in units of log 2 (exp2 is one instruction)
     const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
     const float gv = g[gi], bv = beta[gi];
-    const float gcum = 1.44269504f * wave_inclusive_scan(lane < len ? gv : 0.0f), bz = lane < len ? bv : 0.0f;
+    const float gcum = 1.44269504f * wave_cumulative_decay(lane < len ? gv : 0.0f), bz = lane < len ? bv : 0.0f;
     s_gamma[lane] = gcum;
     s_beta[lane] = bz;
     float* fact = reinterpret_cast<float*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES + T_BYTES);
@@ -210,14 +215,14 @@ __global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k
     if (t == 1) {  // rows j (tile 0), columns i (tile 1): i > j always
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * __builtin_amdgcn_exp2f(gc - gr4[r / 4][r % 4]);
+        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * safe_exp2(gc - gr4[r / 4][r % 4]);
     } else {       // rows i, columns j of a diagonal block; the mask goes on the exponent (branch-free)
       float* blk = t == 0 ? s_A11 : s_A22;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int il = acc_row(r, hh);
         blk[il * SB + ln] = acc[r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
-                            __builtin_amdgcn_exp2f(il > ln ? gr4[r / 4][r % 4] - gc : -1e30f);
+                            safe_exp2(il > ln ? gr4[r / 4][r % 4] - gc : 1.0f);
       }
     }
   }
@@ -546,7 +551,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       grow = __shfl(gv, srow);
       const float brow = __shfl(bv, srow);
       const float rk = l2_factor(kss2, l2norm);
-      const float ekr = __builtin_amdgcn_exp2f(grow) * rk, dkr = __builtin_amdgcn_exp2f(g_last - grow) * rk;
+      const float ekr = __builtin_amdgcn_exp2f(grow) * rk, dkr = safe_exp2(g_last - grow) * rk;
       if (spart == 0) {
         tl.beta[srow] = brow;
         tl.ek[srow] = ekr;
@@ -618,7 +623,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
             for (int r = 8 * part; r < 8 * part + 8; ++r) {  // the mask goes on the exponent: branch-free
               const int j = 32 * jm + acc_row(r, hh);
-              acc[r] *= fi * rj[r / 4][r % 4] * __builtin_amdgcn_exp2f(i >= j ? gi - gj[r / 4][r % 4] : -1e30f);
+              acc[r] *= fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f);
             }
             frag_store(s_P, f0 + part, lane, acc_to_operand(acc, 8 * part));
           }

@@ -92,6 +92,31 @@ __device__ __forceinline__ float wave_inclusive_scan(float x) {
   return x;
 }
 
+// Inclusive running minimum / maximum over the 64 lanes (same data movement as the prefix sum; exact).
+__device__ __forceinline__ float wave_inclusive_min(float x) {
+  const float inf = __builtin_inff();
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_SHR(1), 0xF>(inf, x));
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_SHR(2), 0xF>(inf, x));
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_SHR(4), 0xF>(inf, x));
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_SHR(8), 0xF>(inf, x));
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_BCAST15, 0xA>(inf, x));
+  x = fminf(x, dpp_f32<GDR_DPP_ROW_BCAST31, 0xC>(inf, x));
+  return x;
+}
+__device__ __forceinline__ float wave_inclusive_max(float x) { return -wave_inclusive_min(-x); }
+
+// In-chunk cumulative log-decay of a wave's 64 tokens (lane = token). A tree-shaped prefix sum is not monotone in
+// floating point: with every g <= 0 a later lane can still come out an ulp ABOVE an earlier one, and the decay ratios
+// e^{gamma_i - gamma_j} are masked wherever that difference is positive (safe_exp), which would drop whole terms.
+// So the non-positive and the positive parts of g are summed separately and each prefix is made exactly monotone by a
+// running minimum / maximum: for g <= 0 the result never increases from one token to the next.
+__device__ __forceinline__ float wave_cumulative_decay(float g) {
+  if (__ballot(g != g)) return wave_inclusive_scan(g);  // a NaN decay poisons everything after it, as in the reference
+  float cum = wave_inclusive_min(wave_inclusive_scan(fminf(g, 0.0f)));
+  if (__ballot(g > 0.0f)) cum += wave_inclusive_max(wave_inclusive_scan(fmaxf(g, 0.0f)));
+  return cum;
+}
+
 // Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every outstanding global load
 // and store of the wave (vmcnt(0)), which would serialise the software prefetch of the next chunk behind each
 // barrier; here only the LDS / scalar counter is drained.

@@ -28,6 +28,47 @@
 //   scan   (sequences cut into segments of 2^p chunks) the same walk over whole segments with the segment
 //          composites (M, N) of the plain rule: leaves every segment's entering level states.
 #include "gdr_chunk_kernels.h"
+#include <mutex>
+
+// Helper stream + fork / join events for the composites that run beside the prep kernel: one set per (device, caller
+// stream), created on first use and kept until the process ends, so that calls on different streams or from different
+// host threads never share an event. hg_side_lock is held while a call enqueues its fork .. join section, which keeps
+// the record / wait pairs of two host threads that use the same caller stream from interleaving.
+struct HgSide {
+  int device;
+  hipStream_t caller, side;
+  hipEvent_t fork, join;
+};
+#define HG_MAX_SIDES 32
+static HgSide hg_sides[HG_MAX_SIDES];
+static int hg_n_sides = 0;
+static std::mutex hg_side_lock;
+
+// (call with hg_side_lock held) the set of this device and caller stream, or nullptr: the call then runs on one stream
+static HgSide* hg_side_for(hipStream_t caller) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  for (int i = 0; i < hg_n_sides; ++i)
+    if (hg_sides[i].device == dev && hg_sides[i].caller == caller) return &hg_sides[i];
+  if (hg_n_sides == HG_MAX_SIDES) return nullptr;
+  HgSide n;
+  n.device = dev;
+  n.caller = caller;
+  if (hipStreamCreateWithFlags(&n.side, hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  if (hipEventCreateWithFlags(&n.fork, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipStreamDestroy(n.side);
+    return nullptr;
+  }
+  if (hipEventCreateWithFlags(&n.join, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipEventDestroy(n.fork);
+    (void)hipStreamDestroy(n.side);
+    return nullptr;
+  }
+  hg_sides[hg_n_sides] = n;
+  return &hg_sides[hg_n_sides++];
+}
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -818,7 +859,10 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   float* Xi = (float*)(ws + w.off_x);
   constexpr int smem_a = GdrSegSmem<KT, VT, false, false>::BYTES, smem_p = HgPrepSmem<KT, VT>::BYTES,
                 smem_w = HgWalkSmem<KT>::BYTES;
-  static bool attr_set = false;
+  static bool attr_set_dev[64];  // the attribute belongs to the device's copy of the kernel
+  int cur_dev = 0;
+  if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev < 0 || cur_dev >= 64) return LAMPA_ERR_LAUNCH;
+  bool& attr_set = attr_set_dev[cur_dev];
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
@@ -839,17 +883,16 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   // workgroups: they run on a second stream (default priority) beside the prep kernel (launched first, which
   // measured slightly better than the other order) and join before the walk.
   // With a profile recording open everything stays on the caller's stream, so that the intervals mean one kernel each.
-  static hipStream_t side = nullptr;
-  static hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   bool overlap = split && !lampa_prof_recording();
-  if (overlap && !side) {
-    if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess ||
-        hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming) != hipSuccess ||
-        hipEventCreateWithFlags(&ev_join, hipEventDisableTiming) != hipSuccess) {
-      side = nullptr;
-      overlap = false;
-    }
+  std::unique_lock<std::mutex> hold(hg_side_lock, std::defer_lock);
+  HgSide* sd = nullptr;
+  if (overlap) {
+    hold.lock();
+    sd = hg_side_for(s);
+    if (!sd) { overlap = false; hold.unlock(); }
   }
+  hipStream_t side = sd ? sd->side : s;
+  hipEvent_t ev_fork = sd ? sd->fork : nullptr, ev_join = sd ? sd->join : nullptr;
   hipStream_t cs = s;  // the stream of the composites
   if (overlap) {
     if (hipEventRecord(ev_fork, s) != hipSuccess || hipStreamWaitEvent(side, ev_fork, 0) != hipSuccess) return LAMPA_ERR_LAUNCH;
@@ -871,7 +914,10 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
     LAMPA_PROF(s, "hgdn_scan_kernel");
     if (overlap && hipEventRecord(ev_join, side) != hipSuccess) return LAMPA_ERR_LAUNCH;
   }
-  if (overlap && hipStreamWaitEvent(s, ev_join, 0) != hipSuccess) return LAMPA_ERR_LAUNCH;
+  if (overlap) {
+    if (hipStreamWaitEvent(s, ev_join, 0) != hipSuccess) return LAMPA_ERR_LAUNCH;
+    hold.unlock();
+  }
   hipLaunchKernelGGL((hgdn_walk_kernel<T, KT, VT>), dim3(segs, HV, VT / 32), dim3(64 * (HG_CW + 2)), smem_w, s, pv,
                      pv.chunk_tok0, pv.chunk_len, (const T*)k, H, rec, Ubw, Oi, split ? (const float*)Xi : (const float*)nullptr, (T*)o,
                      hstates, L, HV);

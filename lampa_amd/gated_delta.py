@@ -119,6 +119,23 @@ class _ForwardOnly(torch.autograd.Function):
         raise NotImplementedError("lampa_amd gated-delta operators are forward-only")
 
 
+def _check_shapes(q, k, v, g, beta, what):
+    """g and beta are per (token, value head): [B, T, HV]. The reference's token-serial kernel also takes a headwise
+    beta [B, T, HV, V] (``gated_delta_rule_ori.py:444-447,515``); that variant is not built, and reading such a tensor
+    with the scalar stride would silently give wrong values, so it is refused."""
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:2] != q.shape[:2]:
+        raise ValueError(f"{what}: expected q, k [B, T, H, K] and v [B, T, HV, V], got {tuple(q.shape)}, "
+                         f"{tuple(k.shape)}, {tuple(v.shape)}")
+    if v.shape[2] % q.shape[2] != 0:
+        raise ValueError(f"{what}: the number of value heads ({v.shape[2]}) must be a multiple of the number of "
+                         f"q/k heads ({q.shape[2]})")
+    if beta.dim() == v.dim():
+        raise NotImplementedError(f"{what}: headwise beta of shape [B, T, HV, V] is not supported; pass beta [B, T, HV]")
+    if tuple(g.shape) != tuple(v.shape[:3]) or tuple(beta.shape) != tuple(v.shape[:3]):
+        raise ValueError(f"{what}: g and beta must have shape {tuple(v.shape[:3])} (= v.shape[:3]), got "
+                         f"{tuple(g.shape)} and {tuple(beta.shape)}")
+
+
 def _check_varlen(q, initial_state, cu_seqlens):
     if cu_seqlens is not None:
         if q.shape[0] != 1:
@@ -135,8 +152,11 @@ def chunk_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g:
                            scale: float = None, initial_state: torch.Tensor = None, output_final_state: bool = False,
                            cu_seqlens: Optional[torch.LongTensor] = None, head_first: bool = False,
                            use_qk_l2norm_in_kernel: bool = False, *, allow_fp32: bool = False):
-    """q, k [B,T,H,K]; v [B,T,H,V]; g (log-decay, <= 0), beta [B,T,H]; returns (o [B,T,H,V] in q.dtype,
-    final_state [N,H,K,V] fp32 or None). See ``gated_delta_rule_ori.py:236-357`` for the argument contract."""
+    """q, k [B,T,H,K]; v [B,T,H,V]; g (log-decay), beta [B,T,H]; returns (o [B,T,H,V] in q.dtype,
+    final_state [N,H,K,V] fp32 or None). See ``gated_delta_rule_ori.py:236-357`` for the argument contract.
+    g is meant to be <= 0; for positive entries the chunk kernels do what the reference's do: every ratio of
+    cumulative decays inside a chunk goes through ``safe_exp`` (``fla_op.py:27-29``), i.e. it is dropped where its
+    exponent is positive."""
     assert q.dtype == k.dtype == v.dtype
     if not allow_fp32:
         assert q.dtype != torch.float32, "ChunkGatedDeltaRuleFunction does not support float32. Please use bfloat16."
@@ -151,6 +171,7 @@ def chunk_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g:
             "This may indicate the inputs were passed in head-first format [B, H, T, ...] "
             "when head_first=False was specified. "
             "Please verify your input tensor format matches the expected shape [B, T, H, ...].")
+    _check_shapes(q, k, v, g, beta, "chunk_gated_delta_rule")
     _check_varlen(q, initial_state, cu_seqlens)
     if scale is None:
         scale = k.shape[-1] ** -0.5
@@ -174,7 +195,8 @@ def fused_recurrent_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.
     else:
         assert scale > 0, "scale must be positive"
     if beta is None:
-        beta = torch.ones_like(q[..., 0])
+        beta = torch.ones_like(g)
+    _check_shapes(q, k, v, g, beta, "fused_recurrent_gated_delta_rule")
     l2norm = L2_RECURRENT if use_qk_l2norm_in_kernel else L2_NONE
     return _ForwardOnly.apply(_recurrent_launch, q, k, v, g, beta, scale, initial_state, output_final_state,
                               cu_seqlens, l2norm)

@@ -1,10 +1,16 @@
 """Hierarchical (level-weighted) gated-delta forward on the GPU behind the reference's operator signature.
 
 ``chunk_h_gated_delta_rule`` (reference ``models/hattention/gated_delta_rule_apis.py:21-134``): same argument names,
-order, defaults and checks. The reference's own chunk pipeline for this operator does not run as shipped
-(``chunkwise_hgdn.py:661`` unpacks the single tensor ``chunk_scaled_dot_kkt_fwd`` returns into two), so the function
-implemented is its specification, ``hattention_recurrent`` (``recurrent.py:169-216``), reached the way the operator
-reaches it: q l2-normalised and scaled, k l2-normalised (``kernel.py:100-101``), lambda divided by ``scale``
+order, defaults and checks. The reference evaluates it with Triton kernels (``chunkwise_hgdn.py:565-791``), which
+cannot run here, so the function implemented is the token loop the reference keeps as its specification,
+``hattention_recurrent`` (``recurrent.py:169-216``). The reference's chunk pipeline is the same function for g <= 0:
+its two inverses ``Aw = (I + tril(beta K K^T))^-1`` and ``Au = (I + tril(beta K K^T . e^{gamma_i - gamma_j}))^-1``
+(``fla_future/chunk_scaled_dot_kkt.py:62-77``, ``chunkwise_hgdn.py:651-676``) are related by
+``Au = diag(e^gamma) Aw diag(e^-gamma)``, so its ``w_new = e^gamma (Aw beta K)`` (``fla_future/chunk_delta_h.py:449-453``)
+equals ``Au diag(beta e^gamma) K``, the W of the one-inverse form used here, and its per-level state passes
+(``chunkwise_hgdn.py:725-760``: sources masked where the level's bit of the chunk index is set, state reset at the end
+of each period) hold exactly the buckets of the token loop's level states. The operator is reached the way the
+reference reaches it: q l2-normalised and scaled, k l2-normalised (``kernel.py:100-101``), lambda divided by ``scale``
 (``gated_delta_rule_apis.py:68-70``; the kernel does it, with the rounding of a division in lambda's dtype), weak
 hierarchy, base 2.
 

@@ -16,7 +16,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import _capi
-from ._capi import check, ptr, require_cuda, stream_of
+from ._capi import LampaError, check, ptr, require_cuda, stream_of
 
 KEY_U32, KEY_I32, KEY_F32 = 0, 1, 2
 
@@ -262,8 +262,15 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
     return ids, keys, meta
 
 
+def _raise_on_overflow(meta: torch.Tensor, strict: bool):
+    if strict and bool(meta[..., -1].any()):
+        raise LampaError("lsh_bucket_sort: the id ranges of a table multiply to more than 2^31 - 1 buckets, so its "
+                         "32-bit bucket key overflowed and the order is meaningless (use a larger w or fewer "
+                         "projections per table)")
+
+
 def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[torch.Tensor] = None,
-                    n_valid=None, return_ids: bool = True, n_passes: int = 0):
+                    n_valid=None, return_ids: bool = True, n_passes: int = 0, strict: bool = False):
     """E2LSH bucketing in one library call: bucket ids -> packed keys -> stable sort permutation per table ->
     (optionally) the hit features in sorted order. No host synchronisation: the sort reads the number of key bits
     from ``meta`` on the device.
@@ -272,7 +279,11 @@ def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[to
     meta [T, 2J+3], feats [T, N, D].
     A batch of events of N hits each (pad shorter ones): coords [E, N, dim], feats [E, N, D], n_valid an int32
     tensor [E] on the device (or None) -> the same entries with a leading event dimension; one set of launches for
-    the whole batch."""
+    the whole batch.
+
+    A table whose id ranges multiply to more than 2^31 - 1 buckets cannot be packed into one 32-bit key: the kernel
+    then sets ``meta[..., -1]`` (overflow) and the order of that table is meaningless. ``strict=True`` reads the flag
+    (one host synchronisation) and raises ``LampaError``; otherwise the caller has to look at the flag."""
     require_cuda(coords, alpha, beta, feats)
     coords = coords.contiguous().float()
     alpha = alpha.contiguous().float()
@@ -309,10 +320,12 @@ def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[to
                                               n_proj, float(w), ptr(ids), ptr(keys), ptr(meta), ptr(perm), ptr(feats),
                                               row_bytes, ptr(fo), n_passes, ptr(ws), ws.numel(), stream_of(coords)),
               "lampa_lsh_bucket_sort_batch")
+        _raise_on_overflow(meta, strict)
         return out
     n_valid = n if n_valid is None else int(n_valid)
     ws = _workspace(check(lib.lampa_lsh_bucket_sort_workspace_bytes(n, n_tables, n_proj), "workspace"), dev)
     check(lib.lampa_lsh_bucket_sort(ptr(coords), n, n_valid, dim, ptr(alpha), ptr(beta), n_tables, n_proj, float(w),
                                     ptr(ids), ptr(keys), ptr(meta), ptr(perm), ptr(feats), row_bytes, ptr(fo), n_passes,
                                     ptr(ws), ws.numel(), stream_of(coords)), "lampa_lsh_bucket_sort")
+    _raise_on_overflow(meta, strict)
     return out

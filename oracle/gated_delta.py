@@ -11,6 +11,11 @@ Four independent statements of the same function, so that each pins the others:
                         ``wy_fast.py:168-189``, ``chunk_delta_h.py:109-189``, ``chunk_o.py:74-111``;
 * ``recurrent_c``       the C restatement in ``gdr_oracle.c`` (fast enough for T = 60000).
 
+``chunk_form(masked=True)`` adds the reference's ``safe_exp`` masking, which only matters for positive g; it is pinned in
+``tests/test_oracle_gdr.py`` by the cases where the masking has a closed form (no effect for g <= 0; a positive g on the
+first token of a chunk masks nothing; one large positive g inside the first chunk acts as a restart of the sequence
+at that token) and by a scalar-loop restatement of the masked kernels.
+
 Shapes follow the reference operators: q, k [B,T,H,K]; v [B,T,HV,V]; g, beta [B,T,HV]; states [N,HV,K,V].
 """
 import ctypes
@@ -100,17 +105,24 @@ def recurrent_matrix(q, k, v, g, beta, scale=None, initial_state=None, cu_seqlen
     return o, final
 
 
-def chunk_stage_one(k, v, g, beta, dtype=torch.float64):
+def safe_exp(x: torch.Tensor) -> torch.Tensor:
+    """``fla_op.py:27-29``: exp(x) where x <= 0, otherwise 0 (the exponent is replaced by -inf)."""
+    return torch.exp(torch.where(x <= 0, x, torch.full_like(x, float("-inf"))))
+
+
+def chunk_stage_one(k, v, g, beta, dtype=torch.float64, masked=False):
     """Intra-chunk quantities of ONE chunk of ONE head: k [C,K], v [C,V], g, beta [C] (already l2-normed k).
 
-    Returns gamma (inclusive cumsum of g), A (strictly lower), Tm = (I + A)^-1, W, U.
+    Returns gamma (inclusive cumsum of g), A (strictly lower), Tm = (I + A)^-1, W, U. ``masked``: the decay ratio
+    inside A goes through ``safe_exp`` as in ``chunk_scaled_dot_kkt.py:65-67`` (a no-op when g <= 0).
     """
     k, v, g, beta = (x.to(dtype) for x in (k, v, g, beta))
     C = k.shape[0]
     gamma = torch.cumsum(g, 0)
     diff = gamma[:, None] - gamma[None, :]
     lower = torch.tril(torch.ones(C, C, dtype=torch.bool), -1)
-    A = torch.where(lower, beta[:, None] * (k @ k.T) * torch.exp(torch.where(lower, diff, 0.0)), 0.0)
+    ratio = safe_exp(diff) if masked else torch.exp(torch.where(lower, diff, 0.0))
+    A = torch.where(lower, beta[:, None] * (k @ k.T) * ratio, 0.0)
     Tm = torch.linalg.solve_triangular(torch.eye(C, dtype=dtype) + A, torch.eye(C, dtype=dtype), upper=False)
     U = Tm @ (beta[:, None] * v)
     W = Tm @ ((beta * torch.exp(gamma))[:, None] * k)
@@ -118,9 +130,16 @@ def chunk_stage_one(k, v, g, beta, dtype=torch.float64):
 
 
 def chunk_form(q, k, v, g, beta, scale=None, initial_state=None, cu_seqlens=None, l2=L2_NONE, chunk=64,
-               dtype=torch.float64):
+               dtype=torch.float64, masked=False):
     """Chunkwise algorithm (chunks never straddle sequences, ``index.py:69-83``; a partial last chunk uses
-    the gamma of its last valid row, ``chunk_delta_h.py:148``)."""
+    the gamma of its last valid row, ``chunk_delta_h.py:148``).
+
+    ``masked=True`` is what the reference's kernels compute for ANY sign of g: the three decay RATIOS go through
+    ``safe_exp`` -- inside A (``chunk_scaled_dot_kkt.py:67``), inside the intra-chunk attention matrix
+    (``chunk_o.py:98``) and on the state update's e^{gamma_last - gamma_j} (``chunk_delta_h.py:152``) -- while
+    e^{gamma_i} (``wy_fast.py:173``, ``chunk_o.py:97``) and e^{gamma_last} (``chunk_delta_h.py:153``) are plain
+    exponentials. With g <= 0 no ratio's exponent is positive and both settings are the same function; with positive
+    g the result depends on where the chunk boundaries fall (chunk = 64 in the reference)."""
     q, k, v, g, beta, scale = _prep(q, k, v, g, beta, scale, l2, dtype)
     B, T, HV, V = v.shape
     K = k.shape[-1]
@@ -135,13 +154,14 @@ def chunk_form(q, k, v, g, beta, scale=None, initial_state=None, cu_seqlens=None
             for c0 in range(t0, t1, chunk):
                 c1 = min(c0 + chunk, t1)
                 qc, kc, vc = q[b, c0:c1, h], k[b, c0:c1, h], v[b, c0:c1, h]
-                gamma, _, _, W, U = chunk_stage_one(kc, vc, g[b, c0:c1, h], beta[b, c0:c1, h], dtype)
+                gamma, _, _, W, U = chunk_stage_one(kc, vc, g[b, c0:c1, h], beta[b, c0:c1, h], dtype, masked)
                 v_new = U - W @ S
                 diff = gamma[:, None] - gamma[None, :]
                 incl = torch.tril(torch.ones(c1 - c0, c1 - c0, dtype=torch.bool))
-                P = torch.where(incl, (qc @ kc.T) * torch.exp(torch.where(incl, diff, 0.0)), 0.0)
+                ratio = safe_exp(diff) if masked else torch.exp(torch.where(incl, diff, 0.0))
+                P = torch.where(incl, (qc @ kc.T) * ratio, 0.0)
                 o[b, c0:c1, h] = scale * (torch.exp(gamma)[:, None] * (qc @ S) + P @ v_new)
-                k_dec = kc * torch.exp(gamma[-1] - gamma)[:, None]
+                k_dec = kc * (safe_exp(gamma[-1] - gamma) if masked else torch.exp(gamma[-1] - gamma))[:, None]
                 S = torch.exp(gamma[-1]) * S + k_dec.T @ v_new
             final[n, h] = S
     return o, final

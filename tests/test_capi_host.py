@@ -141,3 +141,24 @@ def test_operators_refuse_cpu_tensors():
         gd.chunk_gated_delta_rule(x, x, x, g, g)
     with pytest.raises(_capi.LampaError):
         lsh.stable_argsort(torch.zeros(4, dtype=torch.int32))
+
+
+def test_gated_delta_shape_checks_come_before_any_gpu_work():
+    # headwise beta [B, T, HV, V] (gated_delta_rule_ori.py:444-447) is refused rather than read with the wrong stride;
+    # g and beta must be [B, T, HV]
+    from lampa_amd import gated_delta as gd
+
+    q = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16)
+    v = torch.zeros(1, 64, 4, 64, dtype=torch.bfloat16)
+    g = torch.zeros(1, 64, 4)
+    with pytest.raises(NotImplementedError, match="headwise beta"):
+        gd.fused_recurrent_gated_delta_rule(q, q, v, g, torch.zeros(1, 64, 4, 64))
+    with pytest.raises(ValueError, match="g and beta must have shape"):
+        gd.fused_recurrent_gated_delta_rule(q, q, v, g[:, :, :2], g)
+    with pytest.raises(ValueError, match="g and beta must have shape"):
+        gd.chunk_gated_delta_rule(q, q, v, g, g[:, :32])
+    with pytest.raises(ValueError, match="multiple of the number"):
+        gd.chunk_gated_delta_rule(q, q, v[:, :, :3], g[:, :, :3], g[:, :, :3])
+    with pytest.raises(ValueError, match="expected q, k"):
+        gd.chunk_gated_delta_rule(q, q[:, :32], v, g, g)
+

@@ -179,6 +179,30 @@ def test_chunk_argument_checks(device):
         gd.chunk_gated_delta_rule(q.cpu(), k.cpu(), v.cpu(), g.cpu(), beta.cpu())  # no CPU fallback
 
 
+def test_chunk_positive_g_follows_the_reference_masking(device):
+    # g > 0 is outside the operator's intended domain, but the reference's kernels define what happens: every decay
+    # RATIO inside a chunk goes through safe_exp (fla_op.py:27-29). The oracle's chunk form applies the same masking;
+    # positive entries sit on chunk starts (where nothing is masked) and inside chunks (where tokens are cut off).
+    T = 300
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 2, 64, 64, torch.bfloat16, seed=21, g_scale=0.1)
+    g = g.clone()
+    g[0, [64, 128], 0] = 0.5
+    g[0, [5, 70, 71, 190, 299], :] = torch.tensor([0.3, 1.0, 0.2, 0.6, 0.4])[:, None]
+    h0 = 0.1 * torch.randn(1, 2, 64, 64, generator=torch.Generator().manual_seed(2))
+    want_o, want_s = og.chunk_form(q, k, v, g, beta, initial_state=h0, chunk=64, masked=True)
+    plain_o, _ = og.recurrent_delta(q, k, v, g, beta, initial_state=h0)
+    assert (want_o - plain_o).abs().max() > 0.05  # the masking matters on this input
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device), output_final_state=True)
+    _assert_bf16_close(o, want_o, "o")
+    _assert_bf16_close(s, want_s, "state")
+    # the in-kernel l2norm path goes through the same masked ratios
+    want_o, want_s = og.chunk_form(q * 3, k * 2, v, g, beta, chunk=64, masked=True, l2=og.L2_CHUNK)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q * 3, k * 2, v, g, beta), output_final_state=True,
+                                     use_qk_l2norm_in_kernel=True)
+    _assert_bf16_close(o, want_o, "o l2")
+    _assert_bf16_close(s, want_s, "state l2")
+
+
 def test_chunk_matches_token_serial_kernel_on_gpu(device):
     q, k, v, g, beta = _to(device, *synth.gdr_inputs(1, 5000, 4, 64, 64, torch.bfloat16, seed=21, g_scale=0.1))
     o1, s1 = gd.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)

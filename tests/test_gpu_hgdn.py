@@ -218,3 +218,38 @@ def test_full_length_prefill_matches_oracle(device, g_scale):
     assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"o: {max_abs:.3e} {mean_rel:.3e}"
     max_abs, mean_rel = _state_errors(st, want_s, want_c)
     assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"states: {max_abs:.3e} {mean_rel:.3e}"
+
+
+def test_interleaved_calls_on_two_streams(device):
+    # The launcher forks part of its work onto a helper stream; every caller stream has its own helper stream and
+    # events, so calls issued alternately on two streams with nothing between them must each give what a call on its
+    # own gives.
+    cases = [_inputs(1, 4096, 2, 64, 64, torch.bfloat16, seed=70 + i) for i in range(2)]
+    dev_cases = [tuple(x.to(device) for x in c) for c in cases]
+    alone = []
+    for q, k, v, g, beta, lam in dev_cases:
+        o, _ = hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, use_qk_l2norm_in_kernel=True)
+        alone.append(o.clone())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)]
+    old = hgdn.CHUNKS_PER_SEGMENT
+    hgdn.CHUNKS_PER_SEGMENT = 8  # several segments per sequence: the path that uses the helper stream
+    try:
+        ref = []
+        for q, k, v, g, beta, lam in dev_cases:
+            ref.append(hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, use_qk_l2norm_in_kernel=True)[0].clone())
+        torch.cuda.synchronize()
+        outs = [[], []]
+        for rep in range(4):
+            for i in (0, 1):
+                with torch.cuda.stream(streams[i]):
+                    q, k, v, g, beta, lam = dev_cases[i]
+                    outs[i].append(hgdn.chunk_h_gated_delta_rule(q, k, v, g, lam, beta, use_qk_l2norm_in_kernel=True)[0])
+        torch.cuda.synchronize()
+    finally:
+        hgdn.CHUNKS_PER_SEGMENT = old
+    for i in (0, 1):
+        for o in outs[i]:
+            assert torch.equal(o, ref[i])  # same kernels, same data: bit-identical whatever runs beside them
+        max_abs, mean_rel = _errors(ref[i], alone[i].cpu())
+        assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL

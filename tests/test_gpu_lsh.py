@@ -46,6 +46,19 @@ def test_bucket_overflow_flag(device):
     ids = ol.bucket_ids(coords.numpy(), alpha.numpy(), beta.numpy(), 1.0)
     _, want = ol.pack_keys(ids, 1, 2)
     assert np.array_equal(_np(meta), want) and want[0, -1] == 1
+    # the one-call stage reports it on request instead of returning a meaningless order silently
+    from lampa_amd._capi import LampaError
+    with pytest.raises(LampaError, match="overflow"):
+        lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 1.0, 1, 2, strict=True)
+    lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 1.0, 1, 2)  # default: flag only
+
+
+def test_gather_out_of_range_index_reads_zeros(device):
+    src = torch.arange(1, 13, dtype=torch.float32, device=device).reshape(1, 3, 4)
+    idx = torch.tensor([[2, 5, 0, -1]], dtype=torch.int32, device=device)
+    got = lsh.gather_rows(src, idx)
+    want = torch.stack([src[0, 2], torch.zeros(4, device=device), src[0, 0], torch.zeros(4, device=device)])[None]
+    assert torch.equal(got, want)
 
 
 @pytest.mark.parametrize("kind", ["i32", "f32", "u32bits"])

@@ -125,3 +125,101 @@ def test_c_oracle_fp32_and_fp64_on_longer_sequence():
     o3, s3 = og.recurrent_c(q, k, v, g, beta, dtype=torch.float32)
     assert torch.allclose(o1.float(), o2, atol=1e-6) and torch.allclose(s1.float(), s2, atol=1e-6)
     assert torch.allclose(o1.float(), o3, atol=1e-4) and torch.allclose(s1.float(), s3, atol=1e-4)
+
+
+# ---- the reference's safe_exp masking (positive g) -----------------------------------------------------------------
+def test_masked_chunk_form_is_a_noop_for_nonpositive_g():
+    q, k, v, g, beta = _inputs(B=1, T=150, H=2, K=8, V=6, g_scale=0.3)
+    assert (g <= 0).all()
+    o1, s1 = og.chunk_form(q, k, v, g, beta, chunk=64)
+    o2, s2 = og.chunk_form(q, k, v, g, beta, chunk=64, masked=True)
+    assert torch.equal(o1, o2) and torch.equal(s1, s2)
+
+
+def test_positive_g_on_a_chunk_start_masks_nothing():
+    # gamma_i - gamma_j (j < i in one chunk) and gamma_last - gamma_j are sums of g over tokens AFTER j, so the g of a
+    # chunk's first token enters none of the masked ratios: with positive g only there, the masked chunk form must
+    # equal the token loop, which applies e^g whatever its sign.
+    q, k, v, g, beta = _inputs(B=1, T=200, H=2, K=8, V=6, g_scale=0.3)
+    g = g.clone()
+    g[:, 64] = 0.7
+    g[:, 128] = 0.2
+    o1, s1 = og.recurrent_delta(q, k, v, g, beta)
+    o2, s2 = og.chunk_form(q, k, v, g, beta, chunk=64, masked=True)
+    assert torch.allclose(o1, o2, atol=1e-10) and torch.allclose(s1, s2, atol=1e-10)
+    g[:, 70] = 0.7  # ... and inside a chunk it does change the function
+    o3, _ = og.chunk_form(q, k, v, g, beta, chunk=64, masked=True)
+    o4, _ = og.recurrent_delta(q, k, v, g, beta)
+    assert (o3 - o4).abs().max() > 1e-3
+
+
+def test_large_positive_g_inside_first_chunk_restarts_the_sequence():
+    # One g = +40 at token p of the first chunk (zero initial state, every other g <= 0 and small): every ratio that
+    # spans p has a positive exponent and is masked, so tokens >= p neither see tokens < p (A and the attention
+    # matrix are block diagonal) nor do tokens < p reach the final state (their e^{gamma_last - gamma_j} is masked):
+    # outputs from p on and the final state equal those of the sequence that starts at p with its first g set to 0,
+    # and outputs before p are untouched.
+    T, p = 64, 23
+    q, k, v, g, beta = _inputs(B=1, T=T, H=2, K=8, V=6, g_scale=0.05)
+    g = g.clone()
+    g[:, p] = 40.0
+    o, s = og.chunk_form(q, k, v, g, beta, chunk=64, masked=True)
+    g_tail = g[:, p:].clone()
+    g_tail[:, 0] = 0.0
+    # e^{gamma_i} still multiplies (q_i . S_chunk_start) -- S is zero here, so that term vanishes
+    o_tail, s_tail = og.recurrent_delta(q[:, p:], k[:, p:], v[:, p:], g_tail, beta[:, p:])
+    o_head, _ = og.recurrent_delta(q[:, :p], k[:, :p], v[:, :p], g[:, :p], beta[:, :p])
+    assert torch.allclose(o[:, :p], o_head, atol=1e-10)
+    assert torch.allclose(o[:, p:], o_tail, atol=1e-10)
+    assert torch.allclose(s, s_tail, atol=1e-10)
+
+
+def test_masked_chunk_form_against_scalar_loops():
+    # The masked kernels restated with Python scalars, row by row (forward substitution instead of a matrix inverse):
+    #   A_ij = beta_i (k_i.k_j) sexp(gam_i - gam_j), u_i = beta_i v_i - sum_j A_ij u_j, w_i = beta_i e^{gam_i} k_i - sum_j A_ij w_j
+    #   vnew_i = u_i - w_i S, o_i = scale (e^{gam_i} q_i S + sum_{j<=i} (q_i.k_j) sexp(gam_i - gam_j) vnew_j)
+    #   S' = e^{gam_last} S + sum_j sexp(gam_last - gam_j) k_j vnew_j^T
+    import math
+
+    def sexp(x):
+        return math.exp(x) if x <= 0 else 0.0
+
+    T, K, V, C = 21, 3, 2, 8
+    q, k, v, g, beta = _inputs(B=1, T=T, H=1, K=K, V=V, g_scale=0.5, seed=5)
+    g = g.clone()
+    g[0, [3, 9, 10, 18], 0] = torch.tensor([0.4, 1.1, 0.3, 0.9])
+    qq, kk, vv = q[0, :, 0].double().tolist(), k[0, :, 0].double().tolist(), v[0, :, 0].double().tolist()
+    gg, bb = g[0, :, 0].double().tolist(), beta[0, :, 0].double().tolist()
+    scale = 0.61
+    S = [[0.0] * V for _ in range(K)]
+    out = []
+    dot = lambda a, b: sum(x * y for x, y in zip(a, b))
+    for c0 in range(0, T, C):
+        n = min(C, T - c0)
+        gam, run = [], 0.0
+        for i in range(n):
+            run += gg[c0 + i]
+            gam.append(run)
+        u, w = [], []
+        for i in range(n):
+            ui = [bb[c0 + i] * x for x in vv[c0 + i]]
+            wi = [bb[c0 + i] * math.exp(gam[i]) * x for x in kk[c0 + i]]
+            for j in range(i):
+                a = bb[c0 + i] * dot(kk[c0 + i], kk[c0 + j]) * sexp(gam[i] - gam[j])
+                ui = [x - a * y for x, y in zip(ui, u[j])]
+                wi = [x - a * y for x, y in zip(wi, w[j])]
+            u.append(ui)
+            w.append(wi)
+        vnew = [[u[i][c] - sum(w[i][r] * S[r][c] for r in range(K)) for c in range(V)] for i in range(n)]
+        for i in range(n):
+            row = [math.exp(gam[i]) * sum(qq[c0 + i][r] * S[r][c] for r in range(K)) for c in range(V)]
+            for j in range(i + 1):
+                p = dot(qq[c0 + i], kk[c0 + j]) * sexp(gam[i] - gam[j])
+                row = [x + p * y for x, y in zip(row, vnew[j])]
+            out.append([scale * x for x in row])
+        dec = math.exp(gam[-1])
+        S = [[dec * S[r][c] + sum(sexp(gam[-1] - gam[j]) * kk[c0 + j][r] * vnew[j][c] for j in range(n))
+              for c in range(V)] for r in range(K)]
+    o, s = og.chunk_form(q, k, v, g, beta, scale=scale, chunk=C, masked=True)
+    assert torch.allclose(o[0, :, 0], torch.tensor(out, dtype=torch.float64), atol=1e-10)
+    assert torch.allclose(s[0, 0], torch.tensor(S, dtype=torch.float64), atol=1e-10)
