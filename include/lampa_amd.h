@@ -10,7 +10,7 @@
  *   - return value: 0 on success, negative on error (LAMPA_ERR_*). No C++ exception crosses the boundary;
  *   - state the library keeps between calls: the optional profiling recorder; one helper stream with two events per
  *     (device, caller stream) that lampa_hgdn_chunk_fwd creates on first use and keeps until the process ends (calls
- *     on different streams or host threads never share them).
+ *     on different streams or host threads never share them); the fixed scratch array of lampa_sort_pairs_static.
  *     Everything else lives in caller-owned buffers, so calls on different streams do not interfere.
  * The reference (chengjiang123/Lampa) is Python over Triton/ATen, so each entry point names the Python operator or
  * kernel it replaces (file:line in the reference tree).
@@ -107,6 +107,18 @@ int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n);
 int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
                      int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
                      int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* lampa_sort_pairs for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+ * arguments, same kernels and bit-identical results; the ping-pong buffers and histograms live in a fixed 8 MiB array
+ * inside the library image (one copy per GPU, held until the process ends), so the call allocates nothing.
+ * lampa_sort_workspace_bytes(n_segments, n) must not exceed lampa_sort_pairs_static_max_bytes() (8 MiB: e.g. 3
+ * segments of 140 000 keys), otherwise LAMPA_ERR_WORKSPACE. All calls on one GPU share that array: calls that may
+ * overlap on one GPU (different streams or host threads) race and must be serialised by the caller. */
+int64_t lampa_sort_pairs_static_max_bytes(void);
+int lampa_sort_pairs_static(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
+                            int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
+                            int32_t* vals_out, void* stream);
 
 /* dst[s, i, :] = src[s % src_segments, idx[s, i], :]. Replaces batched_index_select / sort_to_buckets /
  * unsort_from_buckets and the points.gather of LSHOrdering (hash_utils.py:83-93; hept.py:9-19;

@@ -34,6 +34,8 @@ _SIGNATURES = {
     "lampa_row_minmax_f32": (_i32, [_vp, _i32, _i64, _vp, _vp]),
     "lampa_sort_workspace_bytes": (_i64, [_i32, _i64]),
     "lampa_sort_pairs": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp]),
+    "lampa_sort_pairs_static_max_bytes": (_i64, []),
+    "lampa_sort_pairs_static": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _vp, _i32, _i32, _vp, _vp]),
     "lampa_gather_rows": (_i32, [_vp, _i32, _i64, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
     "lampa_scatter_rows": (_i32, [_vp, _vp, _i32, _i32, _i64, _i64, _vp, _vp]),
     "lampa_invert_perm": (_i32, [_vp, _i32, _i32, _i64, _vp, _vp]),

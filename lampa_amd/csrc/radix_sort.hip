@@ -12,6 +12,7 @@
 // (written by the key-packing kernel) so that no host synchronisation is needed: then the host launches the worst
 // case and each segment uses only the launches its keys need (see rs_digit).
 #include "common.h"
+#include <mutex>
 
 #define RS_BLOCK 256
 #define RS_WAVES (RS_BLOCK / 64)
@@ -292,25 +293,11 @@ extern "C" int64_t lampa_sort_workspace_bytes(int n_segments, int64_t n) {
   return 4 * pairs + hist;
 }
 
-// keys_in [S, n] (raw 32-bit keys of kind key_kind), vals_in [S, n] or NULL (payload = position), vals_out [S, n].
-// key_bits_dev (nullable): per-segment number of significant key bits in device memory, element s at
-// key_bits_dev[s * key_bits_stride]; otherwise key_bits (host, 1..32) applies to all segments. Signed and float
-// keys always need 32 bits. n_passes in 1..4 with ceil(bits / n_passes) <= 11; 0 picks ceil(key_bits / 11)
-// for host bits and 3 for device bits.
-extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
-                                int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
-                                int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream) {
-  if (!keys_in || !vals_out || n_segments < 1 || n < 0 || n > INT32_MAX) return LAMPA_ERR_INVALID;
-  if (key_kind != KEY_U32 && key_kind != KEY_I32 && key_kind != KEY_F32) return LAMPA_ERR_INVALID;
-  if (key_kind != KEY_U32) { key_bits = 32; key_bits_dev = nullptr; }
-  if (!key_bits_dev && (key_bits < 1 || key_bits > 32)) return LAMPA_ERR_INVALID;
-  const int max_bits = key_bits_dev ? 32 : key_bits;
-  if (n_passes == 0) n_passes = key_bits_dev ? 3 : (max_bits + RS_MAX_DIGIT_BITS - 1) / RS_MAX_DIGIT_BITS;
-  if (n_passes < 1 || n_passes > 4 || (max_bits + n_passes - 1) / n_passes > RS_MAX_DIGIT_BITS)
-    return LAMPA_ERR_INVALID;
-  if (!workspace || workspace_bytes < lampa_sort_workspace_bytes(n_segments, n)) return LAMPA_ERR_WORKSPACE;
-  if (n == 0) return LAMPA_OK;
-  hipStream_t s = (hipStream_t)stream;
+// Enqueues the passes of one sort; `workspace` holds lampa_sort_workspace_bytes(n_segments, n) bytes (checked by the
+// callers). Nothing in it has to start at zero: every histogram row and total that a pass reads is written by that pass.
+static int rs_sort_enqueue(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
+                           int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
+                           int32_t* vals_out, void* workspace, hipStream_t s) {
   const int n_tiles = (int)((n + RS_TILE - 1) / RS_TILE);
   const int64_t pairs = lampa_align_up((int64_t)n_segments * n * 4, 256);
   char* ws = (char*)workspace;
@@ -334,4 +321,76 @@ extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t
     LAMPA_PROF(s, "rs_scatter_kernel");
   }
   return lampa_launch_status();
+}
+
+// Argument checks shared by the two entry points; resolves the automatic pass count.
+static int rs_check_args(const void* keys_in, int key_kind, int n_segments, int64_t n, int& key_bits,
+                         const int32_t*& key_bits_dev, int& n_passes, const int32_t* vals_out) {
+  if (!keys_in || !vals_out || n_segments < 1 || n < 0 || n > INT32_MAX) return LAMPA_ERR_INVALID;
+  if (key_kind != KEY_U32 && key_kind != KEY_I32 && key_kind != KEY_F32) return LAMPA_ERR_INVALID;
+  if (key_kind != KEY_U32) { key_bits = 32; key_bits_dev = nullptr; }
+  if (!key_bits_dev && (key_bits < 1 || key_bits > 32)) return LAMPA_ERR_INVALID;
+  const int max_bits = key_bits_dev ? 32 : key_bits;
+  if (n_passes == 0) n_passes = key_bits_dev ? 3 : (max_bits + RS_MAX_DIGIT_BITS - 1) / RS_MAX_DIGIT_BITS;
+  if (n_passes < 1 || n_passes > 4 || (max_bits + n_passes - 1) / n_passes > RS_MAX_DIGIT_BITS)
+    return LAMPA_ERR_INVALID;
+  return LAMPA_OK;
+}
+
+// keys_in [S, n] (raw 32-bit keys of kind key_kind), vals_in [S, n] or NULL (payload = position), vals_out [S, n].
+// key_bits_dev (nullable): per-segment number of significant key bits in device memory, element s at
+// key_bits_dev[s * key_bits_stride]; otherwise key_bits (host, 1..32) applies to all segments. Signed and float
+// keys always need 32 bits. n_passes in 1..4 with ceil(bits / n_passes) <= 11; 0 picks ceil(key_bits / 11)
+// for host bits and 3 for device bits.
+extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments, int64_t n,
+                                int key_bits, const int32_t* key_bits_dev, int key_bits_stride, int n_passes,
+                                int32_t* vals_out, void* workspace, int64_t workspace_bytes, void* stream) {
+  const int rc = rs_check_args(keys_in, key_kind, n_segments, n, key_bits, key_bits_dev, n_passes, vals_out);
+  if (rc != LAMPA_OK) return rc;
+  if (!workspace || workspace_bytes < lampa_sort_workspace_bytes(n_segments, n)) return LAMPA_ERR_WORKSPACE;
+  if (n == 0) return LAMPA_OK;
+  return rs_sort_enqueue(keys_in, key_kind, vals_in, n_segments, n, key_bits, key_bits_dev, key_bits_stride, n_passes,
+                         vals_out, workspace, (hipStream_t)stream);
+}
+
+// ---- the sort for callers that cannot allocate -------------------------------------------------------------------
+// Same sort, same kernels, but the ping-pong buffers and histograms live in a fixed array of device memory that is
+// part of the library image (every GPU the library runs on holds its own copy until the process ends). The array's
+// name is only a host-side handle: its device address is looked up once per device with hipGetSymbolAddress and that
+// pointer is what the kernels receive.
+#define RS_STATIC_SCRATCH_BYTES (8 << 20)
+#define RS_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char rs_static_scratch[RS_STATIC_SCRATCH_BYTES];
+static void* rs_scratch_ptr[RS_MAX_DEVICES];
+static std::mutex rs_scratch_lock;
+
+// Device address of the current device's copy of the array (nullptr on failure).
+static void* rs_static_scratch_address() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= RS_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(rs_scratch_lock);
+  if (!rs_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(rs_static_scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    rs_scratch_ptr[dev] = p;
+  }
+  return rs_scratch_ptr[dev];
+}
+
+extern "C" int64_t lampa_sort_pairs_static_max_bytes(void) { return RS_STATIC_SCRATCH_BYTES; }
+
+extern "C" int lampa_sort_pairs_static(const void* keys_in, int key_kind, const int32_t* vals_in, int n_segments,
+                                       int64_t n, int key_bits, const int32_t* key_bits_dev, int key_bits_stride,
+                                       int n_passes, int32_t* vals_out, void* stream) {
+  const int rc = rs_check_args(keys_in, key_kind, n_segments, n, key_bits, key_bits_dev, n_passes, vals_out);
+  if (rc != LAMPA_OK) return rc;
+  if (lampa_sort_workspace_bytes(n_segments, n) > RS_STATIC_SCRATCH_BYTES) return LAMPA_ERR_WORKSPACE;
+  if (n == 0) return LAMPA_OK;
+  void* scratch = rs_static_scratch_address();
+  if (!scratch) return LAMPA_ERR_LAUNCH;
+  return rs_sort_enqueue(keys_in, key_kind, vals_in, n_segments, n, key_bits, key_bits_dev, key_bits_stride, n_passes,
+                         vals_out, scratch, (hipStream_t)stream);
 }

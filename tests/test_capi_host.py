@@ -162,3 +162,14 @@ def test_gated_delta_shape_checks_come_before_any_gpu_work():
     with pytest.raises(ValueError, match="expected q, k"):
         gd.chunk_gated_delta_rule(q, q[:, :32], v, g, g)
 
+
+def test_static_sort_symbols_and_limit():
+    lib = _capi.lib()
+    assert lib.lampa_sort_pairs_static_max_bytes() == 8 << 20
+    assert lib.lampa_sort_workspace_bytes(3, 60000) <= lib.lampa_sort_pairs_static_max_bytes()
+    d = ctypes.c_void_p(0x1000)
+    # argument and size checks run before anything touches the GPU
+    assert lib.lampa_sort_pairs_static(None, 1, None, 1, 10, 32, None, 1, 0, d, None) == -1
+    assert lib.lampa_sort_pairs_static(d, 7, None, 1, 10, 32, None, 1, 0, d, None) == -1
+    assert lib.lampa_sort_pairs_static(d, 1, None, 3, 400000, 32, None, 1, 0, d, None) == -2
+    assert lib.lampa_sort_pairs_static(d, 1, None, 3, 0, 32, None, 1, 0, d, None) == 0
