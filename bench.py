@@ -29,7 +29,7 @@ LAYER_FLOP_PER_TOKEN_HEAD = 2 * 64 * (3 * K + 2 * V) + 6 * K * V + (2 * 64 * 64)
 KERNEL_BYTES_PER_TOKEN_HEAD = {            # algorithmic bytes each kernel of the pipeline has to move
     "gdr_segment_kernel<output>": LAYER_BYTES_PER_TOKEN_HEAD,    # reads q, k, v, g, beta and writes o: the whole 520 B
     "gdr_segment_kernel<composite>": 2 * K + 2 * V + 8,           # reads k, v, g, beta
-    "gdr_tinv_kernel": 2 * K + 8,                                 # reads k, g, beta
+    "gdr_local_kernel": 2 * K + 8,                                # reads k, g, beta
 }
 LSH_BYTES_PER_HIT_TABLE = 224
 # HBM bytes per launch at config 2 from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a plain
@@ -37,7 +37,6 @@ LSH_BYTES_PER_HIT_TABLE = 224
 MEASURED_TRAFFIC_BYTES = {
     "gdr_segment_kernel<output>": 350.2e6,
     "gdr_segment_kernel<composite>": 184.1e6,
-    "gdr_tinv_kernel": 141.8e6,
     "gdr_scan_kernel": 24.7e6,
     "gdr_scan2_kernel<group>": 30.9e6,
     "gdr_scan2_kernel<leaf>": 29.1e6,
@@ -164,7 +163,7 @@ def main():
     # ---- what the output pass's access pattern costs with no arithmetic (memory-only twin of that kernel: same rows
     #      of q, k, v, the per-chunk records and the o rows per workgroup and chunk; whole chunks only) ----
     n_chunks_probe = T // 64
-    rec = torch.zeros(n_chunks_probe * H * 6656, dtype=torch.uint8, device=dev)
+    rec = torch.zeros(n_chunks_probe * H * 6912, dtype=torch.uint8, device=dev)
     o_probe = torch.empty_like(vd)
     cps_probe = gd._default_chunks_per_segment([(T + 63) // 64], H, 2 * torch.cuda.get_device_properties(dev).multi_processor_count)
 
@@ -181,7 +180,7 @@ def main():
     ev1.record()
     torch.cuda.synchronize()
     probe_us = 1e3 * ev0.elapsed_time(ev1) / 100
-    probe_bytes = n_chunks_probe * H * (4 * 64 * 64 * 2 + 6656)
+    probe_bytes = n_chunks_probe * H * (4 * 64 * 64 * 2 + 6912)
     roofline["memory_only_twin"] = {
         "us": round(probe_us, 2), "bytes": probe_bytes, "GB/s": round(probe_bytes / (probe_us * 1e-6) / 1e9, 1),
         "kernel_over_twin": round(stage_us.get("gdr_segment_kernel<output>", float("nan")) / probe_us, 3),

@@ -53,9 +53,9 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
-    hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv, tf, H, HV,
-                       l2norm);
-    LAMPA_PROF(s, "gdr_tinv_kernel");
+    hipLaunchKernelGGL((gdr_local_kernel<T, T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv.chunk_tok0,
+                       pv.chunk_len, tf, H, HV, l2norm);
+    LAMPA_PROF(s, "gdr_local_kernel");
     if (segs > n_seq) {
       hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
                          (const T*)q, (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nc, Dc,
@@ -75,16 +75,16 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   if (two_level) {
     // long sequences: group composites, then every group's scan (which walks the earlier groups' composites first)
     const dim3 block(64 * (KT / 32));
-    hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
+    hipLaunchKernelGGL((gdr_scan2_kernel<T, KT, VT, 4, SCAN_GROUP>), dim3((KT + VT) / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc,
                        Nc, Dc, (const float*)nullptr, (float*)nullptr, Gm, Gn, Gd, HV, 0, gmax);
     LAMPA_PROF(s, "gdr_scan2_kernel<group>");
     if (!walk_in_output) {
-      hipLaunchKernelGGL((gdr_scan2_kernel<KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc,
+      hipLaunchKernelGGL((gdr_scan2_kernel<T, KT, VT, 4, SCAN_LEAF>), dim3(VT / 32 * gmax, n_seq, HV), block, 0, s, pv, Mc, Nc,
                          Dc, h0, Si, Gm, Gn, Gd, HV, segs, gmax);
       LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
     }
   } else {
-    hipLaunchKernelGGL((gdr_scan_kernel<KT, VT, (KT == 64 ? 4 : 4)>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
+    hipLaunchKernelGGL((gdr_scan_kernel<T, KT, VT, 4>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
                        pv, Mc, Nc, Dc, h0, Si, HV, segs);
     LAMPA_PROF(s, "gdr_scan_kernel");
   }
@@ -131,3 +131,9 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
 #undef GDR_CASE
   return LAMPA_ERR_UNSUPPORTED;
 }
+
+#ifdef EXP_STAMP
+extern "C" int lampa_dbg_stamps(unsigned long long* out) {
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(gdr_dbg), sizeof(unsigned long long) * 2 * 8 * 64) == hipSuccess ? 0 : -1;
+}
+#endif

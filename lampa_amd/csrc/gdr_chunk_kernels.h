@@ -31,6 +31,7 @@
 // both operands agree, every A operand is read from LDS in that slot order (ld_kappa).
 #pragma once
 #include "gdr_common.h"
+#include "gdr_ops.h"
 #include "gdr_plan.h"
 
 // Device pointers to the tables of the plan (resolved on the host, so that a kernel reaches an entry with one
@@ -55,7 +56,7 @@ static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_d
 // Record of one chunk and head: T, then the chunk's cumulative log-decay (units of log 2) and beta per token, fp32
 // [64] each. The segment kernels take the two factor rows from here: in g and beta themselves a head's 64 values sit
 // 4 bytes apart in rows that interleave all heads, so every workgroup would fetch the sectors of all of them.
-#define REC_BYTES (T_BYTES + 2 * 64 * 4)
+#define REC_BYTES (T_BYTES + 3 * 64 * 4)  // (third row: the l2-norm factors of the k rows, written by gdr_local_kernel)
 #define GDR_SCAN_GROUP 8  // segments per group of the two-level scan; a multiple of its ring depth
 
 __device__ __forceinline__ bf16x8 frag_load(const unsigned char* base, int frag, int lane) {
@@ -132,204 +133,322 @@ __device__ __forceinline__ bf16x8 raw_to_bf16(typename Raw8<T>::type v, float& s
   return out;
 }
 
+// Raw input piece (type T) -> operand piece (type OT) (+ its sum of squares when the rows get l2-normalised): a bit
+// copy when the operands keep the input type, a conversion otherwise.
+template <typename T, typename OT>
+__device__ __forceinline__ typename OpVec<OT>::x8 raw_to_op(typename Raw8<T>::type v, float& ss, bool want_ss) {
+  typename OpVec<OT>::x8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float f = (float)v[e];
+    if (want_ss) ss = __builtin_fmaf(f, f, ss);
+    if constexpr (!__is_same(T, OT)) out[e] = (OT)f;
+  }
+  if constexpr (__is_same(T, OT)) out = __builtin_bit_cast(typename OpVec<OT>::x8, v);
+  return out;
+}
+
 // ---- T = (I + A)^-1 ------------------------------------------------------------------------------------------
-// One WAVE per (chunk, head), one wave per workgroup: the forward substitution is a single-wave job, so many small
-// workgroups per CU keep every SIMD busy. The k tile never touches LDS: the MFMA operand fragments of K K^T are
-// 16-byte global loads (lane = row, its half of each 16-wide contraction step). LDS holds only the two diagonal
-// blocks (fp32) and the per-token factors, all wave-private (LDS operations of one wave complete in order).
-// T is stored as three row-major 32x32 bf16 blocks: T11 | T21 | T22 (the upper-right block is zero and not kept).
-template <typename T, int KT>
-__global__ void __launch_bounds__(64, 3) gdr_tinv_kernel(const T* __restrict__ k, const float* __restrict__ g,
-                                                         const float* __restrict__ beta, const GdrPlanView pv,
-                                                         unsigned char* __restrict__ tmat, int H, int HV, int l2norm) {
-  constexpr int SB = 36, NK = KT / 16;
-  // diagonal blocks of A, later of T. ONE array: the forward substitution indexes it with the lane's block, and
-  // two separate arrays would make the compiler read both and select per value.
-  __shared__ __align__(16) float s_Ad[2 * 32 * SB];
-  __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64];
+// c ? a : b on two accumulator registers. Written plainly, "c ? acc[i] : acc[j]" is folded into acc[c ? i : j], a
+// register-indexed access that costs a 16-way compare-and-select chain; hiding one operand keeps it one v_cndmask.
+__device__ __forceinline__ float gdr_pick(bool c, float a, float b) {
+  asm volatile("" : "+v"(a));
+  return c ? a : b;
+}
+
+// n consecutive floats (n = 1..4) from LDS into the first n components of a vector: exactly the bytes needed, so that
+// partially used vectors of neighbouring loads never share (and wait for) a register
+template <int N>
+__device__ __forceinline__ f32x4 lds_ld_n(const float* p) {
+  f32x4 out;
+  if constexpr (N >= 4) {
+    out = *reinterpret_cast<const f32x4*>(p);
+  } else if constexpr (N == 3) {
+    typedef float f32x3 __attribute__((ext_vector_type(3)));
+    const f32x3 t3 = *reinterpret_cast<const f32x3*>(p);
+    out[0] = t3[0]; out[1] = t3[1]; out[2] = t3[2]; out[3] = 0.0f;
+  } else if constexpr (N == 2) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 t2 = *reinterpret_cast<const f32x2*>(p);
+    out[0] = t2[0]; out[1] = t2[1]; out[2] = 0.0f; out[3] = 0.0f;
+  } else {
+    out[0] = *p; out[1] = 0.0f; out[2] = 0.0f; out[3] = 0.0f;
+  }
+  return out;
+}
+
+// One wave per (chunk, head), many per CU (every step is a short dependent chain on one wave, so it needs other waves
+// to fill the gaps): K K^T on MFMA with operand fragments loaded straight from HBM (the k tile never touches LDS),
+// gating, T by forward substitution on the four 16x16 diagonal blocks at once (lane = block and column: 15 dependent
+// steps) and two levels of MFMA merges T21 = -T22 (A21 T11), each product a single fp16 instruction (T is rounded to
+// the operand type OT afterwards, the coarser or an equal rounding). LDS holds the two diagonal 32x32 blocks in fp32
+// and the per-token factor rows, all wave-private. Output: the record of the chunk and head.
+template <typename T, typename OT, int KT>
+__global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ k, const float* __restrict__ g,
+                                                          const float* __restrict__ beta,
+                                                          const int32_t* __restrict__ chunk_tok0,
+                                                          const int32_t* __restrict__ chunk_len,
+                                                          unsigned char* __restrict__ rec, int H, int HV, int l2norm) {
+  using X8 = typename OpVec<T>::x8;    // input fragments (the K K^T products run in the input type)
+  using O8 = typename OpVec<OT>::x8;   // record elements
+  using O2 = typename OpVec<OT>::x2;
+  constexpr int SB = 36, NKS = KT / 16;
+  __shared__ __align__(16) float s_Ad[2 * 32 * SB];  // the two diagonal 32x32 blocks of A, later of T
+  __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64], s_ra[64], s_ca[64];
   float* s_A11 = s_Ad;
   float* s_A22 = s_Ad + 32 * SB;
-
   const int chunk = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
-  const int tok0 = pv.chunk_tok0[chunk];
-  const int len = pv.chunk_len[chunk];
+  const int tok0 = chunk_tok0[chunk], len = chunk_len[chunk];
   const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;
+  const bool want_ss = l2norm != GDR_L2_NONE;
 
-  // operand fragments of the k tile: f[tm][ks] = k[32 tm + ln][16 ks + 8 hh .. + 7]; rows past the end of a
-  // partial chunk behave as k = 0, g = 0, beta = 0
-  typename Raw8<T>::type raw[2][NK];
+  // operand fragments of the k tile: fk[tm][ks] = k[32 tm + ln][16 ks + 8 hh .. + 7]; rows past the end of a partial
+  // chunk behave as k = 0, g = 0, beta = 0
+  X8 fk[2][NKS];
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm) {
-    const T* kp = k + ((size_t)(tok0 + min(32 * tm + ln, len - 1)) * H + h) * KT + 8 * hh;
+    const size_t row = (size_t)(tok0 + min(32 * tm + ln, len - 1)) * H + h;
 #pragma unroll
-    for (int ks = 0; ks < NK; ++ks) raw[tm][ks] = *reinterpret_cast<const typename Raw8<T>::type*>(kp + 16 * ks);
+    for (int ks = 0; ks < NKS; ++ks) fk[tm][ks] = *reinterpret_cast<const X8*>(k + row * KT + 16 * ks + 8 * hh);
   }
-  {  // gamma is kept in units of log 2 (exp2 is one instruction)
-    const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
-    const float gv = g[gi], bv = beta[gi];
-    const float gcum = 1.44269504f * wave_cumulative_decay(lane < len ? gv : 0.0f), bz = lane < len ? bv : 0.0f;
-    s_gamma[lane] = gcum;
-    s_beta[lane] = bz;
-    float* fact = reinterpret_cast<float*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES + T_BYTES);
-    fact[lane] = gcum;
-    fact[64 + lane] = bz;
-  }
-  bf16x8 f[2][NK];
-  {
-    typename Raw8<T>::type zero;
+  const size_t gi = (size_t)(tok0 + min(lane, len - 1)) * HV + hv;
+  const float rg = g[gi], rb = beta[gi];
+  if (len < 64) {
+    X8 zero;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) zero[e] = (T)0.0f;
+    for (int x = 0; x < 8; ++x) zero[x] = (T)0.0f;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) fk[tm][ks] = 32 * tm + ln < len ? fk[tm][ks] : zero;
+  }
+  float rk2[2] = {1.0f, 1.0f};
+  if (want_ss) {
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {
       float ss = 0.0f;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks)
-        f[tm][ks] = raw_to_bf16<T>(32 * tm + ln < len ? raw[tm][ks] : zero, ss, l2norm != GDR_L2_NONE);
+      for (int ks = 0; ks < NKS; ++ks) ss = op_sumsq<T>(fk[tm][ks], ss);
       ss += __shfl_xor(ss, 32);
-      s_rk[32 * tm + ln] = l2_factor(ss, l2norm);
+      rk2[tm] = l2_factor(ss, l2norm);
     }
   }
+  f32x16 accA[3];
+#pragma unroll
+  for (int tt = 0; tt < 3; ++tt) {
+    const int tr = tt == 2 ? 1 : 0, tc = tt == 0 ? 0 : 1;  // tiles (0,0), (0,1) = A21^T, (1,1)
+    accA[tt] = zero16();
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) accA[tt] = mfma32(fk[tr][ks], fk[tc][ks], accA[tt]);
+  }
+  // per-token factors, lane = token (gamma in units of log 2)
+  float gcum = 1.44269504f * wave_cumulative_decay(lane < len ? rg : 0.0f);
+  // The product must be ROUNDED before it enters any difference of two gammas: contracted into it as an fma, the
+  // difference of equal gammas comes out as a rounding residual of either sign, and a positive exponent is masked to
+  // zero. The empty asm hides the product from the compiler.
+  asm volatile("" : "+v"(gcum));
+  const float bz = lane < len ? rb : 0.0f;
+  const float g_last = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gcum), 63));
+  const float rk_tok = hh ? rk2[1] : rk2[0];
+  {
+    float* fact = reinterpret_cast<float*>(rec + ((size_t)chunk * HV + hv) * REC_BYTES + T_BYTES);
+    fact[lane] = gcum;
+    fact[64 + lane] = bz;
+    fact[128 + lane] = rk_tok;
+  }
+  // Fast gating: e^{gamma_i - gamma_j} = E_i / E_j with E = e^{gamma - gamma_ref}, gamma_ref = gamma_last / 2, as long as
+  // no exponent can leave the fp32 range (total decay of the chunk above 2^-120) and no g is positive (then every ratio
+  // has to go through safe_exp one by one).
+  const bool fast = !__ballot(rg > 0.0f && lane < len) && g_last > -120.0f;
+  const float E = __builtin_amdgcn_exp2f(gcum - 0.5f * g_last), iE = __builtin_amdgcn_exp2f(0.5f * g_last - gcum);
+  s_gamma[lane] = gcum;
+  s_beta[lane] = bz;
+  s_rk[lane] = rk_tok;
+  s_ra[lane] = bz * rk_tok * E;
+  s_ca[lane] = rk_tok * iE;
   lds_fence();
-
-  // A = strict_lower(beta_i rk_i rk_j (k_i . k_j) e^{gamma_i - gamma_j}). The diagonal blocks go to LDS; the
-  // off-diagonal block is computed transposed (rows j < 32, columns i >= 32) and stays in registers, because an
-  // accumulator that holds A21^T is, rounded to bf16, the A operand of A21 X.
   f32x16 a21t;
+  if (fast) {
 #pragma unroll
-  for (int t = 0; t < 3; ++t) {
-    const int tr = t == 2 ? 1 : 0, tc = t == 0 ? 0 : 1;  // accumulator rows / columns: (0,0), (0,1) = A21^T, (1,1)
-    f32x4 gr4[4], rr4[4], br4[4];
+    for (int tt = 0; tt < 3; ++tt) {
+      const int tr = tt == 2 ? 1 : 0, tc = tt == 0 ? 0 : 1;
+      f32x4 rowa[4], rowc[4];
 #pragma unroll
-    for (int b4 = 0; b4 < 4; ++b4) {
-      gr4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tr + 8 * b4 + 4 * hh]);
-      rr4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tr + 8 * b4 + 4 * hh]);
-      br4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tr + 8 * b4 + 4 * hh]);
+      for (int b4 = 0; b4 < 4; ++b4) {
+        rowa[b4] = *reinterpret_cast<const f32x4*>(&s_ra[32 * tr + 8 * b4 + 4 * hh]);
+        rowc[b4] = *reinterpret_cast<const f32x4*>(&s_ca[32 * tr + 8 * b4 + 4 * hh]);
+      }
+      const int cidx = 32 * tc + ln;
+      const float cola = s_ca[cidx], cola_t = s_ra[cidx];
+      lds_fence();
+      if (tt == 1) {  // A21^T: rows j (tile 0), columns i (tile 1): A_ij = ra_i ca_j (k_i.k_j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) a21t[r] = accA[1][r] * cola_t * rowc[r / 4][r % 4];
+      } else {        // diagonal blocks: rows i, columns j, strictly lower
+        float* blk = tt == 0 ? s_A11 : s_A22;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int il = acc_row(r, hh);
+          blk[il * SB + ln] = il > ln ? accA[tt][r] * cola * rowa[r / 4][r % 4] : 0.0f;
+        }
+      }
     }
-    const int cidx = 32 * tc + ln;
-    const float gc = s_gamma[cidx], rc = s_rk[cidx], bc = s_beta[cidx];
-    lds_fence();
-    f32x16 acc = zero16();
+  } else {
 #pragma unroll
-    for (int ks = 0; ks < NK; ++ks) acc = mfma32(f[tr][ks], f[tc][ks], acc);
-    if (t == 1) {  // rows j (tile 0), columns i (tile 1): i > j always
+    for (int tt = 0; tt < 3; ++tt) {
+      const int tr = tt == 2 ? 1 : 0, tc = tt == 0 ? 0 : 1;
+      f32x4 gr4[4], rr4[4], br4[4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        a21t[r] = acc[r] * (bc * rc) * rr4[r / 4][r % 4] * safe_exp2(gc - gr4[r / 4][r % 4]);
-    } else {       // rows i, columns j of a diagonal block; the mask goes on the exponent (branch-free)
-      float* blk = t == 0 ? s_A11 : s_A22;
+      for (int b4 = 0; b4 < 4; ++b4) {
+        gr4[b4] = *reinterpret_cast<const f32x4*>(&s_gamma[32 * tr + 8 * b4 + 4 * hh]);
+        rr4[b4] = *reinterpret_cast<const f32x4*>(&s_rk[32 * tr + 8 * b4 + 4 * hh]);
+        br4[b4] = *reinterpret_cast<const f32x4*>(&s_beta[32 * tr + 8 * b4 + 4 * hh]);
+      }
+      const int cidx = 32 * tc + ln;
+      const float gc = s_gamma[cidx], rc = s_rk[cidx], bc = s_beta[cidx];
+      lds_fence();
+      if (tt == 1) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int il = acc_row(r, hh);
-        blk[il * SB + ln] = acc[r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
-                            safe_exp2(il > ln ? gr4[r / 4][r % 4] - gc : 1.0f);
+        for (int r = 0; r < 16; ++r)
+          a21t[r] = accA[1][r] * (bc * rc) * rr4[r / 4][r % 4] * safe_exp2(gc - gr4[r / 4][r % 4]);
+      } else {
+        float* blk = tt == 0 ? s_A11 : s_A22;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int il = acc_row(r, hh);
+          blk[il * SB + ln] = accA[tt][r] * (br4[r / 4][r % 4] * rr4[r / 4][r % 4] * rc) *
+                              safe_exp2(il > ln ? gr4[r / 4][r % 4] - gc : 1.0f);
+        }
       }
     }
   }
   lds_fence();
-
-  // T as a 2x2 block matrix of 32x32 blocks: T11, T22 by forward substitution -- lane 32b + c owns column c of
-  // block b, every lane of a half-wave reads the same A element (LDS broadcast), fp32 throughout;
-  // T21 = -T22 (A21 T11) with two MFMA products whose operands are split into bf16 high and remainder parts.
-  const int b = hh, c = ln;
-  float* Ab = s_Ad + b * (32 * SB);
+  // ---- the four 16x16 diagonal blocks by forward substitution: lane 16 b + c owns column c of block b (block b = rows
+  //      and columns 16 (b % 2) .. + 15 of the 32x32 diagonal block b / 2), fp32 throughout
   {
-    float x[32];
-    f32x4 rowbuf[2][8];  // rows i and i+1: the next row loads while this one is reduced
-    rowbuf[1][0] = *reinterpret_cast<const f32x4*>(Ab + 1 * SB);
+    const int b4 = lane >> 4, c = lane & 15;
+    float* Ab = s_Ad + (b4 >> 1) * (32 * SB) + (16 * (b4 & 1)) * SB + 16 * (b4 & 1);
+    float x[16];
+    // every row this lane needs, requested at once (row i: columns 0 .. i-1, exactly those)
+    f32x4 rows[16][4];
+#define GDR_ROW(i)                                                                                    \
+  {                                                                                                   \
+    constexpr int full = (i) / 4, rem = (i) % 4;                                                      \
+    _Pragma("unroll") for (int qq = 0; qq < full; ++qq) rows[i][qq] = lds_ld_n<4>(Ab + (i) * SB + 4 * qq); \
+    if constexpr (rem > 0) rows[i][full] = lds_ld_n<rem>(Ab + (i) * SB + 4 * full);                   \
+  }
+    GDR_ROW(1) GDR_ROW(2) GDR_ROW(3) GDR_ROW(4) GDR_ROW(5) GDR_ROW(6) GDR_ROW(7) GDR_ROW(8)
+    GDR_ROW(9) GDR_ROW(10) GDR_ROW(11) GDR_ROW(12) GDR_ROW(13) GDR_ROW(14) GDR_ROW(15)
+#undef GDR_ROW
     x[0] = (c == 0) ? 1.0f : 0.0f;
 #pragma unroll
-    for (int i = 1; i < 32; ++i) {
-      if (i + 1 < 32) {
-#pragma unroll
-        for (int q = 0; q < (i + 1 + 3) / 4; ++q)
-          rowbuf[(i + 1) & 1][q] = *reinterpret_cast<const f32x4*>(Ab + (i + 1) * SB + 4 * q);
-      }
+    for (int i = 1; i < 16; ++i) {
+      // the terms with x[0 .. i-2] first, the one that waits for x[i-1] last
       float acc0 = (i == c) ? 1.0f : 0.0f, acc1 = 0.0f;
 #pragma unroll
-      for (int j = 0; j < i; ++j) {
-        if (j & 1) acc1 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc1);
-        else acc0 = __builtin_fmaf(-rowbuf[i & 1][j / 4][j % 4], x[j], acc0);
+      for (int j = 0; j + 1 < i; ++j) {
+        if (j & 1) acc1 = __builtin_fmaf(-rows[i][j / 4][j % 4], x[j], acc1);
+        else acc0 = __builtin_fmaf(-rows[i][j / 4][j % 4], x[j], acc0);
       }
-      x[i] = acc0 + acc1;
-      // pins the order "loads of row i+1, arithmetic of row i": without it the compiler either serialises every
-      // load behind a wait or hoists all the loads to the top and spills
-      asm volatile("" : "+v"(x[i]) : : "memory");
+      x[i] = __builtin_fmaf(-rows[i][(i - 1) / 4][(i - 1) % 4], x[i - 1], acc0 + acc1);
     }
-    lds_fence();  // every lane is done reading A11 / A22 before they are overwritten
+    lds_fence();
 #pragma unroll
-    for (int i = 0; i < 32; ++i) Ab[i * SB + c] = x[i];  // fp32 T11 / T22 in place of A11 / A22
+    for (int i = 0; i < 16; ++i) Ab[i * SB + c] = x[i];  // T in place of A
   }
   lds_fence();
-
-  f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
+  // ---- first merge, both 32x32 diagonal blocks in ONE 32x32x16 product per stage: operand row / column ln = 16 B + i
+  //      belongs to diagonal block B; the quadrants (B, B) of the result are the two products wanted. fp16 operands: T is
+  //      rounded to the input type afterwards, which is the coarser rounding for bf16 inputs and the same for fp16.
+  {
+    const int B = ln >> 4, i = ln & 15;
+    float* blk = s_Ad + B * (32 * SB);
+    f16x8 a1, b1, a2, b2;
+    const f32x4 p0 = *reinterpret_cast<const f32x4*>(blk + (16 + i) * SB + 4 * hh);       // A21'[i][slots]
+    const f32x4 p1 = *reinterpret_cast<const f32x4*>(blk + (16 + i) * SB + 8 + 4 * hh);
+    const f32x4 q0 = *reinterpret_cast<const f32x4*>(blk + (16 + i) * SB + 16 + 4 * hh);  // T22'[i][slots]
+    const f32x4 q1 = *reinterpret_cast<const f32x4*>(blk + (16 + i) * SB + 24 + 4 * hh);
+    float colv[8];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {  // Y = A21 T11: A from the A21^T accumulator, T11 rows in the same slot order
-    bf16x8 ahi, alo, bhi, blo;
+    for (int qq = 0; qq < 8; ++qq) colv[qq] = blk[kappa(hh, qq) * SB + i];                  // T11'[slots][i]
+    lds_fence();
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const float av = a21t[8 * ks + q];
-      const float bv = s_A11[(16 * ks + kappa(hh, q)) * SB + ln];
-      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
-      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
-      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    for (int qq = 0; qq < 4; ++qq) {
+      a1[qq] = (_Float16)p0[qq]; a1[4 + qq] = (_Float16)p1[qq];
+      a2[qq] = (_Float16)q0[qq]; a2[4 + qq] = (_Float16)q1[qq];
     }
-    y0 = mfma32(ahi, bhi, y0);
-    y1 = mfma32(alo, bhi, y1);
-    y2 = mfma32(ahi, blo, y2);
+#pragma unroll
+    for (int qq = 0; qq < 8; ++qq) b1[qq] = (_Float16)colv[qq];
+    const f32x16 y = mfma32(a1, b1, zero16());  // quadrant (B, B): A21' T11'
+#pragma unroll
+    for (int qq = 0; qq < 8; ++qq) b2[qq] = (_Float16)gdr_pick(B != 0, y[8 + qq], y[qq]);
+    const f32x16 z = mfma32(a2, b2, zero16());  // quadrant (B, B): T22' (A21' T11')
+#pragma unroll
+    for (int qq = 0; qq < 8; ++qq)              // T21'[row][i] = -z: rows 16 B + kappa(hh, qq) of the product
+      blk[(16 + kappa(hh, qq)) * SB + i] = -gdr_pick(B != 0, z[8 + qq], z[qq]);
   }
-  f32x16 t0 = zero16(), t1 = zero16(), t2 = zero16();
+  lds_fence();
+  // ---- second merge: T21 = -T22 (A21 T11), A21 from the transposed accumulator
+  f32x16 y = zero16(), t21 = zero16();
+  {
+    float colv[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) y0[r] += y1[r] + y2[r];
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {  // T22 Y, Y taken straight from the accumulator as the B operand
-    bf16x8 ahi, alo, bhi, blo;
-    const f32x4 a0 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
-    const f32x4 a1 = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
+      for (int qq = 0; qq < 8; ++qq) colv[8 * ks + qq] = s_A11[(16 * ks + kappa(hh, qq)) * SB + ln];
+    f32x4 rowv[4];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const float av = q < 4 ? a0[q % 4] : a1[q % 4];
-      const float bv = y0[8 * ks + q];
-      const __bf16 ah = (__bf16)av, bh = (__bf16)bv;
-      ahi[q] = ah; alo[q] = (__bf16)(av - (float)ah);
-      bhi[q] = bh; blo[q] = (__bf16)(bv - (float)bh);
+    for (int ks = 0; ks < 2; ++ks) {
+      rowv[2 * ks + 0] = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 4 * hh]);
+      rowv[2 * ks + 1] = *reinterpret_cast<const f32x4*>(&s_A22[ln * SB + 16 * ks + 8 + 4 * hh]);
     }
-    t0 = mfma32(ahi, bhi, t0);
-    t1 = mfma32(alo, bhi, t1);
-    t2 = mfma32(ahi, blo, t2);
+    lds_fence();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      f16x8 bb;
+#pragma unroll
+      for (int qq = 0; qq < 8; ++qq) bb[qq] = (_Float16)colv[8 * ks + qq];
+      y = mfma32(acc_to_op<_Float16>(a21t, 8 * ks), bb, y);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      f16x8 aa;
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) { aa[qq] = (_Float16)rowv[2 * ks][qq]; aa[4 + qq] = (_Float16)rowv[2 * ks + 1][qq]; }
+      t21 = mfma32(aa, acc_to_op<_Float16>(y, 8 * ks), t21);
+    }
   }
-
-  // T -> HBM: the diagonal blocks from LDS in 16-byte pieces; T21 from the accumulator, two columns per store
-  // (lanes 2j and 2j+1 swap one value of every adjacent row pair, as in the segment kernel's output)
-  __bf16* out = reinterpret_cast<__bf16*>(tmat + ((size_t)chunk * HV + hv) * REC_BYTES);
+  // ---- T -> HBM: the diagonal blocks from LDS in 16-byte pieces; T21 from the accumulator, two columns per store
+  //      (lanes 2j and 2j+1 swap one value of every adjacent row pair)
+  OT* out = reinterpret_cast<OT*>(rec + ((size_t)chunk * HV + hv) * REC_BYTES);
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
     const float* src = blk == 0 ? s_A11 : s_A22;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int piece = lane + 64 * j, row = piece >> 2, part = piece & 3;
+    for (int jj = 0; jj < 2; ++jj) {
+      const int piece = lane + 64 * jj, row = piece >> 2, part = piece & 3;
       const f32x4 lo = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part]);
       const f32x4 hi = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part + 4]);
-      bf16x8 pk;
+      O8 pk;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { pk[e] = (__bf16)lo[e]; pk[4 + e] = (__bf16)hi[e]; }
-      *reinterpret_cast<bf16x8*>(out + (blk == 0 ? 0 : 2048) + row * 32 + 8 * part) = pk;
+      for (int e4 = 0; e4 < 4; ++e4) { pk[e4] = (OT)lo[e4]; pk[4 + e4] = (OT)hi[e4]; }
+      *reinterpret_cast<O8*>(out + (blk == 0 ? 0 : 2048) + row * 32 + 8 * part) = pk;
     }
   }
   {
     const bool odd = ln & 1;
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int pr = 0; pr < 8; ++pr) {
       const int r0 = 2 * pr, r1 = r0 + 1;
-      const float x0 = -(t0[r0] + (t1[r0] + t2[r0])), x1 = -(t0[r1] + (t1[r1] + t2[r1]));
-      const float keep = odd ? x1 : x0;
-      const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
-      bf16x2 pk;
-      pk[0] = (__bf16)(odd ? got : keep);
-      pk[1] = (__bf16)(odd ? keep : got);
+      const float x0 = -t21[r0], x1 = -t21[r1];
+      const float keep = gdr_pick(odd, x1, x0);
+      const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, gdr_pick(odd, x0, x1));
+      O2 pk;
+      pk[0] = (OT)(odd ? got : keep);
+      pk[1] = (OT)(odd ? keep : got);
       const int row = acc_row(r0, hh) + (odd ? 1 : 0);
-      *reinterpret_cast<bf16x2*>(out + 1024 + row * 32 + (ln & ~1)) = pk;
+      *reinterpret_cast<O2*>(out + 1024 + row * 32 + (ln & ~1)) = pk;
     }
   }
 }
@@ -371,13 +490,14 @@ struct GdrSegSmem {
 };
 
 // pointers into one of the two tile sets
-struct GdrTiles {
+template <typename OT>
+struct GdrTilesT {
   // k = the raw k tile; or (composite pass with SCALED tiles) k = diag(ek) K and kd = diag(dk) K, rounded to bf16
   // once: the stagers fold the per-token gate and norm factors into the tiles, so the chain waves neither read nor
   // apply them. That takes a third of the chain waves' LDS traffic away and pays when many short segments share the
   // CUs; with few long segments (one workgroup per CU) the stagers' extra work is the longer pole, so the
   // hierarchical forward instantiates the composite pass with SCALED = false.
-  __bf16 *k, *kd, *v, *t;
+  OT *k, *kd, *v, *t;
   float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
 };
 
@@ -413,7 +533,7 @@ __device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int
   return out;
 }
 
-template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B>
+template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B, typename OT = T>
 __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
@@ -424,6 +544,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
                        float* __restrict__ ht, int H, int HV, float scale, int l2norm,
                        const unsigned char* __restrict__ Mgrp, const unsigned char* __restrict__ Ngrp,
                        const float* __restrict__ Dgrp, const float* __restrict__ h0, int gmax) {
+  // OT: the 16-bit type of every MFMA operand (tiles in LDS, T, R, v_new, P, the state as operand, M' of the
+  // composites): the input type, so that fp16 inputs run on the fp16 MFMA without losing mantissa bits
+  using X8 = typename OpVec<OT>::x8;
+  using X4 = typename OpVec<OT>::x4;
   constexpr bool SCALED = !PASS_B && SCALED_K;
   using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
@@ -431,11 +555,11 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   extern __shared__ __align__(16) unsigned char smem[];
   auto tiles = [&](int par) {
     unsigned char* base = smem + par * SM::TILE_BYTES;
-    GdrTiles t;
-    t.k = reinterpret_cast<__bf16*>(base + SM::T_OFF_K);
-    t.kd = reinterpret_cast<__bf16*>(base + (SCALED ? SM::T_OFF_KD : SM::T_OFF_K));
-    t.v = reinterpret_cast<__bf16*>(base + SM::T_OFF_V);
-    t.t = reinterpret_cast<__bf16*>(base + SM::T_OFF_T);
+    GdrTilesT<OT> t;
+    t.k = reinterpret_cast<OT*>(base + SM::T_OFF_K);
+    t.kd = reinterpret_cast<OT*>(base + (SCALED ? SM::T_OFF_KD : SM::T_OFF_K));
+    t.v = reinterpret_cast<OT*>(base + SM::T_OFF_V);
+    t.t = reinterpret_cast<OT*>(base + SM::T_OFF_T);
     t.beta = reinterpret_cast<float*>(base + SM::T_OFF_F);
     t.ek = t.beta + 64;
     t.dk = t.beta + 128;
@@ -444,7 +568,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     t.misc = t.beta + 320;
     return t;
   };
-  __bf16* s_q = reinterpret_cast<__bf16*>(smem + SM::OFF_Q);
+  OT* s_q = reinterpret_cast<OT*>(smem + SM::OFF_Q);
   unsigned char* s_P = smem + SM::OFF_P;
   T* s_o = reinterpret_cast<T*>(smem + SM::OFF_O);
   float* s_qs = reinterpret_cast<float*>(smem + SM::OFF_QF);  // scale e^{gamma_i} rq_i
@@ -469,7 +593,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     // registers after the row norms are known, and the next k loads must already be on their way by then
     typename Raw8<T>::type rk0_[KU], rk1_[SCALED ? KU : 1], rv_[VU];
     typename Raw8<T>::type rq0_[PASS_B ? KU : 1], rq1_[PASS_B ? KU : 1];  // q of even / odd chunks of the segment
-    bf16x8 rt_[3];
+    X8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
@@ -485,7 +609,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
 #pragma unroll
       for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
-      const bf16x8* tp = reinterpret_cast<const bf16x8*>(tmat + ((size_t)c * HV + hv) * REC_BYTES);
+      const X8* tp = reinterpret_cast<const X8*>(tmat + ((size_t)c * HV + hv) * REC_BYTES);
 #pragma unroll
       for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
     };
@@ -520,28 +644,28 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       }
     };
     auto stage_data = [&](int c, int par, typename Raw8<T>::type* rk_) {
-      const GdrTiles tl = tiles(par);
+      const GdrTilesT<OT> tl = tiles(par);
       zero_dead_rows(c, rk_, KU);
       zero_dead_rows(c, rv_, VU);
 #pragma unroll
       for (int j = 0; j < 3; ++j)
-        *reinterpret_cast<bf16x8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
+        *reinterpret_cast<X8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
       kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u) {
-        const bf16x8 piece = raw_to_bf16<T>(rk_[u], kss, want_ss);
-        if constexpr (!SCALED) *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
+        const X8 piece = raw_to_op<T, OT>(rk_[u], kss, want_ss);
+        if constexpr (!SCALED) *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
       }
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         float unused = 0.0f;
-        *reinterpret_cast<bf16x8*>(&tl.v[srow * SV + spart * (VT / 2) + 8 * u]) =
-            raw_to_bf16<T>(rv_[u], unused, false);
+        *reinterpret_cast<X8*>(&tl.v[srow * SV + spart * (VT / 2) + 8 * u]) =
+            raw_to_op<T, OT>(rv_[u], unused, false);
       }
     };
     // per-token factors of chunk c (gate, beta, norms) into tile set par
     auto stage_factors = [&](int c, int par, const typename Raw8<T>::type* rk_) {
-      const GdrTiles tl = tiles(par);
+      const GdrTilesT<OT> tl = tiles(par);
       // in-chunk cumulative log-decay in units of log 2 (exp2 is a single instruction) and beta, lane = token; both
       // come ready from the chunk's record (zero decay increment and zero beta past the end of a partial chunk)
       const float bv = rb, gv = rg;
@@ -564,15 +688,15 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
           const typename Raw8<T>::type piece = rk_[u];  // (dead rows were zeroed by stage_data)
-          bf16x8 pe, pd;
+          X8 pe, pd;
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float f = (float)piece[e];
-            pe[e] = (__bf16)(f * ekr);
-            pd[e] = (__bf16)(f * dkr);
+            pe[e] = (OT)(f * ekr);
+            pd[e] = (OT)(f * dkr);
           }
-          *reinterpret_cast<bf16x8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = pe;
-          *reinterpret_cast<bf16x8*>(&tl.kd[srow * SK + spart * (KT / 2) + 8 * u]) = pd;
+          *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = pe;
+          *reinterpret_cast<X8*>(&tl.kd[srow * SK + spart * (KT / 2) + 8 * u]) = pd;
         }
       }
     };
@@ -581,8 +705,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       float qss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; ++u)
-        *reinterpret_cast<bf16x8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
-            raw_to_bf16<T>(rq_[u], qss, want_ss);
+        *reinterpret_cast<X8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
+            raw_to_op<T, OT>(rq_[u], qss, want_ss);
       qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
       if (spart == 0) {
         const float rq = l2_factor(qss, l2norm);
@@ -593,16 +717,16 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 
     auto build_p = [&](int par) {
       if constexpr (PASS_B) {
-        const GdrTiles tl = tiles(par);
+        const GdrTilesT<OT> tl = tiles(par);
         // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tile 0, stager 1 tile 2,
         // and they share tile 1: both run its four MFMAs, each finishes and stores one of its two fragments.
         auto p_tile = [&](int t, int half) {  // half: -1 = whole tile, 0 / 1 = accumulator registers 0-7 / 8-15
           const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
-          bf16x8 fa[KT / 16], fb[KT / 16];
+          X8 fa[KT / 16], fb[KT / 16];
 #pragma unroll
           for (int ks = 0; ks < KT / 16; ++ks) {
-            fa[ks] = *reinterpret_cast<const bf16x8*>(&tl.k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
-            fb[ks] = *reinterpret_cast<const bf16x8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
+            fa[ks] = *reinterpret_cast<const X8*>(&tl.k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
+            fb[ks] = *reinterpret_cast<const X8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
           }
           f32x4 gj[4], rj[4];  // gamma_j, rk_j of this lane's 16 accumulator rows
 #pragma unroll
@@ -625,7 +749,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
               const int j = 32 * jm + acc_row(r, hh);
               acc[r] *= fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f);
             }
-            frag_store(s_P, f0 + part, lane, acc_to_operand(acc, 8 * part));
+            op_frag_store<OT>(s_P, f0 + part, lane, acc_to_op<OT>(acc, 8 * part));
           }
         };
         p_tile(sw == 0 ? 0 : 2, -1);
@@ -701,14 +825,14 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         S[km][r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + 32 * km + acc_row(r, hh)) * VT + col] : 0.0f;
-    bf16x8 rm[2][NKM * NKS];
+    X8 rm[2][NKM * NKS];
     f32x4 rn[2][NKM * 4];
     float rd[2];
-    auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) __attribute__((always_inline)) {
+    auto issue = [&](int p, X8* m, f32x4* n, float& d) __attribute__((always_inline)) {
       p = uniform(max(0, min(p, nst - 1)));
       const bool top = p < lead;
       const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
-      const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mgrp : Mcomp) + sh * M_BYTES);
+      const X8* M = reinterpret_cast<const X8*>((top ? Mgrp : Mcomp) + sh * M_BYTES);
       const f32x4* N = reinterpret_cast<const f32x4*>((top ? Ngrp : Ncomp) + (sh * (VT / 32) + vslab) * N_BYTES);
 #pragma unroll
       for (int f = 0; f < NKM * NKS; ++f) m[f] = M[f * 64 + lane];
@@ -716,10 +840,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int f = 0; f < NKM * 4; ++f) n[f] = N[f * 64 + lane];
       d = (top ? Dgrp : Dcomp)[sh];
     };
-    auto step = [&](const bf16x8* m, const f32x4* n, float d) __attribute__((always_inline)) {
-      bf16x8 Sb[NKS];
+    auto step = [&](const X8* m, const f32x4* n, float d) __attribute__((always_inline)) {
+      X8 Sb[NKS];
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc_to_op<OT>(S[ks / 2], 8 * (ks % 2));
 #pragma unroll
       for (int km = 0; km < NKM; ++km) {
         f32x16 acc;
@@ -767,26 +891,26 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   // pays the LDS latency once per MFMA.
   if (nc > 0) lds_barrier();  // tiles (c0) are ready
   for (int c = c0; c < c1; ++c) {
-    const GdrTiles tl = tiles((c - c0) & 1);
+    const GdrTilesT<OT> tl = tiles((c - c0) & 1);
     if constexpr (PASS_B) lds_barrier();  // Qb(c) (the chain waves only take part)
-    bf16x8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
-    bf16x8 ft[6];              // T (stage 2), P (output)
+    X8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+    X8 ft[6];              // T (stage 2), P (output)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
-    bf16x8 Sb[KT / 16];
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = op_ld_kappa<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
+    X8 Sb[KT / 16];
 #pragma unroll
-    for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_operand(S[ks / 2], 8 * (ks % 2));
+    for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_op<OT>(S[ks / 2], 8 * (ks % 2));
     lds_fence();
     // batch for stage 2: T fragments and the per-token factors / v tile of stage 1's epilogue
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
       for (int ks = 0; ks < 2 * (tm + 1); ++ks)  // blocks T11 | T21, T22
-        ft[2 * tm + ks] = ld_kappa(tl.t + (tm == 0 ? 0 : (ks < 2 ? 1 : 2)) * 32 * ST, ST, ln, 16 * (ks & 1), hh);
+        ft[2 * tm + ks] = op_ld_kappa<OT>(tl.t + (tm == 0 ? 0 : (ks < 2 ? 1 : 2)) * 32 * ST, ST, ln, 16 * (ks & 1), hh);
     f32x4 be[8], ek[8];
-    bf16x4 vv[8];
+    X4 vv[8];
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
       const int i0 = 8 * t8 + 4 * hh;
@@ -794,9 +918,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       if constexpr (!SCALED) ek[t8] = *reinterpret_cast<const f32x4*>(&tl.ek[i0]);
       // v[8 t8 + 4 hh + e][col]. The M slabs (v = 0) issue the same transposing loads and drop the result with
       // vmask: the load must run with every lane enabled, so it is kept out of any per-wave branch.
-      vv[t8] = ld_col4(tl.v, SV, 32 * vslab, 8 * t8, lane);
+      vv[t8] = op_ld_col4<OT>(tl.v, SV, 32 * vslab, 8 * t8, lane);
     }
-    bf16x8 Rb[4];
+    X8 Rb[4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {  // R = beta (v - ek (K S))
       f32x16 acc = zero16();
@@ -809,36 +933,36 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
           const float ks_ = SCALED ? acc[4 * b4 + e] : ek[4 * tm + b4][e] * acc[4 * b4 + e];
           acc[4 * b4 + e] = be[4 * tm + b4][e] * (vmask * (float)vv[4 * tm + b4][e] - ks_);
         }
-      Rb[2 * tm + 0] = acc_to_operand(acc, 0);
-      Rb[2 * tm + 1] = acc_to_operand(acc, 8);
+      Rb[2 * tm + 0] = acc_to_op<OT>(acc, 0);
+      Rb[2 * tm + 1] = acc_to_op<OT>(acc, 8);
     }
     lds_fence();
     // batch for stage 3: K^T fragments (transposing reads of the row-major k tile) and the decay factors
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = ld_kappa_tr(tl.kd, SK, 32 * km, 16 * ks, lane);
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = op_ld_kappa_tr<OT>(tl.kd, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
     if constexpr (!SCALED) {
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) dk[t8] = *reinterpret_cast<const f32x4*>(&tl.dk[8 * t8 + 4 * hh]);
     }
     const float dec = tl.misc[0];
-    bf16x8 Vb[4], Vsb[4];
+    X8 Vb[4], Vsb[4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {  // v_new = T R (T is lower triangular: tile tm needs 2 (tm + 1) steps)
       f32x16 acc = zero16();
 #pragma unroll
       for (int ks = 0; ks < 2 * (tm + 1); ++ks) acc = mfma32(ft[2 * tm + ks], Rb[ks], acc);
-      Vb[2 * tm + 0] = acc_to_operand(acc, 0);
-      Vb[2 * tm + 1] = acc_to_operand(acc, 8);
+      Vb[2 * tm + 0] = acc_to_op<OT>(acc, 0);
+      Vb[2 * tm + 1] = acc_to_op<OT>(acc, 8);
       if constexpr (!SCALED) {
 #pragma unroll
         for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc[4 * b4 + e] *= dk[4 * tm + b4][e];
-        Vsb[2 * tm + 0] = acc_to_operand(acc, 0);
-        Vsb[2 * tm + 1] = acc_to_operand(acc, 8);
+        Vsb[2 * tm + 0] = acc_to_op<OT>(acc, 0);
+        Vsb[2 * tm + 1] = acc_to_op<OT>(acc, 8);
       } else {  // (the decay factors are in the kd tile)
         Vsb[2 * tm + 0] = Vb[2 * tm + 0];
         Vsb[2 * tm + 1] = Vb[2 * tm + 1];
@@ -859,9 +983,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = ld_kappa(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
 #pragma unroll
-      for (int f = 0; f < 6; ++f) ft[f] = frag_load(s_P, f, lane);
+      for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
       f32x4 qs[8];
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) qs[t8] = *reinterpret_cast<const f32x4*>(&s_qs[8 * t8 + 4 * hh]);
@@ -933,8 +1057,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int r = 0; r < 16; ++r) {
         const int row = 32 * km + acc_row(r, hh);
         const float val = S[km][r] - (row == mcol ? dtot : 0.0f);
-        *reinterpret_cast<__bf16*>(out + ((size_t)((km * (KT / 16) + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) =
-            (__bf16)val;
+        *reinterpret_cast<OT*>(out + ((size_t)((km * (KT / 16) + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) =
+            (OT)val;
       }
     if (wave == 0 && lane == 0) Dcomp[(size_t)seg * HV + hv] = dtot;
   } else {
@@ -964,13 +1088,14 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 // needs the other waves' rows of the state only as B operand: every wave publishes its two operand fragments in
 // LDS (double-buffered by step parity, one LDS-only barrier per step) and starts the step's MFMAs with its own
 // fragments while the others' are on their way.
-template <int KT, int VT, int DEPTH>
+template <typename OT, int KT, int VT, int DEPTH>
 __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanView pv,
                                                                  const unsigned char* __restrict__ Mcomp,
                                                                  const unsigned char* __restrict__ Ncomp,
                                                                  const float* __restrict__ Dcomp,
                                                                  const float* __restrict__ h0,
                                                                  float* __restrict__ Sinit, int HV, int n_segments) {
+  using X8 = typename OpVec<OT>::x8;
   constexpr int NKS = KT / 16;
   constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
   __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
@@ -986,12 +1111,12 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
     for (int r = 0; r < 16; ++r) S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + col];
   }
 
-  bf16x8 rm[DEPTH][NKS];
+  X8 rm[DEPTH][NKS];
   f32x4 rn[DEPTH][4];
   float rd[DEPTH];
-  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+  auto issue = [&](int p, X8* m, f32x4* n, float& d) {
     const size_t sh = (size_t)(seg0 + p) * HV + hv;
-    const bf16x8* M = reinterpret_cast<const bf16x8*>(Mcomp + sh * M_BYTES);
+    const X8* M = reinterpret_cast<const X8*>(Mcomp + sh * M_BYTES);
     const f32x4* N = reinterpret_cast<const f32x4*>(Ncomp + (sh * (VT / 32) + vn) * N_BYTES);
 #pragma unroll
     for (int j = 0; j < NKS; ++j) m[j] = M[(wave * NKS + (2 * wave + j) % NKS) * 64 + lane];  // own fragments first
@@ -1003,7 +1128,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, nsteps - 1)), rm[d], rn[d], rd[d]);
 
-  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+  auto step = [&](int p, X8* m, f32x4* n, float& dd) {
     {  // the state segment seg0 + p starts from; steps past the end write to the spare slot behind the last segment
       const size_t slot = p <= nsteps ? (size_t)(seg0 + p) : (size_t)n_segments;
       f32x4* si = reinterpret_cast<f32x4*>(Sinit + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
@@ -1017,9 +1142,9 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
     }
     const float dec = dd;
     unsigned char* xbuf = s_x[p & 1];
-    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
-    frag_store(xbuf, 2 * wave + 0, lane, own0);
-    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    const X8 own0 = acc_to_op<OT>(S, 0), own1 = acc_to_op<OT>(S, 8);
+    op_frag_store<OT>(xbuf, 2 * wave + 0, lane, own0);
+    op_frag_store<OT>(xbuf, 2 * wave + 1, lane, own1);
     f32x16 acc;
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4)
@@ -1029,7 +1154,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
     acc = mfma32(m[1], own1, acc);
     lds_barrier();
 #pragma unroll
-    for (int j = 2; j < NKS; ++j) acc = mfma32(m[j], frag_load(xbuf, (2 * wave + j) % NKS, lane), acc);
+    for (int j = 2; j < NKS; ++j) acc = mfma32(m[j], op_frag_load<OT>(xbuf, (2 * wave + j) % NKS, lane), acc);
     S = acc;
     issue(max(0, min(p + DEPTH, nsteps - 1)), m, n, dd);
   };
@@ -1063,7 +1188,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
 // Same step code in both modes; loops are branch free with clamped operands and a spare store slot as above.
 enum { SCAN_GROUP = 1, SCAN_LEAF = 2 };
 
-template <int KT, int VT, int DEPTH, int MODE>
+template <typename OT, int KT, int VT, int DEPTH, int MODE>
 __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlanView pv,
                                                                   const unsigned char* __restrict__ Msrc,
                                                                   const unsigned char* __restrict__ Nsrc,
@@ -1072,6 +1197,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
                                                                   float* __restrict__ dst, unsigned char* __restrict__ Mout,
                                                                   unsigned char* __restrict__ Nout, float* __restrict__ Dout,
                                                                   int HV, int spare_slot, int gmax) {
+  using X8 = typename OpVec<OT>::x8;
   constexpr int G = GDR_SCAN_GROUP;
   static_assert(G % DEPTH == 0, "a group must be a whole number of ring rounds");
   constexpr int NKS = KT / 16;
@@ -1107,13 +1233,13 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
       S[r] = h0[(((size_t)seq * HV + hv) * KT + 32 * wave + acc_row(r, hh)) * VT + 32 * vn + ln];
   }
 
-  bf16x8 rm[DEPTH][NKS];
+  X8 rm[DEPTH][NKS];
   f32x4 rn[DEPTH][4];
   float rd[DEPTH];
-  auto issue = [&](int p, bf16x8* m, f32x4* n, float& d) {
+  auto issue = [&](int p, X8* m, f32x4* n, float& d) {
     const bool top = MODE == SCAN_LEAF && p < lead;  // a group composite (read through the *out pointers)
     const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
-    const bf16x8* M = reinterpret_cast<const bf16x8*>((top ? Mout : Msrc) + sh * M_BYTES);
+    const X8* M = reinterpret_cast<const X8*>((top ? Mout : Msrc) + sh * M_BYTES);
     const f32x4* N = reinterpret_cast<const f32x4*>((top ? Nout : Nsrc) + (sh * (VT / 32) + nblk) * N_BYTES);
 #pragma unroll
     for (int f = 0; f < NKS; ++f) m[f] = M[(wave * NKS + (2 * wave + f) % NKS) * 64 + lane];  // own fragments first
@@ -1125,7 +1251,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
   for (int d = 0; d < DEPTH; ++d) issue(max(0, min(d, last)), rm[d], rn[d], rd[d]);
 
   float dprod = 1.0f;
-  auto step = [&](int p, bf16x8* m, f32x4* n, float& dd) {
+  auto step = [&](int p, X8* m, f32x4* n, float& dd) {
     if (MODE != SCAN_GROUP) {
       const size_t slot = (p >= lead && p <= nsteps) ? (size_t)(slot0 + (p - lead)) : (size_t)spare_slot;
       f32x4* si = reinterpret_cast<f32x4*>(dst + ((slot * HV + hv) * (VT / 32) + vn) * (KT * 32));
@@ -1140,9 +1266,9 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
     const float dec = dd;
     dprod *= dec;
     unsigned char* xbuf = s_x[p & 1];
-    const bf16x8 own0 = acc_to_operand(S, 0), own1 = acc_to_operand(S, 8);
-    frag_store(xbuf, 2 * wave + 0, lane, own0);
-    frag_store(xbuf, 2 * wave + 1, lane, own1);
+    const X8 own0 = acc_to_op<OT>(S, 0), own1 = acc_to_op<OT>(S, 8);
+    op_frag_store<OT>(xbuf, 2 * wave + 0, lane, own0);
+    op_frag_store<OT>(xbuf, 2 * wave + 1, lane, own1);
     f32x16 acc;
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4)
@@ -1152,7 +1278,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
     acc = mfma32(m[1], own1, acc);
     lds_barrier();
 #pragma unroll
-    for (int f = 2; f < NKS; ++f) acc = mfma32(m[f], frag_load(xbuf, (2 * wave + f) % NKS, lane), acc);
+    for (int f = 2; f < NKS; ++f) acc = mfma32(m[f], op_frag_load<OT>(xbuf, (2 * wave + f) % NKS, lane), acc);
     S = acc;
     issue(max(0, min(p + DEPTH, last)), m, n, dd);
   };
@@ -1179,7 +1305,7 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan2_kernel(const GdrPlan
       for (int r = 0; r < 16; ++r) {
         const int row = 32 * wave + acc_row(r, hh);
         const float val = S[r] - (row == mcol ? dprod : 0.0f);
-        *reinterpret_cast<__bf16*>(out + ((size_t)((wave * NKS + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) = (__bf16)val;
+        *reinterpret_cast<OT*>(out + ((size_t)((wave * NKS + ks) * 64 + 32 * hs + (row & 31))) * 16 + 2 * slot) = (OT)val;
       }
       if (vn == 0 && tid == 0) Dout[gh] = dprod;
     } else {

@@ -1,0 +1,98 @@
+// MFMA operand helpers of the chunkwise gated-delta kernels, generic in the 16-bit operand type (bf16 or fp16).
+//
+// bf16 inputs run on v_mfma_f32_32x32x16_bf16, fp16 inputs on v_mfma_f32_32x32x16_f16: every operand that the kernels
+// derive (T, W, U, P, the state as operand ...) is rounded to the INPUT type, as the reference's Triton kernels do
+// (b_h.to(b_k.dtype), models/hattention/chunk_delta_h.py:133-151; its caller feeds fp16,
+// models/hattention/modeling_gated_deltaproduct.py:583-587).
+#pragma once
+#include "gdr_common.h"
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+template <typename T>
+struct OpVec {
+  typedef T x8 __attribute__((ext_vector_type(8)));
+  typedef T x4 __attribute__((ext_vector_type(4)));
+  typedef T x2 __attribute__((ext_vector_type(2)));
+};
+
+// 8 accumulator registers [base, base + 8) of a lane, rounded to T: the lane's share of an MFMA operand whose 16-wide
+// contraction step covers accumulator rows 16 (base / 8) .. + 15 in slot order (see acc_to_operand in gdr_common.h).
+// Read as the B operand it is (rows of the accumulator tile = contraction, lane's column = operand column); read as
+// the A operand it is the TRANSPOSE of the tile (operand row = the lane's column).
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 acc_to_op(const f32x16& acc, int base) {
+  typename OpVec<T>::x8 out;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) out[s] = (T)acc[base + s];
+  return out;
+}
+
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 op_frag_load(const unsigned char* base, int frag, int lane) {
+  return *reinterpret_cast<const typename OpVec<T>::x8*>(base + (size_t)frag * 1024 + lane * 16);
+}
+template <typename T>
+__device__ __forceinline__ void op_frag_store(unsigned char* base, int frag, int lane, typename OpVec<T>::x8 v) {
+  *reinterpret_cast<typename OpVec<T>::x8*>(base + (size_t)frag * 1024 + lane * 16) = v;
+}
+
+// A-operand fragment of rows row0 .. row0 + 31 (lane's row = `row`) of a row-major array with `stride` elements per
+// row, contraction step starting at column col0, in accumulator slot order.
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa(const T* arr, int stride, int row, int col0, int hh) {
+  const typename OpVec<T>::x4 lo = *reinterpret_cast<const typename OpVec<T>::x4*>(arr + row * stride + col0 + 4 * hh);
+  const typename OpVec<T>::x4 hi = *reinterpret_cast<const typename OpVec<T>::x4*>(arr + row * stride + col0 + 8 + 4 * hh);
+  typename OpVec<T>::x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
+// ds_read_b64_tr_b16: lane i of every block of 16 lanes receives element (i % 4) of the four 8-byte rows that lanes
+// i/4, i/4 + 4, i/4 + 8 and i/4 + 12 of its block point at. Must be issued with every lane enabled.
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x4 op_lds_read_tr4(const T* p) {
+  typedef short s16x4v __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s16x4v lds_s16x4;
+  return __builtin_bit_cast(typename OpVec<T>::x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p));
+}
+
+// Four consecutive rows row0 + 4 hh .. + 3 of column col0 + (lane % 32) of a row-major tile: lane L of a block of 16
+// points at row L / 4, column group L % 4 of the block's 16 columns.
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x4 op_ld_col4(const T* arr, int stride, int col0, int row0, int lane) {
+  const int L = lane & 15, blk = (lane >> 4) & 1, hh = lane >> 5;
+  return op_lds_read_tr4<T>(arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * (L & 3));
+}
+
+// Fragment of the TRANSPOSE of a row-major tile: operand row (A) / column (B) = tile column col0 + (lane % 32),
+// contraction over the tile rows row0 .. row0 + 15 in accumulator slot order.
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa_tr(const T* arr, int stride, int col0, int row0, int lane) {
+  const int L = lane & 15, blk = (lane >> 4) & 1, hh = lane >> 5;
+  const T* p = arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * (L & 3);
+  const typename OpVec<T>::x4 lo = op_lds_read_tr4<T>(p), hi = op_lds_read_tr4<T>(p + 8 * stride);
+  typename OpVec<T>::x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
+// sum of squares of a 16-byte piece of the input type, accumulated in fp32
+template <typename T>
+__device__ __forceinline__ float op_sumsq(typename OpVec<T>::x8 v, float ss) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float f = (float)v[e];
+    ss = __builtin_fmaf(f, f, ss);
+  }
+  return ss;
+}

@@ -864,7 +864,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev < 0 || cur_dev >= 64) return LAMPA_ERR_LAUNCH;
   bool& attr_set = attr_set_dev[cur_dev];
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false, false>,
+    if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false, false, __bf16>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
         hipFuncSetAttribute((const void*)hgdn_prep_kernel<T, KT, VT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             smem_p) != hipSuccess ||
@@ -875,9 +875,10 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   }
   LAMPA_PROF(s, "start");
   if (chunks == 0) return LAMPA_OK;
-  hipLaunchKernelGGL((gdr_tinv_kernel<T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv, tf, H, HV,
-                     l2norm);
-  LAMPA_PROF(s, "gdr_tinv_kernel");
+  // (the hierarchical kernels keep bf16 operands whatever the input type)
+  hipLaunchKernelGGL((gdr_local_kernel<T, __bf16, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta,
+                     pv.chunk_tok0, pv.chunk_len, tf, H, HV, l2norm);
+  LAMPA_PROF(s, "gdr_local_kernel");
   const bool split = segs > n_seq;
   // The segment composites and their scan depend on T only, like the prep kernel, and are latency bound on a few
   // workgroups: they run on a second stream (default priority) beside the prep kernel (launched first, which
@@ -903,7 +904,7 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
                      scale, l2norm);
   LAMPA_PROF(s, "hgdn_prep_kernel");
   if (split) {
-    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false, false>), dim3(segs, HV),
+    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false, false, __bf16>), dim3(segs, HV),
                        dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, cs, (const T*)q, (const T*)k, (const T*)v, g,
                        beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nm, Dc, (T*)nullptr,
                        (float*)nullptr, H, HV, scale, l2norm, (const unsigned char*)nullptr,

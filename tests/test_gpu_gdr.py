@@ -203,6 +203,27 @@ def test_chunk_positive_g_follows_the_reference_masking(device):
     _assert_bf16_close(s, want_s, "state l2")
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_chunk_fp16_weak_decay_long_sequence(device, D):
+    # fp16 is the type the reference's layer feeds (modeling_gated_deltaproduct.py:583-587). With next to no decay the
+    # state keeps everything it was ever given, the regime in which rounding errors of the operands accumulate the most;
+    # fp16 operands stay fp16 on the MFMA (11-bit mantissa), so the result sits far inside the bf16 contract.
+    T, H = 20000, 2
+    q, k, v, g, beta = synth.gdr_inputs(1, T, H, D, D, torch.float16, seed=D, g_scale=0.003)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), output_final_state=True)
+    assert o.dtype == torch.float16
+    _assert_bf16_close(o, want_o, "fp16 o")
+    _assert_bf16_close(s, want_s, "fp16 state")
+    max_abs, mean_rel = _errors(o, want_o)
+    assert mean_rel <= 1.5e-3, f"fp16 operands should beat the bf16 error level by far: {mean_rel:.3e}"
+    # the same inputs rounded to bf16 go through the bf16 MFMA and stay inside the same contract
+    ob, sb = gd.chunk_gated_delta_rule(*_to(device, q.bfloat16(), k.bfloat16(), v.bfloat16(), g, beta), output_final_state=True)
+    wb_o, wb_s = og.recurrent_c(q.bfloat16(), k.bfloat16(), v.bfloat16(), g, beta)
+    _assert_bf16_close(ob, wb_o, "bf16 o")
+    _assert_bf16_close(sb, wb_s, "bf16 state")
+
+
 def test_chunk_matches_token_serial_kernel_on_gpu(device):
     q, k, v, g, beta = _to(device, *synth.gdr_inputs(1, 5000, 4, 64, 64, torch.bfloat16, seed=21, g_scale=0.1))
     o1, s1 = gd.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
