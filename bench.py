@@ -34,13 +34,29 @@ KERNEL_BYTES_PER_TOKEN_HEAD = {            # algorithmic bytes each kernel of th
 LSH_BYTES_PER_HIT_TABLE = 224
 # HBM bytes per launch at config 2 from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a plain
 # 256 MiB copy gives): profiles/bench_config1_config2_config3_hbm_traffic_pmc.md. Counters cannot be read from inside a run.
-MEASURED_TRAFFIC_BYTES = {
-    "gdr_segment_kernel<output>": 350.2e6,
-    "gdr_segment_kernel<composite>": 184.1e6,
-    "gdr_scan_kernel": 24.7e6,
-    "gdr_scan2_kernel<group>": 30.9e6,
-    "gdr_scan2_kernel<leaf>": 29.1e6,
-}
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "gdr_chunk_fwd_config2_hbm_traffic_pmc.md")
+
+
+def measured_traffic():
+    """HBM bytes per launch of every kernel of the layer from the counter summary under profiles/ (rows
+    `| kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | bytes |` under the line `commit: <hash>`): counters cannot be read
+    from inside a run, so the figure is the last profiled one and says which commit it was measured at."""
+    out, commit = {}, None
+    try:
+        with open(TRAFFIC_PROFILE) as fh:
+            for ln in fh:
+                if ln.lower().startswith("commit:"):
+                    commit = ln.split(":", 1)[1].strip()
+                cells = [c.strip() for c in ln.strip().strip("|").split("|")]
+                if len(cells) == 4 and cells[0].startswith("gdr_"):
+                    try:
+                        out[cells[0]] = float(cells[3])
+                    except ValueError:
+                        pass
+    except OSError:
+        pass
+    return out, commit
 
 
 def _median(xs):
@@ -48,29 +64,35 @@ def _median(xs):
     return xs[len(xs) // 2]
 
 
-def cpu_baseline_gdr(q, k, v, g, beta, sample_tokens):
+def cpu_baseline_gdr(q, k, v, g, beta, sample_tokens, repeats=5, warmups=3):
     """The reference's CPU path for the layer: a token loop in plain PyTorch (port: oracle.gated_delta.recurrent_delta,
-    fp32) on a prefix of the same inputs, scaled to hits/s."""
+    fp32) on a prefix of the same inputs: `warmups` untimed passes over a 256-token prefix, then `repeats` timed passes
+    over the first `sample_tokens` tokens; the median, scaled to hits/s (the loop is serial in the tokens)."""
     import torch
     from oracle import gated_delta as og
 
     sl = slice(0, sample_tokens)
     args = [x[:, sl].float() for x in (q, k, v, g, beta)]
-    og.recurrent_delta(*[a[:, :64] for a in args], dtype=torch.float32)  # warm-up
-    t0 = time.perf_counter()
-    og.recurrent_delta(*args, dtype=torch.float32)
-    dt = time.perf_counter() - t0
+    for _ in range(warmups):
+        og.recurrent_delta(*[a[:, :256] for a in args], dtype=torch.float32)
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        og.recurrent_delta(*args, dtype=torch.float32)
+        times.append(time.perf_counter() - t0)
+    dt = _median(times)
     return sample_tokens / dt, dt
 
 
-def cpu_baseline_lsh(coords, feats, alpha):
-    """The reference's CPU path for the LSH stage in plain PyTorch: bmm -> quantise -> pack -> stable sort -> gather."""
+def cpu_baseline_lsh(coords, feats, alpha, offsets):
+    """The reference's CPU path for the LSH stage in plain PyTorch: bmm -> + offset -> quantise -> pack -> stable sort
+    -> gather (the function the GPU leg computes); 3 untimed passes, then the median of 5."""
     import torch
 
     times = []
-    for _ in range(5):
+    for it in range(8):
         t0 = time.perf_counter()
-        proj = torch.bmm(coords[None], alpha[None])[0]
+        proj = torch.bmm(coords[None], alpha[None])[0] + offsets[None, :]
         ids = torch.floor(proj / W_BUCKET).to(torch.int64).T.reshape(N_TABLES, N_PROJ, -1)
         lo = ids.amin(-1, keepdim=True)
         rng = ids.amax(-1, keepdim=True) - lo + 1
@@ -78,7 +100,8 @@ def cpu_baseline_lsh(coords, feats, alpha):
         keys = ((ids - lo) * stride).sum(1)
         perm = torch.sort(keys, dim=-1, stable=True).indices
         out = feats[None].expand(N_TABLES, -1, -1).gather(1, perm[..., None].expand(-1, -1, feats.shape[-1]))
-        times.append(time.perf_counter() - t0)
+        if it >= 3:
+            times.append(time.perf_counter() - t0)
     del out
     return _median(times)
 
@@ -89,8 +112,11 @@ def main():
     # defaults long enough for the GPU clocks to settle (a layer is ~0.16 ms: 50 + 200 steps take 40 ms)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=T,
-                    help="tokens of the workload the CPU baseline is timed on (default: all of them, about 5-10 s)")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192,
+                    help="prefix of the workload the CPU baseline is timed on (median of 5 passes, scaled linearly)")
+    ap.add_argument("--prewarm-ms", type=float, default=150.0,
+                    help="untimed steps run before the warm-up until this much wall clock has passed, so that the GPU "
+                         "clocks have settled whatever --warmup is")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (for profiler runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run one plain device copy of 256 MiB, the known-size kernel that scales a counter run")
@@ -131,7 +157,15 @@ def main():
     def step():
         return gd.chunk_gated_delta_rule(qd, kd, vd, gd_, bd, output_final_state=True)
 
-    # ---- timed region: exactly K steps ----
+    # ---- clock settling (untimed, stated in the output), then W warm-up steps, then the timed region: exactly K steps ----
+    t_pre = time.perf_counter()
+    n_pre = 0
+    while 1e3 * (time.perf_counter() - t_pre) < args.prewarm_ms:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        n_pre += 20
+    prewarm_ms = 1e3 * (time.perf_counter() - t_pre)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -157,8 +191,10 @@ def main():
     dom_bytes = KERNEL_BYTES_PER_TOKEN_HEAD.get(dominant, LAYER_BYTES_PER_TOKEN_HEAD) * token_heads
     dom_gbs = dom_bytes / (stage_us[dominant] * 1e-6) / 1e9
     layer_us = ms_per_step * 1e3
+    traffic_table, traffic_commit = measured_traffic()
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+                "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic_table.get(dominant),
+                "traffic_measured_at_commit": traffic_commit,
                 "kernel_us": round(stage_us[dominant], 2), "algorithmic_bytes_per_launch": dom_bytes}
     # ---- what the output pass's access pattern costs with no arithmetic (memory-only twin of that kernel: same rows
     #      of q, k, v, the per-chunk records and the o rows per workgroup and chunk; whole chunks only) ----
@@ -392,10 +428,31 @@ def main():
     config0 = {"workload": "config0: token-serial gated delta, B=1 H=4 T=8192 d_k=d_v=32, fp32, zero initial state",
                "us": round(c0_us, 1), "hits_per_s": round(8192 / (c0_us * 1e-6), 1)}
     if not args.no_cpu:
-        c0_cpu_hps, c0_cpu_dt = cpu_baseline_gdr(q0, k0, v0, g0, b0, 8192)
+        c0_cpu_hps, c0_cpu_dt = cpu_baseline_gdr(q0, k0, v0, g0, b0, 8192, repeats=5, warmups=3)
         config0["cpu_baseline"] = {"value": round(c0_cpu_hps, 1), "unit": "hits/s", "seconds": round(c0_cpu_dt, 3),
                                    "cores": torch.get_num_threads(), "kind": "port"}
     del d0
+
+    # ---- config 4: 16 packed events of U[6000, 60000] hits, H = 8, K = V = 128, bf16 (varlen, two-level scan) ----
+    lens4, cu4 = synth.varlen_lengths(16, 6000, 60000, seed=0)
+    T4 = int(cu4[-1])
+    d4 = [x.to(dev) for x in synth.gdr_inputs(1, T4, 8, 128, 128, torch.bfloat16, seed=4)]
+    cu4d = cu4.to(dev)
+    c4_us = time_us(lambda: gd.chunk_gated_delta_rule(*d4, output_final_state=True, cu_seqlens=cu4d), n=20, w=5)
+    _capi.profile_begin()
+    for _ in range(5):
+        gd.chunk_gated_delta_rule(*d4, output_final_state=True, cu_seqlens=cu4d)
+    c4_stage = {}
+    for name, ms in _capi.profile_end(max_entries=64):
+        c4_stage.setdefault(name, []).append(ms)
+    th4 = T4 * 8
+    config4 = {"workload": f"config4: 16 packed events ({T4} tokens), H=8, K=V=128, bf16, cu_seqlens",
+               "us": round(c4_us, 1), "hits_per_s": round(T4 / (c4_us * 1e-6), 1),
+               "hbm_frac": round(1032 * th4 / (c4_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+               "mfma_frac": round(182.9e3 * th4 / (c4_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+               "kernel_us": {n: round(1e3 * sum(v_) / len(v_), 1) for n, v_ in c4_stage.items()},
+               "note": "algorithmic work per token-head: 1032 B and 182.9 kFLOP"}
+    del d4
 
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
@@ -403,12 +460,12 @@ def main():
         cores = torch.get_num_threads()
         n_cpu = min(T, max(64, args.cpu_sample_tokens))
         cpu_hits_per_s, cpu_dt = cpu_baseline_gdr(q, k, v, g, beta, n_cpu)
-        lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha)
+        lsh_cpu_s = cpu_baseline_lsh(coords, feats, alpha, beta_h)
         lsh_info["cpu_baseline_us"] = round(lsh_cpu_s * 1e6, 1)
         # the same loop on one thread, on a shorter prefix (the loop is serial in the tokens: time scales linearly)
-        n_one = min(n_cpu, 8192)
+        n_one = min(n_cpu, 2048)
         torch.set_num_threads(1)
-        one_hits_per_s, one_dt = cpu_baseline_gdr(q, k, v, g, beta, n_one)
+        one_hits_per_s, one_dt = cpu_baseline_gdr(q, k, v, g, beta, n_one, repeats=3, warmups=1)
         torch.set_num_threads(cores)
         cpu_model = ""
         try:
@@ -418,19 +475,22 @@ def main():
             pass
         cpu = {"value": round(cpu_hits_per_s, 1), "unit": "hits/s", "cores": cores, "kind": "port",
                "cpu_model": cpu_model,
-               "one_thread": {"value": round(one_hits_per_s, 1), "sample": f"first {n_one} tokens ({one_dt:.2f} s)"},
-               "sample": f"first {n_cpu} of {T} tokens, all {H} heads, fp32 token loop in PyTorch ({cpu_dt:.2f} s)"
-                         + ("" if n_cpu == T else ", scaled linearly"),
+               "one_thread": {"value": round(one_hits_per_s, 1),
+                              "sample": f"first {n_one} tokens, median of 3 passes ({one_dt:.2f} s each)"},
+               "sample": f"first {n_cpu} of {T} tokens, all {H} heads, fp32 token loop in PyTorch: 3 warm-ups on 256 "
+                         f"tokens, median of 5 timed passes ({cpu_dt:.2f} s each)"
+                         + ("" if n_cpu == T else ", scaled linearly to hits/s"),
                "cpu_count": os.cpu_count()}
 
     out = {
         "metric": "hits/s per gated-delta layer at T=60k (bf16); % HBM and MFMA roofline",
         "value": round(hits_per_s, 1), "unit": "hits/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "prewarm_ms": round(prewarm_ms, 1), "prewarm_steps": n_pre,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0, "config4": config4,
     }
     print(json.dumps(out))
 
