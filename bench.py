@@ -283,6 +283,7 @@ def main():
     lsh_info = {
         "workload": f"config1: N={N_HITS}, {N_TABLES} tables x {N_PROJ} proj, w={W_BUCKET}, {FEAT_DIM} fp32 feats",
         "us_per_event": round(lsh_us, 2), "hits_per_s": round(N_HITS / (lsh_us * 1e-6), 1),
+        "launches_per_event": round(len(lprof) / args.steps, 2),
         "sum_kernel_us": round(lsh_gpu_us, 2), "kernel_us_per_event": lsh_kernel_us,
         "roofline": {"bound": "hbm", "achieved": round(lsh_bytes / (lsh_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(lsh_bytes / (lsh_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),

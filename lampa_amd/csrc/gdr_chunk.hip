@@ -53,8 +53,8 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
-    hipLaunchKernelGGL((gdr_local_kernel<T, T, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta, pv.chunk_tok0,
-                       pv.chunk_len, tf, H, HV, l2norm);
+    hipLaunchKernelGGL((gdr_local_kernel<T, T, KT>), dim3(gdr_local_grid(chunks, HV)), dim3(64), 0, s, (const T*)k, g, beta,
+                       pv.chunk_tok0, pv.chunk_len, tf, chunks, H, HV, l2norm);
     LAMPA_PROF(s, "gdr_local_kernel");
     if (segs > n_seq) {
       hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,

@@ -183,12 +183,15 @@ __device__ __forceinline__ f32x4 lds_ld_n(const float* p) {
 // steps) and two levels of MFMA merges T21 = -T22 (A21 T11), each product a single fp16 instruction (T is rounded to
 // the operand type OT afterwards, the coarser or an equal rounding). LDS holds the two diagonal 32x32 blocks in fp32
 // and the per-token factor rows, all wave-private. Output: the record of the chunk and head.
+static inline int gdr_local_grid(int n_chunks, int HV) { return 8 * ((n_chunks + 7) / 8) * HV; }
+
 template <typename T, typename OT, int KT>
 __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ k, const float* __restrict__ g,
                                                           const float* __restrict__ beta,
                                                           const int32_t* __restrict__ chunk_tok0,
                                                           const int32_t* __restrict__ chunk_len,
-                                                          unsigned char* __restrict__ rec, int H, int HV, int l2norm) {
+                                                          unsigned char* __restrict__ rec, int n_chunks, int H, int HV,
+                                                          int l2norm) {
   using X8 = typename OpVec<T>::x8;    // input fragments (the K K^T products run in the input type)
   using O8 = typename OpVec<OT>::x8;   // record elements
   using O2 = typename OpVec<OT>::x2;
@@ -197,7 +200,11 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
   __shared__ __align__(16) float s_gamma[64], s_beta[64], s_rk[64], s_ra[64], s_ca[64];
   float* s_A11 = s_Ad;
   float* s_A22 = s_Ad + 32 * SB;
-  const int chunk = blockIdx.x, hv = blockIdx.y;
+  // 1-D grid of gdr_local_grid(n_chunks, HV) workgroups. Workgroups go to the 8 XCDs round robin by their id and
+  // every XCD has its own L2: the HV heads of a chunk are given to consecutive workgroups of ONE XCD, because g and
+  // beta are [T, H] rows of which a head uses 4 bytes per 32-byte sector, and the sector should be fetched once.
+  const int chunk = ((int)blockIdx.x / 8 / HV) * 8 + (int)blockIdx.x % 8, hv = ((int)blockIdx.x / 8) % HV;
+  if (chunk >= n_chunks) return;
   const int h = hv / (HV / H);
   const int tok0 = chunk_tok0[chunk], len = chunk_len[chunk];
   const int lane = threadIdx.x, hh = lane >> 5, ln = lane & 31;

@@ -876,8 +876,8 @@ static int hg_launch(const void* q, const void* k, const void* v, const float* g
   LAMPA_PROF(s, "start");
   if (chunks == 0) return LAMPA_OK;
   // (the hierarchical kernels keep bf16 operands whatever the input type)
-  hipLaunchKernelGGL((gdr_local_kernel<T, __bf16, KT>), dim3(chunks, HV), dim3(64), 0, s, (const T*)k, g, beta,
-                     pv.chunk_tok0, pv.chunk_len, tf, H, HV, l2norm);
+  hipLaunchKernelGGL((gdr_local_kernel<T, __bf16, KT>), dim3(gdr_local_grid(chunks, HV)), dim3(64), 0, s, (const T*)k, g,
+                     beta, pv.chunk_tok0, pv.chunk_len, tf, chunks, H, HV, l2norm);
   LAMPA_PROF(s, "gdr_local_kernel");
   const bool split = segs > n_seq;
   // The segment composites and their scan depend on T only, like the prep kernel, and are latency bound on a few

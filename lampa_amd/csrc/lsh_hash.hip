@@ -308,12 +308,38 @@ extern "C" int lampa_sort_pairs(const void* keys_in, int key_kind, const int32_t
 int lampa_gather_rows_grouped(const void* src, int src_segments, int group, int64_t n_src, const void* idx,
                               int idx_bytes, int n_segments, int64_t n, int64_t row_bytes, void* dst, void* stream);
 
+// the one-launch form of the stage (lsh_stage.hip)
+int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables);
+int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t n_valid, const int32_t* n_valid_dev,
+                     int dim, const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                     int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, int32_t* perm_out, const void* feats,
+                     int64_t feat_row_bytes, void* feats_out, void* workspace, int64_t workspace_bytes,
+                     hipStream_t s);
+
+// Enough for either form of the stage: the one-launch kernel, or the separate kernels (key packing + sort).
 extern "C" int64_t lampa_lsh_bucket_sort_batch_workspace_bytes(int n_events, int64_t n_hits, int n_tables, int n_proj) {
-  if (n_events < 1) return LAMPA_ERR_INVALID;
+  if (n_events < 1 || n_tables < 1) return LAMPA_ERR_INVALID;
   const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
   const int64_t b = lampa_sort_workspace_bytes(n_events * n_tables, n_hits);
   if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
-  return n_events * a + b;
+  const int64_t separate = n_events * a + b, fused = lsh_fused_workspace_bytes(n_events, n_hits, n_tables);
+  return separate > fused ? separate : fused;
+}
+
+// Argument checks of the stage (those of the key kernels and of the sort), so that both forms refuse the same calls.
+static int lsh_stage_check(const float* coords, int n_events, int64_t n_hits, int64_t n_valid, int dim,
+                           const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                           const int32_t* keys_out, const int32_t* meta_out, const int32_t* perm_out, const void* feats,
+                           int64_t feat_row_bytes, const void* feats_out, int n_passes) {
+  if (!perm_out || (feats && (!feats_out || feat_row_bytes < 1)) || n_events < 1) return LAMPA_ERR_INVALID;
+  if (!coords || !alpha || !beta || !keys_out || !meta_out) return LAMPA_ERR_INVALID;
+  if (n_events > 65535 || n_hits < 0 || n_valid < 0 || n_valid > n_hits || n_hits > INT32_MAX)
+    return LAMPA_ERR_INVALID;
+  if (dim < 1 || dim > LSH_MAX_DIM || n_tables < 1 || n_proj < 1 || n_proj > LSH_MAX_PROJ ||
+      n_tables * n_proj > LSH_MAX_COLS || !(w > 0.0f))
+    return LAMPA_ERR_INVALID;
+  if (n_passes != 0 && n_passes != 3 && n_passes != 4) return LAMPA_ERR_INVALID;  // 32-bit keys, 11-bit digits
+  return LAMPA_OK;
 }
 
 extern "C" int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj) {
@@ -330,13 +356,21 @@ extern "C" int lampa_lsh_bucket_sort_batch(const float* coords, int n_events, in
                                            int32_t* meta_out, int32_t* perm_out, const void* feats,
                                            int64_t feat_row_bytes, void* feats_out, int n_passes, void* workspace,
                                            int64_t workspace_bytes, void* stream) {
-  if (!perm_out || (feats && (!feats_out || feat_row_bytes < 1)) || n_events < 1) return LAMPA_ERR_INVALID;
+  int rc = lsh_stage_check(coords, n_events, n_hits, n_hits, dim, alpha, beta, n_tables, n_proj, w, keys_out, meta_out,
+                           perm_out, feats, feat_row_bytes, feats_out, n_passes);
+  if (rc != LAMPA_OK) return rc;
   const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
   if (a < 0) return LAMPA_ERR_INVALID;
   const int64_t b = lampa_sort_workspace_bytes(n_events * n_tables, n_hits);
   if (b < 0) return LAMPA_ERR_INVALID;
-  if (!workspace || workspace_bytes < n_events * a + b) return LAMPA_ERR_WORKSPACE;
-  int rc = lsh_bucket_keys_batch(coords, n_events, n_hits, n_hits, n_valid_dev, dim, alpha, beta, n_tables, n_proj, w,
+  if (!workspace || workspace_bytes < lampa_lsh_bucket_sort_batch_workspace_bytes(n_events, n_hits, n_tables, n_proj))
+    return LAMPA_ERR_WORKSPACE;
+  if (n_hits == 0) return LAMPA_OK;
+  rc = lsh_fused_launch(coords, n_events, n_hits, n_hits, n_valid_dev, dim, alpha, beta, n_tables, n_proj, w, ids_out,
+                        keys_out, meta_out, perm_out, feats, feat_row_bytes, feats_out, workspace, workspace_bytes,
+                        (hipStream_t)stream);
+  if (rc != 1) return rc;  // launched (or failed); 1 = this call needs the separate kernels
+  rc = lsh_bucket_keys_batch(coords, n_events, n_hits, n_hits, n_valid_dev, dim, alpha, beta, n_tables, n_proj, w,
                                  ids_out, keys_out, meta_out, workspace, n_events * a, (hipStream_t)stream);
   if (rc != LAMPA_OK) return rc;
   const int stride = 2 * n_proj + 3;
@@ -357,12 +391,20 @@ extern "C" int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_
                                      int32_t* keys_out, int32_t* meta_out, int32_t* perm_out, const void* feats,
                                      int64_t feat_row_bytes, void* feats_out, int n_passes, void* workspace,
                                      int64_t workspace_bytes, void* stream) {
-  if (!perm_out || (feats && (!feats_out || feat_row_bytes < 1))) return LAMPA_ERR_INVALID;
+  int rc = lsh_stage_check(coords, 1, n_hits, n_valid, dim, alpha, beta, n_tables, n_proj, w, keys_out, meta_out, perm_out,
+                           feats, feat_row_bytes, feats_out, n_passes);
+  if (rc != LAMPA_OK) return rc;
   const int64_t a = lampa_lsh_bucket_workspace_bytes(n_hits, n_tables, n_proj);
   const int64_t b = lampa_sort_workspace_bytes(n_tables, n_hits);
   if (a < 0 || b < 0) return LAMPA_ERR_INVALID;
-  if (!workspace || workspace_bytes < a + b) return LAMPA_ERR_WORKSPACE;
-  int rc = lampa_lsh_bucket_keys(coords, n_hits, n_valid, dim, alpha, beta, n_tables, n_proj, w, ids_out, keys_out,
+  if (!workspace || workspace_bytes < lampa_lsh_bucket_sort_workspace_bytes(n_hits, n_tables, n_proj))
+    return LAMPA_ERR_WORKSPACE;
+  if (n_hits == 0) return LAMPA_OK;
+  rc = lsh_fused_launch(coords, 1, n_hits, n_valid, nullptr, dim, alpha, beta, n_tables, n_proj, w, ids_out, keys_out,
+                        meta_out, perm_out, feats, feat_row_bytes, feats_out, workspace, workspace_bytes,
+                        (hipStream_t)stream);
+  if (rc != 1) return rc;  // launched (or failed); 1 = this call needs the separate kernels
+  rc = lampa_lsh_bucket_keys(coords, n_hits, n_valid, dim, alpha, beta, n_tables, n_proj, w, ids_out, keys_out,
                                  meta_out, workspace, a, stream);
   if (rc != LAMPA_OK) return rc;
   const int stride = 2 * n_proj + 3;

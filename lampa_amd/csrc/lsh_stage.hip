@@ -1,0 +1,568 @@
+// The whole E2LSH bucketing stage (hash -> key ranges -> packed keys -> stable radix sort -> feature gather) of one
+// event, or of a few, in ONE kernel launch on gfx950.
+//
+// Why one kernel: for one event of 60 000 hits every step is a few microseconds of work, and a dependent kernel
+// launch costs about as much as the step itself. Here the steps of a segment (a table of an event: its own key
+// ranges, its own sort) are separated by barriers over the segment's tiles instead (a flag per tile; one to two
+// microseconds), and a segment's keys go from the packing step into the first sort pass in registers. What tiles hand
+// to each other (min / max partials, digit counts, the scattered pairs, the permutation) moves through device-scope
+// relaxed atomic stores and loads: such a store is written through, such a load never reads a CU's L1, and the
+// producer waits for its stores to complete before it raises its flag. No fence is used: on this GPU a device-scope
+// release writes back a whole L2 and an acquire invalidates one, several microseconds each (measured), which is more
+// than a step costs.
+//
+// Every tile of every segment of the call is a workgroup, and all of them must be on the GPU at once (a tile waits
+// for the other tiles of its segment): the launcher checks the grid against what the GPU holds and otherwise leaves
+// the call to the separate kernels, which are the better form for large batches anyway (bandwidth, not latency).
+// Every wait is bounded; a tile whose wait runs out marks the segment's meta row (overflow field, bit 1) and goes on
+// with what it has, with every store kept in range.
+//
+// Replaces (reference chengjiang123/Lampa), fused: E2LSH.forward  models/model_utils/hash_utils.py:368-371, the hash
+// range of lsh_mapping  hash_utils.py:334-340, the mixed-radix key of get_geo_shift  models/attention/hept.py:79-88,
+// q_hashed.argsort(dim=-1)  hept.py:138-139 and sort_to_buckets  hept.py:9-14. Same arithmetic contract as
+// lsh_hash.hip (explicit fmaf chain, floorf, saturation) and the same stable order as radix_sort.hip.
+#include "lsh_device.h"
+#include <atomic>
+#include <chrono>
+#include <mutex>
+
+#define LF_BLOCK 256
+#define LF_WAVES (LF_BLOCK / 64)
+#define LF_MAX_DIGIT_BITS 11
+#define LF_MAX_BINS (1 << LF_MAX_DIGIT_BITS)
+#define LF_SPIN_LIMIT (1 << 22)
+#define LF_PARTIAL_STRIDE (2 * LSH_MAX_PROJ)
+
+struct LshFusedArgs {
+  const float* coords; int64_t n_hits; int64_t n_valid; const int32_t* n_valid_dev; int dim;
+  const float* alpha; const float* beta; int n_tables; int n_proj; float inv_w;
+  int32_t* ids; int32_t* keys; int32_t* meta; int32_t* perm;
+  const char* feats; int vec_per_row; char* feats_out;   // rows of vec_per_row 16-byte pieces
+  int n_events; int n_tiles;
+  uint64_t* flags; int32_t* partial; uint32_t* rows; uint32_t* totals; uint2* pairs0; uint2* pairs1;
+  uint32_t gen;
+};
+
+__device__ __forceinline__ void lf_flag_store(uint64_t* p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t lf_flag_load(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Data that tiles exchange inside the kernel goes through device-scope relaxed atomics as well: such a store is
+// written through to the point where all CUs agree, such a load never reads a CU's L1.
+template <typename W>
+__device__ __forceinline__ W lf_load(const W* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename W>
+__device__ __forceinline__ void lf_store(W* p, W v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint2 lf_load_pair(const uint2* p) {
+  const uint64_t v = lf_load(reinterpret_cast<const uint64_t*>(p));
+  return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
+}
+__device__ __forceinline__ void lf_store_pair(uint2* p, uint32_t key, uint32_t val) {
+  lf_store(reinterpret_cast<uint64_t*>(p), (uint64_t)key | ((uint64_t)val << 32));
+}
+
+// Barrier over the n_tiles workgroups of a segment, all on one XCD. Before: this workgroup's stores have reached the
+// L2. After: every tile has got that far, and this CU's L1 holds nothing older. `want` grows by one per barrier; a
+// neighbour can be at most one barrier ahead. Returns false when the bounded wait ran out.
+__device__ __forceinline__ bool lf_barrier(uint64_t* gf, int tile, int n_tiles, uint64_t want) {
+  __shared__ int s_ok;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    if (threadIdx.x == 0) lf_flag_store(gf + tile, want);
+    int spins = 0;
+    bool done;
+    for (;;) {
+      bool ok = true;
+      for (int c = threadIdx.x; c < n_tiles; c += 64) {
+        const uint64_t v = lf_flag_load(gf + c);
+        ok = ok && (v == want || v == want + 1);
+      }
+      done = __all(ok);
+      if (done || ++spins > LF_SPIN_LIMIT) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (threadIdx.x == 0) s_ok = done ? 1 : 0;
+  }
+  __syncthreads();
+  return s_ok != 0;
+}
+
+__device__ __forceinline__ uint32_t lf_wave_inclusive(uint32_t v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(v, off);
+    if (lane >= off) v += up;
+  }
+  return v;
+}
+
+// grid = segments * n_tiles workgroups: workgroup b is tile b % n_tiles of segment b / n_tiles (segment =
+// event * n_tables + table). A tile is 256 * ITEMS hits; element order inside a tile as in the radix sort: wave w owns
+// a quarter of the tile, item k of lane l is at quarter * w + k * 64 + l. Small ITEMS = more, smaller tiles: more CUs
+// and more waves per hit, which is what the latency of one event needs.
+template <int DIM, int ITEMS>
+__global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs a) {
+  __shared__ uint32_t s_bin[LF_WAVES][LF_MAX_BINS];  // per-wave digit counts, later the waves' output bases
+  __shared__ uint32_t s_base[LF_MAX_BINS];           // keys of the segment with a smaller digit
+  __shared__ uint32_t s_tot[LF_MAX_BINS];            // digit totals of the segment; later the tile's permutation
+  __shared__ int32_t s_mm[LF_WAVES][LF_PARTIAL_STRIDE];
+  __shared__ int32_t s_lo[LSH_MAX_PROJ], s_hi[LSH_MAX_PROJ];
+  __shared__ uint32_t s_stride[LSH_MAX_PROJ];
+  __shared__ float s_alpha[LSH_MAX_DIM][LSH_MAX_PROJ], s_beta[LSH_MAX_PROJ];  // the table's projections
+  __shared__ uint32_t s_total;
+  __shared__ int s_bits, s_over;
+  __shared__ uint32_t s_wsum[LF_WAVES];
+  constexpr int XD = DIM ? DIM : LSH_MAX_DIM;
+  constexpr int DPT = LF_MAX_BINS / LF_BLOCK;
+  constexpr int TILE = LF_BLOCK * ITEMS;
+  static_assert(TILE <= LF_MAX_BINS, "the tile's permutation is staged in s_tot");
+
+  const int tile = blockIdx.x % a.n_tiles, seg = blockIdx.x / a.n_tiles;
+  const int n_tiles = a.n_tiles, J = a.n_proj, T = a.n_tables, n_cols = J * T;
+  const int n_hits = (int)a.n_hits, dim = DIM ? DIM : a.dim;
+  const int wave = threadIdx.x >> 6, lane = lane_id();
+  uint64_t* gf = a.flags + (int64_t)seg * n_tiles;
+  int32_t* partial = a.partial + (int64_t)seg * n_tiles * LF_PARTIAL_STRIDE;
+  uint32_t* rows = a.rows + (int64_t)seg * n_tiles * LF_MAX_BINS;
+  uint32_t* totals = a.totals + (int64_t)seg * LF_MAX_BINS;
+  uint2* pairs[2] = {a.pairs0 + (int64_t)seg * n_hits, a.pairs1 + (int64_t)seg * n_hits};
+  uint64_t phase = (uint64_t)a.gen << 32;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  const int ibase = tile * TILE + wave * (TILE / LF_WAVES) + lane;
+
+  {
+    const int ev = seg / T, table = seg - ev * T;
+    const float* coords = a.coords + (int64_t)ev * n_hits * a.dim;
+    const int n_valid = a.n_valid_dev ? a.n_valid_dev[ev] : (int)a.n_valid;
+    bool healthy = true;
+
+    // ---- hash the tile's hits for this table: min / max of every projection's bucket id ----
+    if ((int)threadIdx.x < LSH_MAX_DIM * LSH_MAX_PROJ) {
+      const int d = threadIdx.x / LSH_MAX_PROJ, j = threadIdx.x % LSH_MAX_PROJ;
+      s_alpha[d][j] = (d < dim && j < J) ? a.alpha[d * n_cols + table * J + j] : 0.0f;
+      if (d == 0) s_beta[j] = j < J ? a.beta[table * J + j] : 0.0f;
+    }
+    float x[ITEMS][XD];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int idx = ibase + 64 * k;
+      lsh_load_coords<DIM>(coords, idx < n_valid ? idx : 0, a.dim, x[k]);
+    }
+    __syncthreads();
+    // bucket id of item k for projection j: the chain p = fmaf(x[d], a[d], p) from 0, as everywhere in this library
+    auto bucket_id = [&](int k, int j) -> int32_t {
+      float acc = 0.0f;
+#pragma unroll
+      for (int d = 0; d < XD; ++d)
+        if (DIM || d < dim) acc = __builtin_fmaf(x[k][d], s_alpha[d][j], acc);
+      return lsh_quantise(acc, s_beta[j], a.inv_w);
+    };
+    for (int j = 0; j < J; ++j) {
+      int32_t lo = INT32_MAX, hi = INT32_MIN;
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const int32_t id = bucket_id(k, j);
+        const bool valid = ibase + 64 * k < n_valid;
+        lo = valid ? min(lo, id) : lo;
+        hi = valid ? max(hi, id) : hi;
+      }
+      lo = lsh_wave_extreme<false>(lo);
+      hi = lsh_wave_extreme<true>(hi);
+      if (lane == 63) { s_mm[wave][2 * j] = lo; s_mm[wave][2 * j + 1] = hi; }
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < 2 * J) {
+      const int q = threadIdx.x;
+      int32_t v = s_mm[0][q];
+#pragma unroll
+      for (int w = 1; w < LF_WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
+      lf_store(partial + tile * LF_PARTIAL_STRIDE + q, v);
+    }
+    healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+
+    // ---- ranges, mixed-radix strides, key width (every tile computes them; tile 0 writes the meta row) ----
+    {  // thread t reduces value t % 16 over tiles t / 16, t / 16 + 16, ...: independent loads, one round trip
+      const int q = threadIdx.x & 15;
+      int32_t v = (q & 1) ? INT32_MIN : INT32_MAX;
+      if (q < 2 * J) {
+#pragma unroll 8
+        for (int p = threadIdx.x >> 4; p < n_tiles; p += LF_BLOCK / 16) {
+          const int32_t o = lf_load(partial + p * LF_PARTIAL_STRIDE + q);
+          v = (q & 1) ? max(v, o) : min(v, o);
+        }
+      }
+      int32_t o = __shfl_xor(v, 16);
+      v = (q & 1) ? max(v, o) : min(v, o);
+      o = __shfl_xor(v, 32);
+      v = (q & 1) ? max(v, o) : min(v, o);
+      if (lane < 16) s_mm[wave][lane] = v;
+      __syncthreads();
+      if ((int)threadIdx.x < 2 * J) {
+        v = s_mm[0][q];
+#pragma unroll
+        for (int w = 1; w < LF_WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
+        if (n_valid == 0) v = 0;
+        if (q & 1) s_hi[q >> 1] = v; else s_lo[q >> 1] = v;
+      }
+    }
+    __syncthreads();
+    int32_t* m = a.meta + (int64_t)seg * (2 * J + 3);
+    if (threadIdx.x == 0) {
+      uint64_t total = 1;
+      int overflow = 0;
+      for (int j = 0; j < J; ++j) {
+        const int64_t range = (int64_t)s_hi[j] - (int64_t)s_lo[j] + 1;
+        s_stride[j] = (uint32_t)total;
+        total *= (uint64_t)range;
+        if (total > (uint64_t)INT32_MAX) { overflow = 1; total = (uint64_t)INT32_MAX + 1; }
+        if (tile == 0) {
+          m[j] = s_lo[j];
+          m[J + j] = range > INT32_MAX ? INT32_MAX : (int32_t)range;
+        }
+      }
+      const uint64_t top = (n_valid < n_hits) ? total : total - 1;
+      int bits = min(32, max(1, 64 - (int)__clzll((unsigned long long)top)));  // significant bits of the largest key
+      if (overflow) bits = 32;
+      s_total = (uint32_t)total;
+      s_bits = bits;
+      s_over = overflow;
+      if (tile == 0) {
+        m[2 * J] = total > (uint64_t)INT32_MAX ? INT32_MAX : (int32_t)total;
+        m[2 * J + 1] = bits;
+        m[2 * J + 2] = overflow;
+      }
+    }
+    __syncthreads();
+
+    // ---- bucket ids and packed keys of the tile's hits (padding hits: ids 0, key = total, so they sort last) ----
+    uint32_t key[ITEMS], rank[ITEMS];
+    int32_t val[ITEMS];
+    bool inside[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int idx = ibase + 64 * k;
+      inside[k] = idx < n_hits;
+      const bool valid = idx < n_valid;
+      uint32_t kk = valid ? 0u : s_total;
+      for (int j = 0; j < J; ++j) {
+        int32_t id = 0;
+        if (valid) {
+          id = bucket_id(k, j);
+          kk += ((uint32_t)id - (uint32_t)s_lo[j]) * s_stride[j];
+        }
+        if (a.ids && inside[k]) a.ids[((int64_t)ev * n_cols + table * J + j) * n_hits + idx] = id;
+      }
+      if (inside[k]) a.keys[(int64_t)seg * n_hits + idx] = (int32_t)kk;
+      key[k] = inside[k] ? kk : 0xFFFFFFFFu;
+      val[k] = idx;
+    }
+
+    // ---- stable LSD radix sort of the segment: ceil(bits / 11) passes of equal digit width ----
+    const int bits = s_bits;
+    const int eff = (bits + LF_MAX_DIGIT_BITS - 1) / LF_MAX_DIGIT_BITS, width = (bits + eff - 1) / eff;
+    int32_t* perm = a.perm + (int64_t)seg * n_hits;
+    for (int e = 0; e < eff; ++e) {
+      const int shift = e * width, nbits = min(width, bits - shift), bins = 1 << nbits;
+      const uint32_t mask = (uint32_t)bins - 1u;
+      const bool last = e == eff - 1;
+      for (int d = threadIdx.x; d < bins; d += LF_BLOCK) {
+#pragma unroll
+        for (int w = 0; w < LF_WAVES; ++w) s_bin[w][d] = 0;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t d = (key[k] >> shift) & mask;
+        uint64_t peers = __ballot(inside[k]);
+        for (int b = 0; b < nbits; ++b) {
+          const uint64_t bal = __ballot((d >> b) & 1u);
+          peers &= ((d >> b) & 1u) ? bal : ~bal;
+        }
+        if (!inside[k]) peers = 0;
+        const int leader = peers ? (__ffsll((unsigned long long)peers) - 1) : lane;
+        uint32_t old = 0;
+        if (inside[k] && lane == leader) old = atomicAdd(&s_bin[wave][d], (uint32_t)__popcll(peers));
+        old = __shfl(old, leader);
+        rank[k] = old + (uint32_t)__popcll(peers & lt_mask);
+      }
+      __syncthreads();
+      // the tile's digit counts for the other tiles of the segment
+      for (int d = threadIdx.x; d < bins; d += LF_BLOCK) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < LF_WAVES; ++w) c += s_bin[w][d];
+        lf_store(rows + tile * LF_MAX_BINS + d, c);
+      }
+      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      // Tile t turns the counts of digits t*per .. (t+1)*per - 1 of ALL tiles into prefixes over the tiles (in place)
+      // and their sum into the segment's totals: every tile reads n_tiles * per words instead of n_tiles rows. A wave
+      // takes a digit, its lanes the tiles (128 at a time); four digits per wave are in flight, all loads first.
+      {
+        const int per = (bins + n_tiles - 1) / n_tiles, d0 = tile * per;
+        const int steps = (per + LF_WAVES - 1) / LF_WAVES;
+        for (int s0 = 0; s0 < steps; s0 += 4) {
+          uint32_t carry[4] = {0, 0, 0, 0};
+          for (int p0 = 0; p0 < n_tiles; p0 += 128) {
+            uint32_t c[4][2];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const int p = p0 + 64 * h + lane;
+                c[u][h] = (dd < per && d < bins && p < n_tiles) ? lf_load(rows + p * LF_MAX_BINS + d) : 0u;
+              }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const int p = p0 + 64 * h + lane;
+                const uint32_t incl = lf_wave_inclusive(c[u][h], lane);
+                if (dd < per && d < bins && p < n_tiles) lf_store(rows + p * LF_MAX_BINS + d, carry[u] + incl - c[u][h]);
+                carry[u] += __shfl(incl, 63);
+              }
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+            if (lane == 0 && dd < per && d < bins) lf_store(totals + d, carry[u]);
+          }
+        }
+      }
+      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      // thread t owns digits t, t + 256, ...: keys of the digit in the tiles before this one, and in the segment
+      uint32_t excl[DPT];
+#pragma unroll
+      for (int j = 0; j < DPT; ++j) {
+        const int d = threadIdx.x + j * LF_BLOCK;
+        excl[j] = d < bins ? lf_load(rows + tile * LF_MAX_BINS + d) : 0u;
+        if (d < bins) s_tot[d] = lf_load(totals + d);
+      }
+      __syncthreads();
+      {  // exclusive scan of the digit totals: thread t scans digits 8t .. 8t+7
+        uint32_t dt[DPT], mine = 0;
+#pragma unroll
+        for (int j = 0; j < DPT; ++j) {
+          const int d = threadIdx.x * DPT + j;
+          dt[j] = d < bins ? s_tot[d] : 0u;
+          mine += dt[j];
+        }
+        uint32_t incl = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const uint32_t up = __shfl_up(incl, off);
+          if (lane >= off) incl += up;
+        }
+        if (lane == 63) s_wsum[wave] = incl;
+        __syncthreads();
+        uint32_t run = incl - mine;
+#pragma unroll
+        for (int w = 0; w < LF_WAVES; ++w) run += w < wave ? s_wsum[w] : 0u;
+#pragma unroll
+        for (int j = 0; j < DPT; ++j) {
+          const int d = threadIdx.x * DPT + j;
+          if (d < bins) s_base[d] = run;
+          run += dt[j];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < DPT; ++j) {  // output base of every wave of the tile for every digit
+        const int d = threadIdx.x + j * LF_BLOCK;
+        if (d < bins) {
+          uint32_t run = s_base[d] + excl[j];
+#pragma unroll
+          for (int w = 0; w < LF_WAVES; ++w) {
+            const uint32_t c = s_bin[w][d];
+            s_bin[w][d] = run;
+            run += c;
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        if (inside[k]) {
+          const uint32_t d = (key[k] >> shift) & mask;
+          const uint32_t pos = s_bin[wave][d] + rank[k];
+          if (pos < (uint32_t)n_hits) {  // always, unless a wait was abandoned
+            if (last) lf_store(perm + pos, val[k]);
+            else lf_store_pair(pairs[e & 1] + pos, key[k], (uint32_t)val[k]);
+          }
+        }
+      }
+      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      if (!last) {
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+          const int idx = ibase + 64 * k;
+          const uint2 kv = inside[k] ? lf_load_pair(pairs[e & 1] + idx) : make_uint2(0xFFFFFFFFu, 0u);
+          key[k] = kv.x;
+          val[k] = (int32_t)kv.y;
+        }
+      }
+    }
+
+    // ---- the hit features in sorted order: rows tile*TILE .. of the segment's output ----
+    if (a.feats) {
+      const int row0 = tile * TILE, n_rows = min(TILE, n_hits - row0);
+      for (int r = threadIdx.x; r < n_rows; r += LF_BLOCK) s_tot[r] = (uint32_t)lf_load(perm + row0 + r);
+      __syncthreads();
+      const int vpr = a.vec_per_row, items = n_rows * vpr;
+      const uint4* src = reinterpret_cast<const uint4*>(a.feats) + (int64_t)ev * n_hits * vpr;
+      uint4* dst = reinterpret_cast<uint4*>(a.feats_out) + ((int64_t)seg * n_hits + row0) * vpr;
+      constexpr int GU = 12;  // 16-byte loads in flight per thread: the reads are random rows, a memory latency each
+      for (int it0 = 0; it0 < items; it0 += GU * LF_BLOCK) {
+        uint4 v[GU];
+#pragma unroll
+        for (int u = 0; u < GU; ++u) {
+          const int it = it0 + u * LF_BLOCK + threadIdx.x;
+          v[u] = make_uint4(0, 0, 0, 0);
+          if (it < items) {
+            const int r = it / vpr, piece = it - r * vpr;
+            const uint32_t from = s_tot[r];
+            if (from < (uint32_t)n_hits) v[u] = src[(int64_t)from * vpr + piece];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < GU; ++u) {
+          const int it = it0 + u * LF_BLOCK + threadIdx.x;
+          if (it < items) dst[it] = v[u];
+        }
+      }
+    }
+    // a wait that ran out: say so in the segment's meta row (after tile 0's write of the overflow field, which
+    // happened before the first sort barrier)
+    if (!healthy && threadIdx.x == 0) m[2 * J + 2] = s_over | 2;
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------------------
+#define LF_MAX_DEVICES 64
+struct LfDevice {
+  int state;             // 0 unknown, 1 known
+  int capacity[2][2];    // workgroups the GPU holds at once: [generic dim, dim 4][ITEMS 8, 4]
+};
+static LfDevice lf_dev[LF_MAX_DEVICES];
+static std::mutex lf_lock;
+static std::atomic<uint32_t> lf_generation{0};
+static const int lf_items[2] = {8, 4};
+
+template <int DIM, int ITEMS>
+static int lf_occupancy() {
+  int occ = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, lsh_fused_kernel<DIM, ITEMS>, LF_BLOCK, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    occ = 0;
+  }
+  return occ;
+}
+
+// How many workgroups of each form of the kernel the current GPU holds at once (CUs x workgroups per CU), looked up
+// once per device.
+static const LfDevice* lf_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LF_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(lf_lock);
+  LfDevice& d = lf_dev[dev];
+  if (d.state == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    d.capacity[0][0] = cus * lf_occupancy<0, 8>(); d.capacity[0][1] = cus * lf_occupancy<0, 4>();
+    d.capacity[1][0] = cus * lf_occupancy<4, 8>(); d.capacity[1][1] = cus * lf_occupancy<4, 4>();
+    d.state = 1;
+  }
+  return &d;
+}
+
+static int64_t lf_tiles(int64_t n_hits, int items) {
+  const int64_t tile = (int64_t)LF_BLOCK * items;
+  return n_hits > 0 ? (n_hits + tile - 1) / tile : 1;
+}
+
+// The fused kernel is for calls of at most this many segments (events x tables): beyond it the call cannot fit the
+// GPU at once whatever the event size.
+#define LF_MAX_SEGMENTS 64
+
+// Workspace of the fused kernel: flags | partials | digit counts and totals | two pair buffers, sized for the
+// smallest tile. Zero when the call is too large for the fused kernel.
+int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables) {
+  const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, 4);
+  if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 8) > 4096) return 0;
+  return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256) +
+         lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256);
+}
+
+// Launches the fused kernel when it applies: returns LAMPA_OK after a launch, 1 when the caller has to take the
+// separate kernels (the tiles of the call do not all fit the GPU at once, rows that are not 16-byte pieces), or an
+// error.
+int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t n_valid, const int32_t* n_valid_dev,
+                     int dim, const float* alpha, const float* beta, int n_tables, int n_proj, float w,
+                     int32_t* ids_out, int32_t* keys_out, int32_t* meta_out, int32_t* perm_out, const void* feats,
+                     int64_t feat_row_bytes, void* feats_out, void* workspace, int64_t workspace_bytes,
+                     hipStream_t s) {
+  const int64_t segs = (int64_t)n_events * n_tables;
+  if (n_hits < 1 || n_hits > (1 << 24) || segs > LF_MAX_SEGMENTS) return 1;
+  if (feats && (feat_row_bytes % 16 != 0 || feat_row_bytes / 16 > (1 << 16) || ((uintptr_t)feats % 16) != 0 ||
+                ((uintptr_t)feats_out % 16) != 0))
+    return 1;
+  const int64_t need = lsh_fused_workspace_bytes(n_events, n_hits, n_tables);
+  if (need == 0) return 1;
+  if (workspace_bytes < need) return LAMPA_ERR_WORKSPACE;
+  const LfDevice* d = lf_device();
+  if (!d) return 1;
+  // the smaller tile (more workgroups, shorter steps) when the whole call is then still on the GPU at once
+  const int dsel = dim == 4 ? 1 : 0;
+  int pick = -1;
+  for (int i = 1; i >= 0 && pick < 0; --i)
+    if (segs * lf_tiles(n_hits, lf_items[i]) <= d->capacity[dsel][i]) pick = i;
+  if (pick < 0) return 1;
+  const int items = lf_items[pick];
+  const int64_t tiles = lf_tiles(n_hits, items);
+  LshFusedArgs a;
+  a.coords = coords; a.n_hits = n_hits; a.n_valid = n_valid; a.n_valid_dev = n_valid_dev; a.dim = dim;
+  a.alpha = alpha; a.beta = beta; a.n_tables = n_tables; a.n_proj = n_proj; a.inv_w = 1.0f / w;
+  a.ids = ids_out; a.keys = keys_out; a.meta = meta_out; a.perm = perm_out;
+  a.feats = (const char*)feats; a.vec_per_row = feats ? (int)(feat_row_bytes / 16) : 0; a.feats_out = (char*)feats_out;
+  a.n_events = n_events; a.n_tiles = (int)tiles;
+  char* p = (char*)workspace;
+  a.flags = (uint64_t*)p;   p += lampa_align_up(segs * tiles * 8, 256);
+  a.partial = (int32_t*)p;  p += lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256);
+  a.rows = (uint32_t*)p;    a.totals = a.rows + segs * tiles * LF_MAX_BINS;
+  p += lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256);
+  a.pairs0 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
+  a.pairs1 = (uint2*)p;
+  // a value no earlier call has left in a workspace: the flags need no clearing
+  uint32_t gen = lf_generation.fetch_add(1) + 1;
+  if (gen == 1) {
+    const uint32_t seed = (uint32_t)std::chrono::steady_clock::now().time_since_epoch().count() | 1u;
+    uint32_t expected = 1;
+    lf_generation.compare_exchange_strong(expected, seed);
+    gen = lf_generation.fetch_add(1) + 1;
+  }
+  a.gen = gen;
+  const dim3 grid((unsigned)(segs * tiles)), block(LF_BLOCK);
+  LAMPA_PROF(s, "start");
+#define LF_LAUNCH(DIM, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, ITEMS>), grid, block, 0, s, a)
+  if (dim == 4) {
+    if (items == 8) LF_LAUNCH(4, 8); else LF_LAUNCH(4, 4);
+  } else {
+    if (items == 8) LF_LAUNCH(0, 8); else LF_LAUNCH(0, 4);
+  }
+#undef LF_LAUNCH
+  LAMPA_PROF(s, "lsh_fused_kernel");
+  return lampa_launch_status();
+}

@@ -263,6 +263,10 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
 
 
 def _raise_on_overflow(meta: torch.Tensor, strict: bool):
+    if strict and bool((meta[..., -1] & 2).any()):
+        raise LampaError("lsh_bucket_sort: a workgroup of the one-launch kernel gave up waiting for the other "
+                         "workgroups of its table (the GPU was shared with another kernel that waits in the same way); "
+                         "the outputs of this call are not to be used")
     if strict and bool(meta[..., -1].any()):
         raise LampaError("lsh_bucket_sort: the id ranges of a table multiply to more than 2^31 - 1 buckets, so its "
                          "32-bit bucket key overflowed and the order is meaningless (use a larger w or fewer "
@@ -283,7 +287,13 @@ def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[to
 
     A table whose id ranges multiply to more than 2^31 - 1 buckets cannot be packed into one 32-bit key: the kernel
     then sets ``meta[..., -1]`` (overflow) and the order of that table is meaningless. ``strict=True`` reads the flag
-    (one host synchronisation) and raises ``LampaError``; otherwise the caller has to look at the flag."""
+    (one host synchronisation) and raises ``LampaError``; otherwise the caller has to look at the flag.
+
+    A call of at most 64 tables in total whose tiles all fit the GPU at once (one event of 60 000 hits does, four do)
+    runs as ONE kernel whose workgroups wait for each other; larger calls run as separate kernels. The waits of the
+    one-launch kernel are bounded: should one run out (two such kernels sharing a GPU can starve each other) bit 1 of
+    ``meta[..., -1]`` is set and the outputs are not to be used; ``strict=True`` raises for it as well. Calls that may
+    run at the same time on one GPU (different streams, processes) should be serialised by the caller."""
     require_cuda(coords, alpha, beta, feats)
     coords = coords.contiguous().float()
     alpha = alpha.contiguous().float()

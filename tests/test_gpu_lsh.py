@@ -220,3 +220,48 @@ def test_bucket_sort_batch_of_nine_events_matches_single_events(device):
                               n_valid=int(lens[e]))
         for name in ("ids", "meta", "keys", "perm", "feats"):
             assert np.array_equal(_np(got[name][e]), want[name]), (name, e)
+
+
+def test_one_launch_and_separate_kernels_agree(device):
+    """The stage has two forms: one kernel whose workgroups wait for each other (calls that fit the GPU at once) and
+    separate kernels (everything else). The same event through both must give the same bits: alone (one launch), as
+    one of 32 copies (96 tables: separate kernels), and with feature rows of 100 bytes (not 16-byte pieces: separate
+    kernels); three calls in a row reuse the same workspace memory, whose flags the kernel never clears."""
+    n = 30011
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    coords, feats, _ = synth.collider_event(n, seed=5)
+    cd, fd, ad, bd = coords.to(device), feats.to(device), alpha.to(device), beta.to(device)
+    want = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy())
+    for _ in range(3):
+        one = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, fd, strict=True)
+        for name in ("ids", "meta", "keys", "perm", "feats"):
+            assert np.array_equal(_np(one[name]), want[name]), name
+    many = lsh.lsh_bucket_sort(cd[None].expand(32, -1, -1).contiguous(), ad, bd, 0.5, 3, 4,
+                               fd[None].expand(32, -1, -1).contiguous(), strict=True)
+    for name in ("ids", "meta", "keys", "perm", "feats"):
+        assert torch.equal(many[name][0], one[name]) and torch.equal(many[name][31], one[name]), name
+    f25 = torch.cat([fd, fd[:, :1]], dim=1)
+    odd = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, f25, strict=True)
+    assert torch.equal(odd["perm"], one["perm"]) and torch.equal(odd["feats"][..., :24], one["feats"])
+    four = lsh.lsh_bucket_sort(cd[None].expand(4, -1, -1).contiguous(), ad, bd, 0.5, 3, 4,
+                               fd[None].expand(4, -1, -1).contiguous(), n_valid=torch.tensor([n, 17, 0, 2049]),
+                               strict=True)  # 12 tables in one launch, padded events
+    for e, nv in enumerate([n, 17, 0, 2049]):
+        w = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy(), n_valid=nv)
+        for name in ("ids", "meta", "keys", "perm", "feats"):
+            assert np.array_equal(_np(four[name][e]), w[name]), (name, e)
+
+
+def test_one_launch_generic_dim_and_wide_keys(device):
+    """dim 3 (the generic coordinate path) and a bucket width that makes the keys need three radix passes."""
+    n = 9000
+    gen = torch.Generator().manual_seed(3)
+    coords = torch.randn(n, 3, generator=gen) * 3
+    alpha = torch.randn(3, 6, generator=gen)
+    beta = torch.rand(6, generator=gen) * 0.05
+    feats = torch.randn(n, 8, generator=gen)
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.05, 2, 3, feats.to(device))
+    want = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.05, 2, 3, feats.numpy())
+    assert int(want["meta"][:, -2].max()) > 22 and not want["meta"][:, -1].any()  # more than two 11-bit digits
+    for name in ("ids", "meta", "keys", "perm", "feats"):
+        assert np.array_equal(_np(got[name]), want[name]), name
