@@ -103,7 +103,28 @@ def _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu
 
 
 def _chunk_path_supported(q, v) -> bool:
-    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] in (64, 128) and v.shape[-1] in (64, 128)
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] <= 128 and v.shape[-1] <= 128
+
+
+def _chunk_head_size(d: int) -> int:
+    """The chunk kernels are built for head sizes 64 and 128; a smaller head runs as the next of the two."""
+    return 64 if d <= 64 else 128
+
+
+def _chunk_launch_any_head(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
+    """Head sizes other than 64 / 128 (the reference's layer uses d_k = 16, d_v = 32,
+    ``modeling_gated_deltaproduct.py:583-587``): q, k and v are zero-padded along the head dimension. Zero columns
+    of k and q add nothing to k k^T, q k^T, q S or the norms, zero columns of v give zero columns of the state and
+    of o, so the padded problem contains the original one exactly; `scale` was fixed from the original K."""
+    K, V = q.shape[-1], v.shape[-1]
+    Kp, Vp = _chunk_head_size(K), _chunk_head_size(V)
+    if (Kp, Vp) == (K, V):
+        return _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm)
+    pad = torch.nn.functional.pad
+    h0 = None if initial_state is None else pad(initial_state.to(torch.float32), (0, Vp - V, 0, Kp - K))
+    o, ht = _chunk_launch(pad(q, (0, Kp - K)), pad(k, (0, Kp - K)), pad(v, (0, Vp - V)), g, beta, scale, h0,
+                          output_final_state, cu_seqlens, l2norm)
+    return o[..., :V].contiguous(), None if ht is None else ht[..., :K, :V].contiguous()
 
 
 class _ForwardOnly(torch.autograd.Function):
@@ -176,7 +197,7 @@ def chunk_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g:
     if scale is None:
         scale = k.shape[-1] ** -0.5
     l2norm = L2_CHUNK if use_qk_l2norm_in_kernel else L2_NONE
-    launcher = _chunk_launch if _chunk_path_supported(q, v) else _recurrent_launch
+    launcher = _chunk_launch_any_head if _chunk_path_supported(q, v) else _recurrent_launch
     o, final_state = _ForwardOnly.apply(launcher, q, k, v, g, beta, scale, initial_state, output_final_state,
                                         cu_seqlens, l2norm)
     return o.to(q.dtype), final_state

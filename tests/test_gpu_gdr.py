@@ -224,6 +224,38 @@ def test_chunk_fp16_weak_decay_long_sequence(device, D):
     _assert_bf16_close(sb, wb_s, "bf16 state")
 
 
+@pytest.mark.parametrize("K,V", [(16, 32), (32, 32), (96, 40)])
+def test_chunk_small_heads_long_sequence_fp16(device, K, V):
+    # the head sizes of the reference's own layer (d_k = 16, d_v = 32, fp16: modeling_gated_deltaproduct.py:583-587)
+    # go through the chunk kernels as a zero-padded 64- or 128-wide head, not through the token loop
+    T, H = 30000, 6
+    q, k, v, g, beta = synth.gdr_inputs(1, T, H, K, V, torch.float16, seed=K + V, g_scale=0.05)
+    h0 = torch.randn(1, H, K, V, generator=torch.Generator().manual_seed(1)) * 0.1
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0)
+    dq, dk, dv, dg, db = _to(device, q, k, v, g, beta)
+    o, s = gd.chunk_gated_delta_rule(dq, dk, dv, dg, db, initial_state=h0.to(device), output_final_state=True)
+    assert o.shape == (1, T, H, V) and s.shape == (1, H, K, V) and o.dtype == torch.float16 and o.is_contiguous()
+    _assert_bf16_close(o, want_o, "small-head o")
+    _assert_bf16_close(s, want_s, "small-head state")
+    if (K, V) == (16, 32):  # and it is far quicker than the token loop on the same inputs
+        import time
+        o2, s2 = gd.fused_recurrent_gated_delta_rule(dq[:, :4096], dk[:, :4096], dv[:, :4096], dg[:, :4096],
+                                                     db[:, :4096], initial_state=h0.to(device), output_final_state=True)
+        _assert_bf16_close(o[:, :4096], o2.float().cpu(), "chunk vs token loop")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            gd.chunk_gated_delta_rule(dq, dk, dv, dg, db)
+        torch.cuda.synchronize()
+        t_chunk = (time.perf_counter() - t0) / 5
+        t0 = time.perf_counter()
+        gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
+        torch.cuda.synchronize()
+        t_loop = time.perf_counter() - t0
+        print(f"K=16 V=32 H=6 T=30000 fp16: chunk path {1e6 * t_chunk:.0f} us, token loop {1e6 * t_loop:.0f} us")
+        assert t_chunk * 20 < t_loop
+
+
 def test_chunk_matches_token_serial_kernel_on_gpu(device):
     q, k, v, g, beta = _to(device, *synth.gdr_inputs(1, 5000, 4, 64, 64, torch.bfloat16, seed=21, g_scale=0.1))
     o1, s1 = gd.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
