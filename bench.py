@@ -33,7 +33,7 @@ KERNEL_BYTES_PER_TOKEN_HEAD = {            # algorithmic bytes each kernel of th
 }
 LSH_BYTES_PER_HIT_TABLE = 224
 # HBM bytes per launch at config 2 from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a plain
-# 256 MiB copy gives): profiles/bench_config1_config2_config3_hbm_traffic_pmc.md. Counters cannot be read from inside a run.
+# 256 MiB copy gives), read from the summary below. Counters cannot be read from inside a run.
 TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
                                "gdr_chunk_fwd_config2_hbm_traffic_pmc.md")
 
