@@ -10,7 +10,8 @@
  *   - return value: 0 on success, negative on error (LAMPA_ERR_*). No C++ exception crosses the boundary;
  *   - state the library keeps between calls: the optional profiling recorder; one helper stream with two events per
  *     (device, caller stream) that lampa_hgdn_chunk_fwd creates on first use and keeps until the process ends (calls
- *     on different streams or host threads never share them); the fixed scratch array of lampa_sort_pairs_static.
+ *     on different streams or host threads never share them); the fixed scratch array of lampa_sort_pairs_static;
+ *     per device, how many workgroups of the one-launch LSH kernel the GPU holds (looked up once).
  *     Everything else lives in caller-owned buffers, so calls on different streams do not interfere.
  * The reference (chengjiang123/Lampa) is Python over Triton/ATen, so each entry point names the Python operator or
  * kernel it replaces (file:line in the reference tree).
@@ -74,7 +75,14 @@ int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, 
 /* The whole bucketing stage of one event in one call: lampa_lsh_bucket_keys, then lampa_sort_pairs on the packed
  * keys (digit widths from meta, read on the device), then lampa_gather_rows of the hit features when feats != NULL.
  * Replaces the hash -> argsort -> sort_to_buckets sequence of models/attention/hept.py:127-143.
- * perm_out [n_tables, n_hits] int32; feats [n_hits, feat_row_bytes] -> feats_out [n_tables, n_hits, feat_row_bytes]. */
+ * perm_out [n_tables, n_hits] int32; feats [n_hits, feat_row_bytes] -> feats_out [n_tables, n_hits, feat_row_bytes].
+ * n_passes: 0 (automatic), 3 or 4 sort launches for the 32-bit keys.
+ * A call (this one or the batch form) of at most 64 tables whose tiles all fit the GPU at once, with feature rows made
+ * of 16-byte pieces, runs as ONE kernel whose workgroups wait for the other workgroups of their table (flags in the
+ * workspace; no host-visible state); any other call runs as separate kernels. The results are the same bits. The waits
+ * are bounded: should one run out (two such kernels sharing one GPU at the same time can starve each other), bit 1 of the
+ * table's overflow field in meta_out is set and the outputs of the call are not to be used. Calls of the stage that
+ * could overlap on one GPU should therefore be serialised by the caller. */
 int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj);
 int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_t n_valid, int dim, const float* alpha,
                           const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
