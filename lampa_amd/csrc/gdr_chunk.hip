@@ -42,14 +42,18 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   float* Dc = (float*)(ws + w.off_d);
   float* Si = (float*)(ws + w.off_sinit);
   constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_b = GdrSegSmem<KT, VT, true>::BYTES;
-  static bool attr_set = false;
-  if (!attr_set) {
+  // the dynamic LDS limit is a per-device attribute of a kernel: set once per device and instantiation (a repeated
+  // set by two host threads racing here is harmless)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
+  if (!attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
         hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, true>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
-    attr_set = true;
+    attr_set[dev] = true;
   }
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
@@ -131,9 +135,3 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
 #undef GDR_CASE
   return LAMPA_ERR_UNSUPPORTED;
 }
-
-#ifdef EXP_STAMP
-extern "C" int lampa_dbg_stamps(unsigned long long* out) {
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(gdr_dbg), sizeof(unsigned long long) * 2 * 8 * 64) == hipSuccess ? 0 : -1;
-}
-#endif
