@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
   // blockIdx.z = event of a batch: its own coords, valid count and partials
   coords += (int64_t)blockIdx.z * n_hits * dim;
   partial += (int64_t)blockIdx.z * gridDim.x * n_cols * 2;
-  if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
+  if (n_valid_dev) n_valid = max((int64_t)0, min(n_hits, (int64_t)n_valid_dev[blockIdx.z]));  // a count outside the event is cut
   float x[LSH_MM_ITEMS][LSH_MAX_DIM];
   bool valid[LSH_MM_ITEMS];
 #pragma unroll
@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
   if (ids) ids += (int64_t)blockIdx.z * n_cols * n_hits;
   keys += (int64_t)blockIdx.z * n_tables * n_hits;
   meta += (int64_t)blockIdx.z * n_tables * (2 * n_proj + 3);
-  if (n_valid_dev) n_valid = n_valid_dev[blockIdx.z];
+  if (n_valid_dev) n_valid = max((int64_t)0, min(n_hits, (int64_t)n_valid_dev[blockIdx.z]));  // a count outside the event is cut
   __shared__ int32_t s_lo[LSH_MAX_COLS], s_hi[LSH_MAX_COLS];
   __shared__ uint32_t s_stride[LSH_MAX_COLS];
   __shared__ uint32_t s_total[LSH_MAX_COLS];  // per table

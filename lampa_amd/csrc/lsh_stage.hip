@@ -140,7 +140,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
   {
     const int ev = seg / T, table = seg - ev * T;
     const float* coords = a.coords + (int64_t)ev * n_hits * a.dim;
-    const int n_valid = a.n_valid_dev ? a.n_valid_dev[ev] : (int)a.n_valid;
+    const int n_valid = max(0, min(n_hits, a.n_valid_dev ? a.n_valid_dev[ev] : (int)a.n_valid));  // a count outside the event is cut
     bool healthy = true;
 
     // ---- hash the tile's hits for this table: min / max of every projection's bucket id ----

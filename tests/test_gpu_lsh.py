@@ -265,3 +265,20 @@ def test_one_launch_generic_dim_and_wide_keys(device):
     assert int(want["meta"][:, -2].max()) > 22 and not want["meta"][:, -1].any()  # more than two 11-bit digits
     for name in ("ids", "meta", "keys", "perm", "feats"):
         assert np.array_equal(_np(got[name]), want[name]), name
+
+
+@pytest.mark.parametrize("n_events", [3, 30])
+def test_valid_counts_outside_the_event_are_cut(device, n_events):
+    """Per-event valid counts live in device memory, so the library cannot refuse bad ones: a count beyond the event is
+    taken as the event's length, a negative one as zero (both forms of the stage: 9 and 90 tables)."""
+    n = 3000
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    coords = torch.stack([synth.collider_event(n, seed=40 + e)[0] for e in range(n_events)])
+    feats = torch.stack([synth.collider_event(n, seed=40 + e)[1] for e in range(n_events)])
+    lens = torch.tensor([n + 5000, -7, 17] * (n_events // 3), dtype=torch.int32)
+    got = lsh.lsh_bucket_sort(coords.to(device), alpha.to(device), beta.to(device), 0.5, 3, 4, feats.to(device), n_valid=lens)
+    for e in range(n_events):
+        nv = min(n, max(0, int(lens[e])))
+        want = ol.bucket_sort(coords[e].numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats[e].numpy(), n_valid=nv)
+        for name in ("ids", "meta", "keys", "perm", "feats"):
+            assert np.array_equal(_np(got[name][e]), want[name]), (name, e)
