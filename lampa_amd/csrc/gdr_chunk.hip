@@ -23,7 +23,9 @@ static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, i
   return w;
 }
 
-static bool gdr_chunk_supported(int K, int V) { return (K == 64 || K == 128) && (V == 64 || V == 128); }
+static bool gdr_chunk_supported(int K, int V) {
+  return ((K == 64 || K == 128) && (V == 64 || V == 128)) || (K == 32 && V == 32);
+}
 
 extern "C" int64_t lampa_gdr_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V) {
   if (total_chunks < 0 || n_segments < 0 || HV < 1) return LAMPA_ERR_INVALID;
@@ -122,11 +124,13 @@ extern "C" int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, 
   return gdr_chunk_launch<TT, KK, VV>(q, k, v, g, beta, o, h0, ht, pv, n_seq, chunks, segs, max_nseg, H, HV, scale, \
                                       l2norm, ws, s)
   if (dtype == GDR_BF16) {
+    if (K == 32 && V == 32) GDR_CASE(__bf16, 32, 32);
     if (K == 64 && V == 64) GDR_CASE(__bf16, 64, 64);
     if (K == 64 && V == 128) GDR_CASE(__bf16, 64, 128);
     if (K == 128 && V == 64) GDR_CASE(__bf16, 128, 64);
     if (K == 128 && V == 128) GDR_CASE(__bf16, 128, 128);
   } else {
+    if (K == 32 && V == 32) GDR_CASE(_Float16, 32, 32);
     if (K == 64 && V == 64) GDR_CASE(_Float16, 64, 64);
     if (K == 64 && V == 128) GDR_CASE(_Float16, 64, 128);
     if (K == 128 && V == 64) GDR_CASE(_Float16, 128, 64);

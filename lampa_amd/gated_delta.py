@@ -106,18 +106,21 @@ def _chunk_path_supported(q, v) -> bool:
     return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] <= 128 and v.shape[-1] <= 128
 
 
-def _chunk_head_size(d: int) -> int:
-    """The chunk kernels are built for head sizes 64 and 128; a smaller head runs as the next of the two."""
-    return 64 if d <= 64 else 128
+def _chunk_head_sizes(K: int, V: int):
+    """The chunk kernels are built for K, V in {64, 128} and for K = V = 32; other head sizes run as the next larger
+    built shape."""
+    if K <= 32 and V <= 32:
+        return 32, 32
+    return (64 if K <= 64 else 128), (64 if V <= 64 else 128)
 
 
 def _chunk_launch_any_head(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
-    """Head sizes other than 64 / 128 (the reference's layer uses d_k = 16, d_v = 32,
+    """Head sizes that are not built (the reference's layer uses d_k = 16, d_v = 32,
     ``modeling_gated_deltaproduct.py:583-587``): q, k and v are zero-padded along the head dimension. Zero columns
     of k and q add nothing to k k^T, q k^T, q S or the norms, zero columns of v give zero columns of the state and
     of o, so the padded problem contains the original one exactly; `scale` was fixed from the original K."""
     K, V = q.shape[-1], v.shape[-1]
-    Kp, Vp = _chunk_head_size(K), _chunk_head_size(V)
+    Kp, Vp = _chunk_head_sizes(K, V)
     if (Kp, Vp) == (K, V):
         return _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm)
     pad = torch.nn.functional.pad

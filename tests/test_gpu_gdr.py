@@ -256,6 +256,40 @@ def test_chunk_small_heads_long_sequence_fp16(device, K, V):
         assert t_chunk * 20 < t_loop
 
 
+@pytest.mark.parametrize("T", [1, 64, 65, 200, 1000])
+def test_chunk_32_wide_heads_short_sequences(device, T):
+    # the 32 x 32 build of the chunk kernels: batch 2, grouped value heads, initial state, both l2norm settings
+    gen = torch.Generator().manual_seed(T)
+    B, H, HV = 2, 2, 4
+    q = torch.randn(B, T, H, 32, generator=gen).bfloat16()
+    k = torch.nn.functional.normalize(torch.randn(B, T, H, 32, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(B, T, HV, 32, generator=gen).bfloat16()
+    g = -torch.rand(B, T, HV, generator=gen) * 0.3
+    beta = torch.rand(B, T, HV, generator=gen)
+    h0 = 0.5 * torch.randn(B, HV, 32, 32, generator=gen)
+    for l2, flag in ((og.L2_NONE, False), (og.L2_CHUNK, True)):
+        want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, l2=l2)
+        o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                         output_final_state=True, use_qk_l2norm_in_kernel=flag)
+        _assert_bf16_close(o, want_o, f"o T={T} l2={flag}")
+        _assert_bf16_close(s, want_s, f"state T={T} l2={flag}")
+
+
+def test_chunk_32_wide_heads_varlen_and_many_segments(device, monkeypatch):
+    # packed sequences incl. an empty one; one chunk per segment, so that long sequences take the two-level scan
+    monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", 1)
+    lens = [64 * 30 + 1, 5, 0, 64 * 9, 64 * 26 - 1]
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.long)
+    T = int(cu[-1])
+    q, k, v, g, beta = synth.gdr_inputs(1, T, 3, 32, 32, torch.float16, seed=12, g_scale=0.003)
+    h0 = 0.5 * torch.randn(len(lens), 3, 32, 32, generator=torch.Generator().manual_seed(4))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device), output_final_state=True,
+                                     cu_seqlens=cu.to(device))
+    _assert_bf16_close(o, want_o, "o varlen 32")
+    _assert_bf16_close(s, want_s, "state varlen 32")
+
+
 def test_chunk_matches_token_serial_kernel_on_gpu(device):
     q, k, v, g, beta = _to(device, *synth.gdr_inputs(1, 5000, 4, 64, 64, torch.bfloat16, seed=21, g_scale=0.1))
     o1, s1 = gd.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
