@@ -251,7 +251,7 @@ int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunk
 int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment, int32_t* plan_host);
 
 /* Chunkwise forward (chunk = 64 tokens). Replaces chunk_gated_delta_rule_fwd and the seven Triton kernels it
- * launches (models/hattention/gated_delta_rule_ori.py:29-80). Shapes as above with H <= HV; K, V in {64, 128};
+ * launches (models/hattention/gated_delta_rule_ori.py:29-80). Shapes as above with H <= HV; K, V in {64, 128} or K = V = 32;
  * dtype LAMPA_BF16 or LAMPA_FP16; plan_host / plan_dev: the same plan in host and device memory. */
 int64_t lampa_gdr_chunk_workspace_bytes(int64_t total_chunks, int64_t n_segments, int HV, int K, int V);
 int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta, void* o,

@@ -512,6 +512,12 @@ template <int KT, int VT, bool PASS_B>
 struct GdrSegShape {
   static constexpr int SLABS = PASS_B ? VT / 32 : (KT + VT) / 32;  // chain waves
   static constexpr int WAVES = SLABS + 2;                          // + two stager waves
+  // The k and q tiles are stored swizzled (op_swizzle16 in gdr_ops.h: one conflict-free 16-byte LDS read per operand
+  // fragment instead of two 8-byte reads). It pays in the output pass of the 128-wide heads (-10 %); at K = V = 64
+  // the output pass times the same and the composite pass loses: the wider reads cost it 24 registers, and two of
+  // its six-wave workgroups only share a CU below 128 (the hardware deals a workgroup's waves out to the SIMDs in a
+  // fixed rotation and starts the next workgroup one step further on, so one SIMD carries four of the twelve waves).
+  static constexpr bool SWIZZLED = PASS_B && (KT > 64 || VT > 64);
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -556,6 +562,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   using X8 = typename OpVec<OT>::x8;
   using X4 = typename OpVec<OT>::x4;
   constexpr bool SCALED = !PASS_B && SCALED_K;
+  constexpr bool SWZ = GdrSegShape<KT, VT, PASS_B>::SWIZZLED;
   using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
@@ -659,9 +666,13 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         *reinterpret_cast<X8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
       kss = 0.0f;
 #pragma unroll
-      for (int u = 0; u < KU; ++u) {
-        const X8 piece = raw_to_op<T, OT>(rk_[u], kss, want_ss);
-        if constexpr (!SCALED) *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = piece;
+      for (int u = 0; u < KU; u += 2) {
+        X8 pa = raw_to_op<T, OT>(rk_[u], kss, want_ss), pb = raw_to_op<T, OT>(rk_[u + 1], kss, want_ss);
+        if constexpr (!SCALED) {
+          if constexpr (SWZ) op_swizzle16<OT>(pa, pb);
+          *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = pa;
+          *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u + 8]) = pb;
+        }
       }
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
@@ -711,9 +722,12 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       zero_dead_rows(c, rq_, KU);
       float qss = 0.0f;
 #pragma unroll
-      for (int u = 0; u < KU; ++u)
-        *reinterpret_cast<X8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) =
-            raw_to_op<T, OT>(rq_[u], qss, want_ss);
+      for (int u = 0; u < KU; u += 2) {
+        X8 pa = raw_to_op<T, OT>(rq_[u], qss, want_ss), pb = raw_to_op<T, OT>(rq_[u + 1], qss, want_ss);
+        if constexpr (SWZ) op_swizzle16<OT>(pa, pb);
+        *reinterpret_cast<X8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) = pa;
+        *reinterpret_cast<X8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u + 8]) = pb;
+      }
       qss += dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, qss);
       if (spart == 0) {
         const float rq = l2_factor(qss, l2norm);
@@ -905,7 +919,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = op_ld_kappa<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh)
+                                        : op_ld_kappa<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
     X8 Sb[KT / 16];
 #pragma unroll
     for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_op<OT>(S[ks / 2], 8 * (ks % 2));
@@ -948,7 +963,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = op_ld_kappa_tr<OT>(tl.kd, SK, 32 * km, 16 * ks, lane);
+      for (int ks = 0; ks < 4; ++ks) fk[km * 4 + ks] = op_ld_kappa_tr<OT, SWZ>(tl.kd, SK, 32 * km, 16 * ks, lane);
     f32x4 dk[8];
     if constexpr (!SCALED) {
 #pragma unroll
@@ -990,7 +1005,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh)
+                                        : op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
 #pragma unroll
       for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
       f32x4 qs[8];

@@ -56,6 +56,25 @@ __device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa(const T* arr, int s
   return out;
 }
 
+// Swizzled row-major tiles. The lane's share of a 16-wide contraction step in accumulator slot order is elements
+// 4 hh .. + 3 and 8 + 4 hh .. + 3 of the 16: two 8-byte LDS reads, and the 32 lanes of a half-wave hit every bank pair
+// twice whatever 16-byte aligned row stride the tile has. Tiles that feed such operands are therefore stored with the
+// two middle groups of four of every 16 columns swapped ([0-3 | 8-11 | 4-7 | 12-15]): the share becomes ONE aligned
+// 16-byte piece at column 8 hh of the group (a ds_read_b128, served 16 lanes at a time without conflicts). The writer
+// holds both 8-element pieces of a group in registers, so the swap is a renaming of registers.
+template <typename T>
+__device__ __forceinline__ void op_swizzle16(typename OpVec<T>::x8& a, typename OpVec<T>::x8& b) {
+  typename OpVec<T>::x8 na, nb;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { na[s] = a[s]; na[4 + s] = b[s]; nb[s] = a[4 + s]; nb[4 + s] = b[4 + s]; }
+  a = na;
+  b = nb;
+}
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa_swz(const T* arr, int stride, int row, int col0, int hh) {
+  return *reinterpret_cast<const typename OpVec<T>::x8*>(arr + row * stride + col0 + 8 * hh);
+}
+
 // ds_read_b64_tr_b16: lane i of every block of 16 lanes receives element (i % 4) of the four 8-byte rows that lanes
 // i/4, i/4 + 4, i/4 + 8 and i/4 + 12 of its block point at. Must be issued with every lane enabled.
 template <typename T>
@@ -75,10 +94,12 @@ __device__ __forceinline__ typename OpVec<T>::x4 op_ld_col4(const T* arr, int st
 
 // Fragment of the TRANSPOSE of a row-major tile: operand row (A) / column (B) = tile column col0 + (lane % 32),
 // contraction over the tile rows row0 .. row0 + 15 in accumulator slot order.
-template <typename T>
+// SWZ: the tile is stored swizzled (above): logical column group g of a 16 sits at position [0, 2, 1, 3][g].
+template <typename T, bool SWZ = false>
 __device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa_tr(const T* arr, int stride, int col0, int row0, int lane) {
   const int L = lane & 15, blk = (lane >> 4) & 1, hh = lane >> 5;
-  const T* p = arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * (L & 3);
+  const int g = SWZ ? (((L & 1) << 1) | ((L >> 1) & 1)) : (L & 3);
+  const T* p = arr + (row0 + 4 * hh + (L >> 2)) * stride + col0 + 16 * blk + 4 * g;
   const typename OpVec<T>::x4 lo = op_lds_read_tr4<T>(p), hi = op_lds_read_tr4<T>(p + 8 * stride);
   typename OpVec<T>::x8 out;
 #pragma unroll
