@@ -67,8 +67,8 @@ __device__ __forceinline__ void lf_store_pair(uint2* p, uint32_t key, uint32_t v
   lf_store(reinterpret_cast<uint64_t*>(p), (uint64_t)key | ((uint64_t)val << 32));
 }
 
-// Barrier over the n_tiles workgroups of a segment, all on one XCD. Before: this workgroup's stores have reached the
-// L2. After: every tile has got that far, and this CU's L1 holds nothing older. `want` grows by one per barrier; a
+// Barrier over the n_tiles workgroups of a segment: a flag per tile, every tile polls all of them. Before the flag is
+// raised every thread has waited for its own (written-through) stores to complete. `want` grows by one per barrier; a
 // neighbour can be at most one barrier ahead. Returns false when the bounded wait ran out.
 __device__ __forceinline__ bool lf_barrier(uint64_t* gf, int tile, int n_tiles, uint64_t want) {
   __shared__ int s_ok;
@@ -455,7 +455,14 @@ struct LfDevice {
 };
 static LfDevice lf_dev[LF_MAX_DEVICES];
 static std::mutex lf_lock;
-static std::atomic<uint32_t> lf_generation{0};
+
+// A value that no earlier call of this process has left in a workspace (the flags are compared for equality with
+// generation << 32 | barrier number, so they need no clearing), started from the clock so that a workspace written by
+// another process is no more likely to match.
+static uint32_t lf_next_generation() {
+  static std::atomic<uint32_t> counter{(uint32_t)std::chrono::steady_clock::now().time_since_epoch().count()};
+  return counter.fetch_add(1) + 1;
+}
 static const int lf_items[2] = {8, 4};
 
 template <int DIM, int ITEMS>
@@ -545,15 +552,7 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   p += lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256);
   a.pairs0 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
   a.pairs1 = (uint2*)p;
-  // a value no earlier call has left in a workspace: the flags need no clearing
-  uint32_t gen = lf_generation.fetch_add(1) + 1;
-  if (gen == 1) {
-    const uint32_t seed = (uint32_t)std::chrono::steady_clock::now().time_since_epoch().count() | 1u;
-    uint32_t expected = 1;
-    lf_generation.compare_exchange_strong(expected, seed);
-    gen = lf_generation.fetch_add(1) + 1;
-  }
-  a.gen = gen;
+  a.gen = lf_next_generation();
   const dim3 grid((unsigned)(segs * tiles)), block(LF_BLOCK);
   LAMPA_PROF(s, "start");
 #define LF_LAUNCH(DIM, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, ITEMS>), grid, block, 0, s, a)
