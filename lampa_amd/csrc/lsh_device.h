@@ -9,13 +9,18 @@
 #define LSH_MAX_PROJ 8
 #define LSH_BLOCK 256
 
-__device__ __forceinline__ int32_t lsh_quantise(float p, float b, float inv_w) {
-  float t = (p + b) * inv_w;
+// bucket id of the scaled projection t = (p + b) * inv_w. Monotone non-decreasing on the non-NaN floats (so the
+// smallest / largest id of a set is the id of its smallest / largest t).
+__device__ __forceinline__ int32_t lsh_quantise_scaled(float t) {
   if (t != t) return INT32_MAX;
   float f = floorf(t);
   if (f >= 2147483648.0f) return INT32_MAX;
   if (f <= -2147483648.0f) return INT32_MIN;
   return (int32_t)f;
+}
+__device__ __forceinline__ float lsh_scaled(float p, float b, float inv_w) { return (p + b) * inv_w; }
+__device__ __forceinline__ int32_t lsh_quantise(float p, float b, float inv_w) {
+  return lsh_quantise_scaled(lsh_scaled(p, b, inv_w));
 }
 
 template <int DIM>

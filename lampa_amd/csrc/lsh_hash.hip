@@ -14,6 +14,7 @@
 // A block covers LSH_MM_ITEMS * 256 hits (all coordinate loads of a thread are independent). partial
 // [gridDim.x, n_cols, 2] (min, max) per event; no atomics, no initialisation needed.
 #define LSH_MM_ITEMS 8
+#define LSH_PK_ITEMS 4
 template <int DIM>
 __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __restrict__ coords, int64_t n_hits,
                                                               int64_t n_valid,
@@ -23,6 +24,10 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
                                                               float inv_w, int32_t* __restrict__ partial) {
   __shared__ int32_t s_min[LSH_BLOCK / 64][LSH_MAX_COLS];
   __shared__ int32_t s_max[LSH_BLOCK / 64][LSH_MAX_COLS];
+  // the projections are read from LDS (one broadcast read per use) instead of scalar loads inside the column loop
+  __shared__ float s_alpha[LSH_MAX_DIM * LSH_MAX_COLS], s_beta[LSH_MAX_COLS];
+  for (int i = threadIdx.x; i < dim * n_cols; i += LSH_BLOCK) s_alpha[i] = alpha[i];
+  for (int i = threadIdx.x; i < n_cols; i += LSH_BLOCK) s_beta[i] = beta[i];
   // blockIdx.z = event of a batch: its own coords, valid count and partials
   coords += (int64_t)blockIdx.z * n_hits * dim;
   partial += (int64_t)blockIdx.z * gridDim.x * n_cols * 2;
@@ -36,15 +41,23 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
     lsh_load_coords<DIM>(coords, valid[i] ? n : 0, dim, x[i]);
   }
   const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  // The kernel is bound by its arithmetic (hits x columns), so the extremes are taken on the scaled projections and
+  // only they are quantised: the quantisation is monotone, NaNs (id INT32_MAX) are ignored by fminf / fmaxf and noted
+  // separately. Invalid items hold the coordinates of hit 0, a valid hit, so they need no masking (with no valid hit
+  // at all the packing kernel ignores the partials).
   for (int c = 0; c < n_cols; ++c) {
-    int32_t lo = INT32_MAX, hi = INT32_MIN;
-    const float b = beta[c];
+    const float b = s_beta[c];
+    float tlo = INFINITY, thi = -INFINITY;
+    bool nan_seen = false;
 #pragma unroll
     for (int i = 0; i < LSH_MM_ITEMS; ++i) {
-      const int32_t id = lsh_quantise(lsh_dot<DIM>(x[i], alpha, dim, n_cols, c), b, inv_w);
-      lo = valid[i] ? min(lo, id) : lo;
-      hi = valid[i] ? max(hi, id) : hi;
+      const float t = lsh_scaled(lsh_dot<DIM>(x[i], s_alpha, dim, n_cols, c), b, inv_w);
+      tlo = fminf(tlo, t);
+      thi = fmaxf(thi, t);
+      nan_seen = nan_seen || t != t;
     }
+    int32_t lo = lsh_quantise_scaled(tlo), hi = nan_seen ? INT32_MAX : lsh_quantise_scaled(thi);
     lo = lsh_wave_extreme<false>(lo);
     hi = lsh_wave_extreme<true>(hi);
     if (lane_id() == 63) { s_min[wave][c] = lo; s_max[wave][c] = hi; }
@@ -59,7 +72,7 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_minmax_kernel(const float* __re
 }
 
 // ---- pass 2: reduce the partials, derive the mixed-radix strides, pack the keys of every table ---------
-// grid (ceil(N / 256), 1, events): a hit's coordinates are read once for all tables.
+// grid (ceil(N / (256 * LSH_PK_ITEMS)), 1, events): a hit's coordinates are read once for all tables.
 // meta [n_tables, 2J+3] = lo[J], range[J], total, key_bits, overflow.
 template <int DIM>
 __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __restrict__ coords, int64_t n_hits,
@@ -82,6 +95,9 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
   __shared__ int32_t s_lo[LSH_MAX_COLS], s_hi[LSH_MAX_COLS];
   __shared__ uint32_t s_stride[LSH_MAX_COLS];
   __shared__ uint32_t s_total[LSH_MAX_COLS];  // per table
+  __shared__ float s_alpha[LSH_MAX_DIM * LSH_MAX_COLS], s_beta[LSH_MAX_COLS];  // (as in the min / max kernel)
+  for (int i = threadIdx.x; i < dim * n_cols; i += LSH_BLOCK) s_alpha[i] = alpha[i];
+  for (int i = threadIdx.x; i < n_cols; i += LSH_BLOCK) s_beta[i] = beta[i];
   // column c is reduced by the four threads 4c .. 4c+3 (n_cols <= 64)
   {
     const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
@@ -124,23 +140,37 @@ __global__ void __launch_bounds__(LSH_BLOCK) lsh_pack_kernel(const float* __rest
     }
   }
   __syncthreads();
-  const int64_t n = (int64_t)blockIdx.x * LSH_BLOCK + threadIdx.x;
-  if (n >= n_hits) return;
-  const bool valid = n < n_valid;
-  float x[LSH_MAX_DIM];
-  lsh_load_coords<DIM>(coords, valid ? n : 0, dim, x);
+  // LSH_PK_ITEMS hits per thread: the reduction above is paid once per block, and the coordinate loads of a thread
+  // are independent
+  float x[LSH_PK_ITEMS][LSH_MAX_DIM];
+#pragma unroll
+  for (int i = 0; i < LSH_PK_ITEMS; ++i) {
+    const int64_t n = ((int64_t)blockIdx.x * LSH_PK_ITEMS + i) * LSH_BLOCK + threadIdx.x;
+    lsh_load_coords<DIM>(coords, n < n_valid ? n : 0, dim, x[i]);
+  }
   for (int table = 0; table < n_tables; ++table) {
-    uint32_t key = valid ? 0u : s_total[table];
+    uint32_t key[LSH_PK_ITEMS];
+#pragma unroll
+    for (int i = 0; i < LSH_PK_ITEMS; ++i) key[i] = s_total[table];
     for (int j = 0; j < n_proj; ++j) {
       const int c = table * n_proj + j;
-      int32_t id = 0;
-      if (valid) {
-        id = lsh_quantise(lsh_dot<DIM>(x, alpha, dim, n_cols, c), beta[c], inv_w);
-        key += ((uint32_t)id - (uint32_t)s_lo[c]) * s_stride[c];
+      const float b = s_beta[c];
+      const uint32_t lo = (uint32_t)s_lo[c], stride = s_stride[c];
+#pragma unroll
+      for (int i = 0; i < LSH_PK_ITEMS; ++i) {
+        const int64_t n = ((int64_t)blockIdx.x * LSH_PK_ITEMS + i) * LSH_BLOCK + threadIdx.x;
+        const bool valid = n < n_valid;
+        const int32_t id = valid ? lsh_quantise(lsh_dot<DIM>(x[i], s_alpha, dim, n_cols, c), b, inv_w) : 0;
+        if (j == 0 && valid) key[i] = 0u;
+        if (valid) key[i] += ((uint32_t)id - lo) * stride;
+        if (ids && n < n_hits) ids[(int64_t)c * n_hits + n] = id;
       }
-      if (ids) ids[(int64_t)c * n_hits + n] = id;
     }
-    keys[(int64_t)table * n_hits + n] = (int32_t)key;
+#pragma unroll
+    for (int i = 0; i < LSH_PK_ITEMS; ++i) {
+      const int64_t n = ((int64_t)blockIdx.x * LSH_PK_ITEMS + i) * LSH_BLOCK + threadIdx.x;
+      if (n < n_hits) keys[(int64_t)table * n_hits + n] = (int32_t)key[i];
+    }
   }
 }
 
@@ -218,7 +248,7 @@ static int lsh_bucket_keys_batch(const float* coords, int n_events, int64_t n_hi
   const int64_t per_block = (int64_t)LSH_BLOCK * LSH_MM_ITEMS;
   int blocks_valid = (int)(((n_valid_dev ? n_hits : n_valid) + per_block - 1) / per_block);
   if (blocks_valid < 1) blocks_valid = 1;
-  const int blocks_all = (int)((n_hits + LSH_BLOCK - 1) / LSH_BLOCK);
+  const int blocks_all = (int)((n_hits + LSH_BLOCK * LSH_PK_ITEMS - 1) / (LSH_BLOCK * LSH_PK_ITEMS));
   LAMPA_PROF(s, "start");
   if (dim == 4) {
     hipLaunchKernelGGL(lsh_minmax_kernel<4>, dim3(blocks_valid, 1, n_events), dim3(LSH_BLOCK), 0, s, coords, n_hits,

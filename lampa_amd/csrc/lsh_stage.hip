@@ -156,23 +156,29 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       lsh_load_coords<DIM>(coords, idx < n_valid ? idx : 0, a.dim, x[k]);
     }
     __syncthreads();
-    // bucket id of item k for projection j: the chain p = fmaf(x[d], a[d], p) from 0, as everywhere in this library
-    auto bucket_id = [&](int k, int j) -> int32_t {
+    // scaled projection of item k for column j: the chain p = fmaf(x[d], a[d], p) from 0, as everywhere in this
+    // library, then (p + b) * inv_w; its bucket id is lsh_quantise_scaled of it
+    auto scaled = [&](int k, int j) -> float {
       float acc = 0.0f;
 #pragma unroll
       for (int d = 0; d < XD; ++d)
         if (DIM || d < dim) acc = __builtin_fmaf(x[k][d], s_alpha[d][j], acc);
-      return lsh_quantise(acc, s_beta[j], a.inv_w);
+      return lsh_scaled(acc, s_beta[j], a.inv_w);
     };
+    auto bucket_id = [&](int k, int j) -> int32_t { return lsh_quantise_scaled(scaled(k, j)); };
+    // extremes on the scaled projections, quantised once (the quantisation is monotone; NaNs, id INT32_MAX, are
+    // ignored by fminf / fmaxf and noted separately); items past the valid count hold hit 0, a valid hit
     for (int j = 0; j < J; ++j) {
-      int32_t lo = INT32_MAX, hi = INT32_MIN;
+      float tlo = INFINITY, thi = -INFINITY;
+      bool nan_seen = false;
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
-        const int32_t id = bucket_id(k, j);
-        const bool valid = ibase + 64 * k < n_valid;
-        lo = valid ? min(lo, id) : lo;
-        hi = valid ? max(hi, id) : hi;
+        const float t = scaled(k, j);
+        tlo = fminf(tlo, t);
+        thi = fmaxf(thi, t);
+        nan_seen = nan_seen || t != t;
       }
+      int32_t lo = lsh_quantise_scaled(tlo), hi = nan_seen ? INT32_MAX : lsh_quantise_scaled(thi);
       lo = lsh_wave_extreme<false>(lo);
       hi = lsh_wave_extreme<true>(hi);
       if (lane == 63) { s_mm[wave][2 * j] = lo; s_mm[wave][2 * j + 1] = hi; }
