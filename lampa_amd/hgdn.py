@@ -231,8 +231,7 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
     if not all([q.ndim == 4, q.shape[1] == 1, k.ndim == 4, k.shape[1] == 1, v.ndim == 4, v.shape[1] == 1,
                 beta.ndim == 3, beta.shape[1] == 1, g.ndim == 3, g.shape[1] == 1, l.ndim == 4, l.shape[1] == 1]):
         raise ValueError
-    o = _step(initial_state, q[:, 0], k[:, 0], v[:, 0], g[:, 0], l[:, 0], beta[:, 0], scale, lam_div)
-    return o.unsqueeze(1), initial_state
+    return _step(initial_state, q, k, v, g, l, beta, scale, lam_div, token_dim=True), initial_state
 
 
 def _check_chunk_shapes(T: int, K: int, V: int, L: int) -> None:
@@ -244,16 +243,18 @@ def _check_chunk_shapes(T: int, K: int, V: int, L: int) -> None:
         raise NotImplementedError("hierarchical chunk kernels: at most 4096 chunks per sequence")
 
 
-def _step(hstate: HState, q, k, v, g, l, beta, scale, lam_div) -> torch.Tensor:
+def _step(hstate: HState, q, k, v, g, l, beta, scale, lam_div, token_dim: bool = False) -> torch.Tensor:
     """``hattention_step`` (``kernel.py:577-633``) on ``[B, H, K]`` / ``[B, HV, V]`` / ``[B, HV]`` / ``[B, HV, L]``
-    slices; updates ``hstate`` in place and returns ``o [B, HV, V]``."""
-    if not all([q.ndim == 3, k.ndim == 3, v.ndim == 3, beta.ndim == 2, g.ndim == 2, l.ndim == 3,
+    slices -- or, with ``token_dim``, on the operator's own ``[B, 1, ...]`` tensors, which are the same memory when
+    contiguous (no slicing on the way to the kernel); updates ``hstate`` in place and returns ``o`` shaped like ``v``."""
+    t = 1 if token_dim else 0
+    if not all([q.ndim == 3 + t, k.ndim == 3 + t, v.ndim == 3 + t, beta.ndim == 2 + t, g.ndim == 2 + t, l.ndim == 3 + t,
                 hstate.dtype == torch.float32, q.dtype == k.dtype == v.dtype, hstate.base == 2,
                 hstate.htype == HType.WEAK, hstate.hstruct == HStruct.GDELTA]):
         raise TypeError
     require_cuda(q, k, v, g, l, beta, hstate.states)
-    B, H, K = q.shape
-    HV, V, L = v.shape[1], v.shape[2], l.shape[-1]
+    B, H, K = q.shape[0], q.shape[-2], q.shape[-1]
+    HV, V, L = v.shape[-2], v.shape[-1], l.shape[-1]
     if tuple(hstate.shape) != (B, HV, K, V, L):
         raise ValueError("Shape, dtype or device mismatch")
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
