@@ -171,14 +171,18 @@ def test_steps_from_an_empty_state_any_head_size(device):
                                           initial_state=st, output_final_state=True, use_qk_l2norm_in_kernel=True)
 
 
-def test_step_entry_point_fp32_and_odd_sizes(device):
-    # the C entry point itself: fp32 tokens, K = 24, V = 40 (not a multiple of the 16-column tiles), 9 levels, weights
-    # taken as given (lam_div = 1), recurrent-style l2norm off; ten tokens from an empty state
+@pytest.mark.parametrize("B,T,H,HV,K,V,L", [
+    (2, 10, 2, 4, 24, 40, 9),    # LDS-staged kernel, pieces of 4 columns; K below the number of row groups
+    (2, 10, 2, 4, 24, 30, 9),    # V not a multiple of 4: the register-resident kernel, partial 16-column tile
+    (2, 6, 1, 2, 100, 8, 32),    # 32 levels, two row groups
+    (130, 3, 2, 4, 64, 64, 12),  # a launch large enough for pieces of 8 columns
+])
+def test_step_entry_point_fp32_and_odd_sizes(device, B, T, H, HV, K, V, L):
+    # the C entry point itself: fp32 tokens, weights taken as given (lam_div = 1), l2norm off; T tokens from an empty state
     import ctypes
     from lampa_amd import _capi
     from lampa_amd._capi import ptr
     gen = torch.Generator().manual_seed(11)
-    B, T, H, HV, K, V, L = 2, 10, 2, 4, 24, 40, 9
     q, k = (torch.randn(B, T, H, K, generator=gen) for _ in range(2))
     v = torch.randn(B, T, HV, V, generator=gen)
     g = -0.2 * torch.rand(B, T, HV, generator=gen)
