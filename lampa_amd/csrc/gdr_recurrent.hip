@@ -1,13 +1,15 @@
-// Token-serial gated-delta-rule forward with an fp32 state held in registers (gfx950).
+// Token-serial gated-delta-rule forward with an fp32 state held in registers (gfx950). Two kernels:
 //
-// One wave owns up to 64 value columns of one (sequence, value head): lane = value column, and every lane keeps
-// the K state rows of its column in registers, so the three contractions of a step (S^T k, the rank-one update
-// and S^T q) are per-lane loops with no cross-lane traffic; k_t and q_t are loaded one element per lane,
-// normalised with a wave reduction and broadcast with v_readlane.
+// gdr_recurrent_kernel: one wave owns up to 64 value columns of one (sequence, value head): lane = value column, and
+// every lane keeps the K state rows of its column in registers, so the three contractions of a step (S^T k, the
+// rank-one update and S^T q) are per-lane loops with no cross-lane traffic; k_t and q_t are loaded one element per
+// lane, normalised with a wave reduction and broadcast with v_readlane.
+// gdr_recurrent_split_kernel (further down): 32 columns per wave, the state rows of a column split over the two halves
+// of the wave -- fewer instructions per token and wave, for launches of few waves.
 //
 // Replaces fused_recurrent_gated_delta_rule_fwd_kernel, models/hattention/gated_delta_rule_ori.py:372-464
-// (same order of operations; state layout [N, HV, K, V] fp32; grouped value heads HV >= H).  It is also the
-// fp32 mode of the chunk operator and the on-GPU cross-check of the chunk kernels.
+// (state layout [N, HV, K, V] fp32; grouped value heads HV >= H).  It is also the fp32 mode of the chunk operator and
+// the on-GPU cross-check of the chunk kernels.
 #include "gdr_common.h"
 
 // value of lane `src` (a compile-time constant) in every lane: one v_readlane into a scalar register
@@ -125,12 +127,214 @@ __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__
   }
 }
 
+// ---- the same recurrence with the state rows of a column split over the two halves of the wave ----------------------
+// One wave owns 32 value columns of one (sequence, value head): lane = (half, column), and a lane keeps KT / 2 state
+// rows of its column, so a step is half as many instructions per wave as above and V <= 32 fills the wave; the two
+// partial sums of S^T k and of S^T q meet through one cross-half exchange each. The wave is bound by instruction issue
+// (one wave per SIMD: four cycles per instruction), so everything that is not the recurrence leaves the step: k and q
+// of a group of tokens are loaded 4 elements at a time one group ahead, widened and parked in LDS (a lane reads its
+// KT / 2 values of a token with 16-byte broadcast reads instead of one cross-lane read per element), and the per-token
+// scalars (1 / |k|, scale / |q|, e^g, beta) are computed for the whole group at once, lane = token. The l2 norms are
+// applied as factors on the sums, not on the vectors. K a multiple of 4, q and k 16-byte aligned.
+// x of the lower half of the wave plus x of the upper half, in every lane (one cross-half swap, no LDS)
+__device__ __forceinline__ float rec_half_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // r[0] = lower half's, r[1] = upper half's
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <typename T>
+__device__ __forceinline__ float4 rec_load4(const T* p) {
+  if constexpr (sizeof(T) == 4) {
+    return *reinterpret_cast<const float4*>(p);
+  } else {
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    const vec4 x = *reinterpret_cast<const vec4*>(p);
+    return make_float4(GdrElem<T>::to_float(x[0]), GdrElem<T>::to_float(x[1]), GdrElem<T>::to_float(x[2]),
+                       GdrElem<T>::to_float(x[3]));
+  }
+}
+
+template <typename T, int KT>
+__global__ void __launch_bounds__(64)
+    gdr_recurrent_split_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                               const float* __restrict__ g, const float* __restrict__ beta, T* __restrict__ o,
+                               const float* __restrict__ h0, float* __restrict__ ht,
+                               const int64_t* __restrict__ cu_seqlens, int64_t t_len, int H, int HV, int K, int V,
+                               float scale, int l2norm) {
+  constexpr int RP = KT / 2;                          // state rows per lane
+  constexpr int G = 2048 / KT < 64 ? 2048 / KT : 64;  // tokens per group
+  constexpr int ROW4 = (2 * KT + 4) / 4;              // 16-byte pieces per token in LDS: k | q, padded against conflicts
+  constexpr int PPT = 2 * KT / 4;                     // 4-element pieces of k | q per token
+  constexpr int PIECES = G * PPT / 64;                // pieces per lane and group
+  constexpr int VALS = G * 32 / 64;                   // v elements per lane and group
+  static_assert((G * PPT) % 64 == 0, "group shape");
+  // two buffers of a group each; two more tokens' room behind each group, so that the reads ahead need no bound
+  // (what they return for tokens after the group is never used)
+  __shared__ float4 s_kq[2][(G + 2) * ROW4];
+  __shared__ float4 s_sc[2][G + 2];
+  __shared__ float s_v[2][(G + 2) * 32];
+  const int lane = threadIdx.x, half = lane >> 5, cl = lane & 31;
+  const int col = blockIdx.x * 32 + cl;
+  const bool active = col < V;
+  const int seq = blockIdx.y / HV, hv = blockIdx.y % HV;
+  const int h = hv / (HV / H);
+  const int64_t bos = cu_seqlens ? cu_seqlens[seq] : seq * t_len;
+  const int64_t eos = cu_seqlens ? cu_seqlens[seq + 1] : bos + t_len;
+
+  float S[RP];  // rows half * RP + r
+#pragma unroll
+  for (int r = 0; r < RP; ++r) {
+    const int i = half * RP + r;
+    S[r] = (h0 && active && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + col] : 0.0f;
+  }
+  if (bos < eos) {
+    float4 piece[PIECES];
+    float vals[VALS];
+    float g_tok = 0.0f, b_tok = 0.0f;
+    // loads of the group that starts at token t0: every address is inside the tensors (tokens past the end re-read the
+    // last one, elements past K or V the last element) and what is out of range is replaced when it is parked
+    auto fetch = [&](int64_t t0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int n = 0; n < PIECES; ++n) {
+        const int pi = lane + 64 * n, j = pi / PPT, c = 4 * (pi % PPT);
+        const int64_t t = t0 + j < eos ? t0 + j : eos - 1;
+        const int e = c < KT ? c : c - KT;
+        piece[n] = rec_load4<T>((c < KT ? k : q) + (t * H + h) * K + (e < K ? e : K - 4));
+      }
+#pragma unroll
+      for (int n = 0; n < VALS; ++n) {
+        const int vi = lane + 64 * n, j = vi / 32, cc = blockIdx.x * 32 + vi % 32;
+        const int64_t t = t0 + j < eos ? t0 + j : eos - 1;
+        vals[n] = GdrElem<T>::to_float(v[(t * HV + hv) * V + (cc < V ? cc : V - 1)]);
+      }
+      const int64_t t = t0 + lane < eos ? t0 + lane : eos - 1;
+      g_tok = g[t * HV + hv];
+      b_tok = beta[t * HV + hv];
+    };
+    // the fetched group into LDS buffer `buf`, then its per-token scalars (lane = token)
+    auto commit = [&](int buf, bool live) __attribute__((always_inline)) {
+#pragma unroll
+      for (int n = 0; n < PIECES; ++n) {
+        const int pi = lane + 64 * n, j = pi / PPT, c4 = pi % PPT;
+        const int c = 4 * c4, e = c < KT ? c : c - KT;
+        s_kq[buf][j * ROW4 + c4] = e < K ? piece[n] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      }
+#pragma unroll
+      for (int n = 0; n < VALS; ++n) s_v[buf][lane + 64 * n] = vals[n];
+      if (lane < G) {
+        float kss = 0.0f, qss = 0.0f;
+#pragma unroll
+        for (int c4 = 0; c4 < KT / 4; ++c4) {
+          const float4 a = s_kq[buf][lane * ROW4 + c4], b = s_kq[buf][lane * ROW4 + KT / 4 + c4];
+          kss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+          qss += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+        }
+        float kinv = 1.0f, qinv = 1.0f;
+        if (l2norm == GDR_L2_CHUNK) {
+          kinv = 1.0f / __fsqrt_rn(kss + 1e-6f);
+          qinv = 1.0f / __fsqrt_rn(qss + 1e-6f);
+        } else if (l2norm == GDR_L2_RECURRENT) {
+          kinv = 1.0f / (__fsqrt_rn(kss) + 1e-6f);
+          qinv = 1.0f / (__fsqrt_rn(qss) + 1e-6f);
+        }
+        // a token past the end is a step that changes nothing (d = 0, decay 1), so the steps need no branch
+        s_sc[buf][lane] = live ? make_float4(kinv, qinv * scale, expf(g_tok), b_tok) : make_float4(0.0f, 0.0f, 1.0f, 0.0f);
+      }
+    };
+    // a token's operands: its scalars, this lane's RP elements of k and of q, its v
+    struct Operands {
+      float4 sc, kk[RP / 4], qq[RP / 4];
+      float v;
+    };
+    auto read_token = [&](int buf, int j, Operands& x) __attribute__((always_inline)) {
+      x.sc = s_sc[buf][j];  // 1 / |k|, scale / |q|, e^g, beta
+      const float4* kr = &s_kq[buf][j * ROW4 + half * (RP / 4)];
+#pragma unroll
+      for (int r4 = 0; r4 < RP / 4; ++r4) {
+        x.kk[r4] = kr[r4];
+        x.qq[r4] = kr[KT / 4 + r4];
+      }
+      x.v = s_v[buf][j * 32 + cl];
+    };
+    fetch(bos);
+    commit(0, bos + lane < eos);
+    int buf = 0;
+    for (int64_t t0 = bos; t0 < eos; t0 += G, buf ^= 1) {
+      const bool more = t0 + G < eos;
+      if (more) fetch(t0 + G);
+      const int n_tok = eos - t0 < G ? (int)(eos - t0) : G;
+      // two tokens per round on two operand sets: a token's operands are requested before the arithmetic of the token
+      // before it starts, so their LDS latency hides behind it. The token after the last of an odd count is a step
+      // that changes nothing.
+      auto step = [&](const Operands& x, int64_t t) __attribute__((always_inline)) {
+        float kk[RP], qq[RP];
+#pragma unroll
+        for (int r4 = 0; r4 < RP / 4; ++r4) {
+          kk[4 * r4] = x.kk[r4].x; kk[4 * r4 + 1] = x.kk[r4].y; kk[4 * r4 + 2] = x.kk[r4].z; kk[4 * r4 + 3] = x.kk[r4].w;
+          qq[4 * r4] = x.qq[r4].x; qq[4 * r4 + 1] = x.qq[r4].y; qq[4 * r4 + 2] = x.qq[r4].z; qq[4 * r4 + 3] = x.qq[r4].w;
+        }
+        float dot4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int r = 0; r < RP; ++r) dot4[r & 3] = __builtin_fmaf(S[r], kk[r], dot4[r & 3]);
+        const float dot = rec_half_sum((dot4[0] + dot4[1]) + (dot4[2] + dot4[3]));
+        // S <- e^g S, then d = beta (v - S^T k), S <- S + k d^T, o = S^T q, with k = k_raw / |k|
+        const float4 sc = x.sc;
+        const float d = sc.w * (x.v - sc.z * sc.x * dot);
+        const float dk = d * sc.x;
+        float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int r = 0; r < RP; ++r) {
+          S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
+          out4[r & 3] = __builtin_fmaf(S[r], qq[r], out4[r & 3]);
+        }
+        const float out = rec_half_sum((out4[0] + out4[1]) + (out4[2] + out4[3]));
+        if (active && half == 0 && t < eos) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out * sc.y);
+      };
+      Operands xa, xb;
+      read_token(buf, 0, xa);
+      for (int j = 0; j < n_tok; j += 2) {
+        read_token(buf, j + 1, xb);
+        __builtin_amdgcn_sched_barrier(0);
+        step(xa, t0 + j);
+        read_token(buf, j + 2, xa);
+        __builtin_amdgcn_sched_barrier(0);
+        step(xb, t0 + j + 1);
+      }
+      if (more) commit(buf ^ 1, t0 + G + lane < eos);
+    }
+  }
+  if (ht && active) {
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      const int i = half * RP + r;
+      if (i < K) ht[(((int64_t)seq * HV + hv) * K + i) * V + col] = S[r];
+    }
+  }
+}
+
 template <typename T>
 static int gdr_recurrent_launch(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                 void* o, const float* h0, float* ht, const int64_t* cu, int n_seq, int64_t t_len,
                                 int H, int HV, int K, int V, float scale, int l2norm, hipStream_t s) {
-  const dim3 grid((V + 63) / 64, n_seq * HV), block(64);
   LAMPA_PROF(s, "start");
+  // the split form while its waves (twice as many) still find a SIMD each or nearly so
+  const int64_t split_waves = (int64_t)((V + 31) / 32) * n_seq * HV;
+  if (K % 4 == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) == 0 &&
+      split_waves <= 2048) {
+    const dim3 grid2((V + 31) / 32, n_seq * HV);
+#define GDR_REC_SPLIT(KT)                                                                                          \
+  hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT>), grid2, dim3(64), 0, s, (const T*)q, (const T*)k,         \
+                     (const T*)v, g, beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm)
+    if (K <= 16) GDR_REC_SPLIT(16);
+    else if (K <= 32) GDR_REC_SPLIT(32);
+    else if (K <= 64) GDR_REC_SPLIT(64);
+    else GDR_REC_SPLIT(128);
+#undef GDR_REC_SPLIT
+    LAMPA_PROF(s, "gdr_recurrent_split_kernel");
+    return lampa_launch_status();
+  }
+  const dim3 grid((V + 63) / 64, n_seq * HV), block(64);
 #define GDR_REC_CASE(KT)                                                                                         \
   hipLaunchKernelGGL((gdr_recurrent_kernel<T, KT>), grid, block, 0, s, (const T*)q, (const T*)k, (const T*)v, g, \
                      beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm)

@@ -32,8 +32,11 @@ def _to(dev, *xs):
 
 
 # ------------------------------------------------------------------------------------------------- token-serial
-@pytest.mark.parametrize("K,V,T", [(32, 32, 700), (64, 64, 300), (128, 128, 130), (16, 32, 257)])
+@pytest.mark.parametrize("K,V,T", [(32, 32, 700), (64, 64, 300), (128, 128, 130), (16, 32, 257), (20, 40, 131),
+                                   (30, 70, 90), (8, 8, 65), (100, 24, 64)])
 def test_recurrent_fp32_matches_oracle(device, K, V, T):
+    # K a multiple of 4: the split-wave kernel (groups of 64 / 32 / 16 tokens: T covers whole groups, a partial one, odd
+    # counts); K = 30: the lane-per-column kernel
     q, k, v, g, beta = synth.gdr_inputs(2, T, 3, K, V, torch.float32, seed=K + T, g_scale=0.1)
     h0 = torch.randn(2, 3, K, V, generator=torch.Generator().manual_seed(1))
     for l2, flag in ((og.L2_NONE, False), (og.L2_RECURRENT, True)):
@@ -53,6 +56,28 @@ def test_config0_fp32_plumbing(device):
     assert _errors(o2, want_o)[0] <= FP32_TOL and _errors(s2, want_s)[0] <= FP32_TOL
     with pytest.raises(AssertionError):
         gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta))
+
+
+def test_recurrent_many_short_sequences_both_kernels(device):
+    # 700 sequences x 4 value heads of 0 .. 9 tokens: more waves than the split-wave kernel takes (the lane-per-column
+    # kernel runs); the first 100 sequences alone go to the split-wave kernel; same oracle
+    gen = torch.Generator().manual_seed(8)
+    lens = torch.randint(0, 10, (700,), generator=gen)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), torch.cumsum(lens, 0)])
+    T, H, HV, K, V = int(cu[-1]), 2, 4, 32, 32
+    q, k = (torch.randn(1, T, H, K, generator=gen) for _ in range(2))
+    v = torch.randn(1, T, HV, V, generator=gen)
+    g = -torch.rand(1, T, HV, generator=gen) * 0.3
+    beta = torch.rand(1, T, HV, generator=gen)
+    h0 = torch.randn(700, HV, K, V, generator=gen)
+    for n in (700, 100):
+        Tn = int(cu[n])
+        args = [x[:, :Tn] for x in (q, k, v, g, beta)]
+        want_o, want_s = og.recurrent_c(*args, initial_state=h0[:n], cu_seqlens=cu[:n + 1], l2=og.L2_RECURRENT)
+        o, s = gd.fused_recurrent_gated_delta_rule(*_to(device, *args), initial_state=h0[:n].to(device),
+                                                   output_final_state=True, cu_seqlens=cu[:n + 1].to(device),
+                                                   use_qk_l2norm_in_kernel=True)
+        assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL, n
 
 
 def test_recurrent_varlen_gva_bf16(device):
