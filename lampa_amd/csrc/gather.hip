@@ -13,30 +13,45 @@ __device__ __forceinline__ int64_t gs_index(const void* idx, int64_t i) {
   return (int64_t)reinterpret_cast<const IdxT*>(idx)[i];
 }
 
-// One thread moves one VEC-byte piece of a row. dst[s, n, :] = src[s or 0, idx[s, n], :] when GATHER,
-// dst[s, idx[s, n], :] = src[s, n, :] otherwise.
+// One thread moves GS_UNROLL VEC-byte pieces of rows, a block's worth apart: all their indices are loaded first, then
+// all their source pieces, then they are stored, so a thread has GS_UNROLL independent loads in flight (the kernel is a
+// chain of three dependent memory operations per piece and is bound by how many bytes the chip has in flight, not by
+// the bus). dst[s, n, :] = src[s or 0, idx[s, n], :] when GATHER, dst[s, idx[s, n], :] = src[s, n, :] otherwise.
+#define GS_UNROLL 4
 template <typename VecT, typename IdxT, bool GATHER>
 __global__ void __launch_bounds__(GS_BLOCK) gs_rows_kernel(const char* __restrict__ src, int64_t src_seg_stride,
                                                           int src_segments, int group, const void* __restrict__ idx, int64_t n,
                                                           int64_t n_src, int vec_per_row, char* __restrict__ dst) {
   const int seg = blockIdx.y;
-  const int64_t item = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
-  const int64_t row = item / vec_per_row;
-  const int piece = (int)(item - row * vec_per_row);
-  if (row >= n) return;
-  const int64_t other = gs_index<IdxT>(idx, (int64_t)seg * n + row);
   const int64_t limit = GATHER ? n_src : n;
   const int64_t row_bytes = (int64_t)vec_per_row * (int64_t)sizeof(VecT);
-  if (other < 0 || other >= limit) {
+  const char* src_seg = src + ((seg / group) % src_segments) * src_seg_stride;
+  char* dst_seg = dst + (int64_t)seg * n * row_bytes;
+  int64_t row[GS_UNROLL], other[GS_UNROLL];
+  int piece[GS_UNROLL];
+  bool live[GS_UNROLL], inside[GS_UNROLL];
+#pragma unroll
+  for (int u = 0; u < GS_UNROLL; ++u) {
+    const int64_t item = ((int64_t)blockIdx.x * GS_UNROLL + u) * GS_BLOCK + threadIdx.x;
+    row[u] = item / vec_per_row;
+    piece[u] = (int)(item - row[u] * vec_per_row);
+    live[u] = row[u] < n;
+    other[u] = live[u] ? gs_index<IdxT>(idx, (int64_t)seg * n + row[u]) : 0;
+  }
+  VecT val[GS_UNROLL];
+#pragma unroll
+  for (int u = 0; u < GS_UNROLL; ++u) {
     // an index outside the source: a gathered row reads as zeros (never as whatever the output buffer held), a
     // scattered row is dropped
-    if (GATHER) reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + row) * row_bytes)[piece] = VecT{};
-    return;
+    inside[u] = live[u] && other[u] >= 0 && other[u] < limit;
+    const int64_t from = GATHER ? other[u] : row[u];
+    val[u] = inside[u] ? reinterpret_cast<const VecT*>(src_seg + from * row_bytes)[piece[u]] : VecT{};
   }
-  const int64_t from = GATHER ? other : row, to = GATHER ? row : other;
-  const VecT* s = reinterpret_cast<const VecT*>(src + ((seg / group) % src_segments) * src_seg_stride + from * row_bytes) + piece;
-  VecT* d = reinterpret_cast<VecT*>(dst + ((int64_t)seg * n + to) * row_bytes) + piece;
-  *d = *s;
+#pragma unroll
+  for (int u = 0; u < GS_UNROLL; ++u) {
+    const int64_t to = GATHER ? row[u] : other[u];
+    if (inside[u] || (GATHER && live[u])) reinterpret_cast<VecT*>(dst_seg + to * row_bytes)[piece[u]] = val[u];
+  }
 }
 
 template <typename IdxT>
@@ -59,7 +74,8 @@ static int gs_launch(const void* src, int64_t src_seg_stride, int src_segments, 
   const int vec = a16 ? 16 : (a4 ? 4 : 1);
   const int vec_per_row = (int)(row_bytes / vec);
   const int64_t items = n * vec_per_row;
-  const dim3 grid((unsigned)((items + GS_BLOCK - 1) / GS_BLOCK), n_segments), block(GS_BLOCK);
+  const int64_t per_block = (int64_t)GS_BLOCK * GS_UNROLL;
+  const dim3 grid((unsigned)((items + per_block - 1) / per_block), n_segments), block(GS_BLOCK);
   LAMPA_PROF(s, "start");
   if (vec == 16)
     hipLaunchKernelGGL((gs_rows_kernel<uint4, IdxT, GATHER>), grid, block, 0, s, (const char*)src, src_seg_stride, src_segments,
