@@ -18,8 +18,8 @@ All three branches of the operator are here: outputs only (``hattention_kernel``
 states (``hattention_prefill``, ``kernel.py:467-575``: the whole chunks through the chunk kernels, the remaining
 tokens one by one) and the single-token step on an ``HState`` (``hattention_step``, ``kernel.py:577-633``).
 
-Differences a caller can observe: forward only; the chunk kernels take K = 64 and V in {64, 128} (the single-token step
-takes any K and V, up to 32 levels); ``HState.counts`` lives on the host (the reference keeps it on the device and synchronises
+Differences a caller can observe: forward only; the chunk kernels are built for K = 64 and V in {64, 128}, smaller
+heads are zero-padded to those, larger ones are refused (the single-token step takes any K and V, up to 32 levels); ``HState.counts`` lives on the host (the reference keeps it on the device and synchronises
 on every comparison, ``recurrent.py:44-56``); the step computes its output from the fp32 states, the reference rounds
 them to the output type first (``kernel.py:628-631``).
 """
@@ -209,7 +209,8 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
         _check_chunk_shapes(T, K, V, L)
         if T % 64 != 0:  # chunkwise_hgdn.py:598-601
             raise ValueError(f"T={T} and BT=64")
-        return _ForwardOnly.apply(q, k, v, g, l, beta, scale, lam_div), None
+        pq, pk, pv = _pad_heads(q, k, v)
+        return _ForwardOnly.apply(pq, pk, pv, g, l, beta, scale, lam_div)[..., :V].contiguous(), None
     if initial_state is None:  # hattention_prefill, kernel.py:467-575
         require_cuda(q, k, v, g, l, beta)
         hstate = HState(2, HType.WEAK, HStruct.GDELTA, (B, HV, K, V, L), torch.float32, q.device)
@@ -218,8 +219,13 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
         if T0:
             _check_chunk_shapes(T0, K, V, L)
             cut = lambda x: x[:, :T0]
-            o[:, :T0] = _ForwardOnly.apply(cut(q), cut(k), cut(v), cut(g), cut(l), cut(beta), scale, lam_div,
-                                           hstate.states)
+            pq, pk, pv = _pad_heads(cut(q), cut(k), cut(v))
+            padded = pq.shape[-1] != K or pv.shape[-1] != V
+            states = (torch.zeros(B, HV, pq.shape[-1], pv.shape[-1], L, dtype=torch.float32, device=q.device)
+                      if padded else hstate.states)
+            o[:, :T0] = _ForwardOnly.apply(pq, pk, pv, cut(g), cut(l), cut(beta), scale, lam_div, states)[..., :V]
+            if padded:  # (the padded rows and columns of the states are zero)
+                hstate.states = states[:, :, :K, :V].contiguous()
             # counts after T0 tokens (kernel.py:451-462): the last token alone in level 0, level l > 0 holds 2^(l-1)
             # tokens iff that bit of T0 - 1 is set
             hstate._counts[0] = 1
@@ -234,9 +240,21 @@ def chunk_h_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
     return _step(initial_state, q, k, v, g, l, beta, scale, lam_div, token_dim=True), initial_state
 
 
+def _pad_heads(q, k, v):
+    """The chunk kernels are built for K = 64 and V in {64, 128}; smaller heads are zero-padded along the head
+    dimension: zero columns of k and q add nothing to k k^T, q k^T, q S or the norms, zero columns of v give zero
+    columns of every level state and of o, so the padded problem contains the original one exactly (`scale` is fixed
+    from the original K by the caller)."""
+    K, V = q.shape[-1], v.shape[-1]
+    Kp, Vp = 64, (64 if V <= 64 else 128)
+    pad = torch.nn.functional.pad
+    return (q if K == Kp else pad(q, (0, Kp - K)), k if K == Kp else pad(k, (0, Kp - K)),
+            v if V == Vp else pad(v, (0, Vp - V)))
+
+
 def _check_chunk_shapes(T: int, K: int, V: int, L: int) -> None:
-    if K != 64 or V not in (64, 128):
-        raise NotImplementedError("hierarchical chunk kernels: K = 64 and V in {64, 128} only")
+    if K > 64 or V > 128:
+        raise NotImplementedError("hierarchical chunk kernels: K <= 64 and V <= 128 only")
     if num_levels(T) > L:  # chunkwise_hgdn.py:718-721
         raise ValueError
     if (T // 64) > 4096:

@@ -133,6 +133,25 @@ def test_prefill_returns_the_level_states(device, T, cps):
     assert st.states.shape == (2, 2, 64, 64, lam.shape[-1]) and st.states.dtype == torch.float32
 
 
+@pytest.mark.parametrize("K,V,T", [(16, 32, 640), (32, 32, 300), (48, 96, 256), (64, 40, 200)])
+def test_small_heads_are_padded(device, K, V, T):
+    # head sizes below the built ones (the reference layer's d_k = 16, d_v = 32): outputs alone (whole chunks only) and
+    # the prefill with ragged T, its level states in the caller's K x V
+    q, k, v, g, beta, lam = _inputs(2, T, 2, K, V, torch.bfloat16, seed=K + V, HV=4, g_scale=0.3, L=hgdn.num_levels(T) + 1)
+    scale = K ** -0.5
+    want_o, want_s, want_c = oh.recurrent_c_state(q, k, v, g, beta, lam / scale, scale=scale)
+    d = [x.to(device) for x in (q, k, v, g, lam, beta)]
+    o, st = hgdn.chunk_h_gated_delta_rule(*d, output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o.shape == v.shape and st.states.shape == (2, 4, K, V, lam.shape[-1])
+    max_abs, mean_rel = _errors(o, want_o)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"o: {max_abs:.3e} {mean_rel:.3e}"
+    max_abs, mean_rel = _state_errors(st, want_s, want_c)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, f"states: {max_abs:.3e} {mean_rel:.3e}"
+    if T % 64 == 0:
+        o2, none = hgdn.chunk_h_gated_delta_rule(*d, use_qk_l2norm_in_kernel=True)
+        assert none is None and torch.equal(o2, o)
+
+
 def test_steps_continue_a_prefill(device):
     # 256 tokens through the chunk kernels, then 70 single-token calls with the returned state: one run of 326 tokens
     T0, T1 = 256, 70
