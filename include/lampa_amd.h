@@ -244,6 +244,21 @@ int lampa_gdr_recurrent_fwd(const void* q, const void* k, const void* v, const f
                             const float* h0, float* ht, const int64_t* cu_seqlens, int n_seq, int64_t t_len, int H,
                             int HV, int K, int V, int dtype, float scale, int l2norm, void* stream);
 
+/* The same operator (gated_delta_rule_ori.py:372-520) for a few long sequences, which one or two wavefronts each would
+ * leave the GPU idle with: the caller cuts every sequence into segments and they run in parallel -- every segment's
+ * affine map of its initial state, a short serial pass over the maps, then every segment again from its true initial
+ * state; fp32 throughout, the same results up to fp32 rounding.
+ * cu_seg: device int64 [n_seg+1] token offsets of the segments (every sequence boundary among them; an empty sequence
+ * keeps one empty segment); seq_seg0: device int32 [n_seq+1], first segment of every sequence; seg_out: device int32
+ * [n_seg], the sequence whose last segment this is, else -1. K and V multiples of 4, K <= 128, q and k 16-byte aligned
+ * (LAMPA_ERR_UNSUPPORTED otherwise). workspace: lampa_gdr_recurrent_segmented_workspace_bytes(n_seg, HV, K, V). */
+int64_t lampa_gdr_recurrent_segmented_workspace_bytes(int n_seg, int HV, int K, int V);
+int lampa_gdr_recurrent_segmented_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                      void* o, const float* h0, float* ht, const int64_t* cu_seg,
+                                      const int32_t* seq_seg0, const int32_t* seg_out, int n_seq, int n_seg, int H,
+                                      int HV, int K, int V, int dtype, float scale, int l2norm, void* workspace,
+                                      int64_t workspace_bytes, void* stream);
+
 /* Chunk / segment tables of the chunkwise forward, built on the host from the sequence boundaries.
  * Replaces prepare_chunk_indices / prepare_chunk_offsets (models/hattention/index.py:69-83).
  * cu_seqlens_host: int64 [n_seq+1]; chunks_per_segment: length of a segment of the split-sequence scan in

@@ -155,15 +155,19 @@ __device__ __forceinline__ float4 rec_load4(const T* p) {
   }
 }
 
-template <typename T, int KT>
+// COMPOSITE: the affine map of the sequence instead of its outputs. The state of a gated delta sequence is affine in
+// the state it starts from, S_end = M S_0 + N: the wave's columns are columns of [M | N] (V = K + the value width),
+// started from [I | 0], the M columns see v = 0; nothing is written but ht (fp32 [n_seq, HV, K, V]). ht_map (nullable)
+// gives the row of ht that a sequence's final state goes to (negative: not stored).
+template <typename T, int KT, bool COMPOSITE>
 __global__ void __launch_bounds__(64)
     gdr_recurrent_split_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                const float* __restrict__ g, const float* __restrict__ beta, T* __restrict__ o,
                                const float* __restrict__ h0, float* __restrict__ ht,
                                const int64_t* __restrict__ cu_seqlens, int64_t t_len, int H, int HV, int K, int V,
-                               float scale, int l2norm) {
+                               float scale, int l2norm, const int32_t* __restrict__ ht_map) {
   constexpr int RP = KT / 2;                          // state rows per lane
-  constexpr int G = 2048 / KT < 64 ? 2048 / KT : 64;  // tokens per group
+  constexpr int G = 1024 / KT < 64 ? 1024 / KT : 64;  // tokens per group (LDS for one wave per SIMD of a CU)
   constexpr int ROW4 = (2 * KT + 4) / 4;              // 16-byte pieces per token in LDS: k | q, padded against conflicts
   constexpr int PPT = 2 * KT / 4;                     // 4-element pieces of k | q per token
   constexpr int PIECES = G * PPT / 64;                // pieces per lane and group
@@ -182,11 +186,14 @@ __global__ void __launch_bounds__(64)
   const int64_t bos = cu_seqlens ? cu_seqlens[seq] : seq * t_len;
   const int64_t eos = cu_seqlens ? cu_seqlens[seq + 1] : bos + t_len;
 
+  const int v_dim = COMPOSITE ? V - K : V;   // width of a row of v
+  const int v_col = COMPOSITE ? col - K : col;  // this lane's column of v (negative: an M column, v = 0)
   float S[RP];  // rows half * RP + r
 #pragma unroll
   for (int r = 0; r < RP; ++r) {
     const int i = half * RP + r;
-    S[r] = (h0 && active && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + col] : 0.0f;
+    if constexpr (COMPOSITE) S[r] = (i == col && col < K) ? 1.0f : 0.0f;
+    else S[r] = (h0 && active && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + col] : 0.0f;
   }
   if (bos < eos) {
     float4 piece[PIECES];
@@ -200,13 +207,15 @@ __global__ void __launch_bounds__(64)
         const int pi = lane + 64 * n, j = pi / PPT, c = 4 * (pi % PPT);
         const int64_t t = t0 + j < eos ? t0 + j : eos - 1;
         const int e = c < KT ? c : c - KT;
-        piece[n] = rec_load4<T>((c < KT ? k : q) + (t * H + h) * K + (e < K ? e : K - 4));
+        if (COMPOSITE && c >= KT) piece[n] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);  // (q is not used)
+        else piece[n] = rec_load4<T>((c < KT ? k : q) + (t * H + h) * K + (e < K ? e : K - 4));
       }
 #pragma unroll
       for (int n = 0; n < VALS; ++n) {
-        const int vi = lane + 64 * n, j = vi / 32, cc = blockIdx.x * 32 + vi % 32;
+        const int vi = lane + 64 * n, j = vi / 32;
+        const int cc = (int)blockIdx.x * 32 + vi % 32 - (COMPOSITE ? K : 0);
         const int64_t t = t0 + j < eos ? t0 + j : eos - 1;
-        vals[n] = GdrElem<T>::to_float(v[(t * HV + hv) * V + (cc < V ? cc : V - 1)]);
+        vals[n] = GdrElem<T>::to_float(v[(t * HV + hv) * v_dim + max(0, min(cc, v_dim - 1))]);
       }
       const int64_t t = t0 + lane < eos ? t0 + lane : eos - 1;
       g_tok = g[t * HV + hv];
@@ -221,7 +230,10 @@ __global__ void __launch_bounds__(64)
         s_kq[buf][j * ROW4 + c4] = e < K ? piece[n] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
       }
 #pragma unroll
-      for (int n = 0; n < VALS; ++n) s_v[buf][lane + 64 * n] = vals[n];
+      for (int n = 0; n < VALS; ++n) {
+        const int cc = (int)blockIdx.x * 32 + (lane + 64 * n) % 32 - (COMPOSITE ? K : 0);
+        s_v[buf][lane + 64 * n] = (COMPOSITE && cc < 0) ? 0.0f : vals[n];
+      }
       if (lane < G) {
         float kss = 0.0f, qss = 0.0f;
 #pragma unroll
@@ -282,14 +294,19 @@ __global__ void __launch_bounds__(64)
         const float4 sc = x.sc;
         const float d = sc.w * (x.v - sc.z * sc.x * dot);
         const float dk = d * sc.x;
-        float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (COMPOSITE) {
 #pragma unroll
-        for (int r = 0; r < RP; ++r) {
-          S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
-          out4[r & 3] = __builtin_fmaf(S[r], qq[r], out4[r & 3]);
+          for (int r = 0; r < RP; ++r) S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
+        } else {
+          float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int r = 0; r < RP; ++r) {
+            S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
+            out4[r & 3] = __builtin_fmaf(S[r], qq[r], out4[r & 3]);
+          }
+          const float out = rec_half_sum((out4[0] + out4[1]) + (out4[2] + out4[3]));
+          if (active && half == 0 && t < eos) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out * sc.y);
         }
-        const float out = rec_half_sum((out4[0] + out4[1]) + (out4[2] + out4[3]));
-        if (active && half == 0 && t < eos) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out * sc.y);
       };
       Operands xa, xb;
       read_token(buf, 0, xa);
@@ -304,11 +321,12 @@ __global__ void __launch_bounds__(64)
       if (more) commit(buf ^ 1, t0 + G + lane < eos);
     }
   }
-  if (ht && active) {
+  const int out_row = ht_map ? ht_map[seq] : seq;
+  if (ht && active && out_row >= 0) {
 #pragma unroll
     for (int r = 0; r < RP; ++r) {
       const int i = half * RP + r;
-      if (i < K) ht[(((int64_t)seq * HV + hv) * K + i) * V + col] = S[r];
+      if (i < K) ht[(((int64_t)out_row * HV + hv) * K + i) * V + col] = S[r];
     }
   }
 }
@@ -316,7 +334,8 @@ __global__ void __launch_bounds__(64)
 template <typename T>
 static int gdr_recurrent_launch(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                 void* o, const float* h0, float* ht, const int64_t* cu, int n_seq, int64_t t_len,
-                                int H, int HV, int K, int V, float scale, int l2norm, hipStream_t s) {
+                                int H, int HV, int K, int V, float scale, int l2norm, hipStream_t s,
+                                const int32_t* ht_map = nullptr) {
   LAMPA_PROF(s, "start");
   // the split form while its waves (twice as many) still find a SIMD each or nearly so
   const int64_t split_waves = (int64_t)((V + 31) / 32) * n_seq * HV;
@@ -324,8 +343,8 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
       split_waves <= 2048) {
     const dim3 grid2((V + 31) / 32, n_seq * HV);
 #define GDR_REC_SPLIT(KT)                                                                                          \
-  hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT>), grid2, dim3(64), 0, s, (const T*)q, (const T*)k,         \
-                     (const T*)v, g, beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm)
+  hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false>), grid2, dim3(64), 0, s, (const T*)q, (const T*)k,  \
+                     (const T*)v, g, beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm, ht_map)
     if (K <= 16) GDR_REC_SPLIT(16);
     else if (K <= 32) GDR_REC_SPLIT(32);
     else if (K <= 64) GDR_REC_SPLIT(64);
@@ -344,6 +363,203 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
 #undef GDR_REC_CASE
   LAMPA_PROF(s, "gdr_recurrent_kernel");
   return lampa_launch_status();
+}
+
+// ---- long sequences in parallel ---------------------------------------------------------------------------------
+// A token-serial kernel gives a (sequence, head) to one or two waves, so a few long sequences leave the chip idle. The
+// state a run of tokens ends with is affine in the state it starts from, so the sequences are cut into segments:
+//   A  every segment's map [M | N] from [I | 0]            (gdr_recurrent_split_kernel<COMPOSITE>, K + V columns)
+//   S  S_{p+1} = M_p S_p + N_p over a sequence's segments  (gdr_segment_scan_kernel, serial, small)
+//   B  every segment again from the state it really starts with, writing o (the plain kernel, segments as sequences)
+// all in fp32: the same function as the token loop up to fp32 rounding.
+
+// 32 columns of the state per workgroup (lane = column, 8 row groups); mn [n_seg, HV, K, K + V], sinit [n_seg, HV, K, V].
+// A step is short (KT / 8 rows x KT multiply-adds per thread), so what counts is that nothing serial is left in it but
+// that: M_p is loaded with 16-byte accesses into registers DEPTH segments ahead (its 1 - 2 us of memory latency would
+// otherwise be paid once per segment), parked in LDS, and every thread reads the rows it needs from there as
+// broadcasts; loop bounds are compile-time (K is padded to KT with zeros in LDS). LDS: M [KT][KT + 4] | S [KT][33].
+template <int KT, int DEPTH>
+__global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __restrict__ mn, const float* __restrict__ h0,
+                                                              const int32_t* __restrict__ seq_seg0, int HV, int K, int V,
+                                                              float* __restrict__ sinit) {
+  constexpr int MS = KT + 4;             // row stride of M in LDS (floats)
+  constexpr int K4 = KT / 4;             // 16-byte pieces per row of M
+  constexpr int RPB = 256 / K4 < KT ? 256 / K4 : KT;  // rows of M that the workgroup loads at once
+  constexpr int MREGS = (KT + RPB - 1) / RPB;         // such batches = pieces per thread
+  constexpr int NR = KT / 8;                          // rows of the new column per thread (rg, rg + 8, ...)
+  static_assert(KT % 8 == 0, "eight row groups");
+  extern __shared__ float4 s_scan4[];
+  float* s_M = reinterpret_cast<float*>(s_scan4);
+  float* s_S = s_M + KT * MS;
+  const int tid = threadIdx.x, c = tid & 31, rg = tid >> 5;
+  const int seq = blockIdx.y, hv = blockIdx.z;
+  const int col = blockIdx.x * 32 + c;
+  const bool active = col < V;
+  const int colc = active ? col : V - 1;  // (idle lanes shadow the last column and store nothing)
+#pragma unroll
+  for (int n = 0; n < NR; ++n) {
+    const int i = rg + 8 * n;
+    s_S[i * 33 + c] = (h0 && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + colc] : 0.0f;
+  }
+  const int p0 = seq_seg0[seq], p1 = seq_seg0[seq + 1];
+  const int W = K + V;
+  const int my_row = tid / K4, my_c4 = tid % K4;
+  const bool loader = my_row < RPB;
+  float4 mreg[DEPTH][MREGS];
+  float nreg[DEPTH][NR];
+  // M_p and this thread's entries of N_p into register set `slot` (zeros past K). Every step issues the same memory
+  // operations (a segment index past the end is clamped: its loads are never used), so that the waits the compiler
+  // places count exactly and the loads issued ahead stay in flight across the steps.
+  auto fetch = [&](int p, int slot) __attribute__((always_inline)) {
+    p = min(p, p1 - 1);
+    const float* M = mn + ((int64_t)p * HV + hv) * K * W;
+    // (unconditional loads from clamped addresses; what lies past K is replaced by zero when the values are used: a
+    // branch or a select at the load would make the wave wait for it at once)
+#pragma unroll
+    for (int u = 0; u < MREGS; ++u)
+      mreg[slot][u] = *reinterpret_cast<const float4*>(M + (int64_t)min(u * RPB + my_row, K - 1) * W + min(4 * my_c4, K - 4));
+#pragma unroll
+    for (int n = 0; n < NR; ++n) nreg[slot][n] = M[(int64_t)min(rg + 8 * n, K - 1) * W + K + colc];
+  };
+  // the state segment p starts from. Every lane stores every time (a lane past V or a row past K repeats the last
+  // column's / row's store with the same value): a store under a condition becomes a branch, and then the compiler can
+  // no longer count the memory operations in flight and waits for the loads issued ahead much too early.
+  auto store_start = [&](int p) __attribute__((always_inline)) {
+    float* out = sinit + ((int64_t)p * HV + hv) * K * V;
+#pragma unroll
+    for (int n = 0; n < NR; ++n) {
+      const int i = min(rg + 8 * n, K - 1);
+      out[(int64_t)i * V + colc] = s_S[i * 33 + c];
+    }
+  };
+  // one step: the state segment p starts from is stored, then S <- M_p S + N_p from register set `slot`, which is then
+  // loaded again for segment p + DEPTH
+  auto advance = [&](int p, int slot) __attribute__((always_inline)) {
+    store_start(p);
+#pragma unroll
+    for (int u = 0; u < MREGS; ++u) {
+      const int i = u * RPB + my_row;
+      const bool inside = i < K && 4 * my_c4 < K;
+      if (loader && i < KT)
+        *reinterpret_cast<float4*>(s_M + i * MS + 4 * my_c4) = inside ? mreg[slot][u] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    float acc[NR];
+#pragma unroll
+    for (int n = 0; n < NR; ++n) acc[n] = rg + 8 * n < K ? nreg[slot][n] : 0.0f;
+    lds_barrier();  // M_p is in LDS (an LDS-only barrier: the loads issued ahead stay in flight)
+    fetch(p + DEPTH, slot);
+#pragma unroll 2
+    for (int l0 = 0; l0 < KT; l0 += 4) {
+      const float s0 = s_S[l0 * 33 + c], s1 = s_S[(l0 + 1) * 33 + c], s2 = s_S[(l0 + 2) * 33 + c],
+                  s3 = s_S[(l0 + 3) * 33 + c];
+#pragma unroll
+      for (int n = 0; n < NR; ++n) {
+        // (rows rg + 8 n, n < NR, all lie below KT: no bound, a bound would put every read into a branch of its own)
+        const float4 m = *reinterpret_cast<const float4*>(s_M + (rg + 8 * n) * MS + l0);
+        acc[n] = __builtin_fmaf(m.w, s3, __builtin_fmaf(m.z, s2, __builtin_fmaf(m.y, s1, __builtin_fmaf(m.x, s0, acc[n]))));
+      }
+    }
+    lds_barrier();  // every thread has read the old column and M_p
+#pragma unroll
+    for (int n = 0; n < NR; ++n) s_S[(rg + 8 * n) * 33 + c] = acc[n];
+    lds_barrier();
+  };
+  if (p0 >= p1) return;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) fetch(p0 + d, d);
+  __syncthreads();
+  int p = p0;
+  for (; p + DEPTH < p1; p += DEPTH) {  // DEPTH steps on fixed register sets (no moves: a move would wait for its load)
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) advance(p + d, d);
+  }
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (p + d + 1 < p1) advance(p + d, d);
+  store_start(p1 - 1);
+}
+
+template <typename T>
+static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                   void* o, const float* h0, float* ht, const int64_t* cu_seg,
+                                   const int32_t* seq_seg0, const int32_t* seg_out, int n_seq, int n_seg, int H, int HV,
+                                   int K, int V, float scale, int l2norm, float* mn, float* sinit, hipStream_t s) {
+  static bool attr_set[64] = {};  // per device: the widest scan's dynamic LDS limit (a repeated set is harmless)
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
+  if (!attr_set[dev]) {
+    if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (128 * 132 + 128 * 33) * (int)sizeof(float)) != hipSuccess)
+      return LAMPA_ERR_LAUNCH;
+    attr_set[dev] = true;
+  }
+  LAMPA_PROF(s, "start");
+  const dim3 grid_a((K + V + 31) / 32, n_seg * HV), grid_b((V + 31) / 32, n_seg * HV);
+#define GDR_REC_SEG(KT)                                                                                              \
+  do {                                                                                                               \
+    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, true>), grid_a, dim3(64), 0, s, (const T*)k, (const T*)k,  \
+                       (const T*)v, g, beta, (T*)nullptr, (const float*)nullptr, mn, cu_seg, (int64_t)0, H, HV, K,   \
+                       K + V, scale, l2norm, (const int32_t*)nullptr);                                               \
+    LAMPA_PROF(s, "gdr_recurrent_split_kernel<composite>");                                                          \
+    hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1)>),                            \
+                       dim3((V + 31) / 32, n_seq, HV), dim3(256), (KT * (KT + 4) + KT * 33) * sizeof(float), s, mn,  \
+                       h0, seq_seg0, HV, K, V, sinit);                                                               \
+    LAMPA_PROF(s, "gdr_segment_scan_kernel");                                                                        \
+    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false>), grid_b, dim3(64), 0, s, (const T*)q, (const T*)k, \
+                       (const T*)v, g, beta, (T*)o, sinit, ht, cu_seg, (int64_t)0, H, HV, K, V, scale, l2norm,       \
+                       seg_out);                                                                                     \
+    LAMPA_PROF(s, "gdr_recurrent_split_kernel");                                                                     \
+  } while (0)
+  if (K <= 16) GDR_REC_SEG(16);
+  else if (K <= 32) GDR_REC_SEG(32);
+  else if (K <= 64) GDR_REC_SEG(64);
+  else GDR_REC_SEG(128);
+#undef GDR_REC_SEG
+  return lampa_launch_status();
+}
+
+// Workspace of lampa_gdr_recurrent_segmented_fwd: the segments' maps [n_seg, HV, K, K + V] and the states they start
+// from [n_seg, HV, K, V], fp32.
+extern "C" int64_t lampa_gdr_recurrent_segmented_workspace_bytes(int n_seg, int HV, int K, int V) {
+  if (n_seg < 0 || HV < 1 || K < 1 || V < 1) return LAMPA_ERR_INVALID;
+  return lampa_align_up((int64_t)n_seg * HV * K * (K + V) * 4, 256) + lampa_align_up((int64_t)n_seg * HV * K * V * 4, 256);
+}
+
+// lampa_gdr_recurrent_fwd for a few long sequences: the caller cuts every sequence into segments (cu_seg: device int64,
+// n_seg + 1 token offsets, every sequence boundary among them; seq_seg0: device int32, n_seq + 1, first segment of
+// every sequence; seg_out: device int32, n_seg, the sequence whose last segment this is, else -1) and the segments run
+// in parallel. Same arguments and results otherwise; K and V multiples of 4, q and k 16-byte aligned, K <= 128.
+extern "C" int lampa_gdr_recurrent_segmented_fwd(const void* q, const void* k, const void* v, const float* g,
+                                                 const float* beta, void* o, const float* h0, float* ht,
+                                                 const int64_t* cu_seg, const int32_t* seq_seg0, const int32_t* seg_out,
+                                                 int n_seq, int n_seg, int H, int HV, int K, int V, int dtype,
+                                                 float scale, int l2norm, void* workspace, int64_t workspace_bytes,
+                                                 void* stream) {
+  if (!q || !k || !v || !g || !beta || !o || !cu_seg || !seq_seg0 || !seg_out) return LAMPA_ERR_INVALID;
+  if (n_seq < 0 || n_seg < n_seq || H < 1 || HV < H || HV % H != 0 || K < 1 || V < 1) return LAMPA_ERR_INVALID;
+  if (l2norm < 0 || l2norm > 2) return LAMPA_ERR_INVALID;
+  if (K > 128 || K % 4 != 0 || V % 4 != 0 ||
+      ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) != 0)
+    return LAMPA_ERR_UNSUPPORTED;
+  if (n_seq == 0 || n_seg == 0) return LAMPA_OK;
+  if (!workspace || workspace_bytes < lampa_gdr_recurrent_segmented_workspace_bytes(n_seg, HV, K, V))
+    return LAMPA_ERR_WORKSPACE;
+  float* mn = (float*)workspace;
+  float* sinit = (float*)((char*)workspace + lampa_align_up((int64_t)n_seg * HV * K * (K + V) * 4, 256));
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case GDR_BF16:
+      return gdr_recurrent_segmented<__bf16>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H,
+                                             HV, K, V, scale, l2norm, mn, sinit, s);
+    case GDR_FP16:
+      return gdr_recurrent_segmented<_Float16>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H,
+                                               HV, K, V, scale, l2norm, mn, sinit, s);
+    case GDR_FP32:
+      return gdr_recurrent_segmented<float>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H, HV,
+                                            K, V, scale, l2norm, mn, sinit, s);
+    default:
+      return LAMPA_ERR_INVALID;
+  }
 }
 
 // q, k [total_tokens, H, K]; v, o [total_tokens, HV, V]; g, beta fp32 [total_tokens, HV]; h0, ht fp32

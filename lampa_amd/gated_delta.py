@@ -66,10 +66,70 @@ def _plan(cu_host, device, n_value_heads: int, head_dims):
     return host, dev
 
 
+# Token-serial operator: sequences at least this long are cut into segments that run in parallel when the launch
+# would otherwise occupy less than a quarter of the chip (None: never).
+SEGMENT_MIN_TOKENS: Optional[int] = 512
+
+_segment_cache = {}
+
+
+def _segment_tables(cu_host, seg_len: int, device):
+    """Device tables of ``lampa_gdr_recurrent_segmented_fwd``: every sequence cut into segments of ``seg_len`` tokens
+    (an empty sequence keeps one empty segment, so that its final state is still written)."""
+    key = (tuple(cu_host), seg_len, str(device))
+    hit = _segment_cache.get(key)
+    if hit is not None:
+        return hit
+    cu_seg, seq_seg0, seg_out = [], [], []
+    for s, (a, b) in enumerate(zip(cu_host[:-1], cu_host[1:])):
+        seq_seg0.append(len(cu_seg))
+        starts = list(range(a, b, seg_len)) or [a]
+        cu_seg.extend(starts)
+        seg_out.extend([-1] * (len(starts) - 1) + [s])
+    seq_seg0.append(len(cu_seg))
+    cu_seg.append(cu_host[-1])
+    tables = (torch.tensor(cu_seg, dtype=torch.int64).to(device), torch.tensor(seq_seg0, dtype=torch.int32).to(device),
+              torch.tensor(seg_out, dtype=torch.int32).to(device), len(seg_out))
+    if len(_segment_cache) > 64:
+        _segment_cache.clear()
+    _segment_cache[key] = tables
+    return tables
+
+
+def _recurrent_segmented_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_host, seg_len, l2norm):
+    H, K = q.shape[2], q.shape[3]
+    HV, V = v.shape[2], v.shape[3]
+    n_seq = len(cu_host) - 1
+    cu_seg, seq_seg0, seg_out, n_seg = _segment_tables(cu_host, seg_len, q.device)
+    lib = _capi.lib()
+    ws_bytes = check(lib.lampa_gdr_recurrent_segmented_workspace_bytes(n_seg, HV, K, V),
+                     "lampa_gdr_recurrent_segmented_workspace_bytes")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    o = torch.empty_like(v)
+    ht = torch.empty((n_seq, HV, K, V), dtype=torch.float32, device=q.device) if output_final_state else None
+    h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+    check(lib.lampa_gdr_recurrent_segmented_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(o), ptr(h0), ptr(ht),
+                                                ptr(cu_seg), ptr(seq_seg0), ptr(seg_out), n_seq, n_seg, H, HV, K, V,
+                                                _DTYPES[q.dtype], float(scale), l2norm, ptr(ws), ws_bytes,
+                                                stream_of(q)), "lampa_gdr_recurrent_segmented_fwd")
+    return o, ht
+
+
 def _recurrent_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
     B, T, H, K = q.shape
     HV, V = v.shape[2], v.shape[3]
     n_seq = B if cu_seqlens is None else len(cu_seqlens) - 1
+    slabs = (V + 31) // 32
+    if (SEGMENT_MIN_TOKENS and K % 4 == 0 and V % 4 == 0 and K <= 128 and n_seq * HV * slabs <= 256
+            and q.shape[0] * T >= SEGMENT_MIN_TOKENS and q.data_ptr() % 16 == 0 and k.data_ptr() % 16 == 0):
+        # a few long sequences: one or two waves each would leave most of the chip idle
+        cu_host = [i * T for i in range(B + 1)] if cu_seqlens is None else [int(c) for c in cu_seqlens.tolist()]
+        if max(b - a for a, b in zip(cu_host[:-1], cu_host[1:])) >= SEGMENT_MIN_TOKENS:
+            want = max(1, 1024 // (HV * slabs))  # segments for about one wave per SIMD in the output pass (the scan
+            # between the passes is serial in the segments: no more of them than fill the chip)
+            seg_len = max(128, -(-(cu_host[-1] // want) // 64) * 64)
+            return _recurrent_segmented_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_host,
+                                               seg_len, l2norm)
     o = torch.empty_like(v)
     ht = torch.empty((n_seq, HV, K, V), dtype=torch.float32, device=q.device) if output_final_state else None
     cu = None if cu_seqlens is None else cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()

@@ -80,6 +80,36 @@ def test_recurrent_many_short_sequences_both_kernels(device):
         assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL, n
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_recurrent_long_sequences_run_as_segments(device, dtype):
+    # a few long sequences (one of them empty, one shorter than a segment) are cut into segments that run in parallel;
+    # against the oracle and against the same call with the segments switched off
+    gen = torch.Generator().manual_seed(21)
+    lens = [1500, 0, 77, 2049]
+    cu = torch.tensor([0] + list(np.cumsum(lens)))
+    T, H, HV, K, V = sum(lens), 1, 2, 32, 64
+    q, k = (torch.randn(1, T, H, K, generator=gen).to(dtype) for _ in range(2))
+    v = torch.randn(1, T, HV, V, generator=gen).to(dtype)
+    g = -torch.rand(1, T, HV, generator=gen) * 0.1
+    beta = torch.rand(1, T, HV, generator=gen)
+    h0 = torch.randn(4, HV, K, V, generator=gen)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu, l2=og.L2_RECURRENT)
+    run = lambda: gd.fused_recurrent_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                                      output_final_state=True, cu_seqlens=cu.to(device),
+                                                      use_qk_l2norm_in_kernel=True)
+    o, s = run()
+    old = gd.SEGMENT_MIN_TOKENS
+    gd.SEGMENT_MIN_TOKENS = None
+    try:
+        o1, s1 = run()
+    finally:
+        gd.SEGMENT_MIN_TOKENS = old
+    tol = FP32_TOL if dtype == torch.float32 else 2e-2
+    assert _errors(o, want_o)[0] <= tol and _errors(s, want_s)[0] <= 10 * FP32_TOL
+    assert _errors(o1, want_o)[0] <= tol and _errors(s1, want_s)[0] <= 10 * FP32_TOL
+    assert _errors(o, o1.float().cpu())[0] <= tol and _errors(s, s1.cpu())[0] <= 10 * FP32_TOL
+
+
 def test_recurrent_varlen_gva_bf16(device):
     gen = torch.Generator().manual_seed(3)
     T, H, HV, K, V = 500, 2, 4, 64, 64
@@ -273,12 +303,22 @@ def test_chunk_small_heads_long_sequence_fp16(device, K, V):
             gd.chunk_gated_delta_rule(dq, dk, dv, dg, db)
         torch.cuda.synchronize()
         t_chunk = (time.perf_counter() - t0) / 5
-        t0 = time.perf_counter()
-        gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
-        torch.cuda.synchronize()
-        t_loop = time.perf_counter() - t0
-        print(f"K=16 V=32 H=6 T=30000 fp16: chunk path {1e6 * t_chunk:.0f} us, token loop {1e6 * t_loop:.0f} us")
-        assert t_chunk * 20 < t_loop
+        def loop_time(segments):  # the token-serial operator, as parallel segments or as one serial run per head
+            old = gd.SEGMENT_MIN_TOKENS
+            gd.SEGMENT_MIN_TOKENS = old if segments else None
+            try:
+                gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
+                torch.cuda.synchronize()
+                return time.perf_counter() - t0
+            finally:
+                gd.SEGMENT_MIN_TOKENS = old
+        t_seg, t_loop = loop_time(True), loop_time(False)
+        print(f"K=16 V=32 H=6 T=30000 fp16: chunk path {1e6 * t_chunk:.0f} us, token loop in segments "
+              f"{1e6 * t_seg:.0f} us, serial {1e6 * t_loop:.0f} us")
+        assert t_chunk * 20 < t_loop and t_chunk < t_seg < t_loop
 
 
 @pytest.mark.parametrize("T", [1, 64, 65, 200, 1000])
