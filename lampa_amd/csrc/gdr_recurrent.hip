@@ -373,29 +373,50 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
 //   B  every segment again from the state it really starts with, writing o (the plain kernel, segments as sequences)
 // all in fp32: the same function as the token loop up to fp32 rounding.
 
-// 32 columns of the state per workgroup (lane = column, 8 row groups); mn [n_seg, HV, K, K + V], sinit [n_seg, HV, K, V].
-// A step is short (KT / 8 rows x KT multiply-adds per thread), so what counts is that nothing serial is left in it but
-// that: M_p is loaded with 16-byte accesses into registers DEPTH segments ahead (its 1 - 2 us of memory latency would
-// otherwise be paid once per segment), parked in LDS, and every thread reads the rows it needs from there as
-// broadcasts; loop bounds are compile-time (K is padded to KT with zeros in LDS). LDS: M [KT][KT + 4] | S [KT][33].
+// 32 columns of the state per workgroup; mn [n_seg, HV, K, K + V], sinit [n_seg, HV, K, V]. A step is short, so what
+// counts is that nothing serial is left in it but the product itself:
+//  - M_p is loaded with 16-byte accesses into registers DEPTH segments ahead (its 1 - 2 us of memory latency would
+//    otherwise be paid once per segment) and parked in LDS; the register sets are fixed per step of an unrolled group
+//    (moving a set would wait for its load), and every memory operation of a step is unconditional (under a condition
+//    it becomes a branch, after which the compiler no longer counts the operations in flight and drains them);
+//  - M_p S runs on the fp32 MFMA (v_mfma_f32_32x32x2f32: 4 bytes per lane and operand from LDS). As multiply-adds with
+//    M read as broadcasts it was bound by LDS bandwidth (512 KB per step at K = 64: 4.8 us). The four waves split the
+//    product into row tiles of 32 and, where there are fewer than four of those, into parts of the contraction whose
+//    partial tiles are added afterwards;
+//  - LDS-only barriers.
+// LDS: M [max(KT, 32)][KT + 4] | S [KT][33] | partial tiles [KS][max(KT, 32)][33], floats.
+typedef float rs_f32x16 __attribute__((ext_vector_type(16)));
+template <int KT>
+struct RsScanShape {
+  static constexpr int RT = KT >= 32 ? KT / 32 : 1;  // row tiles of 32
+  static constexpr int KS = 4 / RT;                  // parts of the contraction (one wave each)
+  static constexpr int ROWS = RT * 32;
+  static constexpr int MS = KT + 4;                  // row stride of M in LDS (floats)
+  static constexpr size_t LDS_BYTES = ((size_t)ROWS * MS + (size_t)KT * 33 + (size_t)KS * ROWS * 33) * sizeof(float);
+};
+
 template <int KT, int DEPTH>
 __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __restrict__ mn, const float* __restrict__ h0,
                                                               const int32_t* __restrict__ seq_seg0, int HV, int K, int V,
                                                               float* __restrict__ sinit) {
-  constexpr int MS = KT + 4;             // row stride of M in LDS (floats)
-  constexpr int K4 = KT / 4;             // 16-byte pieces per row of M
-  constexpr int RPB = 256 / K4 < KT ? 256 / K4 : KT;  // rows of M that the workgroup loads at once
-  constexpr int MREGS = (KT + RPB - 1) / RPB;         // such batches = pieces per thread
-  constexpr int NR = KT / 8;                          // rows of the new column per thread (rg, rg + 8, ...)
-  static_assert(KT % 8 == 0, "eight row groups");
+  using SH = RsScanShape<KT>;
+  constexpr int MS = SH::MS, RT = SH::RT, KS = SH::KS, ROWS = SH::ROWS;
+  constexpr int K4 = KT / 4;                          // 16-byte pieces per row of M
+  constexpr int RPB = 256 / K4 < ROWS ? 256 / K4 : ROWS;  // rows of M that the workgroup stores to LDS at once
+  constexpr int MREGS = (ROWS + RPB - 1) / RPB;       // such batches = pieces per thread
+  constexpr int NR = KT / 8;                          // rows of the new column per thread in the combine step
+  constexpr int KL = KT / KS;                         // contraction length of a wave
+  static_assert(KT % 8 == 0 && KL % 2 == 0, "shape");
   extern __shared__ float4 s_scan4[];
   float* s_M = reinterpret_cast<float*>(s_scan4);
-  float* s_S = s_M + KT * MS;
+  float* s_S = s_M + ROWS * MS;
+  float* s_P = s_S + KT * 33;
   const int tid = threadIdx.x, c = tid & 31, rg = tid >> 5;
+  const int wave = tid >> 6, ln = tid & 31, hh = (tid >> 5) & 1;
+  const int rt = wave % RT, ks = wave / RT;
   const int seq = blockIdx.y, hv = blockIdx.z;
   const int col = blockIdx.x * 32 + c;
-  const bool active = col < V;
-  const int colc = active ? col : V - 1;  // (idle lanes shadow the last column and store nothing)
+  const int colc = col < V ? col : V - 1;  // (lanes past V shadow the last column: same loads, same stores)
 #pragma unroll
   for (int n = 0; n < NR; ++n) {
     const int i = rg + 8 * n;
@@ -407,23 +428,18 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
   const bool loader = my_row < RPB;
   float4 mreg[DEPTH][MREGS];
   float nreg[DEPTH][NR];
-  // M_p and this thread's entries of N_p into register set `slot` (zeros past K). Every step issues the same memory
-  // operations (a segment index past the end is clamped: its loads are never used), so that the waits the compiler
-  // places count exactly and the loads issued ahead stay in flight across the steps.
+  // M_p and this thread's entries of N_p into register set `slot`: unconditional loads from clamped addresses (a
+  // segment index past the end, a row or column past K); what lies past K is replaced by zero when it is used
   auto fetch = [&](int p, int slot) __attribute__((always_inline)) {
     p = min(p, p1 - 1);
     const float* M = mn + ((int64_t)p * HV + hv) * K * W;
-    // (unconditional loads from clamped addresses; what lies past K is replaced by zero when the values are used: a
-    // branch or a select at the load would make the wave wait for it at once)
 #pragma unroll
     for (int u = 0; u < MREGS; ++u)
       mreg[slot][u] = *reinterpret_cast<const float4*>(M + (int64_t)min(u * RPB + my_row, K - 1) * W + min(4 * my_c4, K - 4));
 #pragma unroll
     for (int n = 0; n < NR; ++n) nreg[slot][n] = M[(int64_t)min(rg + 8 * n, K - 1) * W + K + colc];
   };
-  // the state segment p starts from. Every lane stores every time (a lane past V or a row past K repeats the last
-  // column's / row's store with the same value): a store under a condition becomes a branch, and then the compiler can
-  // no longer count the memory operations in flight and waits for the loads issued ahead much too early.
+  // the state segment p starts from (every lane stores every time: rows past K repeat the last row's store)
   auto store_start = [&](int p) __attribute__((always_inline)) {
     float* out = sinit + ((int64_t)p * HV + hv) * K * V;
 #pragma unroll
@@ -440,7 +456,7 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
     for (int u = 0; u < MREGS; ++u) {
       const int i = u * RPB + my_row;
       const bool inside = i < K && 4 * my_c4 < K;
-      if (loader && i < KT)
+      if (loader && i < ROWS)
         *reinterpret_cast<float4*>(s_M + i * MS + 4 * my_c4) = inside ? mreg[slot][u] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     float acc[NR];
@@ -448,20 +464,39 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
     for (int n = 0; n < NR; ++n) acc[n] = rg + 8 * n < K ? nreg[slot][n] : 0.0f;
     lds_barrier();  // M_p is in LDS (an LDS-only barrier: the loads issued ahead stay in flight)
     fetch(p + DEPTH, slot);
-#pragma unroll 2
-    for (int l0 = 0; l0 < KT; l0 += 4) {
-      const float s0 = s_S[l0 * 33 + c], s1 = s_S[(l0 + 1) * 33 + c], s2 = s_S[(l0 + 2) * 33 + c],
-                  s3 = s_S[(l0 + 3) * 33 + c];
+    {
+      // this wave's tile: rows 32 rt .., contraction indices ks KL .. ; step s takes the indices s (lanes 0-31) and
+      // KL / 2 + s (lanes 32-63) of that range, so that a lane walks consecutive addresses
+      const float* ap = s_M + (32 * rt + ln) * MS + ks * KL + hh * (KL / 2);
+      const float* bp = s_S + (ks * KL + hh * (KL / 2)) * 33 + ln;
+      rs_f32x16 t;
 #pragma unroll
-      for (int n = 0; n < NR; ++n) {
-        // (rows rg + 8 n, n < NR, all lie below KT: no bound, a bound would put every read into a branch of its own)
-        const float4 m = *reinterpret_cast<const float4*>(s_M + (rg + 8 * n) * MS + l0);
-        acc[n] = __builtin_fmaf(m.w, s3, __builtin_fmaf(m.z, s2, __builtin_fmaf(m.y, s1, __builtin_fmaf(m.x, s0, acc[n]))));
+      for (int r = 0; r < 16; ++r) t[r] = 0.0f;
+#pragma unroll
+      for (int s0 = 0; s0 < KL / 2; s0 += 8) {  // operands of eight steps, then their MFMAs
+        float av[8], bv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < KL / 2) {
+            av[u] = ap[s0 + u];
+            bv[u] = bp[(s0 + u) * 33];
+          }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < KL / 2) t = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u], t, 0, 0, 0);
       }
-    }
-    lds_barrier();  // every thread has read the old column and M_p
+      float* pp = s_P + (ks * ROWS + 32 * rt + 4 * hh) * 33 + ln;  // accumulator register r: row 8 (r / 4) + 4 hh + r % 4
 #pragma unroll
-    for (int n = 0; n < NR; ++n) s_S[(rg + 8 * n) * 33 + c] = acc[n];
+      for (int r = 0; r < 16; ++r) pp[(8 * (r / 4) + (r % 4)) * 33] = t[r];
+    }
+    lds_barrier();  // the partial tiles are in LDS; every wave has read the old S and M_p
+#pragma unroll
+    for (int n = 0; n < NR; ++n) {
+      const int i = rg + 8 * n;
+#pragma unroll
+      for (int part = 0; part < KS; ++part) acc[n] += s_P[(part * ROWS + i) * 33 + c];
+      s_S[i * 33 + c] = acc[n];
+    }
     lds_barrier();
   };
   if (p0 >= p1) return;
@@ -469,7 +504,7 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
   for (int d = 0; d < DEPTH; ++d) fetch(p0 + d, d);
   __syncthreads();
   int p = p0;
-  for (; p + DEPTH < p1; p += DEPTH) {  // DEPTH steps on fixed register sets (no moves: a move would wait for its load)
+  for (; p + DEPTH < p1; p += DEPTH) {  // DEPTH steps on fixed register sets
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) advance(p + d, d);
   }
@@ -489,7 +524,7 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
   if (!attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (128 * 132 + 128 * 33) * (int)sizeof(float)) != hipSuccess)
+                            (int)RsScanShape<128>::LDS_BYTES) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
     attr_set[dev] = true;
   }
@@ -502,8 +537,8 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
                        K + V, scale, l2norm, (const int32_t*)nullptr);                                               \
     LAMPA_PROF(s, "gdr_recurrent_split_kernel<composite>");                                                          \
     hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1)>),                            \
-                       dim3((V + 31) / 32, n_seq, HV), dim3(256), (KT * (KT + 4) + KT * 33) * sizeof(float), s, mn,  \
-                       h0, seq_seg0, HV, K, V, sinit);                                                               \
+                       dim3((V + 31) / 32, n_seq, HV), dim3(256), RsScanShape<KT>::LDS_BYTES, s, mn, h0, seq_seg0,   \
+                       HV, K, V, sinit);                                                                             \
     LAMPA_PROF(s, "gdr_segment_scan_kernel");                                                                        \
     hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false>), grid_b, dim3(64), 0, s, (const T*)q, (const T*)k, \
                        (const T*)v, g, beta, (T*)o, sinit, ht, cu_seg, (int64_t)0, H, HV, K, V, scale, l2norm,       \
