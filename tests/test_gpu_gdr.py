@@ -363,6 +363,19 @@ def test_chunk_matches_token_serial_kernel_on_gpu(device):
     _assert_bf16_close(s1, s2.cpu(), "state")
 
 
+@pytest.mark.parametrize("g_scale", [1.0, 0.003])
+def test_fp32_mode_at_the_config2_shape(device, g_scale):
+    # the fp32 mode of the chunk operator (allow_fp32) at the headline shape, T = 60000, d = 64 (four heads): fp32 inputs
+    # through the token-serial kernels as parallel segments, 1e-4 against the fp64 token loop, with strong and weak decay
+    q, k, v, g, beta = synth.gdr_inputs(1, 60000, 4, 64, 64, torch.float32, seed=5, g_scale=g_scale)
+    h0 = 0.5 * torch.randn(1, 4, 64, 64, generator=torch.Generator().manual_seed(6))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, l2=og.L2_CHUNK)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                     output_final_state=True, allow_fp32=True, use_qk_l2norm_in_kernel=True)
+    assert o.dtype == torch.float32
+    assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL
+
+
 def test_config2_full_size(device):
     # B=1, H=8, T=60000, d=64, bf16 q/k/v, fp32 g/beta, tokens in the LSH-sorted order of a config-1 event
     from lampa_amd import lsh
