@@ -426,8 +426,23 @@ def main():
         return 1e6 * (time.perf_counter() - t_) / n
 
     c0_us = time_us(lambda: gd.fused_recurrent_gated_delta_rule(*d0, output_final_state=True))
+    _capi.profile_begin()
+    for _ in range(5):
+        gd.fused_recurrent_gated_delta_rule(*d0, output_final_state=True)
+    c0_stage = {}
+    for name, ms in _capi.profile_end(max_entries=64):
+        if name != "start":
+            c0_stage[name] = c0_stage.get(name, 0.0) + 1e3 * ms / 5
+    # the same operator in fp32 at the headline shape (the fp32 mode of the chunk operator, allow_fp32=True)
+    d2f = [x.to(dev) for x in synth.gdr_inputs(1, T, H, K, V, torch.float32, seed=0)]
+    f32_us = time_us(lambda: gd.chunk_gated_delta_rule(*d2f, output_final_state=True, allow_fp32=True), n=5, w=2)
+    del d2f
     config0 = {"workload": "config0: token-serial gated delta, B=1 H=4 T=8192 d_k=d_v=32, fp32, zero initial state",
-               "us": round(c0_us, 1), "hits_per_s": round(8192 / (c0_us * 1e-6), 1)}
+               "us": round(c0_us, 1), "hits_per_s": round(8192 / (c0_us * 1e-6), 1),
+               "kernel_us": {n: round(v_, 1) for n, v_ in c0_stage.items()},
+               "fp32_mode_at_config2_shape": {"us": round(f32_us, 1), "hits_per_s": round(T / (f32_us * 1e-6), 1)},
+               "note": "the sequence is cut into segments that run in parallel: every segment's affine map, a serial "
+                       "scan over the maps, then every segment from its true initial state; fp32 throughout"}
     if not args.no_cpu:
         c0_cpu_hps, c0_cpu_dt = cpu_baseline_gdr(q0, k0, v0, g0, b0, 8192, repeats=5, warmups=3)
         config0["cpu_baseline"] = {"value": round(c0_cpu_hps, 1), "unit": "hits/s", "seconds": round(c0_cpu_dt, 3),
