@@ -259,7 +259,7 @@ extern "C" int lampa_proj_conv_fwd(const void* x, int64_t x_stride, int64_t n_to
 #define NP_OUT 128     // output columns (4 waves x 32)
 #define NP_LDA (NP_KMAX + 8)
 
-__global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restrict__ o, const __bf16* __restrict__ g,
+__global__ void __launch_bounds__(256, 2) pc_norm_proj_kernel(const __bf16* __restrict__ o, const __bf16* __restrict__ g,
                                                           int64_t g_stride, const float* __restrict__ norm_w,
                                                           const __bf16* __restrict__ W, int64_t n_tokens, float eps,
                                                           __bf16* __restrict__ y, const __bf16* __restrict__ residual,
@@ -285,29 +285,41 @@ __global__ void __launch_bounds__(256) pc_norm_proj_kernel(const __bf16* __restr
 #pragma unroll
   for (int c = 0; c < 8; ++c) nw[c] = norm_w ? norm_w[8 * sub + c] : 1.0f;
 
+  // (the loads of four passes are issued before the first is used: two memory round trips per tile, not one per pass;
+  // all eight at once would cost the second workgroup per CU its registers)
   auto stage = [&](int64_t t0, int buf) {
-#pragma unroll 2
-    for (int pass = 0; pass < 8; ++pass) {
-      const int r = 32 * pass + rrow;           // (token, head) row of the tile: token r / 8, head r % 8
-      const int tok = r >> 3, head = r & 7;
-      int64_t t = t0 + tok;
-      t = t < n_tokens ? t : n_tokens - 1;
-      const bf16x8 ov = *reinterpret_cast<const bf16x8*>(o + t * NP_KMAX + head * NP_D + 8 * sub);
-      const bf16x8 gv = *reinterpret_cast<const bf16x8*>(g + t * g_stride + head * NP_D + 8 * sub);
-      float x[8], ss = 0.0f;
 #pragma unroll
-      for (int c = 0; c < 8; ++c) { x[c] = (float)ov[c]; ss = __builtin_fmaf(x[c], x[c], ss); }
-      ss += __shfl_xor(ss, 1);
-      ss += __shfl_xor(ss, 2);
-      ss += __shfl_xor(ss, 4);
-      const float rstd = 1.0f / sqrtf(ss * (1.0f / NP_D) + eps);
-      bf16x8 out;
+    for (int p0 = 0; p0 < 8; p0 += 4) {
+      bf16x8 ovs[4], gvs[4];
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const float gc = (float)gv[c];
-        out[c] = (__bf16)(x[c] * rstd * nw[c] * gc * pc_sigmoid(gc));
+      for (int u = 0; u < 4; ++u) {
+        const int r = 32 * (p0 + u) + rrow;       // (token, head) row of the tile: token r / 8, head r % 8
+        const int tok = r >> 3, head = r & 7;
+        int64_t t = t0 + tok;
+        t = t < n_tokens ? t : n_tokens - 1;
+        ovs[u] = *reinterpret_cast<const bf16x8*>(o + t * NP_KMAX + head * NP_D + 8 * sub);
+        gvs[u] = *reinterpret_cast<const bf16x8*>(g + t * g_stride + head * NP_D + 8 * sub);
       }
-      *reinterpret_cast<bf16x8*>(&s_a[buf][tok * NP_LDA + head * NP_D + 8 * sub]) = out;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int r = 32 * (p0 + u) + rrow;
+        const int tok = r >> 3, head = r & 7;
+        const bf16x8 ov = ovs[u], gv = gvs[u];
+        float x[8], ss = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { x[c] = (float)ov[c]; ss = __builtin_fmaf(x[c], x[c], ss); }
+        ss += __shfl_xor(ss, 1);
+        ss += __shfl_xor(ss, 2);
+        ss += __shfl_xor(ss, 4);
+        const float rstd = 1.0f / sqrtf(ss * (1.0f / NP_D) + eps);
+        bf16x8 out;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const float gc = (float)gv[c];
+          out[c] = (__bf16)(x[c] * rstd * nw[c] * gc * pc_sigmoid(gc));
+        }
+        *reinterpret_cast<bf16x8*>(&s_a[buf][tok * NP_LDA + head * NP_D + 8 * sub]) = out;
+      }
     }
   };
 
