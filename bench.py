@@ -199,7 +199,7 @@ def main():
     # ---- what the output pass's access pattern costs with no arithmetic (memory-only twin of that kernel: same rows
     #      of q, k, v, the per-chunk records and the o rows per workgroup and chunk; whole chunks only) ----
     n_chunks_probe = T // 64
-    rec = torch.zeros(n_chunks_probe * H * 6912, dtype=torch.uint8, device=dev)
+    rec = torch.zeros(n_chunks_probe * H * 5376, dtype=torch.uint8, device=dev)
     o_probe = torch.empty_like(vd)
     cps_probe = gd._default_chunks_per_segment([(T + 63) // 64], H, 2 * torch.cuda.get_device_properties(dev).multi_processor_count)
 
@@ -216,7 +216,7 @@ def main():
     ev1.record()
     torch.cuda.synchronize()
     probe_us = 1e3 * ev0.elapsed_time(ev1) / 100
-    probe_bytes = n_chunks_probe * H * (4 * 64 * 64 * 2 + 6912)
+    probe_bytes = n_chunks_probe * H * (4 * 64 * 64 * 2 + 4608)  # q, k, v, o rows and the T blocks of the record
     roofline["memory_only_twin"] = {
         "us": round(probe_us, 2), "bytes": probe_bytes, "GB/s": round(probe_bytes / (probe_us * 1e-6) / 1e9, 1),
         "kernel_over_twin": round(stage_us.get("gdr_segment_kernel<output>", float("nan")) / probe_us, 3),

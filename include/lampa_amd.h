@@ -312,9 +312,9 @@ int lampa_profile_begin(void);
 int lampa_profile_end(int max_entries, float* ms, const char** names);
 
 /* Memory-only twin of the chunk pipeline's output pass (a benchmarking aid with no counterpart in the reference):
- * the same loads and stores per (segment, head) workgroup and chunk (k, v, q rows, the 6912-byte record of the chunk
+ * the same loads and stores per (segment, head) workgroup and chunk (k, v, q rows, the T blocks of the 5376-byte record of the chunk
  * and head, the o rows) with no arithmetic, for K = V = 64 and 2-byte elements on one dense sequence of
- * n_chunks * 64 tokens. q, k, v, o [n_chunks * 64, H, 64]; records n_chunks * H * 6912 bytes of any content; o is
+ * n_chunks * 64 tokens. q, k, v, o [n_chunks * 64, H, 64]; records n_chunks * H * 5376 bytes of any content; o is
  * overwritten. Its duration is what that access pattern costs on the memory system alone. */
 int lampa_gdr_traffic_probe(const void* q, const void* k, const void* v, const void* records, void* o, int n_chunks,
                             int H, int chunks_per_segment, void* stream);

@@ -52,7 +52,29 @@ static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_d
   return pv;
 }
 
-#define T_BYTES (3 * 32 * 32 * 2)  // T of one chunk and head in HBM: bf16 blocks T11 | T21 | T22, 32x32 row-major each
+// T of one chunk and head in HBM, 16-bit elements: the lower-triangular blocks T11 and T22 packed by rows in 16-byte
+// pieces of 8 columns -- row r keeps its pieces 0 .. r / 8 (rows 0-7 one piece, 8-15 two, 16-23 three, 24-31 four: 80
+// of the 128 pieces of a 32x32 block; what lies above the diagonal inside a kept piece is stored as the zero it is)
+// -- after the full block T21, 32x32 row-major: T21 | T11 packed | T22 packed (so that the 128 threads that stage a
+// record read pieces t, 128 + t and 256 + t % 32 of it: two of the three loads share their address).
+#define T_DIAG_PIECES 80
+#define T_OFF_21 0
+#define T_OFF_11 (32 * 32 * 2)
+#define T_OFF_22 (T_OFF_11 + T_DIAG_PIECES * 16)
+#define T_BYTES (T_OFF_22 + T_DIAG_PIECES * 16)
+// (row, 8-column piece) of piece p of a packed block
+__device__ __forceinline__ void tri_piece(int p, int& row, int& part) {
+  const int x2 = p - 8, x3 = p - 24, x4 = p - 48;
+  const int q3 = (x3 * 11) >> 5;  // x3 / 3 for 0 <= x3 < 24
+  row = p < 8 ? p : p < 24 ? 8 + (x2 >> 1) : p < 48 ? 16 + q3 : 24 + (x4 >> 2);
+  part = p < 8 ? 0 : p < 24 ? (x2 & 1) : p < 48 ? x3 - 3 * q3 : (x4 & 3);
+}
+// (row, piece) of the u-th of the 48 pieces of a 32x32 block that lie entirely above the diagonal
+__device__ __forceinline__ void tri_upper_piece(int u, int& row, int& part) {
+  const int q3 = (u * 11) >> 5, x2 = u - 24;
+  row = u < 24 ? q3 : u < 40 ? 8 + (x2 >> 1) : 16 + (u - 40);
+  part = u < 24 ? 1 + (u - 3 * q3) : u < 40 ? 2 + (x2 & 1) : 3;
+}
 // Record of one chunk and head: T, then the chunk's cumulative log-decay (units of log 2) and beta per token, fp32
 // [64] each. The segment kernels take the two factor rows from here: in g and beta themselves a head's 64 values sit
 // 4 bytes apart in rows that interleave all heads, so every workgroup would fetch the sectors of all of them.
@@ -434,13 +456,17 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
     const float* src = blk == 0 ? s_A11 : s_A22;
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
-      const int piece = lane + 64 * jj, row = piece >> 2, part = piece & 3;
-      const f32x4 lo = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part]);
-      const f32x4 hi = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part + 4]);
-      O8 pk;
+      const int piece = lane + 64 * jj;  // of the packed block
+      if (piece < T_DIAG_PIECES) {
+        int row, part;
+        tri_piece(piece, row, part);
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part]);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(&src[row * SB + 8 * part + 4]);
+        O8 pk;
 #pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4) { pk[e4] = (OT)lo[e4]; pk[4 + e4] = (OT)hi[e4]; }
-      *reinterpret_cast<O8*>(out + (blk == 0 ? 0 : 2048) + row * 32 + 8 * part) = pk;
+        for (int e4 = 0; e4 < 4; ++e4) { pk[e4] = (OT)lo[e4]; pk[4 + e4] = (OT)hi[e4]; }
+        *reinterpret_cast<O8*>(out + (blk == 0 ? T_OFF_11 : T_OFF_22) / 2 + 8 * piece) = pk;
+      }
     }
   }
   {
@@ -455,7 +481,7 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
       pk[0] = (OT)(odd ? got : keep);
       pk[1] = (OT)(odd ? keep : got);
       const int row = acc_row(r0, hh) + (odd ? 1 : 0);
-      *reinterpret_cast<O2*>(out + 1024 + row * 32 + (ln & ~1)) = pk;
+      *reinterpret_cast<O2*>(out + T_OFF_21 / 2 + row * 32 + (ln & ~1)) = pk;
     }
   }
 }
@@ -610,6 +636,30 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     X8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
+    // where this thread's pieces of the packed diagonal blocks of T go in the LDS tile; the pieces above the diagonal
+    // are never staged and are zeroed once, in both tile sets
+    int ta_off, tb_off;  // element offsets into the T area of a tile set of this thread's two packed pieces
+    {
+      int row, part;
+      const int da = stid, db = 128 + (stid & 31);  // indices among the 160 packed pieces (T11: 0 .. 79, T22: 80 .. 159)
+      tri_piece(da < T_DIAG_PIECES ? da : da - T_DIAG_PIECES, row, part);
+      ta_off = ((da < T_DIAG_PIECES ? 0 : 2) * 32 + row) * ST + 8 * part;
+      tri_piece(db - T_DIAG_PIECES, row, part);
+      tb_off = (2 * 32 + row) * ST + 8 * part;
+    }
+    if (stid < 128 - T_DIAG_PIECES) {
+      int ur, up;
+      tri_upper_piece(stid, ur, up);
+      X8 z8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z8[e] = (OT)0.0f;
+#pragma unroll
+      for (int par = 0; par < 2; ++par) {
+        OT* tt = tiles(par).t;
+        *reinterpret_cast<X8*>(&tt[(0 * 32 + ur) * ST + 8 * up]) = z8;
+        *reinterpret_cast<X8*>(&tt[(2 * 32 + ur) * ST + 8 * up]) = z8;
+      }
+    }
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
     auto issue_tiles = [&](int c, typename Raw8<T>::type* rk_) {  // k, v, T
@@ -623,9 +673,12 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int u = 0; u < KU; ++u) rk_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(kb + koff + 8 * u);
 #pragma unroll
       for (int u = 0; u < VU; ++u) rv_[u] = *reinterpret_cast<const typename Raw8<T>::type*>(vb + voff + 8 * u);
+      // three pieces per thread, unconditional loads (the last 32 pieces are loaded by four threads each, which then
+      // store the same values to the same place)
       const X8* tp = reinterpret_cast<const X8*>(tmat + ((size_t)c * HV + hv) * REC_BYTES);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) rt_[j] = tp[stid + 128 * j];  // block j (T11, T21, T22), row stid / 4
+      rt_[0] = tp[stid];                    // T21
+      rt_[1] = tp[128 + stid];              // packed diagonal pieces 0 .. 127 (T11, then the first 48 of T22)
+      rt_[2] = tp[256 + (stid & 31)];       // packed diagonal pieces 128 .. 159 (the rest of T22), four times over
     };
     auto issue_gb = [&](int c) {  // cumulative log-decay and beta of the chunk's tokens (lane = token)
       c = uniform(c);
@@ -661,9 +714,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const GdrTilesT<OT> tl = tiles(par);
       zero_dead_rows(c, rk_, KU);
       zero_dead_rows(c, rv_, VU);
-#pragma unroll
-      for (int j = 0; j < 3; ++j)
-        *reinterpret_cast<X8*>(&tl.t[(j * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[j];
+      *reinterpret_cast<X8*>(&tl.t[(1 * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[0];
+      *reinterpret_cast<X8*>(&tl.t[ta_off]) = rt_[1];
+      *reinterpret_cast<X8*>(&tl.t[tb_off]) = rt_[2];
       kss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; u += 2) {

@@ -173,8 +173,10 @@ __global__ void __launch_bounds__(256)
     bf16x8 tp0, tp1;
     {
       const bf16x8* tp = reinterpret_cast<const bf16x8*>(rec_in);
+      // T21 (128 pieces) | T11 packed (80) | T22 packed (80): every thread takes piece tid (T21, T11, the first 48 of
+      // T22), threads 0 .. 31 also the last 32 of T22 (the others repeat them); unconditional loads
       tp0 = tp[tid];
-      tp1 = tp[256 + (tid & 127)];
+      tp1 = tp[256 + (tid & 31)];
       size_t li[NLAM];
 #pragma unroll
       for (int j = 0; j < NLAM; ++j) {
@@ -200,9 +202,29 @@ __global__ void __launch_bounds__(256)
       }
     }
     {
-      const int p0 = tid, p1 = 256 + tid;
-      *reinterpret_cast<bf16x8*>(&s_t[((p0 >> 7) * 32 + ((p0 & 127) >> 2)) * ST + 8 * (p0 & 3)]) = tp0;
-      if (tid < 128) *reinterpret_cast<bf16x8*>(&s_t[((p1 >> 7) * 32 + ((p1 & 127) >> 2)) * ST + 8 * (p1 & 3)]) = tp1;
+      // the pieces to their rows of the LDS tile (rows 0-31 T11, 32-63 T21, 64-95 T22); the 48 pieces above the
+      // diagonal of either packed block are zero
+      int r0, c0, r1, c1;
+      if (tid < 128) {  // a piece of T21
+        r0 = 32 + (tid >> 2);
+        c0 = tid & 3;
+      } else {
+        const int d = tid - 128;  // among the 160 packed pieces
+        tri_piece(d < T_DIAG_PIECES ? d : d - T_DIAG_PIECES, r0, c0);
+        r0 += d < T_DIAG_PIECES ? 0 : 64;
+      }
+      tri_piece(128 + (tid & 31) - T_DIAG_PIECES, r1, c1);
+      *reinterpret_cast<bf16x8*>(&s_t[r0 * ST + 8 * c0]) = tp0;
+      *reinterpret_cast<bf16x8*>(&s_t[(64 + r1) * ST + 8 * c1]) = tp1;
+      if (tid < 128 - T_DIAG_PIECES) {
+        int ur, up;
+        tri_upper_piece(tid, ur, up);
+        bf16x8 z8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) z8[e] = (__bf16)0.0f;
+        *reinterpret_cast<bf16x8*>(&s_t[ur * ST + 8 * up]) = z8;
+        *reinterpret_cast<bf16x8*>(&s_t[(64 + ur) * ST + 8 * up]) = z8;
+      }
     }
     const bool want_ss = l2norm != GDR_L2_NONE;
     bf16x8 kb[KU], qb[KU];

@@ -54,11 +54,11 @@ extern "C" int lampa_profile_end(int max_entries, float* ms, const char** names)
 // ---- memory-only twin of the output pass ----------------------------------------------------------------------------
 // The loads and stores of the chunk pipeline's output pass (K = V = 64, 2-byte elements, one dense sequence of whole
 // chunks) with no arithmetic at all: per (segment, head) workgroup and chunk, 128 threads fetch the chunk's k, v and q
-// rows (128 bytes per row and head, rows one token apart) and the 6 KiB of T in its record one chunk ahead, the other 128
+// rows (128 bytes per row and head, rows one token apart) and the 4.5 KiB of T in its record one chunk ahead, the other 128
 // threads store the o rows. Its duration is what this access pattern costs on the memory system alone, i.e. the
 // practical floor of the output pass (the algorithmic roofline assumes 8 TB/s for any pattern).
 typedef unsigned int prof_u32x4 __attribute__((ext_vector_type(4)));
-#define PROBE_REC_U4 432  // 6912-byte record of a chunk and head, in 16-byte units (the first 6144 bytes are read: T)
+#define PROBE_REC_U4 336  // 5376-byte record of a chunk and head, in 16-byte units (the first 288 are read: T)
 
 __global__ void __launch_bounds__(256, 2)
     gdr_traffic_probe_kernel(const prof_u32x4* __restrict__ q, const prof_u32x4* __restrict__ k,
@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(256, 2)
       for (int u = 0; u < 4; ++u) { buf[u] = k[base + u]; buf[4 + u] = v[base + u]; buf[8 + u] = q[base + u]; }
       const prof_u32x4* rp = rec + ((size_t)c * H + h) * PROBE_REC_U4;
 #pragma unroll
-      for (int j = 0; j < 3; ++j) buf[12 + j] = rp[tid + 128 * j];
+      for (int j = 0; j < 3; ++j) buf[12 + j] = rp[min(tid + 128 * j, 287)];  // (threads past the end repeat the last piece)
     };
     issue(c0);
     for (int c = c0; c < c1; ++c) {
@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(256, 2)
   }
 }
 
-// q, k, v, o: [n_chunks * 64, H, 64] 2-byte elements; records: n_chunks * H * 6912 bytes (any content). o is
+// q, k, v, o: [n_chunks * 64, H, 64] 2-byte elements; records: n_chunks * H * 5376 bytes (any content). o is
 // overwritten with a pattern. One launch = one pass.
 extern "C" int lampa_gdr_traffic_probe(const void* q, const void* k, const void* v, const void* records, void* o,
                                        int n_chunks, int H, int chunks_per_segment, void* stream) {

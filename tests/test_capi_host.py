@@ -97,7 +97,8 @@ def test_plan_rejects_bad_input(lib):
 def test_hierarchical_forward_argument_checks(lib):
     """Every check of lampa_hgdn_chunk_fwd runs on the host before the first launch (dummy, never dereferenced
     device addresses; the plan is real)."""
-    assert lib.lampa_hgdn_chunk_workspace_bytes(938, 30, 8, 64, 64) > 938 * 8 * (24 * 1024 + 2 * 64 * 64 * 4)
+    # at least the chunk records (5376 B), the walk records (> 16 KiB) and two fp32 K x V tiles per chunk and head
+    assert lib.lampa_hgdn_chunk_workspace_bytes(938, 30, 8, 64, 64) > 938 * 8 * (5376 + 16 * 1024 + 2 * 64 * 64 * 4)
     assert lib.lampa_hgdn_chunk_workspace_bytes(938, 30, 8, 128, 128) == -4
     assert lib.lampa_hgdn_chunk_workspace_bytes(-1, 30, 8, 64, 64) == -1
     d = ctypes.c_void_p(0x1000)  # 16-byte aligned dummy
