@@ -259,6 +259,28 @@ int lampa_gdr_recurrent_segmented_fwd(const void* q, const void* k, const void* 
                                       int HV, int K, int V, int dtype, float scale, int l2norm, void* workspace,
                                       int64_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------- gated-delta backward */
+
+/* Gradients of the gated-delta forward (lampa_gdr_chunk_fwd and lampa_gdr_recurrent_fwd compute the same function)
+ * with respect to q, k, v, g, beta and the initial state, given dout = d o and dht = d (final state). Replaces
+ * chunk_gated_delta_rule_bwd (models/hattention/gated_delta_rule_ori.py:83-160) together with the l2norm_bwd calls of
+ * ChunkGatedDeltaRuleFunction.backward (gated_delta_rule_ori.py:205-233): with l2norm != 0 the gradients are those of
+ * the un-normalised q and k. fp32 arithmetic; token-serial inside segments that run in parallel.
+ * q, k, dq, dk [total_tokens, H, K]; v, dout, dv [total_tokens, HV, V] (dtype LAMPA_BF16/FP16/FP32); g, beta, dg, dbeta
+ * fp32 [total_tokens, HV]; h0, dht, dh0 fp32 [n_seq, HV, K, V], each nullable (zero initial state; no gradient into
+ * the final state; d h0 not wanted).
+ * The caller cuts every sequence into segments as for lampa_gdr_recurrent_segmented_fwd (cu_seg, seq_seg0) and adds
+ * the tables of the pass that runs backwards: seq_seg0_rev device int32 [n_seq+1] = seq_seg0[s] + s, and seg_rev device
+ * int32 [n_seg] = seq_seg0_rev[s] + (last segment of s) - p for segment p of sequence s.
+ * K <= 128, K and V multiples of 4, q and k 16-byte aligned, at most 64 value heads per q/k head, n_seq <= 65535
+ * (LAMPA_ERR_UNSUPPORTED otherwise). workspace: lampa_gdr_bwd_workspace_bytes(total_tokens, n_seq, n_seg, HV, K, V). */
+int64_t lampa_gdr_bwd_workspace_bytes(int64_t total_tokens, int n_seq, int n_seg, int HV, int K, int V);
+int lampa_gdr_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* h0,
+                  const void* dout, const float* dht, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+                  const int64_t* cu_seg, const int32_t* seq_seg0, const int32_t* seq_seg0_rev, const int32_t* seg_rev,
+                  int64_t total_tokens, int n_seq, int n_seg, int H, int HV, int K, int V, int dtype, float scale,
+                  int l2norm, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Chunk / segment tables of the chunkwise forward, built on the host from the sequence boundaries.
  * Replaces prepare_chunk_indices / prepare_chunk_offsets (models/hattention/index.py:69-83).
  * cu_seqlens_host: int64 [n_seq+1]; chunks_per_segment: length of a segment of the split-sequence scan in

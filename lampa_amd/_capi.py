@@ -57,6 +57,8 @@ _SIGNATURES = {
     "lampa_gdr_recurrent_segmented_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "lampa_gdr_recurrent_segmented_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                                  _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),
+    "lampa_gdr_bwd_workspace_bytes": (_i64, [_i64, _i32, _i32, _i32, _i32, _i32]),
+    "lampa_gdr_bwd": (_i32, [_vp] * 18 + [_i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),
     "lampa_profile_begin": (_i32, []),
     "lampa_profile_end": (_i32, [_i32, _vp, _vp]),
     "lampa_gdr_traffic_probe": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),

@@ -553,6 +553,69 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
   return lampa_launch_status();
 }
 
+// The first two launches above on their own, for the backward pass (gdr_backward.hip), which needs the maps and the
+// states the segments start from but not the outputs; the scan is also run a second time there, over the transposed
+// maps in reverse segment order.
+static int gdr_scan_attr() {
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
+  if (!attr_set[dev]) {
+    if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)RsScanShape<128>::LDS_BYTES) != hipSuccess)
+      return LAMPA_ERR_LAUNCH;
+    attr_set[dev] = true;
+  }
+  return LAMPA_OK;
+}
+
+template <typename T>
+static void gdr_segment_maps_typed(const void* k, const void* v, const float* g, const float* beta,
+                                   const int64_t* cu_seg, int n_seg, int H, int HV, int K, int V, int l2norm, float* mn,
+                                   hipStream_t s) {
+  const dim3 grid_a((K + V + 31) / 32, n_seg * HV);
+#define GDR_REC_MAPS(KT)                                                                                            \
+  hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, true>), grid_a, dim3(64), 0, s, (const T*)k, (const T*)k,   \
+                     (const T*)v, g, beta, (T*)nullptr, (const float*)nullptr, mn, cu_seg, (int64_t)0, H, HV, K,    \
+                     K + V, 1.0f, l2norm, (const int32_t*)nullptr)
+  if (K <= 16) GDR_REC_MAPS(16);
+  else if (K <= 32) GDR_REC_MAPS(32);
+  else if (K <= 64) GDR_REC_MAPS(64);
+  else GDR_REC_MAPS(128);
+#undef GDR_REC_MAPS
+}
+
+int gdr_segment_maps(const void* k, const void* v, const float* g, const float* beta, const int64_t* cu_seg, int n_seg,
+                     int H, int HV, int K, int V, int dtype, int l2norm, float* mn, hipStream_t s) {
+  LAMPA_PROF(s, "start");
+  switch (dtype) {
+    case GDR_BF16: gdr_segment_maps_typed<__bf16>(k, v, g, beta, cu_seg, n_seg, H, HV, K, V, l2norm, mn, s); break;
+    case GDR_FP16: gdr_segment_maps_typed<_Float16>(k, v, g, beta, cu_seg, n_seg, H, HV, K, V, l2norm, mn, s); break;
+    case GDR_FP32: gdr_segment_maps_typed<float>(k, v, g, beta, cu_seg, n_seg, H, HV, K, V, l2norm, mn, s); break;
+    default: return LAMPA_ERR_INVALID;
+  }
+  LAMPA_PROF(s, "gdr_recurrent_split_kernel<composite>");
+  return lampa_launch_status();
+}
+
+int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, int n_seq, int HV, int K, int V,
+                     float* sinit, hipStream_t s) {
+  const int rc = gdr_scan_attr();
+  if (rc != LAMPA_OK) return rc;
+  LAMPA_PROF(s, "start");
+  const dim3 grid((V + 31) / 32, n_seq, HV);
+#define GDR_REC_SCAN(KT)                                                                                       \
+  hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1)>), grid, dim3(256),         \
+                     RsScanShape<KT>::LDS_BYTES, s, mn, h0, seq_seg0, HV, K, V, sinit)
+  if (K <= 16) GDR_REC_SCAN(16);
+  else if (K <= 32) GDR_REC_SCAN(32);
+  else if (K <= 64) GDR_REC_SCAN(64);
+  else GDR_REC_SCAN(128);
+#undef GDR_REC_SCAN
+  LAMPA_PROF(s, "gdr_segment_scan_kernel");
+  return lampa_launch_status();
+}
+
 // Workspace of lampa_gdr_recurrent_segmented_fwd: the segments' maps [n_seg, HV, K, K + V] and the states they start
 // from [n_seg, HV, K, V], fp32.
 extern "C" int64_t lampa_gdr_recurrent_segmented_workspace_bytes(int n_seg, int HV, int K, int V) {

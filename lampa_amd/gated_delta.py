@@ -6,7 +6,8 @@ defaults, checks and return tuples.  The arithmetic runs in hand-written gfx950 
 C ABI of ``liblampa_amd.so``; there is no Triton, no PyTorch fallback and no CPU path.
 
 Differences that a caller can observe, all additive:
-* forward only -- ``backward`` raises ``NotImplementedError``;
+* ``chunk_gated_delta_rule`` is differentiable (``lampa_gdr_bwd``: fp32, token-serial inside parallel segments);
+  ``fused_recurrent_gated_delta_rule``'s backward raises ``NotImplementedError`` as the reference's does;
 * ``allow_fp32=True`` lets ``chunk_gated_delta_rule`` accept float32 q/k/v (the reference rejects them); they
   are evaluated by the token-serial fp32 kernel;
 * head sizes other than 64 / 128 are evaluated by the token-serial kernel as well (correct, slower).
@@ -190,17 +191,106 @@ def _chunk_launch_any_head(q, k, v, g, beta, scale, initial_state, output_final_
     return o[..., :V].contiguous(), None if ht is None else ht[..., :K, :V].contiguous()
 
 
-class _ForwardOnly(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, launcher, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
-        require_cuda(q, k, v, g, beta, initial_state)
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
-        return launcher(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm)
+# Backward pass: about this many (segment, value head, 16-column slab) units, one wavefront each.
+BACKWARD_UNITS = 2048
+
+_backward_tables_cache = {}
+
+
+def _backward_tables(cu_host, seg_len: int, device):
+    """The segment tables of ``lampa_gdr_bwd``: those of the segmented forward plus, for the pass that runs backwards,
+    one extra row per sequence (``seq_seg0_rev``) and every segment's row counted from its sequence's end."""
+    key = (tuple(cu_host), seg_len, str(device))
+    hit = _backward_tables_cache.get(key)
+    if hit is not None:
+        return hit
+    cu_seg, seq_seg0, _, n_seg = _segment_tables(cu_host, seg_len, device)
+    first = seq_seg0.tolist()
+    rev0 = [p + s for s, p in enumerate(first)]
+    seg_rev = []
+    for s in range(len(first) - 1):
+        seg_rev.extend(rev0[s] + (first[s + 1] - 1) - p for p in range(first[s], first[s + 1]))
+    tables = (cu_seg, seq_seg0, torch.tensor(rev0, dtype=torch.int32).to(device),
+              torch.tensor(seg_rev, dtype=torch.int32).to(device), n_seg)
+    if len(_backward_tables_cache) > 64:
+        _backward_tables_cache.clear()
+    _backward_tables_cache[key] = tables
+    return tables
+
+
+def _backward_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, do, dht):
+    """Gradients (dq, dk, dv, dg, dbeta, dh0) through ``lampa_gdr_bwd``. Head sizes that are not multiples of 4 are
+    zero-padded (zero columns of q, k and v change neither the function nor the other columns' gradients)."""
+    B, T, H, K = q.shape
+    HV, V = v.shape[2], v.shape[3]
+    if K > 128:
+        raise NotImplementedError(f"backward of the gated-delta operators is built for K <= 128, got K = {K}")
+    Kp, Vp = -(-K // 4) * 4, -(-V // 4) * 4
+    pad = torch.nn.functional.pad
+    if (Kp, Vp) != (K, V):
+        q, k, v, do = pad(q, (0, Kp - K)), pad(k, (0, Kp - K)), pad(v, (0, Vp - V)), pad(do, (0, Vp - V))
+        initial_state = None if initial_state is None else pad(initial_state, (0, Vp - V, 0, Kp - K))
+        dht = None if dht is None else pad(dht, (0, Vp - V, 0, Kp - K))
+    q, k, v, do = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
+    cu_host = [i * T for i in range(B + 1)] if cu_seqlens is None else [int(c) for c in cu_seqlens.tolist()]
+    n_seq, total = len(cu_host) - 1, B * T
+    slabs = (Vp + 15) // 16
+    want = max(1, BACKWARD_UNITS // (HV * slabs))
+    seg_len = max(64, -(-(total // want) // 64) * 64)
+    cu_seg, seq_seg0, seq_seg0_rev, seg_rev, n_seg = _backward_tables(cu_host, seg_len, q.device)
+    lib = _capi.lib()
+    ws_bytes = check(lib.lampa_gdr_bwd_workspace_bytes(total, n_seq, n_seg, HV, Kp, Vp), "lampa_gdr_bwd_workspace_bytes")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dg, dbeta = torch.empty_like(g), torch.empty_like(beta)
+    h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+    dht = None if dht is None else dht.to(torch.float32).contiguous()
+    dh0 = None if h0 is None else torch.empty_like(h0)
+    check(lib.lampa_gdr_bwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(do), ptr(dht), ptr(dq), ptr(dk),
+                            ptr(dv), ptr(dg), ptr(dbeta), ptr(dh0), ptr(cu_seg), ptr(seq_seg0), ptr(seq_seg0_rev),
+                            ptr(seg_rev), total, n_seq, n_seg, H, HV, Kp, Vp, _DTYPES[q.dtype], float(scale), l2norm,
+                            ptr(ws), ws_bytes, stream_of(q)), "lampa_gdr_bwd")
+    if (Kp, Vp) != (K, V):
+        dq, dk, dv = dq[..., :K].contiguous(), dk[..., :K].contiguous(), dv[..., :V].contiguous()
+        dh0 = None if dh0 is None else dh0[..., :K, :V].contiguous()
+    return dq, dk, dv, dg, dbeta, dh0
+
+
+class _GatedDelta(torch.autograd.Function):
+    """Forward through ``launcher``; backward through ``lampa_gdr_bwd`` (``ChunkGatedDeltaRuleFunction``,
+    ``gated_delta_rule_ori.py:163-233``). ``differentiable=False`` keeps the reference's behaviour for the fused
+    recurrent operator, whose backward raises (``gated_delta_rule_ori.py:555-562``)."""
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("lampa_amd gated-delta operators are forward-only")
+    def forward(ctx, launcher, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm,
+                differentiable):
+        require_cuda(q, k, v, g, beta, initial_state)
+        ctx.g_dtype, ctx.beta_dtype = g.dtype, beta.dtype
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        g, beta = g.to(torch.float32).contiguous(), beta.to(torch.float32).contiguous()
+        ctx.differentiable = differentiable
+        if differentiable:
+            ctx.save_for_backward(q, k, v, g, beta, initial_state, cu_seqlens)
+            ctx.scale, ctx.l2norm = scale, l2norm
+        o, ht = launcher(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm)
+        ctx.o_shape, ctx.o_dtype = o.shape, o.dtype
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        if not ctx.differentiable:
+            raise NotImplementedError(
+                "Backward pass is not implemented yet and we do not have plans to implement it "
+                "because we haven't figured out how to compute dg without materializing the full "
+                "hidden states for all time steps.")
+        q, k, v, g, beta, initial_state, cu_seqlens = ctx.saved_tensors
+        if do is None:
+            do = torch.zeros(ctx.o_shape, dtype=ctx.o_dtype, device=q.device)
+        dq, dk, dv, dg, dbeta, dh0 = _backward_launch(q, k, v, g, beta, ctx.scale, initial_state, cu_seqlens,
+                                                      ctx.l2norm, do.to(v.dtype), dht)
+        if dh0 is not None:
+            dh0 = dh0.to(initial_state.dtype)
+        return (None, dq, dk, dv, dg.to(ctx.g_dtype), dbeta.to(ctx.beta_dtype), None, dh0, None, None, None, None)
 
 
 def _check_shapes(q, k, v, g, beta, what):
@@ -261,8 +351,8 @@ def chunk_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g:
         scale = k.shape[-1] ** -0.5
     l2norm = L2_CHUNK if use_qk_l2norm_in_kernel else L2_NONE
     launcher = _chunk_launch_any_head if _chunk_path_supported(q, v) else _recurrent_launch
-    o, final_state = _ForwardOnly.apply(launcher, q, k, v, g, beta, scale, initial_state, output_final_state,
-                                        cu_seqlens, l2norm)
+    o, final_state = _GatedDelta.apply(launcher, q, k, v, g, beta, scale, initial_state, output_final_state,
+                                       cu_seqlens, l2norm, True)
     return o.to(q.dtype), final_state
 
 
@@ -282,5 +372,5 @@ def fused_recurrent_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.
         beta = torch.ones_like(g)
     _check_shapes(q, k, v, g, beta, "fused_recurrent_gated_delta_rule")
     l2norm = L2_RECURRENT if use_qk_l2norm_in_kernel else L2_NONE
-    return _ForwardOnly.apply(_recurrent_launch, q, k, v, g, beta, scale, initial_state, output_final_state,
-                              cu_seqlens, l2norm)
+    return _GatedDelta.apply(_recurrent_launch, q, k, v, g, beta, scale, initial_state, output_final_state,
+                             cu_seqlens, l2norm, False)
