@@ -174,3 +174,27 @@ def test_static_sort_symbols_and_limit():
     assert lib.lampa_sort_pairs_static(d, 7, None, 1, 10, 32, None, 1, 0, d, None) == -1
     assert lib.lampa_sort_pairs_static(d, 1, None, 3, 400000, 32, None, 1, 0, d, None) == -2
     assert lib.lampa_sort_pairs_static(d, 1, None, 3, 0, 32, None, 1, 0, d, None) == 0
+
+
+def test_backward_argument_checks_and_tables(lib):
+    """lampa_gdr_bwd refuses bad arguments before any GPU work; the workspace grows with its parts; the tables of the
+    pass that runs backwards give every sequence one extra row and count its segments from the end."""
+    from lampa_amd import gated_delta as gd
+    small = lib.lampa_gdr_bwd_workspace_bytes(1024, 1, 4, 2, 64, 64)
+    # maps, start states, reverse maps, end states, a state per 8 tokens, the partial dq / dk per 16-column slab
+    assert small > 4 * (4 * 2 * 64 * 128 + 4 * 2 * 64 * 64 + 5 * 2 * 64 * 128 + 5 * 2 * 64 * 64
+                        + 128 * 2 * 64 * 64 + 2 * 4 * 1024 * 2 * 64)
+    assert lib.lampa_gdr_bwd_workspace_bytes(2048, 1, 4, 2, 64, 64) > small
+    assert lib.lampa_gdr_bwd_workspace_bytes(1024, 1, 4, 2, 256, 64) == -1
+    nulls = [None] * 18
+    assert lib.lampa_gdr_bwd(*nulls, 16, 1, 1, 1, 1, 64, 64, 0, 1.0, 0, None, 0, None) == -1
+    fake = [ctypes.c_void_p(4096)] * 18  # never dereferenced: the checks below come first
+    assert lib.lampa_gdr_bwd(*fake, 16, 1, 1, 1, 1, 62, 64, 0, 1.0, 0, None, 0, None) == -4   # K not a multiple of 4
+    assert lib.lampa_gdr_bwd(*fake, 16, 1, 1, 1, 1, 256, 64, 0, 1.0, 0, None, 0, None) == -4  # K > 128
+    assert lib.lampa_gdr_bwd(*fake, 16, 1, 1, 3, 4, 64, 64, 0, 1.0, 0, None, 0, None) == -1   # HV not a multiple of H
+    assert lib.lampa_gdr_bwd(*fake, 16, 1, 1, 1, 1, 64, 64, 0, 1.0, 3, None, 0, None) == -1   # unknown normalisation
+    assert lib.lampa_gdr_bwd(*fake, 16, 1, 1, 1, 1, 64, 64, 0, 1.0, 0, None, 0, None) == -2   # no workspace
+    cu_seg, seq_seg0, rev0, seg_rev, n_seg = gd._backward_tables([0, 0, 130, 194], 64, "cpu")
+    assert n_seg == 5 and cu_seg.tolist() == [0, 0, 64, 128, 130, 194]
+    assert seq_seg0.tolist() == [0, 1, 4, 5] and rev0.tolist() == [0, 2, 6, 8]
+    assert seg_rev.tolist() == [0, 4, 3, 2, 6]  # every sequence's last segment on its first row

@@ -1,0 +1,134 @@
+"""GPU parity of the gated-delta backward pass (``lampa_gdr_bwd`` behind ``chunk_gated_delta_rule``'s autograd) against
+the gradient oracle (``oracle.gated_delta_bwd.backward_manual``, float64 on the same, already rounded, inputs).
+
+Tolerances: the kernels compute in fp32 from the inputs as given, so fp32 inputs must agree to 1e-4 (max-abs relative
+to the largest entry of the gradient; 1e-5 mean-relative); with bf16 / fp16 inputs dq, dk and dv are rounded to that
+type on output (mean-relative 5e-3, the forward's bound), dg, dbeta and d(initial state) stay fp32 (1e-4).
+"""
+import pytest
+import torch
+
+from lampa_amd import gated_delta as gd
+from oracle import gated_delta as og
+from oracle import gated_delta_bwd as ob
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("dq", "dk", "dv", "dg", "dbeta", "dh0")
+
+
+def _inputs(B, T, H, HV, K, V, dtype, seed, unit, g_scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    if unit:
+        q, k = q / q.norm(dim=-1, keepdim=True), k / k.norm(dim=-1, keepdim=True)
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g = -g_scale * torch.nn.functional.softplus(torch.randn(B, T, HV, generator=gen))
+    beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
+    do = torch.randn(B, T, HV, V, generator=gen)
+    return [x.to(dtype) for x in (q, k, v)] + [g, beta, do.to(dtype)], gen
+
+
+def _gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, l2, scale=None):
+    args = [x.to(device).requires_grad_(True) for x in (q, k, v, g, beta)]
+    h0d = None if h0 is None else h0.to(device).requires_grad_(True)
+    o, ht = gd.chunk_gated_delta_rule(*args, scale=scale, initial_state=h0d, output_final_state=dht is not None,
+                                      cu_seqlens=None if cu is None else cu.to(device), use_qk_l2norm_in_kernel=l2,
+                                      allow_fp32=True)
+    loss = (o.float() * do.to(device).float()).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.to(device)).sum()
+    loss.backward()
+    return [a.grad for a in args] + [None if h0d is None else h0d.grad]
+
+
+def _check(got, want, dtype):
+    for name, a, b in zip(NAMES, got, want):
+        if b is None:
+            assert a is None, name
+            continue
+        a = a.double().cpu()
+        assert a.shape == b.shape, name
+        diff = (a - b).abs()
+        rel_max = diff.max().item() / b.abs().max().clamp_min(1e-30).item()
+        rel_mean = (diff.mean() / b.abs().mean().clamp_min(1e-30)).item()
+        rounded = dtype != torch.float32 and name in ("dq", "dk", "dv")
+        assert rel_max <= (2e-2 if rounded else 1e-4) and rel_mean <= (5e-3 if rounded else 1e-5), \
+            f"{name}: max {rel_max:.3e} mean {rel_mean:.3e}"
+
+
+@pytest.mark.parametrize("K,V,H,HV", [(16, 32, 2, 4), (64, 64, 2, 2), (128, 128, 1, 2), (32, 48, 1, 1), (24, 40, 2, 2),
+                                      (10, 6, 1, 3), (128, 20, 1, 1)])
+@pytest.mark.parametrize("l2", [False, True])
+def test_gradients_fp32_match_oracle(device, K, V, H, HV, l2):
+    """Equal-length batches with an initial state and a gradient into the final state; T = 75 leaves a partial block of
+    8 tokens and a partial segment; head sizes on and off the kernels' shapes (10 x 6 is zero-padded to 12 x 8)."""
+    (q, k, v, g, beta, do), gen = _inputs(2, 75, H, HV, K, V, torch.float32, K + V, unit=not l2)
+    h0 = 0.5 * torch.randn(2, HV, K, V, generator=gen)
+    dht = torch.randn(2, HV, K, V, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, do, dht, 0.37, h0, None, og.L2_CHUNK if l2 else og.L2_NONE)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, None, l2, scale=0.37), want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_gradients_varlen_segments(device, dtype, monkeypatch):
+    """Packed sequences (an empty one, one shorter than a block, lengths off the block and segment sizes), cut into
+    segments of 64 tokens so that the reverse maps and the reverse scan carry the state gradient over many segments."""
+    monkeypatch.setattr(gd, "BACKWARD_UNITS", 1 << 20)
+    lens = [0, 5, 333, 64, 1, 500, 97]
+    T = sum(lens)
+    (q, k, v, g, beta, do), gen = _inputs(1, T, 2, 4, 32, 32, dtype, 7, unit=False)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.long)
+    h0 = 0.5 * torch.randn(len(lens), 4, 32, 32, generator=gen)
+    dht = torch.randn(len(lens), 4, 32, 32, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, do, dht, None, h0, cu, og.L2_CHUNK)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, True), want, dtype)
+
+
+def test_gradients_without_states_and_with_unused_output(device):
+    """No initial state (no d h0), no final state; and a loss that uses the final state only (d o is zero)."""
+    (q, k, v, g, beta, do), gen = _inputs(1, 200, 1, 2, 64, 64, torch.float32, 3, unit=True)
+    want = ob.backward_manual(q, k, v, g, beta, do, None, None, None, None, og.L2_NONE)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, None, None, None, False), want, torch.float32)
+    dht = torch.randn(1, 2, 64, 64, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, torch.zeros_like(do), dht, None, None, None, og.L2_NONE)
+    args = [x.to(device).requires_grad_(True) for x in (q, k, v, g, beta)]
+    _, ht = gd.chunk_gated_delta_rule(*args, output_final_state=True, allow_fp32=True)
+    (ht * dht.to(device)).sum().backward()
+    _check([a.grad for a in args] + [None], want, torch.float32)
+
+
+def test_gradients_long_sequence_weak_decay(device):
+    """4 096 tokens with g of the order of -0.003 per token: the state and its gradient carry over hundreds of tokens
+    and through every segment."""
+    (q, k, v, g, beta, do), gen = _inputs(1, 4096, 1, 2, 64, 64, torch.bfloat16, 11, unit=False, g_scale=0.003)
+    h0 = 0.5 * torch.randn(1, 2, 64, 64, generator=gen)
+    dht = torch.randn(1, 2, 64, 64, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, do, dht, None, h0, None, og.L2_CHUNK)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, None, True), want, torch.bfloat16)
+
+
+def test_gradients_do_not_depend_on_the_segmentation_at_full_size(device, monkeypatch):
+    """Config-2 shape (60 032 tokens, 8 heads, K = V = 64, bf16), too long for the float64 loop: the same gradients from
+    63 segments per head and from 8 (fp32 rounding apart), and linear in (d o, d final state)."""
+    (q, k, v, g, beta, do), gen = _inputs(1, 60032, 8, 8, 64, 64, torch.bfloat16, 5, unit=False)
+    dht = torch.randn(1, 8, 64, 64, generator=gen)
+    a = _gpu_grads(device, q, k, v, g, beta, do, None, dht, None, True)
+    monkeypatch.setattr(gd, "BACKWARD_UNITS", 256)
+    b = _gpu_grads(device, q, k, v, g, beta, do, None, dht, None, True)
+    for name, x, y in zip(NAMES[:5], a, b):
+        x, y = x.float(), y.float()
+        assert torch.isfinite(x).all(), name
+        rounded = name in ("dq", "dk", "dv")  # bf16 outputs: one rounding step apart at most
+        assert (x - y).abs().max().item() <= (1e-2 if rounded else 2e-4) * y.abs().max().item(), name
+    c = _gpu_grads(device, q, k, v, g, beta, (2 * do.float()).to(do.dtype), None, 2 * dht, None, True)
+    for name, x, y in zip(NAMES[3:5], b[3:5], c[3:5]):  # the fp32 outputs: exactly twice (a power of two)
+        assert torch.equal(2 * x, y), name
+
+
+def test_fused_recurrent_backward_raises_like_the_reference(device):
+    (q, k, v, g, beta, do), _ = _inputs(1, 16, 1, 1, 16, 16, torch.float32, 0, unit=True)
+    args = [x.to(device).requires_grad_(True) for x in (q, k, v, g, beta)]
+    o, _ = gd.fused_recurrent_gated_delta_rule(*args)
+    with pytest.raises(NotImplementedError):
+        o.sum().backward()
