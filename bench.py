@@ -470,6 +470,29 @@ def main():
                "note": "algorithmic work per token-head: 1032 B and 182.9 kFLOP"}
     del d4
 
+    # ---- backward pass of the layer (lampa_gdr_bwd) at the headline shape and at the reference model's head sizes ----
+    def backward_leg(T_, H_, K_, V_, dtype_):
+        qb, kb, vb, gb_, bb = (x.to(dev) for x in synth.gdr_inputs(1, T_, H_, K_, V_, dtype_, seed=0))
+        dob = torch.randn_like(vb)
+        fn = lambda: gd._backward_launch(qb, kb, vb, gb_, bb, K_ ** -0.5, None, None, gd.L2_CHUNK, dob, None)
+        us = time_us(fn, n=5, w=2)
+        _capi.profile_begin()
+        fn()
+        stage = {}
+        for name, ms in _capi.profile_end(max_entries=64):
+            if name != "start":
+                stage[name] = stage.get(name, 0.0) + 1e3 * ms
+        return {"workload": f"gradients of one gated-delta layer, B=1 H={H_} T={T_} K={K_} V={V_}, "
+                            f"{str(dtype_).split('.')[-1]} q/k/v/do, fp32 arithmetic",
+                "us": round(us, 1), "hits_per_s": round(T_ / (us * 1e-6), 1),
+                "kernel_us": {n: round(v_, 1) for n, v_ in stage.items()}}
+
+    backward = {"config2_shape": backward_leg(T, H, K, V, torch.bfloat16),
+                "reference_model_heads": backward_leg(30016, 6, 16, 32, torch.float16),
+                "note": "token-serial inside parallel segments, fp32: forward maps and scan, reverse maps and scan, then "
+                        "every segment forwards (a state kept every 8 tokens) and backwards block by block; dq, dk, dv, "
+                        "dg, dbeta out, q/k normalisation included"}
+
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
     if not args.no_cpu:
@@ -506,7 +529,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0, "config4": config4,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0, "config4": config4, "backward": backward,
     }
     print(json.dumps(out))
 

@@ -15,16 +15,20 @@
 //   2  every segment's H from zero backwards: N'; the linear part is M^T        (gdr_bwd_segment_kernel<COMPOSITE>)
 //   3  H_end over the segments of a sequence, last to first                     (the forward scan kernel on [M^T | N'])
 //   4  every segment: forward once, leaving S at every 8th token in memory; then block by block from the end: the
-//      block's 8 decayed states rebuilt into LDS, then its tokens backwards     (gdr_bwd_segment_kernel)
+//      block's 8 decayed states rebuilt (into a spill area of the workgroup: 32 KB at K = 64, which as LDS would leave
+//      three waves per CU), then its tokens backwards                           (gdr_bwd_segment_kernel)
 //   5  partial sums over the column slabs and grouped value heads, the chain rule of the q/k normalisation, output
 //      types                                                                    (gdr_bwd_finish_kernel)
 // A wave owns 16 value columns of one (segment, value head): lane = (row group, column), a lane keeps K / 4 rows of
-// its column of S and of H in registers. Sums over the rows of a column cross the four row groups (two exchanges);
-// sums over the columns (dk, dq) go through LDS; db and dg are reduced once per block.
+// its column of S and of H in registers. Sums over the rows of a column cross the four row groups (two register
+// swaps); sums over the columns (dk, dq) go through LDS; db and dg are reduced once per block. A token's step is a
+// chain of dependent LDS round trips, so the kernel lives on waves per SIMD: at most GB_MAX_GRID workgroups of one wave
+// walk through the (segment, head, slab) units.
 #include "gdr_common.h"
 
 #define GB_BT 8     // tokens per block: states kept in LDS at a time, distance of the states kept in memory
 #define GB_COLS 16  // value columns per wave
+#define GB_MAX_GRID 4096  // workgroups of the segment kernel (each owns a spill area for a block's states)
 
 template <typename T>
 __device__ __forceinline__ float4 gb_load4(const T* p) {
@@ -45,9 +49,9 @@ struct GbShape {
   static constexpr int LPT = KT / 8;                   // lanes that load one token's k (8 elements each)
   static constexpr int PASSES = (GB_BT * LPT + 63) / 64;
   static constexpr int C_GROUP = KR * GB_COLS + 16;    // floats per row group in the column-sum buffer (+16: banks)
-  // LDS (floats): decayed states of the block [GB_BT][Q4][64][4] | k [GB_BT][KT] | q | v [GB_BT][16] | do | w |
-  // (a, b) [GB_BT][4] | column sums [2][4][C_GROUP] | db / dg partials [GB_BT][2][64]
-  static constexpr int OFF_K = GB_BT * KT * GB_COLS;
+  // LDS (floats): k [GB_BT][KT] | q | v [GB_BT][16] | do | w | (a, b) [GB_BT][4] | column sums [2][4][C_GROUP] |
+  // db / dg partials [GB_BT][2][64]
+  static constexpr int OFF_K = 0;
   static constexpr int OFF_Q = OFF_K + GB_BT * KT;
   static constexpr int OFF_V = OFF_Q + GB_BT * KT;
   static constexpr int OFF_DO = OFF_V + GB_BT * GB_COLS;
@@ -58,6 +62,7 @@ struct GbShape {
   static constexpr int FLOATS = OFF_RED + GB_BT * 2 * 64;
   static constexpr size_t LDS_BYTES = (size_t)FLOATS * sizeof(float);
   static constexpr int CKPT = KT * GB_COLS;            // floats of one stored state slab
+  static constexpr int HIST = GB_BT * CKPT;            // a block's decayed states (per workgroup, in memory)
 };
 
 template <typename T>
@@ -71,6 +76,8 @@ struct GbArgs {
   const float* mn;          // forward maps [n_seg, HV, K, K + V]
   float* mn_rev;            // COMPOSITE: rows [HV, K, K + V] = [M^T | N']
   float* ckpt;              // states at every GB_BT-th token of every (segment, head, slab)
+  float* hist;              // per workgroup: the decayed states of the block it works on, [GB_BT][Q4][64][4]
+  int64_t units;            // n_seg * HV * slabs (segment, head, slab) units, dealt to the workgroups round robin
   T* dv;
   float *dq_part, *dk_part; // [slabs, total, HV, K]
   float *db_part, *dg_part; // [slabs, total, HV]
@@ -80,19 +87,21 @@ struct GbArgs {
   int l2norm;
 };
 
-__device__ __forceinline__ float gb_rows_sum(float x) {  // over the four row groups of a column (lanes 16 apart)
-  x += __shfl_xor(x, 16);
-  x += __shfl_xor(x, 32);
-  return x;
+// x summed over the four row groups of a column (lanes 16 apart), in every lane: two register swaps, no LDS
+// (permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second, so the two
+// results are (x of row 0 | 0 | 2 | 2) and (1 | 1 | 3 | 3); permlane32_swap does the same with the halves of the wave)
+__device__ __forceinline__ float gb_rows_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 template <typename T, int KT, bool COMPOSITE>
-__global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) {
+__device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float* lds) {
   using SH = GbShape<KT>;
   constexpr int KR = SH::KR, Q4 = SH::Q4, LPT = SH::LPT, PASSES = SH::PASSES, CG = SH::C_GROUP;
-  extern __shared__ float4 s_gb4[];
-  float* lds = reinterpret_cast<float*>(s_gb4);
-  float* s_hist = lds;
   float* s_k = lds + SH::OFF_K;
   float* s_q = lds + SH::OFF_Q;
   float* s_v = lds + SH::OFF_V;
@@ -103,7 +112,10 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
   float* s_red = lds + SH::OFF_RED;
 
   const int lane = threadIdx.x, rg = lane >> 4, j = lane & 15;
-  int64_t bid = blockIdx.x;
+  // the block's decayed states: every lane reads back exactly the 16-byte pieces it wrote (a spill area of its own,
+  // rewritten block after block, so it stays in the caches)
+  float* hist = A.hist + (int64_t)blockIdx.x * SH::HIST + lane * 4;
+  int64_t bid = unit;
   const int slab = (int)(bid % A.slabs);
   bid /= A.slabs;
   const int hv = (int)(bid % A.HV);
@@ -226,7 +238,7 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
     if (keep) {
 #pragma unroll
       for (int m = 0; m < Q4; ++m)
-        *reinterpret_cast<float4*>(s_hist + ((tok * Q4 + m) * 64 + lane) * 4) =
+        *reinterpret_cast<float4*>(hist + (tok * Q4 + m) * 256) =
             make_float4(S[4 * m], S[4 * m + 1], S[4 * m + 2], S[4 * m + 3]);
     }
     const float w = gb_rows_sum((wp[0] + wp[1]) + (wp[2] + wp[3]));
@@ -234,6 +246,7 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
     const float u = bt * (s_v[tok * GB_COLS + j] - w);
 #pragma unroll
     for (int r = 0; r < KR; ++r) S[r] = __builtin_fmaf(kr[r], u, S[r]);
+    __builtin_amdgcn_sched_barrier(0);  // (the next token's operands are not hoisted above this one)
   };
 
   float Hs[KR];
@@ -266,6 +279,7 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
         const float bdu = bt * gb_rows_sum((dup[0] + dup[1]) + (dup[2] + dup[3]));
 #pragma unroll
         for (int r = 0; r < KR; ++r) Hs[r] = a * __builtin_fmaf(-bdu, kr[r], Hs[r]);
+        __builtin_amdgcn_sched_barrier(0);  // (the next token's operands are not hoisted above this one)
       }
       lds_barrier();
     }
@@ -321,6 +335,9 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
 #pragma unroll
       for (int tok = 0; tok < GB_BT; ++tok) fwd_step(tok, S, true);
       lds_barrier();
+      float4 sdn[Q4];
+#pragma unroll
+      for (int m = 0; m < Q4; ++m) sdn[m] = *reinterpret_cast<const float4*>(hist + ((GB_BT - 1) * Q4 + m) * 256);
 #pragma unroll
       for (int tok = GB_BT - 1; tok >= 0; --tok) {
         const int64_t t = tb + tok;
@@ -331,9 +348,10 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
         read_rows(s_k + tok * KT, kr);
         read_rows(s_q + tok * KT, qr);
 #pragma unroll
-        for (int m = 0; m < Q4; ++m) {
-          const float4 x = *reinterpret_cast<const float4*>(s_hist + ((tok * Q4 + m) * 64 + lane) * 4);
+        for (int m = 0; m < Q4; ++m) {  // this token's decayed state; the previous token's is asked for now
+          const float4 x = sdn[m];
           Sd[4 * m] = x.x; Sd[4 * m + 1] = x.y; Sd[4 * m + 2] = x.z; Sd[4 * m + 3] = x.w;
+          if (tok > 0) sdn[m] = *reinterpret_cast<const float4*>(hist + ((tok - 1) * Q4 + m) * 256);
         }
         float dup[4] = {0.0f, 0.0f, 0.0f, 0.0f}, pgp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -383,6 +401,15 @@ __global__ void __launch_bounds__(64) gdr_bwd_segment_kernel(const GbArgs<T> A) 
       }
       lds_barrier();
     }
+  }
+}
+
+template <typename T, int KT, bool COMPOSITE>
+__global__ void __launch_bounds__(64, (KT <= 64 ? 2 : 1)) gdr_bwd_segment_kernel(const GbArgs<T> A) {
+  extern __shared__ float4 s_gb4[];
+  for (int64_t unit = blockIdx.x; unit < A.units; unit += gridDim.x) {
+    gb_unit<T, KT, COMPOSITE>(A, unit, reinterpret_cast<float*>(s_gb4));
+    lds_barrier();
   }
 }
 
@@ -468,7 +495,7 @@ __global__ void __launch_bounds__(256) gdr_bwd_dh0_kernel(const float* __restric
 static int gb_padded_k(int K) { return K <= 16 ? 16 : K <= 32 ? 32 : K <= 64 ? 64 : 128; }
 
 struct GbWorkspace {
-  int64_t mn, sinit, mn_rev, hends, ckpt, dq_part, dk_part, db_part, dg_part, bytes;
+  int64_t mn, sinit, mn_rev, hends, ckpt, hist, dq_part, dk_part, db_part, dg_part, bytes;
 };
 static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int K, int V) {
   const int slabs = (V + GB_COLS - 1) / GB_COLS;
@@ -484,6 +511,7 @@ static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int
   w.mn_rev = take((int64_t)(n_seg + n_seq) * HV * K * (K + V));
   w.hends = take((int64_t)(n_seg + n_seq) * HV * K * V);
   w.ckpt = take((total / GB_BT + n_seg + 1) * HV * slabs * (int64_t)gb_padded_k(K) * GB_COLS);
+  w.hist = take((int64_t)GB_MAX_GRID * GB_BT * gb_padded_k(K) * GB_COLS);
   w.dq_part = take((int64_t)slabs * total * HV * K);
   w.dk_part = take((int64_t)slabs * total * HV * K);
   w.db_part = take((int64_t)slabs * total * HV);
@@ -527,16 +555,15 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
   a.q = (const T*)q; a.k = (const T*)k; a.v = (const T*)v; a.dout = (const T*)dout;
   a.g = g; a.beta = beta;
   a.sinit = sinit; a.hend = hends; a.seg_rev = seg_rev; a.cu_seg = cu_seg;
-  a.mn = mn; a.mn_rev = mn_rev; a.ckpt = (float*)(ws + w.ckpt);
+  a.mn = mn; a.mn_rev = mn_rev; a.ckpt = (float*)(ws + w.ckpt); a.hist = (float*)(ws + w.hist);
   a.dv = (T*)dv;
   a.dq_part = (float*)(ws + w.dq_part); a.dk_part = (float*)(ws + w.dk_part);
   a.db_part = (float*)(ws + w.db_part); a.dg_part = (float*)(ws + w.dg_part);
   a.total = total;
   a.H = H; a.HV = HV; a.K = K; a.V = V; a.slabs = (V + GB_COLS - 1) / GB_COLS;
   a.scale = scale; a.l2norm = l2norm;
-  const int64_t units = (int64_t)n_seg * HV * a.slabs;
-  if (units > 0x7fffffff) return LAMPA_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)units);
+  a.units = (int64_t)n_seg * HV * a.slabs;
+  const dim3 grid((unsigned)(a.units < GB_MAX_GRID ? a.units : GB_MAX_GRID));
 #define GB_SEG(KT, COMP) \
   hipLaunchKernelGGL((gdr_bwd_segment_kernel<T, KT, COMP>), grid, dim3(64), GbShape<KT>::LDS_BYTES, s, a)
 #define GB_SEG_ANY(COMP)                \
