@@ -15,8 +15,9 @@
 //   2  every segment's H from zero backwards: N'; the linear part is M^T        (gdr_bwd_segment_kernel<COMPOSITE>)
 //   3  H_end over the segments of a sequence, last to first                     (the forward scan kernel on [M^T | N'])
 //   4  every segment: forward once, leaving S at every 8th token in memory; then block by block from the end: the
-//      block's 8 decayed states rebuilt (into a spill area of the workgroup: 32 KB at K = 64, which as LDS would leave
-//      three waves per CU), then its tokens backwards                           (gdr_bwd_segment_kernel)
+//      block's 8 decayed states rebuilt (every second one into a spill area of the workgroup -- all eight are 32 KB at
+//      K = 64, which as LDS would leave three waves per CU --, the others from those by one more step on the way
+//      back), then its tokens backwards                                         (gdr_bwd_segment_kernel)
 //   5  partial sums over the column slabs and grouped value heads, the chain rule of the q/k normalisation, output
 //      types                                                                    (gdr_bwd_finish_kernel)
 // A wave owns 16 value columns of one (segment, value head): lane = (row group, column), a lane keeps K / 4 rows of
@@ -62,7 +63,7 @@ struct GbShape {
   static constexpr int FLOATS = OFF_RED + GB_BT * 2 * 64;
   static constexpr size_t LDS_BYTES = (size_t)FLOATS * sizeof(float);
   static constexpr int CKPT = KT * GB_COLS;            // floats of one stored state slab
-  static constexpr int HIST = GB_BT * CKPT;            // a block's decayed states (per workgroup, in memory)
+  static constexpr int HIST = GB_BT / 2 * CKPT;        // every second decayed state of a block (per workgroup, in memory)
 };
 
 template <typename T>
@@ -76,7 +77,7 @@ struct GbArgs {
   const float* mn;          // forward maps [n_seg, HV, K, K + V]
   float* mn_rev;            // COMPOSITE: rows [HV, K, K + V] = [M^T | N']
   float* ckpt;              // states at every GB_BT-th token of every (segment, head, slab)
-  float* hist;              // per workgroup: the decayed states of the block it works on, [GB_BT][Q4][64][4]
+  float* hist;              // per workgroup: decayed states of the block it works on, [GB_BT / 2][Q4][64][4]
   int64_t units;            // n_seg * HV * slabs (segment, head, slab) units, dealt to the workgroups round robin
   T* dv;
   float *dq_part, *dk_part; // [slabs, total, HV, K]
@@ -97,6 +98,10 @@ __device__ __forceinline__ float gb_rows_sum(float x) {
   const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
+
+// A workgroup is one wave, and a wave's LDS instructions execute in the order they were issued: what one lane wrote is
+// there for another lane's later read without a barrier or a wait. Only the compiler has to keep that order.
+__device__ __forceinline__ void gb_wave_fence() { asm volatile("" ::: "memory"); }
 
 template <typename T, int KT, bool COMPOSITE>
 __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float* lds) {
@@ -214,7 +219,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
       s_sc[lane * 4] = live ? expf(greg) : 1.0f;
       s_sc[lane * 4 + 1] = live ? breg : 0.0f;
     }
-    lds_barrier();
+    gb_wave_fence();
   };
   auto read_rows = [&](const float* base, float (&x)[KR]) __attribute__((always_inline)) {
 #pragma unroll
@@ -235,10 +240,10 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
       S[r] *= a;
       wp[r & 3] = __builtin_fmaf(S[r], kr[r], wp[r & 3]);
     }
-    if (keep) {
+    if (keep && (tok & 1) == 0) {  // every second decayed state is kept; the way back rebuilds the one after it
 #pragma unroll
       for (int m = 0; m < Q4; ++m)
-        *reinterpret_cast<float4*>(hist + (tok * Q4 + m) * 256) =
+        *reinterpret_cast<float4*>(hist + ((tok >> 1) * Q4 + m) * 256) =
             make_float4(S[4 * m], S[4 * m + 1], S[4 * m + 2], S[4 * m + 3]);
     }
     const float w = gb_rows_sum((wp[0] + wp[1]) + (wp[2] + wp[3]));
@@ -281,7 +286,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
         for (int r = 0; r < KR; ++r) Hs[r] = a * __builtin_fmaf(-bdu, kr[r], Hs[r]);
         __builtin_amdgcn_sched_barrier(0);  // (the next token's operands are not hoisted above this one)
       }
-      lds_barrier();
+      gb_wave_fence();
     }
     const int W = K + V;
     float* out = A.mn_rev + ((int64_t)A.seg_rev[seg] * HV + hv) * K * W;
@@ -314,7 +319,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
       for (int r = 0; r < KR; ++r) ck[b * ck_stride + r * 64] = S[r];
 #pragma unroll
       for (int tok = 0; tok < GB_BT; ++tok) fwd_step(tok, S, false);
-      lds_barrier();
+      gb_wave_fence();
     }
     // ---- block by block from the end ---------------------------------------------------------------------------------
     float Sn[KR];
@@ -334,10 +339,11 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
       }
 #pragma unroll
       for (int tok = 0; tok < GB_BT; ++tok) fwd_step(tok, S, true);
-      lds_barrier();
+      gb_wave_fence();
       float4 sdn[Q4];
 #pragma unroll
-      for (int m = 0; m < Q4; ++m) sdn[m] = *reinterpret_cast<const float4*>(hist + ((GB_BT - 1) * Q4 + m) * 256);
+      for (int m = 0; m < Q4; ++m)
+        sdn[m] = *reinterpret_cast<const float4*>(hist + (((GB_BT - 2) >> 1) * Q4 + m) * 256);
 #pragma unroll
       for (int tok = GB_BT - 1; tok >= 0; --tok) {
         const int64_t t = tb + tok;
@@ -347,11 +353,27 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
         float kr[KR], qr[KR], Sd[KR];
         read_rows(s_k + tok * KT, kr);
         read_rows(s_q + tok * KT, qr);
+        if (tok & 1) {
+          // an odd token's decayed state from the kept one of the token before: one forward step, the same operations
+          // in the same order as on the way forth
+          float kp[KR];
+          read_rows(s_k + (tok - 1) * KT, kp);
+          const float up = s_sc[(tok - 1) * 4 + 1] * (s_v[(tok - 1) * GB_COLS + j] - s_w[(tok - 1) * GB_COLS + j]);
 #pragma unroll
-        for (int m = 0; m < Q4; ++m) {  // this token's decayed state; the previous token's is asked for now
-          const float4 x = sdn[m];
-          Sd[4 * m] = x.x; Sd[4 * m + 1] = x.y; Sd[4 * m + 2] = x.z; Sd[4 * m + 3] = x.w;
-          if (tok > 0) sdn[m] = *reinterpret_cast<const float4*>(hist + ((tok - 1) * Q4 + m) * 256);
+          for (int m = 0; m < Q4; ++m) {
+            const float4 x = sdn[m];
+            Sd[4 * m] = a * __builtin_fmaf(kp[4 * m], up, x.x);
+            Sd[4 * m + 1] = a * __builtin_fmaf(kp[4 * m + 1], up, x.y);
+            Sd[4 * m + 2] = a * __builtin_fmaf(kp[4 * m + 2], up, x.z);
+            Sd[4 * m + 3] = a * __builtin_fmaf(kp[4 * m + 3], up, x.w);
+          }
+        } else {
+#pragma unroll
+          for (int m = 0; m < Q4; ++m) {  // a kept state; the one two tokens back is asked for now
+            const float4 x = sdn[m];
+            Sd[4 * m] = x.x; Sd[4 * m + 1] = x.y; Sd[4 * m + 2] = x.z; Sd[4 * m + 3] = x.w;
+            if (tok >= 2) sdn[m] = *reinterpret_cast<const float4*>(hist + (((tok - 2) >> 1) * Q4 + m) * 256);
+          }
         }
         float dup[4] = {0.0f, 0.0f, 0.0f, 0.0f}, pgp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -371,7 +393,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
           s_c[(4 + rg) * CG + r * GB_COLS + j] = __builtin_fmaf(Hs[r], u, -bdu * Sd[r]);        // dk
           Hs[r] = a * __builtin_fmaf(-bdu, kr[r], Hs[r]);
         }
-        lds_barrier();
+        gb_wave_fence();
 #pragma unroll
         for (int o = lane; o < 2 * KT; o += 64) {  // the sums over this wave's 16 columns, one (gradient, row) per lane
           const int which = o / KT, i = o % KT;
@@ -381,7 +403,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
                             (((x2.x + x2.y) + (x2.z + x2.w)) + ((x3.x + x3.y) + (x3.z + x3.w)));
           if (i < K && live) (which ? A.dk_part : A.dq_part)[(((int64_t)slab * total + t) * HV + hv) * K + i] = sum;
         }
-        lds_barrier();
+        gb_wave_fence();
       }
       {  // db and dg of the block's tokens: 8 lanes per token
         const int tok = lane >> 3, sub = lane & 7;
@@ -399,7 +421,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
           A.dg_part[((int64_t)slab * total + tb + tok) * HV + hv] = sg;
         }
       }
-      lds_barrier();
+      gb_wave_fence();
     }
   }
 }
@@ -409,7 +431,7 @@ __global__ void __launch_bounds__(64, (KT <= 64 ? 2 : 1)) gdr_bwd_segment_kernel
   extern __shared__ float4 s_gb4[];
   for (int64_t unit = blockIdx.x; unit < A.units; unit += gridDim.x) {
     gb_unit<T, KT, COMPOSITE>(A, unit, reinterpret_cast<float*>(s_gb4));
-    lds_barrier();
+    gb_wave_fence();
   }
 }
 
@@ -444,8 +466,18 @@ __global__ void __launch_bounds__(256) gdr_bwd_finish_kernel(const T* __restrict
       dy[n] = 0.0f;
       if (i < K) {
         x[n] = GdrElem<T>::to_float(x_in[(t * H + h) * K + i]);
-        for (int s = 0; s < slabs; ++s)
-          for (int gq = 0; gq < G; ++gq) dy[n] += part[(((int64_t)s * total + t) * HV + h * G + gq) * K + i];
+        // the partial sums of this entry: (slab, value head of the group), four loads in flight at a time
+        const int n_part = slabs * G;
+        for (int c0 = 0; c0 < n_part; c0 += 4) {
+          float p4[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int c = min(c0 + u, n_part - 1), sl = c / G, gq = c - sl * G;
+            p4[u] = part[(((int64_t)sl * total + t) * HV + h * G + gq) * K + i];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) dy[n] += c0 + u < n_part ? p4[u] : 0.0f;
+        }
       }
     }
     if (l2norm != GDR_L2_NONE) {
@@ -511,7 +543,7 @@ static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int
   w.mn_rev = take((int64_t)(n_seg + n_seq) * HV * K * (K + V));
   w.hends = take((int64_t)(n_seg + n_seq) * HV * K * V);
   w.ckpt = take((total / GB_BT + n_seg + 1) * HV * slabs * (int64_t)gb_padded_k(K) * GB_COLS);
-  w.hist = take((int64_t)GB_MAX_GRID * GB_BT * gb_padded_k(K) * GB_COLS);
+  w.hist = take((int64_t)GB_MAX_GRID * (GB_BT / 2) * gb_padded_k(K) * GB_COLS);
   w.dq_part = take((int64_t)slabs * total * HV * K);
   w.dk_part = take((int64_t)slabs * total * HV * K);
   w.db_part = take((int64_t)slabs * total * HV);
