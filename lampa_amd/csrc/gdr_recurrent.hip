@@ -143,6 +143,11 @@ __device__ __forceinline__ float rec_half_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+template <bool B>
+struct RecLazy {
+  static constexpr bool value = B;
+};
+
 template <typename T>
 __device__ __forceinline__ float4 rec_load4(const T* p) {
   if constexpr (sizeof(T) == 4) {
@@ -178,6 +183,7 @@ __global__ void __launch_bounds__(64)
   __shared__ float4 s_kq[2][(G + 2) * ROW4];
   __shared__ float4 s_sc[2][G + 2];
   __shared__ float s_v[2][(G + 2) * 32];
+  __shared__ float s_fold[2];  // per group: the decay over the whole group if it runs in the lazy form, else 0
   const int lane = threadIdx.x, half = lane >> 5, cl = lane & 31;
   const int col = blockIdx.x * 32 + cl;
   const bool active = col < V;
@@ -234,6 +240,15 @@ __global__ void __launch_bounds__(64)
         const int cc = (int)blockIdx.x * 32 + (lane + 64 * n) % 32 - (COMPOSITE ? K : 0);
         s_v[buf][lane + 64 * n] = (COMPOSITE && cc < 0) ? 0.0f : vals[n];
       }
+      // The decay is not applied to the state token by token: within a group the registers hold S / c_j, c_j = the
+      // decay from the group's start up to token j, and c_j goes into the token's scalars instead (a multiply per
+      // state element and token less); the state is brought back to scale once per group. With more than e^60 of
+      // decay (or growth) inside one group 1 / c_j would leave the fp32 range: such a group runs in the direct form.
+      const float g_use = (lane < G && live) ? g_tok : 0.0f;
+      const float cum = wave_inclusive_scan(g_use);
+      const float span = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_inclusive_scan(fabsf(g_use))), 63));
+      const bool lazy = span <= 60.0f;  // (false for a NaN as well)
+      if (lane == G - 1) s_fold[buf] = lazy ? expf(cum) : 0.0f;
       if (lane < G) {
         float kss = 0.0f, qss = 0.0f;
 #pragma unroll
@@ -251,7 +266,13 @@ __global__ void __launch_bounds__(64)
           qinv = 1.0f / (__fsqrt_rn(qss) + 1e-6f);
         }
         // a token past the end is a step that changes nothing (d = 0, decay 1), so the steps need no branch
-        s_sc[buf][lane] = live ? make_float4(kinv, qinv * scale, expf(g_tok), b_tok) : make_float4(0.0f, 0.0f, 1.0f, 0.0f);
+        // direct: 1 / |k|, scale / |q|, e^g, beta; lazy: c / |k|, c scale / |q|, 1 / (c |k|), beta
+        float4 sc = live ? make_float4(kinv, qinv * scale, expf(g_tok), b_tok) : make_float4(0.0f, 0.0f, 1.0f, 0.0f);
+        if (lazy) {
+          const float c = expf(cum), rc = expf(-cum);
+          sc = live ? make_float4(kinv * c, qinv * scale * c, kinv * rc, b_tok) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        s_sc[buf][lane] = sc;
       }
     };
     // a token's operands: its scalars, this lane's RP elements of k and of q, its v
@@ -260,7 +281,7 @@ __global__ void __launch_bounds__(64)
       float v;
     };
     auto read_token = [&](int buf, int j, Operands& x) __attribute__((always_inline)) {
-      x.sc = s_sc[buf][j];  // 1 / |k|, scale / |q|, e^g, beta
+      x.sc = s_sc[buf][j];  // the token's four scalars (direct or lazy form, see commit)
       const float4* kr = &s_kq[buf][j * ROW4 + half * (RP / 4)];
 #pragma unroll
       for (int r4 = 0; r4 < RP / 4; ++r4) {
@@ -279,44 +300,56 @@ __global__ void __launch_bounds__(64)
       // two tokens per round on two operand sets: a token's operands are requested before the arithmetic of the token
       // before it starts, so their LDS latency hides behind it. The token after the last of an odd count is a step
       // that changes nothing.
-      auto step = [&](const Operands& x, int64_t t) __attribute__((always_inline)) {
-        float kk[RP], qq[RP];
+      auto run_group = [&](auto lazy_tag) __attribute__((always_inline)) {
+        constexpr bool LAZY = decltype(lazy_tag)::value;
+        auto step = [&](const Operands& x, int64_t t) __attribute__((always_inline)) {
+          float kk[RP], qq[RP];
 #pragma unroll
-        for (int r4 = 0; r4 < RP / 4; ++r4) {
-          kk[4 * r4] = x.kk[r4].x; kk[4 * r4 + 1] = x.kk[r4].y; kk[4 * r4 + 2] = x.kk[r4].z; kk[4 * r4 + 3] = x.kk[r4].w;
-          qq[4 * r4] = x.qq[r4].x; qq[4 * r4 + 1] = x.qq[r4].y; qq[4 * r4 + 2] = x.qq[r4].z; qq[4 * r4 + 3] = x.qq[r4].w;
-        }
-        float dot4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int r = 0; r < RP; ++r) dot4[r & 3] = __builtin_fmaf(S[r], kk[r], dot4[r & 3]);
-        const float dot = rec_half_sum((dot4[0] + dot4[1]) + (dot4[2] + dot4[3]));
-        // S <- e^g S, then d = beta (v - S^T k), S <- S + k d^T, o = S^T q, with k = k_raw / |k|
-        const float4 sc = x.sc;
-        const float d = sc.w * (x.v - sc.z * sc.x * dot);
-        const float dk = d * sc.x;
-        if constexpr (COMPOSITE) {
-#pragma unroll
-          for (int r = 0; r < RP; ++r) S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
-        } else {
-          float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-          for (int r = 0; r < RP; ++r) {
-            S[r] = __builtin_fmaf(kk[r], dk, sc.z * S[r]);
-            out4[r & 3] = __builtin_fmaf(S[r], qq[r], out4[r & 3]);
+          for (int r4 = 0; r4 < RP / 4; ++r4) {
+            kk[4 * r4] = x.kk[r4].x; kk[4 * r4 + 1] = x.kk[r4].y; kk[4 * r4 + 2] = x.kk[r4].z; kk[4 * r4 + 3] = x.kk[r4].w;
+            qq[4 * r4] = x.qq[r4].x; qq[4 * r4 + 1] = x.qq[r4].y; qq[4 * r4 + 2] = x.qq[r4].z; qq[4 * r4 + 3] = x.qq[r4].w;
           }
-          const float out = rec_half_sum((out4[0] + out4[1]) + (out4[2] + out4[3]));
-          if (active && half == 0 && t < eos) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out * sc.y);
+          float dot4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int r = 0; r < RP; ++r) dot4[r & 3] = __builtin_fmaf(S[r], kk[r], dot4[r & 3]);
+          const float dot = rec_half_sum((dot4[0] + dot4[1]) + (dot4[2] + dot4[3]));
+          // S <- e^g S, then d = beta (v - S^T k), S <- S + k d^T, o = S^T q, with k = k_raw / |k|; in the lazy form on
+          // S / c_j, where the decay is part of the scalars
+          const float4 sc = x.sc;
+          const float d = LAZY ? sc.w * (x.v - sc.x * dot) : sc.w * (x.v - sc.z * sc.x * dot);
+          const float dk = LAZY ? d * sc.z : d * sc.x;
+          if constexpr (COMPOSITE) {
+#pragma unroll
+            for (int r = 0; r < RP; ++r) S[r] = __builtin_fmaf(kk[r], dk, LAZY ? S[r] : sc.z * S[r]);
+          } else {
+            float out4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int r = 0; r < RP; ++r) {
+              S[r] = __builtin_fmaf(kk[r], dk, LAZY ? S[r] : sc.z * S[r]);
+              out4[r & 3] = __builtin_fmaf(S[r], qq[r], out4[r & 3]);
+            }
+            const float out = rec_half_sum((out4[0] + out4[1]) + (out4[2] + out4[3]));
+            if (active && half == 0 && t < eos) o[(t * HV + hv) * V + col] = GdrElem<T>::from_float(out * sc.y);
+          }
+        };
+        Operands xa, xb;
+        read_token(buf, 0, xa);
+        for (int j = 0; j < n_tok; j += 2) {
+          read_token(buf, j + 1, xb);
+          __builtin_amdgcn_sched_barrier(0);
+          step(xa, t0 + j);
+          read_token(buf, j + 2, xa);
+          __builtin_amdgcn_sched_barrier(0);
+          step(xb, t0 + j + 1);
         }
       };
-      Operands xa, xb;
-      read_token(buf, 0, xa);
-      for (int j = 0; j < n_tok; j += 2) {
-        read_token(buf, j + 1, xb);
-        __builtin_amdgcn_sched_barrier(0);
-        step(xa, t0 + j);
-        read_token(buf, j + 2, xa);
-        __builtin_amdgcn_sched_barrier(0);
-        step(xb, t0 + j + 1);
+      const float fold = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_fold[buf])));
+      if (fold != 0.0f) {
+        run_group(RecLazy<true>{});
+#pragma unroll
+        for (int r = 0; r < RP; ++r) S[r] *= fold;  // back to scale: S = c_last (S / c_last)
+      } else {
+        run_group(RecLazy<false>{});
       }
       if (more) commit(buf ^ 1, t0 + G + lane < eos);
     }

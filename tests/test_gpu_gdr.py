@@ -80,6 +80,36 @@ def test_recurrent_many_short_sequences_both_kernels(device):
         assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL, n
 
 
+@pytest.mark.parametrize("K,V", [(16, 32), (64, 64), (128, 16)])
+def test_recurrent_strong_mixed_and_positive_decay(device, K, V):
+    """The split kernel keeps the state divided by the decay accumulated inside a group of tokens and falls back to the
+    plain form for a group whose decay would leave the fp32 range: runs of g = -9 per token (e^-144 over 16 tokens)
+    between runs of weak decay, a stretch of g = -100 (e^g = 0 in fp32: the state is wiped) and a few positive g, with
+    and without segments."""
+    gen = torch.Generator().manual_seed(K)
+    T, H = 1100, 2
+    q, k = (torch.randn(1, T, H, K, generator=gen) for _ in range(2))
+    v = torch.randn(1, T, H, V, generator=gen)
+    g = -0.05 * torch.rand(1, T, H, generator=gen)
+    g[:, 100:180] = -9.0
+    g[:, 300:303] = -100.0
+    g[:, 400:520:7] = 0.3
+    g[:, 700:900, 1] = -4.0 * torch.rand(200, generator=gen)
+    beta = torch.rand(1, T, H, generator=gen)
+    h0 = torch.randn(1, H, K, V, generator=gen)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, l2=og.L2_RECURRENT)
+    for seg_min in (512, None):
+        old = gd.SEGMENT_MIN_TOKENS
+        gd.SEGMENT_MIN_TOKENS = seg_min
+        try:
+            o, s = gd.fused_recurrent_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device),
+                                                       output_final_state=True, use_qk_l2norm_in_kernel=True)
+        finally:
+            gd.SEGMENT_MIN_TOKENS = old
+        assert torch.isfinite(o).all() and torch.isfinite(s).all()
+        assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL, seg_min
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_recurrent_long_sequences_run_as_segments(device, dtype):
     # a few long sequences (one of them empty, one shorter than a segment) are cut into segments that run in parallel;
