@@ -164,7 +164,7 @@ __device__ __forceinline__ float4 rec_load4(const T* p) {
 // the state it starts from, S_end = M S_0 + N: the wave's columns are columns of [M | N] (V = K + the value width),
 // started from [I | 0], the M columns see v = 0; nothing is written but ht (fp32 [n_seq, HV, K, V]). ht_map (nullable)
 // gives the row of ht that a sequence's final state goes to (negative: not stored).
-template <typename T, int KT, bool COMPOSITE>
+template <typename T, int KT, bool COMPOSITE, bool SHORT_GROUPS = false>
 __global__ void __launch_bounds__(64)
     gdr_recurrent_split_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                const float* __restrict__ g, const float* __restrict__ beta, T* __restrict__ o,
@@ -172,7 +172,10 @@ __global__ void __launch_bounds__(64)
                                const int64_t* __restrict__ cu_seqlens, int64_t t_len, int H, int HV, int K, int V,
                                float scale, int l2norm, const int32_t* __restrict__ ht_map) {
   constexpr int RP = KT / 2;                          // state rows per lane
-  constexpr int G = 1024 / KT < 64 ? 1024 / KT : 64;  // tokens per group (LDS for one wave per SIMD of a CU)
+  // tokens per group: 24 KB of LDS per wave at K >= 64 (six waves per CU); SHORT_GROUPS halves that for launches of
+  // more waves than that holds at once (built for KT = 64, where eight then fit and a launch of 2016 waves needs one
+  // round instead of two: 1.11 -> 0.73 ms; with fewer waves the longer groups are faster, 207 against 230 us)
+  constexpr int G = (SHORT_GROUPS ? 512 : 1024) / KT < 64 ? (SHORT_GROUPS ? 512 : 1024) / KT : 64;
   constexpr int ROW4 = (2 * KT + 4) / 4;              // 16-byte pieces per token in LDS: k | q, padded against conflicts
   constexpr int PPT = 2 * KT / 4;                     // 4-element pieces of k | q per token
   constexpr int PIECES = G * PPT / 64;                // pieces per lane and group
@@ -364,6 +367,9 @@ __global__ void __launch_bounds__(64)
   }
 }
 
+// more waves than six per CU of the 256 (what the long groups' LDS holds at once)
+static inline bool gdr_rec_short_groups(const dim3& grid) { return (int64_t)grid.x * grid.y > 6 * 256; }
+
 template <typename T>
 static int gdr_recurrent_launch(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                 void* o, const float* h0, float* ht, const int64_t* cu, int n_seq, int64_t t_len,
@@ -380,8 +386,13 @@ static int gdr_recurrent_launch(const void* q, const void* k, const void* v, con
                      (const T*)v, g, beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm, ht_map)
     if (K <= 16) GDR_REC_SPLIT(16);
     else if (K <= 32) GDR_REC_SPLIT(32);
-    else if (K <= 64) GDR_REC_SPLIT(64);
-    else GDR_REC_SPLIT(128);
+    else if (K <= 64) {
+      if (gdr_rec_short_groups(grid2))
+        hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, 64, false, true>), grid2, dim3(64), 0, s, (const T*)q,
+                           (const T*)k, (const T*)v, g, beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm,
+                           ht_map);
+      else GDR_REC_SPLIT(64);
+    } else GDR_REC_SPLIT(128);
 #undef GDR_REC_SPLIT
     LAMPA_PROF(s, "gdr_recurrent_split_kernel");
     return lampa_launch_status();
@@ -563,9 +574,10 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
   }
   LAMPA_PROF(s, "start");
   const dim3 grid_a((K + V + 31) / 32, n_seg * HV), grid_b((V + 31) / 32, n_seg * HV);
-#define GDR_REC_SEG(KT)                                                                                              \
+#define GDR_REC_SEG(KT) GDR_REC_SEG2(KT, false, false)
+#define GDR_REC_SEG2(KT, SHORT_A, SHORT_B)                                                                           \
   do {                                                                                                               \
-    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, true>), grid_a, dim3(64), 0, s, (const T*)k, (const T*)k,  \
+    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, true, SHORT_A>), grid_a, dim3(64), 0, s, (const T*)k, (const T*)k,  \
                        (const T*)v, g, beta, (T*)nullptr, (const float*)nullptr, mn, cu_seg, (int64_t)0, H, HV, K,   \
                        K + V, scale, l2norm, (const int32_t*)nullptr);                                               \
     LAMPA_PROF(s, "gdr_recurrent_split_kernel<composite>");                                                          \
@@ -573,16 +585,22 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
                        dim3((V + 31) / 32, n_seq, HV), dim3(256), RsScanShape<KT>::LDS_BYTES, s, mn, h0, seq_seg0,   \
                        HV, K, V, sinit);                                                                             \
     LAMPA_PROF(s, "gdr_segment_scan_kernel");                                                                        \
-    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false>), grid_b, dim3(64), 0, s, (const T*)q, (const T*)k, \
+    hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false, SHORT_B>), grid_b, dim3(64), 0, s, (const T*)q, (const T*)k, \
                        (const T*)v, g, beta, (T*)o, sinit, ht, cu_seg, (int64_t)0, H, HV, K, V, scale, l2norm,       \
                        seg_out);                                                                                     \
     LAMPA_PROF(s, "gdr_recurrent_split_kernel");                                                                     \
   } while (0)
+  const bool short_a = gdr_rec_short_groups(grid_a), short_b = gdr_rec_short_groups(grid_b);
   if (K <= 16) GDR_REC_SEG(16);
   else if (K <= 32) GDR_REC_SEG(32);
-  else if (K <= 64) GDR_REC_SEG(64);
-  else GDR_REC_SEG(128);
+  else if (K <= 64) {
+    if (short_a && short_b) GDR_REC_SEG2(64, true, true);
+    else if (short_a) GDR_REC_SEG2(64, true, false);
+    else if (short_b) GDR_REC_SEG2(64, false, true);
+    else GDR_REC_SEG(64);
+  } else GDR_REC_SEG(128);
 #undef GDR_REC_SEG
+#undef GDR_REC_SEG2
   return lampa_launch_status();
 }
 
@@ -613,8 +631,13 @@ static void gdr_segment_maps_typed(const void* k, const void* v, const float* g,
                      K + V, 1.0f, l2norm, (const int32_t*)nullptr)
   if (K <= 16) GDR_REC_MAPS(16);
   else if (K <= 32) GDR_REC_MAPS(32);
-  else if (K <= 64) GDR_REC_MAPS(64);
-  else GDR_REC_MAPS(128);
+  else if (K <= 64) {
+    if (gdr_rec_short_groups(grid_a))
+      hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, 64, true, true>), grid_a, dim3(64), 0, s, (const T*)k,
+                         (const T*)k, (const T*)v, g, beta, (T*)nullptr, (const float*)nullptr, mn, cu_seg, (int64_t)0,
+                         H, HV, K, K + V, 1.0f, l2norm, (const int32_t*)nullptr);
+    else GDR_REC_MAPS(64);
+  } else GDR_REC_MAPS(128);
 #undef GDR_REC_MAPS
 }
 
