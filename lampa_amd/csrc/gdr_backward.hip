@@ -29,6 +29,10 @@
 
 #define GB_BT 8     // tokens per block: states kept in LDS at a time, distance of the states kept in memory
 #define GB_COLS 16  // value columns per wave
+// what the segment kernel writes once and reads once or never (the states every GB_BT tokens, the partial dq / dk)
+// goes around the caches' replacement order, which leaves the L2 to the spill areas (segment kernel 2.45 -> 2.32 ms)
+#define GB_STREAM_STORE(v, p) __builtin_nontemporal_store((v), (p))
+#define GB_STREAM_LOAD(p) __builtin_nontemporal_load(p)
 #define GB_MAX_GRID 4096  // workgroups of the segment kernel (each owns a spill area for a block's states)
 
 template <typename T>
@@ -316,7 +320,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
       commit(b);
       fetch(b + 1);
 #pragma unroll
-      for (int r = 0; r < KR; ++r) ck[b * ck_stride + r * 64] = S[r];
+      for (int r = 0; r < KR; ++r) GB_STREAM_STORE(S[r], &ck[b * ck_stride + r * 64]);
 #pragma unroll
       for (int tok = 0; tok < GB_BT; ++tok) fwd_step(tok, S, false);
       gb_wave_fence();
@@ -326,7 +330,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
     if (n_blk > 0) {
       fetch(n_blk - 1);
 #pragma unroll
-      for (int r = 0; r < KR; ++r) Sn[r] = ck[(n_blk - 1) * ck_stride + r * 64];
+      for (int r = 0; r < KR; ++r) Sn[r] = GB_STREAM_LOAD(&ck[(n_blk - 1) * ck_stride + r * 64]);
     }
     for (int b = n_blk - 1; b >= 0; --b) {
       const int64_t tb = t0 + (int64_t)b * GB_BT;
@@ -335,7 +339,7 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         S[r] = Sn[r];
-        Sn[r] = ck[max(b - 1, 0) * ck_stride + r * 64];
+        Sn[r] = GB_STREAM_LOAD(&ck[max(b - 1, 0) * ck_stride + r * 64]);
       }
 #pragma unroll
       for (int tok = 0; tok < GB_BT; ++tok) fwd_step(tok, S, true);
@@ -401,7 +405,8 @@ __device__ __forceinline__ void gb_unit(const GbArgs<T>& A, int64_t unit, float*
           const float4 x0 = p[0], x1 = p[1], x2 = p[2], x3 = p[3];
           const float sum = (((x0.x + x0.y) + (x0.z + x0.w)) + ((x1.x + x1.y) + (x1.z + x1.w))) +
                             (((x2.x + x2.y) + (x2.z + x2.w)) + ((x3.x + x3.y) + (x3.z + x3.w)));
-          if (i < K && live) (which ? A.dk_part : A.dq_part)[(((int64_t)slab * total + t) * HV + hv) * K + i] = sum;
+          if (i < K && live)
+            GB_STREAM_STORE(sum, &(which ? A.dk_part : A.dq_part)[(((int64_t)slab * total + t) * HV + hv) * K + i]);
         }
         gb_wave_fence();
       }
