@@ -85,6 +85,20 @@ def test_gradients_varlen_segments(device, dtype, monkeypatch):
     _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, True), want, dtype)
 
 
+def test_gradients_many_short_sequences_more_units_than_workgroups(device):
+    """700 packed sequences of 1 .. 20 tokens: 700 segments x 4 heads x 2 slabs = 5 600 units for the segment kernel's
+    4 096 workgroups, so some workgroups take a second unit (and reuse their spill area and LDS for it)."""
+    gen = torch.Generator().manual_seed(13)
+    lens = torch.randint(1, 21, (700,), generator=gen).tolist()
+    T = sum(lens)
+    (q, k, v, g, beta, do), gen = _inputs(1, T, 2, 4, 16, 32, torch.float32, 17, unit=False)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.long)
+    h0 = 0.5 * torch.randn(700, 4, 16, 32, generator=gen)
+    dht = torch.randn(700, 4, 16, 32, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, do, dht, None, h0, cu, og.L2_CHUNK)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, True), want, torch.float32)
+
+
 def test_gradients_without_states_and_with_unused_output(device):
     """No initial state (no d h0), no final state; and a loss that uses the final state only (d o is zero)."""
     (q, k, v, g, beta, do), gen = _inputs(1, 200, 1, 2, 64, 64, torch.float32, 3, unit=True)
