@@ -12,7 +12,7 @@
  *     (device, caller stream) that lampa_hgdn_chunk_fwd creates on first use and keeps until the process ends (calls
  *     on different streams or host threads never share them); the fixed scratch array of lampa_sort_pairs_static;
  *     per device, how many workgroups of the one-launch LSH kernel the GPU holds (looked up once) and a flag that the
- *     dynamic-LDS limits of the chunk and step kernels have been raised (set on the first call on that device).
+ *     dynamic-LDS limits of the chunk, step, scan and backward kernels have been raised (set on the first call there).
  *     Everything else lives in caller-owned buffers, so calls on different streams do not interfere.
  * The reference (chengjiang123/Lampa) is Python over Triton/ATen, so each entry point names the Python operator or
  * kernel it replaces (file:line in the reference tree).
