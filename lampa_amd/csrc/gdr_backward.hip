@@ -27,8 +27,9 @@
 // walk through the (segment, head, slab) units.
 #include "gdr_common.h"
 
-#define GB_BT 8     // tokens per block: states kept in LDS at a time, distance of the states kept in memory
+#define GB_BT 8     // tokens per block: decayed states rebuilt at a time, distance of the states kept in memory
 #define GB_COLS 16  // value columns per wave
+#define GB_FIN_TOKENS 4  // tokens per wave of the finish kernel
 // what the segment kernel writes once and reads once or never (the states every GB_BT tokens, the partial dq / dk)
 // goes around the caches' replacement order, which leaves the L2 to the spill areas (segment kernel 2.45 -> 2.32 ms)
 #define GB_STREAM_STORE(v, p) __builtin_nontemporal_store((v), (p))
@@ -455,9 +456,9 @@ __global__ void __launch_bounds__(256) gdr_bwd_finish_kernel(const T* __restrict
                                                             int slabs, int l2norm) {
   const int64_t wave = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
   const int lane = threadIdx.x & 63;
-  if (wave >= total * H) return;
-  const int64_t t = wave / H;
   const int h = (int)(wave % H), G = HV / H;
+  // GB_FIN_TOKENS consecutive tokens per wave (a wave per token is over before its loads are back)
+  for (int64_t t = wave / H * GB_FIN_TOKENS; t < min(total, (wave / H + 1) * GB_FIN_TOKENS); ++t) {
 #pragma unroll
   for (int which = 0; which < 2; ++which) {
     const T* x_in = which ? k : q;
@@ -516,6 +517,7 @@ __global__ void __launch_bounds__(256) gdr_bwd_finish_kernel(const T* __restrict
     }
     dbeta[t * HV + hv] = sb;
     dg[t * HV + hv] = sg;
+  }
   }
 }
 
@@ -622,7 +624,7 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
   LAMPA_PROF(s, "gdr_bwd_segment_kernel");
 #undef GB_SEG_ANY
 #undef GB_SEG
-  const int64_t waves = total * H;
+  const int64_t waves = (total + GB_FIN_TOKENS - 1) / GB_FIN_TOKENS * H;
   hipLaunchKernelGGL((gdr_bwd_finish_kernel<T>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, (const T*)q,
                      (const T*)k, a.dq_part, a.dk_part, a.db_part, a.dg_part, (T*)dq, (T*)dk, dbeta, dg, total, H, HV, K,
                      a.slabs, l2norm);
