@@ -534,7 +534,7 @@ __global__ void __launch_bounds__(256) gdr_bwd_dh0_kernel(const float* __restric
 static int gb_padded_k(int K) { return K <= 16 ? 16 : K <= 32 ? 32 : K <= 64 ? 64 : 128; }
 
 struct GbWorkspace {
-  int64_t mn, sinit, mn_rev, hends, ckpt, hist, dq_part, dk_part, db_part, dg_part, bytes;
+  int64_t mn, sinit, mn_rev, hends, groups, ckpt, hist, dq_part, dk_part, db_part, dg_part, bytes;
 };
 static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int K, int V) {
   const int slabs = (V + GB_COLS - 1) / GB_COLS;
@@ -549,6 +549,7 @@ static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int
   w.sinit = take((int64_t)n_seg * HV * K * V);
   w.mn_rev = take((int64_t)(n_seg + n_seq) * HV * K * (K + V));
   w.hends = take((int64_t)(n_seg + n_seq) * HV * K * V);
+  w.groups = take(gdr_scan_group_floats(n_seg + n_seq, HV, K, V));
   w.ckpt = take((total / GB_BT + n_seg + 1) * HV * slabs * (int64_t)gb_padded_k(K) * GB_COLS);
   w.hist = take((int64_t)GB_MAX_GRID * (GB_BT / 2) * gb_padded_k(K) * GB_COLS);
   w.dq_part = take((int64_t)slabs * total * HV * K);
@@ -587,7 +588,8 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
   float* hends = (float*)(ws + w.hends);
   int rc = gdr_segment_maps(k, v, g, beta, cu_seg, n_seg, H, HV, K, V, dtype, l2norm, mn, s);
   if (rc != LAMPA_OK) return rc;
-  rc = gdr_segment_scan(mn, h0, seq_seg0, n_seq, HV, K, V, sinit, s);
+  float* groups = gdr_scan_group_floats(n_seg + n_seq, HV, K, V) ? (float*)(ws + w.groups) : nullptr;
+  rc = gdr_segment_scan(mn, h0, seq_seg0, n_seq, n_seg, HV, K, V, sinit, groups, s);
   if (rc != LAMPA_OK) return rc;
 
   GbArgs<T> a;
@@ -617,7 +619,7 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
   LAMPA_PROF(s, "gdr_bwd_segment_kernel<composite>");
   rc = lampa_launch_status();
   if (rc != LAMPA_OK) return rc;
-  rc = gdr_segment_scan(mn_rev, dht, seq_seg0_rev, n_seq, HV, K, V, hends, s);
+  rc = gdr_segment_scan(mn_rev, dht, seq_seg0_rev, n_seq, n_seg + n_seq, HV, K, V, hends, groups, s);
   if (rc != LAMPA_OK) return rc;
   LAMPA_PROF(s, "start");
   GB_SEG_ANY(false);

@@ -129,8 +129,12 @@ __device__ __forceinline__ void lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)
 
 // Pieces of the segmented token-serial forward (gdr_recurrent.hip) that the backward pass (gdr_backward.hip) runs on
 // their own: every segment's affine map [M | N] (mn [n_seg, HV, K, K + V], fp32), and the serial product of the maps
-// over each sequence's segments (sinit [n_seg, HV, K, V]: the state each segment starts from; h0 nullable).
+// over each sequence's segments (sinit [n_seg, HV, K, V]: the state each segment starts from; h0 nullable), for a few
+// long sequences in three launches over groups of segments (`groups`: scratch of gdr_scan_group_floats floats or NULL).
 int gdr_segment_maps(const void* k, const void* v, const float* g, const float* beta, const int64_t* cu_seg, int n_seg,
                      int H, int HV, int K, int V, int dtype, int l2norm, float* mn, hipStream_t s);
-int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, int n_seq, int HV, int K, int V,
-                     float* sinit, hipStream_t s);
+int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, int n_seq, int n_seg, int HV, int K,
+                     int V, float* sinit, float* groups, hipStream_t s);
+// floats of the `groups` area (the groups' maps and start states of the scan's three-launch form; 0: not used at this
+// size, pass NULL)
+int64_t gdr_scan_group_floats(int n_seg, int HV, int K, int V);

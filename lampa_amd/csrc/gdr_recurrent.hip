@@ -439,10 +439,22 @@ struct RsScanShape {
   static constexpr size_t LDS_BYTES = ((size_t)ROWS * MS + (size_t)KT * 33 + (size_t)KS * ROWS * 33) * sizeof(float);
 };
 
-template <int KT, int DEPTH>
+// What a workgroup's range of maps is (blockIdx.y) and what it writes:
+//   RS_PLAIN    a sequence's segments; the state each segment starts from (the last map is not applied)
+//   RS_COMPOSE  group `grp` (gs consecutive segments) of sequence `seq`, blockIdx.y = seq * maxg + grp, on the K + V
+//               columns of [I | 0]: every map of the group is applied and only the result, the group's own map
+//               [M | N], is stored (template COMPOSE; V counts all K + V columns there)
+//   RS_GROUPS   a sequence's groups, the maps being the groups' maps: the state each group starts from
+//   RS_WITHIN   a group's segments from the state the group starts with (h0 row = blockIdx.y)
+// A long sequence is scanned as RS_COMPOSE -> RS_GROUPS -> RS_WITHIN: three launches of about sqrt(n) dependent steps
+// each instead of one of n.
+enum { RS_PLAIN = 0, RS_COMPOSE = 1, RS_GROUPS = 2, RS_WITHIN = 3 };
+
+template <int KT, int DEPTH, bool COMPOSE = false>
 __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __restrict__ mn, const float* __restrict__ h0,
                                                               const int32_t* __restrict__ seq_seg0, int HV, int K, int V,
-                                                              float* __restrict__ sinit) {
+                                                              float* __restrict__ sinit, int mode, int gs, int maxg,
+                                                              int W) {
   using SH = RsScanShape<KT>;
   constexpr int MS = SH::MS, RT = SH::RT, KS = SH::KS, ROWS = SH::ROWS;
   constexpr int K4 = KT / 4;                          // 16-byte pieces per row of M
@@ -458,16 +470,36 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
   const int tid = threadIdx.x, c = tid & 31, rg = tid >> 5;
   const int wave = tid >> 6, ln = tid & 31, hh = (tid >> 5) & 1;
   const int rt = wave % RT, ks = wave / RT;
-  const int seq = blockIdx.y, hv = blockIdx.z;
+  const int hv = blockIdx.z;
   const int col = blockIdx.x * 32 + c;
   const int colc = col < V ? col : V - 1;  // (lanes past V shadow the last column: same loads, same stores)
+  // the range of maps [p0, p1) and the row of h0
+  int p0, p1, row0 = blockIdx.y;
+  if (mode == RS_PLAIN) {
+    p0 = seq_seg0[blockIdx.y];
+    p1 = seq_seg0[blockIdx.y + 1];
+  } else if (mode == RS_GROUPS) {
+    const int n = seq_seg0[blockIdx.y + 1] - seq_seg0[blockIdx.y];
+    p0 = blockIdx.y * maxg;
+    p1 = p0 + (n + gs - 1) / gs;
+  } else {  // a group of a sequence
+    const int seq = blockIdx.y / maxg, grp = blockIdx.y - seq * maxg;
+    const int s1 = seq_seg0[seq + 1];
+    p0 = seq_seg0[seq] + grp * gs;
+    p1 = min(p0 + gs, s1);
+  }
+  if (p0 >= p1) return;
+  const int p_last = p1 - 1;      // the last map that exists in the range
+  if (COMPOSE) p1 += 1;           // one more (virtual) segment, so that the loop below applies all of them
 #pragma unroll
   for (int n = 0; n < NR; ++n) {
     const int i = rg + 8 * n;
-    s_S[i * 33 + c] = (h0 && i < K) ? h0[(((int64_t)seq * HV + hv) * K + i) * V + colc] : 0.0f;
+    if (COMPOSE) s_S[i * 33 + c] = (i == col && col < K) ? 1.0f : 0.0f;
+    else s_S[i * 33 + c] = (h0 && i < K) ? h0[(((int64_t)row0 * HV + hv) * K + i) * V + colc] : 0.0f;
   }
-  const int p0 = seq_seg0[seq], p1 = seq_seg0[seq + 1];
-  const int W = K + V;
+  // the column of the maps' N part that goes with this column of the state (COMPOSE: none for the first K columns)
+  const int ncol = COMPOSE ? min(max(col - K, 0), W - K - 1) : colc;
+  const bool has_n = !COMPOSE || col >= K;
   const int my_row = tid / K4, my_c4 = tid % K4;
   const bool loader = my_row < RPB;
   float4 mreg[DEPTH][MREGS];
@@ -475,16 +507,17 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
   // M_p and this thread's entries of N_p into register set `slot`: unconditional loads from clamped addresses (a
   // segment index past the end, a row or column past K); what lies past K is replaced by zero when it is used
   auto fetch = [&](int p, int slot) __attribute__((always_inline)) {
-    p = min(p, p1 - 1);
+    p = min(p, p_last);
     const float* M = mn + ((int64_t)p * HV + hv) * K * W;
 #pragma unroll
     for (int u = 0; u < MREGS; ++u)
       mreg[slot][u] = *reinterpret_cast<const float4*>(M + (int64_t)min(u * RPB + my_row, K - 1) * W + min(4 * my_c4, K - 4));
 #pragma unroll
-    for (int n = 0; n < NR; ++n) nreg[slot][n] = M[(int64_t)min(rg + 8 * n, K - 1) * W + K + colc];
+    for (int n = 0; n < NR; ++n) nreg[slot][n] = M[(int64_t)min(rg + 8 * n, K - 1) * W + K + ncol];
   };
   // the state segment p starts from (every lane stores every time: rows past K repeat the last row's store)
   auto store_start = [&](int p) __attribute__((always_inline)) {
+    if (COMPOSE) return;
     float* out = sinit + ((int64_t)p * HV + hv) * K * V;
 #pragma unroll
     for (int n = 0; n < NR; ++n) {
@@ -505,7 +538,7 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
     }
     float acc[NR];
 #pragma unroll
-    for (int n = 0; n < NR; ++n) acc[n] = rg + 8 * n < K ? nreg[slot][n] : 0.0f;
+    for (int n = 0; n < NR; ++n) acc[n] = (has_n && rg + 8 * n < K) ? nreg[slot][n] : 0.0f;
     lds_barrier();  // M_p is in LDS (an LDS-only barrier: the loads issued ahead stay in flight)
     fetch(p + DEPTH, slot);
     {
@@ -543,7 +576,6 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
     }
     lds_barrier();
   };
-  if (p0 >= p1) return;
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) fetch(p0 + d, d);
   __syncthreads();
@@ -556,22 +588,22 @@ __global__ void __launch_bounds__(256) gdr_segment_scan_kernel(const float* __re
   for (int d = 0; d < DEPTH; ++d)
     if (p + d + 1 < p1) advance(p + d, d);
   store_start(p1 - 1);
+  if (COMPOSE) {  // the group's map, in the layout of the segments' maps
+    float* out = sinit + ((int64_t)blockIdx.y * HV + hv) * K * W;
+#pragma unroll
+    for (int n = 0; n < NR; ++n) {
+      const int i = min(rg + 8 * n, K - 1);
+      out[(int64_t)i * W + colc] = s_S[i * 33 + c];
+    }
+  }
 }
 
 template <typename T>
 static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                    void* o, const float* h0, float* ht, const int64_t* cu_seg,
                                    const int32_t* seq_seg0, const int32_t* seg_out, int n_seq, int n_seg, int H, int HV,
-                                   int K, int V, float scale, int l2norm, float* mn, float* sinit, hipStream_t s) {
-  static bool attr_set[64] = {};  // per device: the widest scan's dynamic LDS limit (a repeated set is harmless)
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
-  if (!attr_set[dev]) {
-    if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)RsScanShape<128>::LDS_BYTES) != hipSuccess)
-      return LAMPA_ERR_LAUNCH;
-    attr_set[dev] = true;
-  }
+                                   int K, int V, float scale, int l2norm, float* mn, float* sinit, float* groups,
+                                   hipStream_t s) {
   LAMPA_PROF(s, "start");
   const dim3 grid_a((K + V + 31) / 32, n_seg * HV), grid_b((V + 31) / 32, n_seg * HV);
 #define GDR_REC_SEG(KT) GDR_REC_SEG2(KT, false, false)
@@ -581,10 +613,9 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
                        (const T*)v, g, beta, (T*)nullptr, (const float*)nullptr, mn, cu_seg, (int64_t)0, H, HV, K,   \
                        K + V, scale, l2norm, (const int32_t*)nullptr);                                               \
     LAMPA_PROF(s, "gdr_recurrent_split_kernel<composite>");                                                          \
-    hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1)>),                            \
-                       dim3((V + 31) / 32, n_seq, HV), dim3(256), RsScanShape<KT>::LDS_BYTES, s, mn, h0, seq_seg0,   \
-                       HV, K, V, sinit);                                                                             \
-    LAMPA_PROF(s, "gdr_segment_scan_kernel");                                                                        \
+    if (gdr_segment_scan(mn, h0, seq_seg0, n_seq, n_seg, HV, K, V, sinit, groups, s) != LAMPA_OK)                    \
+      return LAMPA_ERR_LAUNCH;                                                                                       \
+    LAMPA_PROF(s, "start");                                                                                          \
     hipLaunchKernelGGL((gdr_recurrent_split_kernel<T, KT, false, SHORT_B>), grid_b, dim3(64), 0, s, (const T*)q, (const T*)k, \
                        (const T*)v, g, beta, (T*)o, sinit, ht, cu_seg, (int64_t)0, H, HV, K, V, scale, l2norm,       \
                        seg_out);                                                                                     \
@@ -608,12 +639,14 @@ static int gdr_recurrent_segmented(const void* q, const void* k, const void* v, 
 // states the segments start from but not the outputs; the scan is also run a second time there, over the transposed
 // maps in reverse segment order.
 static int gdr_scan_attr() {
-  static bool attr_set[64] = {};
+  static bool attr_set[64] = {};  // per device: the widest scans' dynamic LDS limit (a repeated set is harmless)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
   if (!attr_set[dev]) {
-    if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)RsScanShape<128>::LDS_BYTES) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)RsScanShape<128>::LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute((const void*)gdr_segment_scan_kernel<128, 1, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)RsScanShape<128>::LDS_BYTES) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
     attr_set[dev] = true;
   }
@@ -654,19 +687,56 @@ int gdr_segment_maps(const void* k, const void* v, const float* g, const float* 
   return lampa_launch_status();
 }
 
-int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, int n_seq, int HV, int K, int V,
-                     float* sinit, hipStream_t s) {
+// Group slots of the three-launch scan: at most GDR_SCAN_GROUP_SEQS sequences of together at most
+// GDR_SCAN_GROUP_SEGS segments take it; groups of gs = ceil(sqrt(n_seg / n_seq)) segments, at most
+// maxg = ceil(n_seg / gs) of them in a sequence however the segments are spread, so n_seq * maxg <=
+// n_seq^1.5 sqrt(n_seg) + n_seq slots of a map [K, K + V] and a state [K, V] each.
+#define GDR_SCAN_GROUP_SEQS 4
+#define GDR_SCAN_GROUP_SEGS 4096
+int64_t gdr_scan_group_floats(int n_seg, int HV, int K, int V) {
+  if (n_seg > GDR_SCAN_GROUP_SEGS) return 0;
+  int64_t root = 1;
+  while (root * root < n_seg) ++root;
+  return (8 * root + GDR_SCAN_GROUP_SEQS) * HV * K * (int64_t)(K + 2 * V);
+}
+
+int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, int n_seq, int n_seg, int HV, int K,
+                     int V, float* sinit, float* groups, hipStream_t s) {
   const int rc = gdr_scan_attr();
   if (rc != LAMPA_OK) return rc;
+  const int W = K + V;
+#define GDR_REC_SCAN(KT, COMPOSE, GRID, MAPS, H0, COLS, OUT, MODE, GS, MAXG)                                      \
+  hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1), COMPOSE>), GRID, dim3(256),   \
+                     RsScanShape<KT>::LDS_BYTES, s, MAPS, H0, seq_seg0, HV, K, COLS, OUT, MODE, GS, MAXG, W)
+#define GDR_REC_SCAN_ANY(...)                        \
+  do {                                               \
+    if (K <= 16) GDR_REC_SCAN(16, __VA_ARGS__);      \
+    else if (K <= 32) GDR_REC_SCAN(32, __VA_ARGS__); \
+    else if (K <= 64) GDR_REC_SCAN(64, __VA_ARGS__); \
+    else GDR_REC_SCAN(128, __VA_ARGS__);             \
+  } while (0)
+  // a few long sequences: groups of about sqrt(segments per sequence) segments, three launches of that many steps
+  if (groups && n_seq <= GDR_SCAN_GROUP_SEQS && n_seg <= GDR_SCAN_GROUP_SEGS && n_seg >= 24 * n_seq) {
+    int gs = 1;
+    while (gs * gs * n_seq < n_seg) ++gs;
+    const int maxg = (n_seg + gs - 1) / gs;
+    float* gmaps = groups;                                                  // [n_seq * maxg, HV, K, K + V]
+    float* gstart = groups + (int64_t)n_seq * maxg * HV * K * W;            // [n_seq * maxg, HV, K, V]
+    LAMPA_PROF(s, "start");
+    const dim3 grid_a((W + 31) / 32, n_seq * maxg, HV), grid_b((V + 31) / 32, n_seq, HV),
+        grid_c((V + 31) / 32, n_seq * maxg, HV);
+    GDR_REC_SCAN_ANY(true, grid_a, mn, (const float*)nullptr, W, gmaps, RS_COMPOSE, gs, maxg);
+    LAMPA_PROF(s, "gdr_segment_scan_kernel<compose>");
+    GDR_REC_SCAN_ANY(false, grid_b, (const float*)gmaps, h0, V, gstart, RS_GROUPS, gs, maxg);
+    LAMPA_PROF(s, "gdr_segment_scan_kernel<groups>");
+    GDR_REC_SCAN_ANY(false, grid_c, mn, (const float*)gstart, V, sinit, RS_WITHIN, gs, maxg);
+    LAMPA_PROF(s, "gdr_segment_scan_kernel<within>");
+    return lampa_launch_status();
+  }
   LAMPA_PROF(s, "start");
   const dim3 grid((V + 31) / 32, n_seq, HV);
-#define GDR_REC_SCAN(KT)                                                                                       \
-  hipLaunchKernelGGL((gdr_segment_scan_kernel<KT, (KT <= 32 ? 4 : KT == 64 ? 2 : 1)>), grid, dim3(256),         \
-                     RsScanShape<KT>::LDS_BYTES, s, mn, h0, seq_seg0, HV, K, V, sinit)
-  if (K <= 16) GDR_REC_SCAN(16);
-  else if (K <= 32) GDR_REC_SCAN(32);
-  else if (K <= 64) GDR_REC_SCAN(64);
-  else GDR_REC_SCAN(128);
+  GDR_REC_SCAN_ANY(false, grid, mn, h0, V, sinit, RS_PLAIN, 0, 1);
+#undef GDR_REC_SCAN_ANY
 #undef GDR_REC_SCAN
   LAMPA_PROF(s, "gdr_segment_scan_kernel");
   return lampa_launch_status();
@@ -676,7 +746,8 @@ int gdr_segment_scan(const float* mn, const float* h0, const int32_t* seq_seg0, 
 // from [n_seg, HV, K, V], fp32.
 extern "C" int64_t lampa_gdr_recurrent_segmented_workspace_bytes(int n_seg, int HV, int K, int V) {
   if (n_seg < 0 || HV < 1 || K < 1 || V < 1) return LAMPA_ERR_INVALID;
-  return lampa_align_up((int64_t)n_seg * HV * K * (K + V) * 4, 256) + lampa_align_up((int64_t)n_seg * HV * K * V * 4, 256);
+  return lampa_align_up((int64_t)n_seg * HV * K * (K + V) * 4, 256) + lampa_align_up((int64_t)n_seg * HV * K * V * 4, 256) +
+         lampa_align_up(gdr_scan_group_floats(n_seg, HV, K, V) * 4, 256);
 }
 
 // lampa_gdr_recurrent_fwd for a few long sequences: the caller cuts every sequence into segments (cu_seg: device int64,
@@ -700,17 +771,19 @@ extern "C" int lampa_gdr_recurrent_segmented_fwd(const void* q, const void* k, c
     return LAMPA_ERR_WORKSPACE;
   float* mn = (float*)workspace;
   float* sinit = (float*)((char*)workspace + lampa_align_up((int64_t)n_seg * HV * K * (K + V) * 4, 256));
+  float* groups = (float*)((char*)sinit + lampa_align_up((int64_t)n_seg * HV * K * V * 4, 256));
+  if (gdr_scan_group_floats(n_seg, HV, K, V) == 0) groups = nullptr;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case GDR_BF16:
       return gdr_recurrent_segmented<__bf16>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H,
-                                             HV, K, V, scale, l2norm, mn, sinit, s);
+                                             HV, K, V, scale, l2norm, mn, sinit, groups, s);
     case GDR_FP16:
       return gdr_recurrent_segmented<_Float16>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H,
-                                               HV, K, V, scale, l2norm, mn, sinit, s);
+                                               HV, K, V, scale, l2norm, mn, sinit, groups, s);
     case GDR_FP32:
       return gdr_recurrent_segmented<float>(q, k, v, g, beta, o, h0, ht, cu_seg, seq_seg0, seg_out, n_seq, n_seg, H, HV,
-                                            K, V, scale, l2norm, mn, sinit, s);
+                                            K, V, scale, l2norm, mn, sinit, groups, s);
     default:
       return LAMPA_ERR_INVALID;
   }
