@@ -127,8 +127,8 @@ def _recurrent_launch(q, k, v, g, beta, scale, initial_state, output_final_state
         cu_host = [i * T for i in range(B + 1)] if cu_seqlens is None else [int(c) for c in cu_seqlens.tolist()]
         if max(b - a for a, b in zip(cu_host[:-1], cu_host[1:])) >= SEGMENT_MIN_TOKENS:
             want = max(1, 1024 // (HV * slabs))  # segments for about one wave per SIMD in the output pass (the scan
-            # between the passes is serial in the segments: no more of them than fill the chip)
-            seg_len = max(128, -(-(cu_host[-1] // want) // 64) * 64)
+            # between the passes is serial in the groups of segments: no more of them than fill the chip)
+            seg_len = max(64, -(-(cu_host[-1] // want) // 64) * 64)
             return _recurrent_segmented_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_host,
                                                seg_len, l2norm)
     o = torch.empty_like(v)
