@@ -110,6 +110,26 @@ def test_recurrent_strong_mixed_and_positive_decay(device, K, V):
         assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL, seg_min
 
 
+def test_recurrent_segments_scanned_in_groups_unbalanced_sequences(device):
+    """Four sequences of very different lengths (one empty, one of two segments) cut into 32-token segments: 129 segments,
+    so the scan over them runs as groups' maps -> groups' start states -> segments inside the groups, with groups that
+    are full, partial, single and absent."""
+    gen = torch.Generator().manual_seed(31)
+    lens = [3000, 0, 40, 1000]
+    cu_host = [0] + list(np.cumsum(lens))
+    T, H, HV, K, V = sum(lens), 1, 2, 32, 48
+    q, k = (torch.randn(1, T, H, K, generator=gen) for _ in range(2))
+    v = torch.randn(1, T, HV, V, generator=gen)
+    g = -torch.rand(1, T, HV, generator=gen) * 0.05
+    beta = torch.rand(1, T, HV, generator=gen)
+    h0 = torch.randn(4, HV, K, V, generator=gen)
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=torch.tensor(cu_host),
+                                    l2=og.L2_RECURRENT)
+    o, s = gd._recurrent_segmented_launch(*_to(device, q, k, v, g, beta), K ** -0.5, h0.to(device), True,
+                                          [int(c) for c in cu_host], 32, gd.L2_RECURRENT)
+    assert _errors(o, want_o)[0] <= FP32_TOL and _errors(s, want_s)[0] <= FP32_TOL
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_recurrent_long_sequences_run_as_segments(device, dtype):
     # a few long sequences (one of them empty, one shorter than a segment) are cut into segments that run in parallel;

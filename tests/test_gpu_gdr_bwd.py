@@ -99,6 +99,21 @@ def test_gradients_many_short_sequences_more_units_than_workgroups(device):
     _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, True), want, torch.float32)
 
 
+def test_gradients_scans_in_groups_unbalanced_sequences(device, monkeypatch):
+    """Three sequences (one empty, one of a single short segment) cut into 64-token segments, 75 of them: both scans of
+    the backward pass (forward, and reversed with one extra row per sequence) run in their three-launch form over groups
+    of segments."""
+    monkeypatch.setattr(gd, "BACKWARD_UNITS", 1 << 20)
+    lens = [0, 4700, 30]
+    T = sum(lens)
+    (q, k, v, g, beta, do), gen = _inputs(1, T, 1, 2, 16, 16, torch.float32, 23, unit=False, g_scale=0.05)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.long)
+    h0 = 0.5 * torch.randn(3, 2, 16, 16, generator=gen)
+    dht = torch.randn(3, 2, 16, 16, generator=gen)
+    want = ob.backward_manual(q, k, v, g, beta, do, dht, None, h0, cu, og.L2_CHUNK)
+    _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, True), want, torch.float32)
+
+
 def test_gradients_without_states_and_with_unused_output(device):
     """No initial state (no d h0), no final state; and a loss that uses the final state only (d o is zero)."""
     (q, k, v, g, beta, do), gen = _inputs(1, 200, 1, 2, 64, 64, torch.float32, 3, unit=True)
