@@ -347,22 +347,21 @@ def test_chunk_small_heads_long_sequence_fp16(device, K, V):
         o2, s2 = gd.fused_recurrent_gated_delta_rule(dq[:, :4096], dk[:, :4096], dv[:, :4096], dg[:, :4096],
                                                      db[:, :4096], initial_state=h0.to(device), output_final_state=True)
         _assert_bf16_close(o[:, :4096], o2.float().cpu(), "chunk vs token loop")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(5):
-            gd.chunk_gated_delta_rule(dq, dk, dv, dg, db)
-        torch.cuda.synchronize()
-        t_chunk = (time.perf_counter() - t0) / 5
+        def timed(fn, n):  # warm calls first (tables, workspace), then the average of n
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n
+        t_chunk = timed(lambda: gd.chunk_gated_delta_rule(dq, dk, dv, dg, db), 10)
         def loop_time(segments):  # the token-serial operator, as parallel segments or as one serial run per head
             old = gd.SEGMENT_MIN_TOKENS
             gd.SEGMENT_MIN_TOKENS = old if segments else None
             try:
-                gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-                gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db)
-                torch.cuda.synchronize()
-                return time.perf_counter() - t0
+                return timed(lambda: gd.fused_recurrent_gated_delta_rule(dq, dk, dv, dg, db), 10 if segments else 1)
             finally:
                 gd.SEGMENT_MIN_TOKENS = old
         t_seg, t_loop = loop_time(True), loop_time(False)
