@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(256, 2)
       for (int j = 0; j < 4; ++j) {
         const int piece = t + 128 * j, row = piece >> 3, part = piece & 7;
         const prof_u32x4 val = {(unsigned)c, (unsigned)row, (unsigned)part, 0u};
-        o[((size_t)(c * 64 + row) * H + h) * 8 + part] = val;
+        __builtin_nontemporal_store(val, &o[((size_t)(c * 64 + row) * H + h) * 8 + part]);  // as the output pass stores o
       }
       __syncthreads();
     }
