@@ -82,8 +82,9 @@ int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, 
  * of 16-byte pieces, runs as ONE kernel whose workgroups wait for the other workgroups of their table (flags in the
  * workspace; no host-visible state); any other call runs as separate kernels. The results are the same bits. The waits
  * are bounded: should one run out (two such kernels sharing one GPU at the same time can starve each other), bit 1 of the
- * table's overflow field in meta_out is set and the outputs of the call are not to be used. Calls of the stage that
- * could overlap on one GPU should therefore be serialised by the caller. */
+ * table's overflow field in meta_out is set, the table's perm_out rows are all -1 and its feats_out rows all zero (every
+ * kernel still ends normally): the failure shows in the outputs themselves. Calls of the stage that could overlap on one
+ * GPU should therefore be serialised by the caller. */
 int64_t lampa_lsh_bucket_sort_workspace_bytes(int64_t n_hits, int n_tables, int n_proj);
 int lampa_lsh_bucket_sort(const float* coords, int64_t n_hits, int64_t n_valid, int dim, const float* alpha,
                           const float* beta, int n_tables, int n_proj, float w, int32_t* ids_out, int32_t* keys_out,
@@ -244,6 +245,14 @@ int lampa_gdr_recurrent_fwd(const void* q, const void* k, const void* v, const f
                             const float* h0, float* ht, const int64_t* cu_seqlens, int n_seq, int64_t t_len, int H,
                             int HV, int K, int V, int dtype, float scale, int l2norm, void* stream);
 
+/* The same operator with one beta per value column: beta fp32 [tokens, HV, V]. Replaces the IS_BETA_HEADWISE branch of
+ * fused_recurrent_gated_delta_rule_fwd_kernel (gated_delta_rule_ori.py:415-418,444-448), which its wrapper takes when
+ * beta.ndim == v.ndim (gated_delta_rule_ori.py:515). Every other argument as for lampa_gdr_recurrent_fwd. */
+int lampa_gdr_recurrent_headwise_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                     void* o, const float* h0, float* ht, const int64_t* cu_seqlens, int n_seq,
+                                     int64_t t_len, int H, int HV, int K, int V, int dtype, float scale, int l2norm,
+                                     void* stream);
+
 /* The same operator (gated_delta_rule_ori.py:372-520) for a few long sequences, which one or two wavefronts each would
  * leave the GPU idle with: the caller cuts every sequence into segments and they run in parallel -- every segment's
  * affine map of its initial state, a short serial pass over the maps, then every segment again from its true initial
@@ -324,6 +333,13 @@ int lampa_hgdn_chunk_fwd(const void* q, const void* k, const void* v, const floa
 int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g, const float* beta, const void* lam,
                     int lam_dtype, float lam_div, float* states, void* o, int B, int H, int HV, int K, int V, int L, int z,
                     int dtype, float scale, int l2norm, void* stream);
+
+/* Process-wide switches of the one-launch form of lampa_lsh_bucket_sort[_batch] (no counterpart in the reference).
+ * enabled = 0: every call takes the separate kernels (what a caller retries with after a call came back with bit 1 of
+ * an overflow field set). wait_limit: polls a workgroup spends in one wait for the other workgroups of its table
+ * before it gives up; < 0 = the built-in bound; 0 = give up at once, which lets a test reach the give-up path from the
+ * host with every kernel still ending normally. */
+int lampa_lsh_one_launch_config(int enabled, int64_t wait_limit);
 
 /* ------------------------------------------------------------------------------------------------- profiling */
 

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "lampa_lsh_bucket_sort_batch_workspace_bytes": (_i64, [_i32, _i64, _i32, _i32]),
     "lampa_lsh_bucket_sort_batch": (_i32, [_vp, _i32, _i64, _vp, _i32, _vp, _vp, _i32, _i32, _f32, _vp, _vp, _vp, _vp,
                                            _vp, _i64, _vp, _i32, _vp, _i64, _vp]),
+    "lampa_lsh_one_launch_config": (_i32, [_i32, _i64]),
     "lampa_lsh_project_f32": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "lampa_lsh_ordering_keys": (_i32, [_vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp]),
     "lampa_row_minmax_f32": (_i32, [_vp, _i32, _i64, _vp, _vp]),
@@ -54,6 +55,8 @@ _SIGNATURES = {
     "lampa_gdr_gates_fwd": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i32, _f32, _i32, _vp, _vp, _vp]),
     "lampa_gdr_recurrent_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32,
                                        _i32, _i32, _f32, _i32, _vp]),
+    "lampa_gdr_recurrent_headwise_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32,
+                                                _i32, _i32, _i32, _f32, _i32, _vp]),
     "lampa_gdr_recurrent_segmented_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "lampa_gdr_recurrent_segmented_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                                  _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),

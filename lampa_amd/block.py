@@ -128,9 +128,22 @@ class LshgdBlock(nn.Module):
 
     @torch.no_grad()
     def order(self, coords: torch.Tensor) -> torch.Tensor:
-        """Sequence order of the hits: the stable bucket-sort permutation of the first hash table (int32 [N])."""
-        out = lsh.lsh_bucket_sort(coords.float(), self.lsh_alpha, self.lsh_beta, self.bucket_width,
-                                  self.n_tables, self.n_proj, return_ids=False)
+        """Sequence order of the hits: the stable bucket-sort permutation of the first hash table (int32 [N]). The flag
+        field of the stage is read once per event (one small copy to the host): when a workgroup of the one-launch
+        kernel gave up a wait (``lsh.META_GAVE_UP``) the stage runs again as separate kernels, which wait for nothing; a
+        key that does not fit 32 bits raises."""
+        args = (coords.float(), self.lsh_alpha, self.lsh_beta, self.bucket_width, self.n_tables, self.n_proj)
+        out = lsh.lsh_bucket_sort(*args, return_ids=False)
+        flags = lsh.decode_meta_flags(out["meta"])
+        if bool(flags["gave_up"].any()):
+            lsh.one_launch_config(enabled=False)
+            try:
+                out = lsh.lsh_bucket_sort(*args, return_ids=False, strict=True)
+            finally:
+                lsh.one_launch_config(enabled=True)
+        elif bool(flags["key_overflow"][0]):
+            raise lsh.LampaError("LshgdBlock: the bucket key of the first hash table does not fit 32 bits; the "
+                                 "sequence order would be meaningless")
         return out["perm"][0]
 
     @torch.no_grad()

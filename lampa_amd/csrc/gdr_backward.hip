@@ -26,6 +26,7 @@
 // chain of dependent LDS round trips, so the kernel lives on waves per SIMD: at most GB_MAX_GRID workgroups of one wave
 // walk through the (segment, head, slab) units.
 #include "gdr_common.h"
+#include <mutex>
 
 #define GB_BT 8     // tokens per block: decayed states rebuilt at a time, distance of the states kept in memory
 #define GB_COLS 16  // value columns per wave
@@ -560,6 +561,12 @@ static GbWorkspace gb_workspace(int64_t total, int n_seq, int n_seg, int HV, int
   return w;
 }
 
+// d(initial state) of sequences without tokens: a copy of d(final state), or zero
+__global__ void gdr_bwd_dh0_empty_kernel(const float* __restrict__ dht, float* __restrict__ dh0, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dh0[i] = dht ? dht[i] : 0.0f;
+}
+
 extern "C" int64_t lampa_gdr_bwd_workspace_bytes(int64_t total_tokens, int n_seq, int n_seg, int HV, int K, int V) {
   if (total_tokens < 0 || n_seq < 0 || n_seg < 0 || HV < 1 || K < 1 || V < 1 || K > 128) return LAMPA_ERR_INVALID;
   return gb_workspace(total_tokens, n_seq, n_seg, HV, K, V).bytes;
@@ -572,8 +579,10 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
                   int64_t total, int n_seq, int n_seg, int H, int HV, int K, int V, int dtype, float scale, int l2norm,
                   char* ws, const GbWorkspace& w, hipStream_t s) {
   static bool attr_set[64] = {};  // per device: the widest kernels' dynamic LDS limit
+  static std::mutex attr_lock;    // (several host threads may call at once)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
+  std::unique_lock<std::mutex> hold(attr_lock);
   if (!attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)gdr_bwd_segment_kernel<T, 128, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)GbShape<128>::LDS_BYTES) != hipSuccess ||
@@ -582,6 +591,7 @@ static int gb_run(const void* q, const void* k, const void* v, const float* g, c
       return LAMPA_ERR_LAUNCH;
     attr_set[dev] = true;
   }
+  hold.unlock();
   float* mn = (float*)(ws + w.mn);
   float* sinit = (float*)(ws + w.sinit);
   float* mn_rev = (float*)(ws + w.mn_rev);
@@ -662,7 +672,17 @@ extern "C" int lampa_gdr_bwd(const void* q, const void* k, const void* v, const 
   if (K > 128 || K % 4 != 0 || V % 4 != 0 || HV / H > 64 || n_seq > 65535 ||
       ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) != 0)
     return LAMPA_ERR_UNSUPPORTED;
-  if (n_seq == 0 || n_seg == 0 || total_tokens == 0) return LAMPA_OK;
+  if (n_seq == 0) return LAMPA_OK;
+  if (n_seg == 0 || total_tokens == 0) {
+    // no tokens: the final state is the initial state, so d(initial state) = d(final state) (zero when none is given)
+    if (dh0) {
+      const int64_t n = (int64_t)n_seq * HV * K * V;
+      hipLaunchKernelGGL(gdr_bwd_dh0_empty_kernel, dim3((unsigned)((n + 255) / 256 < 1024 ? (n + 255) / 256 : 1024)),
+                         dim3(256), 0, (hipStream_t)stream, dht, dh0, n);
+      return lampa_launch_status();
+    }
+    return LAMPA_OK;
+  }
   const GbWorkspace w = gb_workspace(total_tokens, n_seq, n_seg, HV, K, V);
   if (!workspace || workspace_bytes < w.bytes) return LAMPA_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;

@@ -1,6 +1,7 @@
 // Host side of the chunkwise gated-delta-rule forward: workspace layout, launch sequence and the C entry points.
 // The kernels (and the description of the algorithm) are in gdr_chunk_kernels.h.
 #include "gdr_chunk_kernels.h"
+#include <mutex>
 
 struct GdrWorkspace {
   int64_t off_t, off_m, off_n, off_d, off_sinit, off_gm, off_gn, off_gd, max_groups, bytes;
@@ -44,11 +45,12 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   float* Dc = (float*)(ws + w.off_d);
   float* Si = (float*)(ws + w.off_sinit);
   constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_b = GdrSegSmem<KT, VT, true>::BYTES;
-  // the dynamic LDS limit is a per-device attribute of a kernel: set once per device and instantiation (a repeated
-  // set by two host threads racing here is harmless)
+  // the dynamic LDS limit is a per-device attribute of a kernel: set once per device and instantiation
   static bool attr_set[64] = {};
+  static std::mutex attr_lock;  // (several host threads may call at once)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAMPA_ERR_LAUNCH;
+  std::unique_lock<std::mutex> hold(attr_lock);
   if (!attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
@@ -57,6 +59,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       return LAMPA_ERR_LAUNCH;
     attr_set[dev] = true;
   }
+  hold.unlock();
   LAMPA_PROF(s, "start");
   if (chunks > 0) {
     hipLaunchKernelGGL((gdr_local_kernel<T, T, KT>), dim3(gdr_local_grid(chunks, HV)), dim3(64), 0, s, (const T*)k, g, beta,

@@ -17,7 +17,9 @@ __device__ __forceinline__ float bcast(float x, int src) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
 }
 
-template <typename T, int KT>
+// BETA_V: beta holds one value per value column, [tokens, HV, V] (IS_BETA_HEADWISE of the reference kernel,
+// gated_delta_rule_ori.py:415-418,444-448), instead of one per (token, value head).
+template <typename T, int KT, bool BETA_V = false>
 __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                           const T* __restrict__ v, const float* __restrict__ g,
                                                           const float* __restrict__ beta, T* __restrict__ o,
@@ -55,7 +57,8 @@ __global__ void __launch_bounds__(64) gdr_recurrent_kernel(const T* __restrict__
       x.qv[r] = i < K ? GdrElem<T>::to_float(q[(t * H + h) * K + i]) : 0.0f;
     }
     x.g = g[t * HV + hv];
-    x.b = beta[t * HV + hv];
+    if constexpr (BETA_V) x.b = active ? beta[(t * HV + hv) * V + col] : 0.0f;
+    else x.b = beta[t * HV + hv];
     x.v = active ? GdrElem<T>::to_float(v[(t * HV + hv) * V + col]) : 0.0f;
   };
   auto step = [&](int64_t t, const Tok& x) __attribute__((always_inline)) {
@@ -813,6 +816,52 @@ extern "C" int lampa_gdr_recurrent_fwd(const void* q, const void* k, const void*
     case GDR_FP32:
       return gdr_recurrent_launch<float>(q, k, v, g, beta, o, h0, ht, cu_seqlens, n_seq, t_len, H, HV, K, V, scale,
                                          l2norm, s);
+    default:
+      return LAMPA_ERR_INVALID;
+  }
+}
+
+// The same operator with one beta per value column: beta fp32 [total_tokens, HV, V] (the reference kernel's
+// IS_BETA_HEADWISE, gated_delta_rule_ori.py:415-418,444-448). Always the lane-per-column kernel: a lane owns one
+// value column, so its beta is one more load per token.
+template <typename T>
+static int gdr_recurrent_headwise_launch(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                         void* o, const float* h0, float* ht, const int64_t* cu, int n_seq,
+                                         int64_t t_len, int H, int HV, int K, int V, float scale, int l2norm,
+                                         hipStream_t s) {
+  LAMPA_PROF(s, "start");
+  const dim3 grid((V + 63) / 64, n_seq * HV), block(64);
+#define GDR_REC_CASE(KT)                                                                                              \
+  hipLaunchKernelGGL((gdr_recurrent_kernel<T, KT, true>), grid, block, 0, s, (const T*)q, (const T*)k, (const T*)v, g, \
+                     beta, (T*)o, h0, ht, cu, t_len, H, HV, K, V, scale, l2norm)
+  if (K <= 32) GDR_REC_CASE(32);
+  else if (K <= 64) GDR_REC_CASE(64);
+  else GDR_REC_CASE(128);
+#undef GDR_REC_CASE
+  LAMPA_PROF(s, "gdr_recurrent_kernel<headwise beta>");
+  return lampa_launch_status();
+}
+
+extern "C" int lampa_gdr_recurrent_headwise_fwd(const void* q, const void* k, const void* v, const float* g,
+                                                const float* beta, void* o, const float* h0, float* ht,
+                                                const int64_t* cu_seqlens, int n_seq, int64_t t_len, int H, int HV,
+                                                int K, int V, int dtype, float scale, int l2norm, void* stream) {
+  if (!q || !k || !v || !g || !beta || !o) return LAMPA_ERR_INVALID;
+  if (n_seq < 0 || H < 1 || HV < H || HV % H != 0 || K < 1 || V < 1 || t_len < 0) return LAMPA_ERR_INVALID;
+  if (K > 128) return LAMPA_ERR_UNSUPPORTED;
+  if (l2norm < 0 || l2norm > 2) return LAMPA_ERR_INVALID;
+  if (n_seq == 0) return LAMPA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case GDR_BF16:
+      return gdr_recurrent_headwise_launch<__bf16>(q, k, v, g, beta, o, h0, ht, cu_seqlens, n_seq, t_len, H, HV, K, V,
+                                                   scale, l2norm, s);
+    case GDR_FP16:
+      return gdr_recurrent_headwise_launch<_Float16>(q, k, v, g, beta, o, h0, ht, cu_seqlens, n_seq, t_len, H, HV, K,
+                                                     V, scale, l2norm, s);
+    case GDR_FP32:
+      return gdr_recurrent_headwise_launch<float>(q, k, v, g, beta, o, h0, ht, cu_seqlens, n_seq, t_len, H, HV, K, V,
+                                                  scale, l2norm, s);
     default:
       return LAMPA_ERR_INVALID;
   }

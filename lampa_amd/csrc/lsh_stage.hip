@@ -40,7 +40,9 @@ struct LshFusedArgs {
   const char* feats; int vec_per_row; char* feats_out;   // rows of vec_per_row 16-byte pieces
   int n_events; int n_tiles;
   uint64_t* flags; int32_t* partial; uint32_t* rows; uint32_t* totals; uint2* pairs0; uint2* pairs1;
+  uint32_t* failed;     // one word per segment: holds `gen` once a tile of the segment has given up a wait in this call
   uint32_t gen;
+  int spin_limit;       // polls a tile spends in one wait before it gives up
 };
 
 __device__ __forceinline__ void lf_flag_store(uint64_t* p, uint64_t v) {
@@ -69,23 +71,25 @@ __device__ __forceinline__ void lf_store_pair(uint2* p, uint32_t key, uint32_t v
 
 // Barrier over the n_tiles workgroups of a segment: a flag per tile, every tile polls all of them. Before the flag is
 // raised every thread has waited for its own (written-through) stores to complete. `want` grows by one per barrier; a
-// neighbour can be at most one barrier ahead. Returns false when the bounded wait ran out.
-__device__ __forceinline__ bool lf_barrier(uint64_t* gf, int tile, int n_tiles, uint64_t want) {
+// neighbour can be at most one barrier ahead. Returns false when the bounded wait ran out (after `limit` polls). A
+// tile that has already given up a wait (`healthy` false) still raises its flag, so that the others do not wait for
+// it, and polls no more: one starved call costs one wait, not one per barrier.
+__device__ __forceinline__ bool lf_barrier(uint64_t* gf, int tile, int n_tiles, uint64_t want, int limit, bool healthy) {
   __shared__ int s_ok;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x < 64) {
     if (threadIdx.x == 0) lf_flag_store(gf + tile, want);
     int spins = 0;
-    bool done;
-    for (;;) {
+    bool done = false;
+    for (; healthy && limit > 0;) {  // (a limit of 0 gives up at once, whatever the other tiles have done)
       bool ok = true;
       for (int c = threadIdx.x; c < n_tiles; c += 64) {
         const uint64_t v = lf_flag_load(gf + c);
         ok = ok && (v == want || v == want + 1);
       }
       done = __all(ok);
-      if (done || ++spins > LF_SPIN_LIMIT) break;
+      if (done || ++spins > limit) break;
       __builtin_amdgcn_s_sleep(1);
     }
     if (threadIdx.x == 0) s_ok = done ? 1 : 0;
@@ -142,6 +146,13 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
     const float* coords = a.coords + (int64_t)ev * n_hits * a.dim;
     const int n_valid = max(0, min(n_hits, a.n_valid_dev ? a.n_valid_dev[ev] : (int)a.n_valid));  // a count outside the event is cut
     bool healthy = true;
+    // barrier number `want` of the segment; the first wait that runs out is made known to the segment's other tiles
+    // (the word is written through before this tile raises its next flag, which the others wait for)
+    auto lf_sync = [&](uint64_t want) -> bool {
+      const bool ok = lf_barrier(gf, tile, n_tiles, want, a.spin_limit, healthy);
+      if (healthy && !ok && threadIdx.x == 0) lf_store(a.failed + seg, a.gen);
+      return ok;
+    };
 
     // ---- hash the tile's hits for this table: min / max of every projection's bucket id ----
     if ((int)threadIdx.x < LSH_MAX_DIM * LSH_MAX_PROJ) {
@@ -191,7 +202,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       for (int w = 1; w < LF_WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
       lf_store(partial + tile * LF_PARTIAL_STRIDE + q, v);
     }
-    healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+    healthy = lf_sync(++phase);
 
     // ---- ranges, mixed-radix strides, key width (every tile computes them; tile 0 writes the meta row) ----
     {  // thread t reduces value t % 16 over tiles t / 16, t / 16 + 16, ...: independent loads, one round trip
@@ -306,7 +317,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         for (int w = 0; w < LF_WAVES; ++w) c += s_bin[w][d];
         lf_store(rows + tile * LF_MAX_BINS + d, c);
       }
-      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      healthy = lf_sync(++phase);
       // Tile t turns the counts of digits t*per .. (t+1)*per - 1 of ALL tiles into prefixes over the tiles (in place)
       // and their sum into the segment's totals: every tile reads n_tiles * per words instead of n_tiles rows. A wave
       // takes a digit, its lanes the tiles (128 at a time); four digits per wave are in flight, all loads first.
@@ -345,7 +356,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
           }
         }
       }
-      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      healthy = lf_sync(++phase);
       // thread t owns digits t, t + 256, ...: keys of the digit in the tiles before this one, and in the segment
       uint32_t excl[DPT];
 #pragma unroll
@@ -402,12 +413,12 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
           const uint32_t d = (key[k] >> shift) & mask;
           const uint32_t pos = s_bin[wave][d] + rank[k];
           if (pos < (uint32_t)n_hits) {  // always, unless a wait was abandoned
-            if (last) lf_store(perm + pos, val[k]);
+            if (last) { if (healthy) lf_store(perm + pos, val[k]); }
             else lf_store_pair(pairs[e & 1] + pos, key[k], (uint32_t)val[k]);
           }
         }
       }
-      healthy = lf_barrier(gf, tile, n_tiles, ++phase) && healthy;
+      healthy = lf_sync(++phase);
       if (!last) {
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
@@ -419,10 +430,21 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       }
     }
 
+    // A wait that ran out, here or (seen through the segment's word after the last barrier) in another tile: the
+    // segment's order cannot be trusted. Every tile that knows then writes -1 over the segment's WHOLE permutation
+    // (other tiles scatter into every part of it, and a tile that has given up scatters into it no more, so the tile
+    // that finishes last leaves it all -1) and zeros over its own rows of the sorted features, so that the failure
+    // shows in the outputs themselves and not only in the meta row. (Only a tile that had already left the last
+    // barrier when another gave up at that same barrier does not know; all scatters were complete by then.)
+    const bool poisoned = !healthy || lf_load(a.failed + seg) == a.gen;
+    const int row0 = tile * TILE, n_rows = max(0, min(TILE, n_hits - row0));
+    if (poisoned)
+      for (int r = threadIdx.x; r < n_hits; r += LF_BLOCK) lf_store(perm + r, (int32_t)-1);
+
     // ---- the hit features in sorted order: rows tile*TILE .. of the segment's output ----
     if (a.feats) {
-      const int row0 = tile * TILE, n_rows = min(TILE, n_hits - row0);
-      for (int r = threadIdx.x; r < n_rows; r += LF_BLOCK) s_tot[r] = (uint32_t)lf_load(perm + row0 + r);
+      for (int r = threadIdx.x; r < n_rows; r += LF_BLOCK)
+        s_tot[r] = poisoned ? 0xFFFFFFFFu : (uint32_t)lf_load(perm + row0 + r);
       __syncthreads();
       const int vpr = a.vec_per_row, items = n_rows * vpr;
       const uint4* src = reinterpret_cast<const uint4*>(a.feats) + (int64_t)ev * n_hits * vpr;
@@ -449,7 +471,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
     }
     // a wait that ran out: say so in the segment's meta row (after tile 0's write of the overflow field, which
     // happened before the first sort barrier)
-    if (!healthy && threadIdx.x == 0) m[2 * J + 2] = s_over | 2;
+    if (poisoned && threadIdx.x == 0) m[2 * J + 2] = s_over | 2;
   }
 }
 
@@ -470,6 +492,17 @@ static uint32_t lf_next_generation() {
   return counter.fetch_add(1) + 1;
 }
 static const int lf_items[2] = {8, 4};
+
+// Process-wide switches of the one-launch form (lampa_lsh_one_launch_config): whether it is used at all, and the
+// number of polls a tile spends in one wait (< 0: LF_SPIN_LIMIT).
+static std::atomic<int> lf_enabled{1};
+static std::atomic<int64_t> lf_wait_limit{-1};
+
+extern "C" int lampa_lsh_one_launch_config(int enabled, int64_t wait_limit) {
+  lf_enabled.store(enabled ? 1 : 0);
+  lf_wait_limit.store(wait_limit);
+  return LAMPA_OK;
+}
 
 template <int DIM, int ITEMS>
 static int lf_occupancy() {
@@ -516,7 +549,8 @@ int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables) {
   const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, 4);
   if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 8) > 4096) return 0;
   return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256) +
-         lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256);
+         lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256) +
+         lampa_align_up(segs * 4, 256);
 }
 
 // Launches the fused kernel when it applies: returns LAMPA_OK after a launch, 1 when the caller has to take the
@@ -528,6 +562,7 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
                      int64_t feat_row_bytes, void* feats_out, void* workspace, int64_t workspace_bytes,
                      hipStream_t s) {
   const int64_t segs = (int64_t)n_events * n_tables;
+  if (!lf_enabled.load()) return 1;
   if (n_hits < 1 || n_hits > (1 << 24) || segs > LF_MAX_SEGMENTS) return 1;
   if (feats && (feat_row_bytes % 16 != 0 || feat_row_bytes / 16 > (1 << 16) || ((uintptr_t)feats % 16) != 0 ||
                 ((uintptr_t)feats_out % 16) != 0))
@@ -557,8 +592,11 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   a.rows = (uint32_t*)p;    a.totals = a.rows + segs * tiles * LF_MAX_BINS;
   p += lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256);
   a.pairs0 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
-  a.pairs1 = (uint2*)p;
+  a.pairs1 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
+  a.failed = (uint32_t*)p;
   a.gen = lf_next_generation();
+  const int64_t limit = lf_wait_limit.load();
+  a.spin_limit = limit < 0 ? LF_SPIN_LIMIT : (int)(limit > LF_SPIN_LIMIT ? LF_SPIN_LIMIT : limit);
   const dim3 grid((unsigned)(segs * tiles)), block(LF_BLOCK);
   LAMPA_PROF(s, "start");
 #define LF_LAUNCH(DIM, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, ITEMS>), grid, block, 0, s, a)

@@ -9,8 +9,9 @@ Differences that a caller can observe, all additive:
 * ``chunk_gated_delta_rule`` is differentiable (``lampa_gdr_bwd``: fp32, token-serial inside parallel segments);
   ``fused_recurrent_gated_delta_rule``'s backward raises ``NotImplementedError`` as the reference's does;
 * ``allow_fp32=True`` lets ``chunk_gated_delta_rule`` accept float32 q/k/v (the reference rejects them); they
-  are evaluated by the token-serial fp32 kernel;
-* head sizes other than 64 / 128 are evaluated by the token-serial kernel as well (correct, slower).
+  are evaluated by the token-serial fp32 kernel (long sequences cut into segments that run in parallel);
+* head sizes up to 128 other than the built ones (K, V in {64, 128} and 32 x 32) are zero-padded along the head
+  dimension to the next built shape and run on the same chunk kernels; larger heads take the token-serial kernel.
 """
 import ctypes
 import math
@@ -29,6 +30,23 @@ _DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 CHUNKS_PER_SEGMENT: Optional[int] = None
 
 _plan_cache = {}
+
+
+def _sequence_bounds(cu_seqlens, B: int, T: int):
+    """Token boundaries of the sequences as a Python list. ``cu_seqlens`` must start at 0, never decrease and end at
+    the number of tokens that were passed (B * T): the kernels index q, k, v and the outputs with these numbers, so a
+    boundary beyond the tensors would be an out-of-range access on the GPU, and tokens outside every sequence would
+    keep uninitialised outputs and gradients."""
+    if cu_seqlens is None:
+        return [i * T for i in range(B + 1)]
+    cu = [int(c) for c in cu_seqlens.tolist()]
+    if len(cu) < 2:
+        raise ValueError(f"cu_seqlens must hold at least two entries (one sequence), got {len(cu)}")
+    if cu[0] != 0 or cu[-1] != B * T or any(b < a for a, b in zip(cu[:-1], cu[1:])):
+        raise ValueError(f"cu_seqlens must start at 0, be non-decreasing and end at the number of tokens ({B * T}); "
+                         f"got first = {cu[0]}, last = {cu[-1]}"
+                         + ("" if all(b >= a for a, b in zip(cu[:-1], cu[1:])) else ", not monotone"))
+    return cu
 
 
 def _default_chunks_per_segment(chunks_per_seq, n_value_heads: int, slots: int) -> int:
@@ -121,33 +139,33 @@ def _recurrent_launch(q, k, v, g, beta, scale, initial_state, output_final_state
     HV, V = v.shape[2], v.shape[3]
     n_seq = B if cu_seqlens is None else len(cu_seqlens) - 1
     slabs = (V + 31) // 32
-    if (SEGMENT_MIN_TOKENS and K % 4 == 0 and V % 4 == 0 and K <= 128 and n_seq * HV * slabs <= 256
+    headwise = beta.dim() == 4  # one beta per value column (the reference's IS_BETA_HEADWISE)
+    if (not headwise and SEGMENT_MIN_TOKENS and K % 4 == 0 and V % 4 == 0 and K <= 128 and n_seq * HV * slabs <= 256
             and q.shape[0] * T >= SEGMENT_MIN_TOKENS and q.data_ptr() % 16 == 0 and k.data_ptr() % 16 == 0):
         # a few long sequences: one or two waves each would leave most of the chip idle
-        cu_host = [i * T for i in range(B + 1)] if cu_seqlens is None else [int(c) for c in cu_seqlens.tolist()]
+        cu_host = _sequence_bounds(cu_seqlens, B, T)
         if max(b - a for a, b in zip(cu_host[:-1], cu_host[1:])) >= SEGMENT_MIN_TOKENS:
             want = max(1, 1024 // (HV * slabs))  # segments for about one wave per SIMD in the output pass (the scan
             # between the passes is serial in the groups of segments: no more of them than fill the chip)
             seg_len = max(64, -(-(cu_host[-1] // want) // 64) * 64)
             return _recurrent_segmented_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_host,
                                                seg_len, l2norm)
+    if cu_seqlens is not None:
+        _sequence_bounds(cu_seqlens, B, T)
     o = torch.empty_like(v)
     ht = torch.empty((n_seq, HV, K, V), dtype=torch.float32, device=q.device) if output_final_state else None
     cu = None if cu_seqlens is None else cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
     h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-    check(_capi.lib().lampa_gdr_recurrent_fwd(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(o), ptr(h0), ptr(ht),
-                                              ptr(cu), n_seq, T, H, HV, K, V, _DTYPES[q.dtype], float(scale), l2norm,
-                                              stream_of(q)), "lampa_gdr_recurrent_fwd")
+    fn = _capi.lib().lampa_gdr_recurrent_headwise_fwd if headwise else _capi.lib().lampa_gdr_recurrent_fwd
+    check(fn(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(o), ptr(h0), ptr(ht), ptr(cu), n_seq, T, H, HV, K, V,
+             _DTYPES[q.dtype], float(scale), l2norm, stream_of(q)), "lampa_gdr_recurrent_fwd")
     return o, ht
 
 
 def _chunk_launch(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm):
     B, T, H, K = q.shape
     HV, V = v.shape[2], v.shape[3]
-    if cu_seqlens is None:
-        cu_host = [i * T for i in range(B + 1)]
-    else:
-        cu_host = [int(c) for c in cu_seqlens.tolist()]
+    cu_host = _sequence_bounds(cu_seqlens, B, T)
     n_seq = len(cu_host) - 1
     plan_host, plan_dev = _plan(cu_host, q.device, HV, (K, V))
     chunks, segs = int(plan_host[1]), int(plan_host[2])
@@ -232,7 +250,7 @@ def _backward_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm,
         initial_state = None if initial_state is None else pad(initial_state, (0, Vp - V, 0, Kp - K))
         dht = None if dht is None else pad(dht, (0, Vp - V, 0, Kp - K))
     q, k, v, do = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
-    cu_host = [i * T for i in range(B + 1)] if cu_seqlens is None else [int(c) for c in cu_seqlens.tolist()]
+    cu_host = _sequence_bounds(cu_seqlens, B, T)
     n_seq, total = len(cu_host) - 1, B * T
     slabs = (Vp + 15) // 16
     want = max(1, BACKWARD_UNITS // (HV * slabs))
@@ -284,6 +302,12 @@ class _GatedDelta(torch.autograd.Function):
                 "because we haven't figured out how to compute dg without materializing the full "
                 "hidden states for all time steps.")
         q, k, v, g, beta, initial_state, cu_seqlens = ctx.saved_tensors
+        if bool((g > 0).any()):
+            # the forward masks decay ratios with a positive exponent (safe_exp); the gradients here are those of the
+            # unmasked recurrence, which is the same function only for g <= 0
+            raise ValueError("chunk_gated_delta_rule backward: g has positive entries; the gradients are defined for "
+                             "log-decays g <= 0 only (the forward masks decay ratios with positive exponents, the "
+                             "backward pass differentiates the unmasked recurrence)")
         if do is None:
             do = torch.zeros(ctx.o_shape, dtype=ctx.o_dtype, device=q.device)
         dq, dk, dv, dg, dbeta, dh0 = _backward_launch(q, k, v, g, beta, ctx.scale, initial_state, cu_seqlens,
@@ -293,21 +317,21 @@ class _GatedDelta(torch.autograd.Function):
         return (None, dq, dk, dv, dg.to(ctx.g_dtype), dbeta.to(ctx.beta_dtype), None, dh0, None, None, None, None)
 
 
-def _check_shapes(q, k, v, g, beta, what):
+def _check_shapes(q, k, v, g, beta, what, headwise_beta_ok=False):
     """g and beta are per (token, value head): [B, T, HV]. The reference's token-serial kernel also takes a headwise
-    beta [B, T, HV, V] (``gated_delta_rule_ori.py:444-447,515``); that variant is not built, and reading such a tensor
-    with the scalar stride would silently give wrong values, so it is refused."""
+    beta [B, T, HV, V] (``gated_delta_rule_ori.py:444-447,515``), and so does ``fused_recurrent_gated_delta_rule`` here;
+    the chunk operator has no such form (the reference asserts ``len(beta.shape) == 3`` there)."""
     if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:2] != q.shape[:2]:
         raise ValueError(f"{what}: expected q, k [B, T, H, K] and v [B, T, HV, V], got {tuple(q.shape)}, "
                          f"{tuple(k.shape)}, {tuple(v.shape)}")
     if v.shape[2] % q.shape[2] != 0:
         raise ValueError(f"{what}: the number of value heads ({v.shape[2]}) must be a multiple of the number of "
                          f"q/k heads ({q.shape[2]})")
-    if beta.dim() == v.dim():
-        raise NotImplementedError(f"{what}: headwise beta of shape [B, T, HV, V] is not supported; pass beta [B, T, HV]")
-    if tuple(g.shape) != tuple(v.shape[:3]) or tuple(beta.shape) != tuple(v.shape[:3]):
-        raise ValueError(f"{what}: g and beta must have shape {tuple(v.shape[:3])} (= v.shape[:3]), got "
-                         f"{tuple(g.shape)} and {tuple(beta.shape)}")
+    beta_shapes = [tuple(v.shape[:3])] + ([tuple(v.shape)] if headwise_beta_ok else [])
+    if tuple(g.shape) != tuple(v.shape[:3]) or tuple(beta.shape) not in beta_shapes:
+        raise ValueError(f"{what}: g must have shape {tuple(v.shape[:3])} (= v.shape[:3]) and beta that shape"
+                         + (f" or {tuple(v.shape)} (one value per value column)" if headwise_beta_ok else "")
+                         + f", got {tuple(g.shape)} and {tuple(beta.shape)}")
 
 
 def _check_varlen(q, initial_state, cu_seqlens):
@@ -361,7 +385,8 @@ def fused_recurrent_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.
                                      initial_state: torch.Tensor = None, output_final_state: bool = False,
                                      cu_seqlens: Optional[torch.LongTensor] = None,
                                      use_qk_l2norm_in_kernel: bool = False):
-    """q, k [B,T,H,K]; v [B,T,HV,V]; g, beta [B,T,HV]; grouped value heads when HV > H. Returns (o [B,T,HV,V],
+    """q, k [B,T,H,K]; v [B,T,HV,V]; g [B,T,HV]; beta [B,T,HV] or, one value per value column, [B,T,HV,V]
+    (``gated_delta_rule_ori.py:444-448,515``); grouped value heads when HV > H. Returns (o [B,T,HV,V],
     final_state [N,HV,K,V] fp32 or None). See ``gated_delta_rule_ori.py:565-667``."""
     _check_varlen(q, initial_state, cu_seqlens)
     if scale is None:
@@ -370,7 +395,7 @@ def fused_recurrent_gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.
         assert scale > 0, "scale must be positive"
     if beta is None:
         beta = torch.ones_like(g)
-    _check_shapes(q, k, v, g, beta, "fused_recurrent_gated_delta_rule")
+    _check_shapes(q, k, v, g, beta, "fused_recurrent_gated_delta_rule", headwise_beta_ok=True)
     l2norm = L2_RECURRENT if use_qk_l2norm_in_kernel else L2_NONE
     return _GatedDelta.apply(_recurrent_launch, q, k, v, g, beta, scale, initial_state, output_final_state,
                              cu_seqlens, l2norm, False)

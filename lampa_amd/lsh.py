@@ -262,12 +262,34 @@ def lsh_bucket_keys(coords: torch.Tensor, alpha: torch.Tensor, beta: torch.Tenso
     return ids, keys, meta
 
 
+META_KEY_OVERFLOW, META_GAVE_UP = 1, 2  # bits of meta[..., -1]
+
+
+def decode_meta_flags(meta) -> dict:
+    """The flag field ``meta[..., -1]`` of every table as booleans: ``key_overflow`` (bit 0: the id ranges of the table
+    multiply to more than 2^31 - 1 buckets, its order is meaningless) and ``gave_up`` (bit 1: a workgroup of the
+    one-launch kernel gave up waiting for the others of its table; the table's perm is then all -1 and its sorted
+    features all zero). Takes the device tensor (one host synchronisation) or anything ``torch.as_tensor`` accepts."""
+    flags = torch.as_tensor(meta)[..., -1].cpu()
+    return {"key_overflow": (flags & META_KEY_OVERFLOW) != 0, "gave_up": (flags & META_GAVE_UP) != 0}
+
+
+def one_launch_config(enabled: bool = True, wait_limit: int = -1) -> None:
+    """Process-wide switches of the one-launch form of the stage (``lampa_lsh_one_launch_config``): ``enabled=False``
+    sends every call to the separate kernels; ``wait_limit`` is the number of polls a workgroup spends in one wait
+    before it gives up (< 0: the built-in bound; 0: give up at once, for tests of the give-up path)."""
+    check(_capi.lib().lampa_lsh_one_launch_config(1 if enabled else 0, int(wait_limit)), "lampa_lsh_one_launch_config")
+
+
 def _raise_on_overflow(meta: torch.Tensor, strict: bool):
-    if strict and bool((meta[..., -1] & 2).any()):
+    if not strict:
+        return
+    flags = decode_meta_flags(meta)
+    if bool(flags["gave_up"].any()):
         raise LampaError("lsh_bucket_sort: a workgroup of the one-launch kernel gave up waiting for the other "
                          "workgroups of its table (the GPU was shared with another kernel that waits in the same way); "
                          "the outputs of this call are not to be used")
-    if strict and bool(meta[..., -1].any()):
+    if bool(flags["key_overflow"].any()):
         raise LampaError("lsh_bucket_sort: the id ranges of a table multiply to more than 2^31 - 1 buckets, so its "
                          "32-bit bucket key overflowed and the order is meaningless (use a larger w or fewer "
                          "projections per table)")
@@ -292,8 +314,9 @@ def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[to
     A call of at most 64 tables in total whose tiles all fit the GPU at once (one event of 60 000 hits does, four do)
     runs as ONE kernel whose workgroups wait for each other; larger calls run as separate kernels. The waits of the
     one-launch kernel are bounded: should one run out (two such kernels sharing a GPU can starve each other) bit 1 of
-    ``meta[..., -1]`` is set and the outputs are not to be used; ``strict=True`` raises for it as well. Calls that may
-    run at the same time on one GPU (different streams, processes) should be serialised by the caller."""
+    ``meta[..., -1]`` is set, the table's ``perm`` is all -1 and its ``feats`` all zero; ``strict=True`` raises for it as
+    well (``decode_meta_flags`` reads the field). Calls that may run at the same time on one GPU (different streams,
+    processes) should be serialised by the caller."""
     require_cuda(coords, alpha, beta, feats)
     coords = coords.contiguous().float()
     alpha = alpha.contiguous().float()

@@ -186,7 +186,8 @@ def quadratic_form(q, k, v, g, beta, scale=None, l2=L2_NONE, dtype=torch.float64
 def recurrent_c(q, k, v, g, beta, scale=None, initial_state=None, cu_seqlens=None, l2=L2_NONE,
                 dtype=torch.float64):
     """``gdr_oracle.c`` through ctypes. Inputs are converted to fp32 arrays (exact for bf16/fp16/fp32 inputs);
-    the state is carried in ``dtype`` (float64 or float32). Returns float32 tensors."""
+    the state is carried in ``dtype`` (float64 or float32). Returns float32 tensors. ``beta`` is [B, T, HV] or, one
+    value per value column, [B, T, HV, V] (``gated_delta_rule_ori.py:444-448``)."""
     B, T, H, K = q.shape
     HV, V = v.shape[2], v.shape[3]
     f = lambda x: np.ascontiguousarray(x.detach().to("cpu", torch.float32).numpy())
@@ -204,5 +205,5 @@ def recurrent_c(q, k, v, g, beta, scale=None, initial_state=None, cu_seqlens=Non
     ht = np.empty((n_seq, HV, K, V), np.float32)
     fn = lib().oracle_gdr_recurrent_f64 if dtype == torch.float64 else lib().oracle_gdr_recurrent_f32
     fn(ptr(qa), ptr(ka), ptr(va), ptr(ga), ptr(ba), ptr(cu), n_seq, H, HV, K, V, ctypes.c_float(scale), l2,
-       ptr(h0), ptr(o), ptr(ht))
+       ptr(h0), ptr(o), ptr(ht), 1 if beta.dim() == 4 else 0)
     return torch.from_numpy(o), torch.from_numpy(ht)

@@ -13,6 +13,8 @@
  *   S   <- S + k_t d^T
  *   o_t =  S^T (scale * q_t)
  * Grouped value heads (HV >= H, HV % H == 0): value head hv reads q/k head hv / (HV / H).
+ * beta_headwise != 0: beta is [tokens, HV, V], one value per value column (IS_BETA_HEADWISE,
+ * gated_delta_rule_ori.py:415-418,444-448); otherwise [tokens, HV].
  * Pins (tests/test_oracle_gdr.py): T=1 closed form, beta=0 pure decay, orthonormal-key recall and
  * overwrite, equality with the quadratic (materialised) form and with the chunk form for several chunk
  * sizes -- all evaluated by the independent numpy/torch restatements in oracle/gated_delta.py.
@@ -24,7 +26,7 @@
 #define DEFINE_GDR(NAME, REAL, EXP, SQRT)                                                                  \
   void NAME(const float* q, const float* k, const float* v, const float* g, const float* beta,             \
             const int64_t* cu_seqlens, int n_seq, int H, int HV, int K, int V, float scale, int l2norm,    \
-            const float* h0, float* o, float* ht) {                                                        \
+            const float* h0, float* o, float* ht, int beta_headwise) {                                     \
     REAL* S = (REAL*)malloc(sizeof(REAL) * (size_t)K * V);                                                 \
     REAL* qn = (REAL*)malloc(sizeof(REAL) * (size_t)K);                                                    \
     REAL* kn = (REAL*)malloc(sizeof(REAL) * (size_t)K);                                                    \
@@ -46,11 +48,11 @@
           if (l2norm == 2) { qi = 1 / (SQRT(qs) + (REAL)1e-6); ki = 1 / (SQRT(ks) + (REAL)1e-6); }         \
           for (int i = 0; i < K; ++i) { qn[i] = (REAL)qt[i] * qi * (REAL)scale; kn[i] = (REAL)kt[i] * ki; }\
           REAL decay = EXP((REAL)g[t * HV + hv]);                                                          \
-          REAL b = (REAL)beta[t * HV + hv];                                                                \
+          const float* bt = beta_headwise ? beta + (t * HV + hv) * V : beta + (t * HV + hv);               \
           for (int j = 0; j < V; ++j) d[j] = 0;                                                            \
           for (int i = 0; i < K; ++i)                                                                      \
             for (int j = 0; j < V; ++j) { S[i * V + j] *= decay; d[j] += S[i * V + j] * kn[i]; }           \
-          for (int j = 0; j < V; ++j) d[j] = b * ((REAL)vt[j] - d[j]);                                     \
+          for (int j = 0; j < V; ++j) d[j] = (REAL)bt[beta_headwise ? j : 0] * ((REAL)vt[j] - d[j]);       \
           float* ot = o + (t * HV + hv) * V;                                                               \
           for (int j = 0; j < V; ++j) {                                                                    \
             REAL acc = 0;                                                                                  \

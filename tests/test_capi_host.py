@@ -145,18 +145,23 @@ def test_operators_refuse_cpu_tensors():
 
 
 def test_gated_delta_shape_checks_come_before_any_gpu_work():
-    # headwise beta [B, T, HV, V] (gated_delta_rule_ori.py:444-447) is refused rather than read with the wrong stride;
-    # g and beta must be [B, T, HV]
+    # g and beta must be [B, T, HV]; the token-serial operator also takes a headwise beta [B, T, HV, V]
+    # (gated_delta_rule_ori.py:444-447), the chunk operator does not (its assert on beta's rank comes first, as in the
+    # reference); a CPU tensor is refused after the shape checks
     from lampa_amd import gated_delta as gd
 
     q = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16)
     v = torch.zeros(1, 64, 4, 64, dtype=torch.bfloat16)
     g = torch.zeros(1, 64, 4)
-    with pytest.raises(NotImplementedError, match="headwise beta"):
+    with pytest.raises(_capi.LampaError):  # headwise beta passes the shape checks and reaches the device check
         gd.fused_recurrent_gated_delta_rule(q, q, v, g, torch.zeros(1, 64, 4, 64))
-    with pytest.raises(ValueError, match="g and beta must have shape"):
+    with pytest.raises(ValueError, match="one value per value column"):
+        gd.fused_recurrent_gated_delta_rule(q, q, v, g, torch.zeros(1, 64, 4, 32))
+    with pytest.raises(AssertionError, match="beta must be of shape"):
+        gd.chunk_gated_delta_rule(q, q, v, g, torch.zeros(1, 64, 4, 64))
+    with pytest.raises(ValueError, match="g must have shape"):
         gd.fused_recurrent_gated_delta_rule(q, q, v, g[:, :, :2], g)
-    with pytest.raises(ValueError, match="g and beta must have shape"):
+    with pytest.raises(ValueError, match="g must have shape"):
         gd.chunk_gated_delta_rule(q, q, v, g, g[:, :32])
     with pytest.raises(ValueError, match="multiple of the number"):
         gd.chunk_gated_delta_rule(q, q, v[:, :, :3], g[:, :, :3], g[:, :, :3])
@@ -198,3 +203,41 @@ def test_backward_argument_checks_and_tables(lib):
     assert n_seg == 5 and cu_seg.tolist() == [0, 0, 64, 128, 130, 194]
     assert seq_seg0.tolist() == [0, 1, 4, 5] and rev0.tolist() == [0, 2, 6, 8]
     assert seg_rev.tolist() == [0, 4, 3, 2, 6]  # every sequence's last segment on its first row
+
+
+def test_lsh_meta_flag_decoding():
+    """Bits of the last field of a table's meta row: 1 = the packed key overflowed 32 bits, 2 = a workgroup of the
+    one-launch kernel gave up a wait (host-side decoding; the GPU test forces the second one)."""
+    import torch
+
+    from lampa_amd import lsh
+
+    meta = torch.zeros(2, 3, 11, dtype=torch.int32)
+    meta[0, 1, -1], meta[1, 0, -1], meta[1, 2, -1] = 1, 2, 3
+    flags = lsh.decode_meta_flags(meta)
+    assert flags["key_overflow"].tolist() == [[False, True, False], [False, False, True]]
+    assert flags["gave_up"].tolist() == [[False, False, False], [True, False, True]]
+    with pytest.raises(lsh.LampaError, match="gave up"):
+        lsh._raise_on_overflow(meta, True)
+    with pytest.raises(lsh.LampaError, match="overflow"):
+        lsh._raise_on_overflow(meta[0], True)
+    lsh._raise_on_overflow(meta, False)
+    assert (lsh.META_KEY_OVERFLOW, lsh.META_GAVE_UP) == (1, 2)
+
+
+def test_sequence_boundaries_are_validated_on_the_host():
+    """cu_seqlens index q, k, v and the outputs inside the kernels: a list that does not start at 0, decreases or does
+    not end at the number of tokens is refused before anything is launched (forward, token-serial and backward
+    launchers all take their boundaries from this function)."""
+    import torch
+
+    from lampa_amd import gated_delta as gd
+
+    assert gd._sequence_bounds(None, 2, 5) == [0, 5, 10]
+    assert gd._sequence_bounds(torch.tensor([0, 3, 3, 10]), 1, 10) == [0, 3, 3, 10]
+    for bad in ([1, 4, 10], [0, 4, 11], [0, 4, 9], [0, 6, 4, 10], [10], [0, -1, 10]):
+        with pytest.raises(ValueError, match="cu_seqlens"):
+            gd._sequence_bounds(torch.tensor(bad), 1, 10)
+    import inspect
+    for launcher in (gd._chunk_launch, gd._recurrent_launch, gd._backward_launch):
+        assert "_sequence_bounds" in inspect.getsource(launcher)

@@ -161,3 +161,15 @@ def test_fused_recurrent_backward_raises_like_the_reference(device):
     o, _ = gd.fused_recurrent_gated_delta_rule(*args)
     with pytest.raises(NotImplementedError):
         o.sum().backward()
+
+
+def test_backward_refuses_positive_log_decay(device):
+    # for g > 0 the chunk forward masks decay ratios with positive exponents (safe_exp) while the backward pass
+    # differentiates the unmasked recurrence: the two would belong to different functions, so backward raises
+    (q, k, v, g, beta, do), _ = _inputs(1, 130, 2, 2, 64, 64, torch.bfloat16, 0, True)
+    g = g.clone()
+    g[0, 70, 1] = 0.25
+    args = [x.to(device).requires_grad_(True) for x in (q, k, v, g, beta)]
+    o, _ = gd.chunk_gated_delta_rule(*args)          # the forward itself accepts it, as the reference's does
+    with pytest.raises(ValueError, match="g <= 0"):
+        o.float().sum().backward()

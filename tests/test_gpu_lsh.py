@@ -282,3 +282,39 @@ def test_valid_counts_outside_the_event_are_cut(device, n_events):
         want = ol.bucket_sort(coords[e].numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats[e].numpy(), n_valid=nv)
         for name in ("ids", "meta", "keys", "perm", "feats"):
             assert np.array_equal(_np(got[name][e]), want[name]), (name, e)
+
+
+def test_one_launch_give_up_path_poisons_the_outputs(device):
+    """The workgroups of the one-launch kernel wait for each other with a bounded number of polls. A limit of zero
+    polls (set from the host; every kernel still ends normally) makes every wait give up: the tables' flag fields then
+    carry bit 1, the permutations are all -1 and the sorted features all zero, ``strict=True`` raises, and the block's
+    ordering step falls back to the separate kernels. Afterwards the default limit gives the exact result again."""
+    from lampa_amd import block as lb
+    from lampa_amd._capi import LampaError
+
+    n = 20000
+    alpha, beta = synth.lsh_params(4, 3, 4, 0.5, 1)
+    coords, feats, _ = synth.collider_event(n, seed=9)
+    cd, fd, ad, bd = coords.to(device), feats.to(device), alpha.to(device), beta.to(device)
+    want = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy())
+    try:
+        lsh.one_launch_config(wait_limit=0)
+        got = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, fd)
+        torch.cuda.synchronize()
+        flags = lsh.decode_meta_flags(got["meta"])
+        assert bool(flags["gave_up"].all())
+        assert bool((got["perm"] == -1).all()) and bool((got["feats"] == 0).all())
+        assert np.array_equal(_np(got["ids"]), want["ids"])  # the bucket ids depend on no other workgroup
+        with pytest.raises(LampaError, match="gave up"):
+            lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, fd, strict=True)
+        # the block reads the flag once per event and sorts again with the separate kernels
+        blk = lb.LshgdBlock().to(device)
+        lsh.one_launch_config(wait_limit=0)
+        order = blk.order(cd)
+        blk_alpha, blk_beta = blk.lsh_alpha.cpu().numpy(), blk.lsh_beta.cpu().numpy()
+        assert np.array_equal(_np(order), ol.bucket_sort(coords.numpy(), blk_alpha, blk_beta, 0.5, 3, 4)["perm"][0])
+    finally:
+        lsh.one_launch_config()
+    again = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, fd, strict=True)
+    for name in ("ids", "meta", "keys", "perm", "feats"):
+        assert np.array_equal(_np(again[name]), want[name]), name

@@ -223,3 +223,27 @@ def test_masked_chunk_form_against_scalar_loops():
     o, s = og.chunk_form(q, k, v, g, beta, scale=scale, chunk=C, masked=True)
     assert torch.allclose(o[0, :, 0], torch.tensor(out, dtype=torch.float64), atol=1e-10)
     assert torch.allclose(s[0, 0], torch.tensor(S, dtype=torch.float64), atol=1e-10)
+
+
+def test_headwise_beta_of_the_token_loop():
+    """One beta per value column (``gated_delta_rule_ori.py:444-448``). Two pins that do not retype the loop: a
+    headwise beta that is constant over the columns is the scalar beta, bit for bit; and since the recurrence acts on
+    every value column of the state independently, column j of the headwise result equals column j of a scalar-beta run
+    with beta[..., j] -- which a wrong index into beta, v or the state would break."""
+    gen = torch.Generator().manual_seed(3)
+    B, T, H, HV, K, V = 2, 37, 2, 4, 8, 5
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g = -torch.rand(B, T, HV, generator=gen)
+    beta = torch.rand(B, T, HV, generator=gen)
+    h0 = torch.randn(B, HV, K, V, generator=gen)
+    o, s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, l2=og.L2_RECURRENT)
+    o2, s2 = og.recurrent_c(q, k, v, g, beta[..., None].expand(B, T, HV, V).contiguous(), initial_state=h0,
+                            l2=og.L2_RECURRENT)
+    assert torch.equal(o, o2) and torch.equal(s, s2)
+    bw = torch.rand(B, T, HV, V, generator=gen)
+    ow, sw = og.recurrent_c(q, k, v, g, bw, initial_state=h0, l2=og.L2_RECURRENT)
+    assert not torch.equal(ow, o)
+    for j in range(V):
+        oj, sj = og.recurrent_c(q, k, v, g, bw[..., j].contiguous(), initial_state=h0, l2=og.L2_RECURRENT)
+        assert torch.equal(ow[..., j], oj[..., j]) and torch.equal(sw[..., j], sj[..., j])
