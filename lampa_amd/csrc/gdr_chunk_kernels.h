@@ -1062,36 +1062,30 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
                                         : op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
 #pragma unroll
       for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
-      f32x4 qs[8];
-#pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) qs[t8] = *reinterpret_cast<const f32x4*>(&s_qs[8 * t8 + 4 * hh]);
+      const float qs0 = s_qs[ln], qs1 = s_qs[32 + ln];  // scale e^{gamma_i} rq_i of this lane's token in either row tile
       lds_fence();
       lds_barrier();  // C(c): the q and P operands of chunk c are in registers
-      // o = qs (Q S_old) + P v_new, packed to the output type two columns at a time: lanes 2j and 2j+1 swap one
-      // value of every adjacent row pair, so the even lane holds both columns of the even row and the odd lane
-      // both columns of the odd row. The slab goes to this wave's own part of the o tile and from there to HBM
-      // in 16-byte pieces.
-      const bool odd = ln & 1;
+      // o^T = S_old^T (qs Q)^T + v_new^T P^T: the state and v_new, which this wave holds in accumulator layout (lane =
+      // value column), are read as the A operands (operand row = value column), the Q and P fragments as the B
+      // operands (operand column = token). The result tile has the TOKEN in the lane and 16 value columns (four runs
+      // of four) in the registers, so the token's factor is one scalar per lane and a run packs into one 8-byte piece
+      // of the token's row without any exchange between lanes. The slab goes to this wave's own part of the o tile
+      // and from there to HBM in 16-byte pieces.
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm) {
         f32x16 a1 = zero16(), a2 = zero16();
 #pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(fk[tm * (KT / 16) + ks], Sb[ks], a1);
+        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(Sb[ks], fk[tm * (KT / 16) + ks], a1);
 #pragma unroll
-        for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(ft[2 * tm + ks], Vb[ks], a2);
+        for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(Vb[ks], ft[2 * tm + ks], a2);
+        const float qsv = tm ? qs1 : qs0;
+        typedef T T4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int pr = 0; pr < 8; ++pr) {
-          const int r0 = 2 * pr, r1 = r0 + 1;
-          const float x0 = qs[4 * tm + r0 / 4][r0 % 4] * a1[r0] + a2[r0];
-          const float x1 = qs[4 * tm + r1 / 4][r1 % 4] * a1[r1] + a2[r1];
-          const float keep = odd ? x1 : x0;
-          const float got = dpp_f32<GDR_DPP_QUAD_XOR1, 0xF>(0.0f, odd ? x0 : x1);
-          typedef T T2 __attribute__((ext_vector_type(2)));
-          T2 pk;
-          pk[0] = GdrElem<T>::from_float(odd ? got : keep);
-          pk[1] = GdrElem<T>::from_float(odd ? keep : got);
-          const int row = 32 * tm + acc_row(r0, hh) + (odd ? 1 : 0);
-          *reinterpret_cast<T2*>(&s_o[row * SV + 32 * vslab + (ln & ~1)]) = pk;
+        for (int b4 = 0; b4 < 4; ++b4) {
+          T4 pk;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pk[e] = GdrElem<T>::from_float(__builtin_fmaf(qsv, a1[4 * b4 + e], a2[4 * b4 + e]));
+          *reinterpret_cast<T4*>(&s_o[(32 * tm + ln) * SV + 32 * vslab + 8 * b4 + 4 * hh]) = pk;
         }
       }
       lds_fence();
