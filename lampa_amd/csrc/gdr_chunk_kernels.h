@@ -496,9 +496,10 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
 // The k, v, T tiles and the per-token factors are DOUBLE-buffered in LDS, so the stagers fill the tiles of chunk c+1
 // while the chain waves work on chunk c; q, P and the o tile exist once. LDS-only barriers per chunk (every barrier is
 // a rendezvous of all waves, so the stagers' work is spread such that they are never the slower side):
-//   Qb(c) (PASS_B) q(c) is staged                         -> the stagers build P(c)
 //   B(c)  the chain waves hold every k / v / T operand of chunk c in registers, and tiles (c+1) [PASS_A: also its
-//         factors] and P(c) are complete                   -> buffer c%2 is free for chunk c+2
+//         factors], q(c) and P(c) are complete             -> buffer c%2 is free for chunk c+2
+//         (a stager stages the q rows of ONE 32-row tile and builds exactly the P tiles of those rows -- stager 0
+//         the tile (0,0), stager 1 the tiles (1,0) and (1,1) -- so no barrier separates staging q from building P)
 //   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
 //                                                          -> the stagers may write q(c+1)
 // Global loads are issued about one chunk period before their data is staged.
@@ -544,6 +545,10 @@ struct GdrSegShape {
   // its six-wave workgroups only share a CU below 128 (the hardware deals a workgroup's waves out to the SIMDs in a
   // fixed rotation and starts the next workgroup one step further on, so one SIMD carries four of the twelve waves).
   static constexpr bool SWIZZLED = PASS_B && (KT > 64 || VT > 64);
+  // Waves per SIMD the register allocation has to leave room for (the second argument of the launch bounds). The
+  // composite pass at K = V = 64 runs two six-wave workgroups per CU, and the hardware's rotation puts four of those
+  // twelve waves on one SIMD: 128 registers each.
+  static constexpr int WAVES_PER_SIMD = (!PASS_B && KT + VT <= 128) ? 4 : 2;  // (with the scaled k tiles)
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -573,7 +578,7 @@ __device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int
 }
 
 template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B, typename OT = T>
-__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
+__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SCALED_K ? GdrSegShape<KT, VT, PASS_B>::WAVES_PER_SIMD : 2))
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
                        const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
@@ -589,6 +594,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   using X4 = typename OpVec<OT>::x4;
   constexpr bool SCALED = !PASS_B && SCALED_K;
   constexpr bool SWZ = GdrSegShape<KT, VT, PASS_B>::SWIZZLED;
+  // Output pass at K <= 64: a stager builds the P tiles of the q rows it staged itself (stager 0 the tile (0,0),
+  // stager 1 the tiles (1,0) and (1,1)), so no barrier separates staging q from building P. At K = 128 a P tile is
+  // twice the work, the two stagers share the middle tile, and the barrier Qb(c) (q(c) is staged) comes back.
+  constexpr bool OWN_Q = KT <= 64;
   using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
   constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
@@ -636,6 +645,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     X8 rt_[3];
     float rg = 0.0f, rb = 0.0f;
     float grow = 0.0f;  // gamma of row srow of the chunk whose tiles were staged last
+    float ghalf = 0.0f;  // half the total log-decay of that chunk
+    bool pfast = false;  // that chunk's P takes the factored gating (stage_factors)
     // where this thread's pieces of the packed diagonal blocks of T go in the LDS tile; the pieces above the diagonal
     // are never staged and are zeroed once, in both tile sets
     int ta_off, tb_off;  // element offsets into the T area of a tile set of this thread's two packed pieces
@@ -662,9 +673,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     }
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
     // a select on a freshly loaded value would make the wave wait for the load at once.
-    auto issue_tiles = [&](int c, typename Raw8<T>::type* rk_) {  // k, v, T
+    // (tok0, len: the chunk's entries of the tables, which the caller holds in scalar registers: fetched here they
+    // would put a dependent scalar-memory round trip in front of every use)
+    auto issue_tiles = [&](int c, int tok0, int len, typename Raw8<T>::type* rk_) {  // k, v, T
       c = uniform(c);
-      const int tok0 = chunk_tok0[c], len = chunk_len[c];
       const T* kb = k + ((size_t)tok0 * H + h) * KT;
       const T* vb = v + ((size_t)tok0 * HV + hv) * VT;
       const int r = min(srow, len - 1);
@@ -686,9 +698,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       rg = fact[lane];
       rb = fact[64 + lane];
     };
-    auto issue_q = [&](int c, typename Raw8<T>::type* rq_) {
-      c = uniform(c);
-      const int tok0 = chunk_tok0[c], len = chunk_len[c];
+    auto issue_q = [&](int tok0, int len, typename Raw8<T>::type* rq_) {
       const T* qb = q + ((size_t)tok0 * H + h) * KT;
       const int koff = min(srow, len - 1) * H * KT + spart * (KT / 2);
 #pragma unroll
@@ -702,18 +712,17 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     float kss = 0.0f;  // sum of squares of this thread's half of k row srow (stage_data -> stage_factors)
     // k, v and T of chunk c from the registers to tile set par
     // rows past the end of a partial chunk become zero (a uniform branch: whole chunks pay nothing for it)
-    auto zero_dead_rows = [&](int c, typename Raw8<T>::type* regs, int n) __attribute__((always_inline)) {
-      const int len = chunk_len[uniform(c)];
+    auto zero_dead_rows = [&](int len, typename Raw8<T>::type* regs, int n) __attribute__((always_inline)) {
       if (len < 64) {
         const bool live = srow < len;
 #pragma unroll
         for (int u = 0; u < n; ++u) regs[u] = live ? regs[u] : zero;
       }
     };
-    auto stage_data = [&](int c, int par, typename Raw8<T>::type* rk_) {
+    auto stage_data = [&](int len, int par, typename Raw8<T>::type* rk_) {
       const GdrTilesT<OT> tl = tiles(par);
-      zero_dead_rows(c, rk_, KU);
-      zero_dead_rows(c, rv_, VU);
+      zero_dead_rows(len, rk_, KU);
+      zero_dead_rows(len, rv_, VU);
       *reinterpret_cast<X8*>(&tl.t[(1 * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[0];
       *reinterpret_cast<X8*>(&tl.t[ta_off]) = rt_[1];
       *reinterpret_cast<X8*>(&tl.t[tb_off]) = rt_[2];
@@ -747,13 +756,25 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       const float brow = __shfl(bv, srow);
       const float rk = l2_factor(kss2, l2norm);
       const float ekr = __builtin_amdgcn_exp2f(grow) * rk, dkr = safe_exp2(g_last - grow) * rk;
+      if constexpr (PASS_B && OWN_Q) {  // (the 128-wide heads have no registers to spare for a second form)
+        // Gating of P in factored form, e^{gamma_i - gamma_j} = E_i / E_j with E = 2^(gamma - gamma_last / 2): one exp2
+        // per token instead of one per element. Allowed while no exponent can leave the fp32 range (the chunk's total
+        // decay above 2^-120) and no log-decay of the chunk is positive (the cumulative sums never rise); otherwise
+        // every ratio goes through safe_exp2 one by one. Lanes past the end of a partial chunk repeat the last sum.
+        const float gprev = __shfl_up(gv, 1);
+        pfast = !__ballot(lane > 0 && gv > gprev) && !__ballot(gv > 0.0f) && g_last > -120.0f;
+        ghalf = 0.5f * g_last;
+      }
       if (spart == 0) {
         tl.beta[srow] = brow;
         tl.ek[srow] = ekr;
         tl.dk[srow] = dkr;
         tl.gamma[srow] = grow;
-        tl.rk[srow] = rk;
-        if (srow == 0) tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
+        tl.rk[srow] = (PASS_B && pfast) ? rk * __builtin_amdgcn_exp2f(ghalf - grow) : rk;  // column factor of P
+        if (srow == 0) {
+          tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
+          tl.misc[1] = (PASS_B && pfast) ? 1.0f : 0.0f;
+        }
       }
       if constexpr (SCALED) {  // the two scaled k tiles, from the raw row that is still in registers
 #pragma unroll
@@ -771,8 +792,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         }
       }
     };
-    auto stage_q = [&](int c, typename Raw8<T>::type* rq_) {
-      zero_dead_rows(c, rq_, KU);
+    auto stage_q = [&](int len, typename Raw8<T>::type* rq_) {
+      zero_dead_rows(len, rq_, KU);
       float qss = 0.0f;
 #pragma unroll
       for (int u = 0; u < KU; u += 2) {
@@ -785,7 +806,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       if (spart == 0) {
         const float rq = l2_factor(qss, l2norm);
         s_qs[srow] = scale * __builtin_amdgcn_exp2f(grow) * rq;
-        s_rq[srow] = rq;
+        s_rq[srow] = pfast ? rq * __builtin_amdgcn_exp2f(grow - ghalf) : rq;  // row factor of P (without scale)
       }
     };
 
@@ -794,6 +815,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
         const GdrTilesT<OT> tl = tiles(par);
         // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tile 0, stager 1 tile 2,
         // and they share tile 1: both run its four MFMAs, each finishes and stores one of its two fragments.
+        const bool fast = OWN_Q && uniform(__float_as_int(tl.misc[1])) != 0;
         auto p_tile = [&](int t, int half) {  // half: -1 = whole tile, 0 / 1 = accumulator registers 0-7 / 8-15
           const int jm = t == 2 ? 1 : 0, tn = t == 0 ? 0 : 1;
           X8 fa[KT / 16], fb[KT / 16];
@@ -802,14 +824,14 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
             fa[ks] = *reinterpret_cast<const X8*>(&tl.k[(32 * jm + ln) * SK + 16 * ks + 8 * hh]);
             fb[ks] = *reinterpret_cast<const X8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
           }
-          f32x4 gj[4], rj[4];  // gamma_j, rk_j of this lane's 16 accumulator rows
+          f32x4 gj[4], rj[4];  // gamma_j (slow path only) and the column factor of this lane's 16 accumulator rows
 #pragma unroll
           for (int b4 = 0; b4 < 4; ++b4) {
-            gj[b4] = *reinterpret_cast<const f32x4*>(&tl.gamma[32 * jm + 8 * b4 + 4 * hh]);
+            if (!fast) gj[b4] = *reinterpret_cast<const f32x4*>(&tl.gamma[32 * jm + 8 * b4 + 4 * hh]);
             rj[b4] = *reinterpret_cast<const f32x4*>(&tl.rk[32 * jm + 8 * b4 + 4 * hh]);
           }
           const int i = 32 * tn + ln;
-          const float gi = tl.gamma[i], fi = scale * s_rq[i];
+          const float gi = fast ? 0.0f : tl.gamma[i], fi = scale * s_rq[i];
           lds_fence();
           f32x16 acc = zero16();
 #pragma unroll
@@ -818,16 +840,30 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
 #pragma unroll
           for (int part = 0; part < 2; ++part) {
             if (half >= 0 && half != part) continue;
+            if (fast) {
 #pragma unroll
-            for (int r = 8 * part; r < 8 * part + 8; ++r) {  // the mask goes on the exponent: branch-free
-              const int j = 32 * jm + acc_row(r, hh);
-              acc[r] *= fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f);
+              for (int r = 8 * part; r < 8 * part + 8; ++r) {
+                const float val = acc[r] * (fi * rj[r / 4][r % 4]);
+                acc[r] = (jm != tn || ln >= acc_row(r, hh)) ? val : 0.0f;  // (the tile below the diagonal is full)
+              }
+            } else {
+#pragma unroll
+              for (int r = 8 * part; r < 8 * part + 8; ++r) {  // the mask goes on the exponent: branch-free
+                const int j = 32 * jm + acc_row(r, hh);
+                acc[r] *= fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f);
+              }
             }
             op_frag_store<OT>(s_P, f0 + part, lane, acc_to_op<OT>(acc, 8 * part));
           }
         };
-        p_tile(sw == 0 ? 0 : 2, -1);
-        p_tile(1, sw);
+        // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero.
+        if constexpr (OWN_Q) {  // a stager builds the tiles whose q rows it staged itself
+          if (sw == 0) p_tile(0, -1);
+          else { p_tile(1, -1); p_tile(2, -1); }
+        } else {                // stager 0 takes tile 0, stager 1 tile 2, and they share tile 1: both run its MFMAs,
+          p_tile(sw == 0 ? 0 : 2, -1);  // each finishes and stores one of its two fragments
+          p_tile(1, sw);
+        }
       }
     };
     // Chunk indices past the end of the segment are clamped (the last chunk is fetched again for nothing), so that
@@ -837,23 +873,30 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     if (nc > 0) {
       typename Raw8<T>::type* const rkA = rk0_;
       typename Raw8<T>::type* const rkB = SCALED ? rk1_ : rk0_;
-      issue_tiles(c0, rkA);
+      // the chunks' table entries live in scalar registers and are fetched a chunk period before their first use
+      const int ca = uniform(c0), cb = uniform(min(c0 + 1, cl)), cc = uniform(min(c0 + 2, cl));
+      const int tk0 = chunk_tok0[ca], ln0 = chunk_len[ca], tk1 = chunk_tok0[cb], ln1 = chunk_len[cb];
+      int ln_c = ln0, ln_c1 = ln1, tk_c2 = chunk_tok0[cc], ln_c2 = chunk_len[cc];  // of chunks c, c + 1, c + 2 (clamped)
+      issue_tiles(c0, tk0, ln0, rkA);
       issue_gb(c0);
-      if constexpr (PASS_B) { issue_q(c0, rq0_); issue_q(min(c0 + 1, cl), rq1_); }
-      stage_data(c0, 0, rkA);
+      if constexpr (PASS_B) { issue_q(tk0, ln0, rq0_); issue_q(tk1, ln1, rq1_); }
+      stage_data(ln0, 0, rkA);
       stage_factors(c0, 0, rkA);
-      issue_tiles(min(c0 + 1, cl), rkB);
+      issue_tiles(min(c0 + 1, cl), tk1, ln1, rkB);
       issue_gb(min(c0 + 1, cl));
       lds_barrier();  // tiles (c0) are ready
       // rk_next holds the raw k rows of chunk c + 1, rk_free is loaded with those of chunk c + 2
       auto one_chunk = [&](int c, int par, typename Raw8<T>::type* rq_, typename Raw8<T>::type* rk_next,
                            typename Raw8<T>::type* rk_free) {
-        if (c + 1 < c1) stage_data(c + 1, par ^ 1, rk_next);
-        issue_tiles(min(c + 2, cl), rk_free);
+        const int cn = uniform(min(c + 3, cl));
+        const int tk_n = chunk_tok0[cn], ln_n = chunk_len[cn];  // used from the next chunk on
+        if (c + 1 < c1) stage_data(ln_c1, par ^ 1, rk_next);
+        issue_tiles(min(c + 2, cl), tk_c2, ln_c2, rk_free);
         if constexpr (PASS_B) {
-          stage_q(c, rq_);
-          issue_q(min(c + 2, cl), rq_);
-          lds_barrier();  // Qb(c)
+          stage_q(ln_c, rq_);
+          issue_q(tk_c2, ln_c2, rq_);
+          if constexpr (OWN_Q) lds_fence();  // this wave's own q rows are in LDS (it builds P from no others)
+          else lds_barrier();                // Qb(c)
           build_p(par);
           lds_barrier();  // B(c)
           if (c + 1 < c1) stage_factors(c + 1, par ^ 1, rk_next);
@@ -864,6 +907,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
           issue_gb(min(c + 2, cl));
           lds_barrier();  // B(c)
         }
+        ln_c = ln_c1; ln_c1 = ln_c2; tk_c2 = tk_n; ln_c2 = ln_n;
       };
       for (int c = c0; c < c1; c += 2) {
         one_chunk(c, 0, rq0_, rkB, rkA);
@@ -963,11 +1007,19 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
   // The LDS operand reads of a stage are issued as one batch one stage ahead of the MFMAs that use them
   // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
   // pays the LDS latency once per MFMA.
+  // The q rows and the P fragments of the output are requested right after B(c), before the state update's MFMAs,
+  // where the registers allow a second set of fragments (K = 64 and below).
+  constexpr bool EARLY_Q = PASS_B && KT <= 64;
+  int o_tok0 = 0, o_len = 0;  // table entries of the chunk whose o rows are stored, fetched a chunk ahead
+  if (PASS_B && nc > 0) { o_tok0 = chunk_tok0[uniform(c0)]; o_len = chunk_len[uniform(c0)]; }
   if (nc > 0) lds_barrier();  // tiles (c0) are ready
   for (int c = c0; c < c1; ++c) {
     const GdrTilesT<OT> tl = tiles((c - c0) & 1);
-    if constexpr (PASS_B) lds_barrier();  // Qb(c) (the chain waves only take part)
+    if constexpr (PASS_B && !OWN_Q) lds_barrier();  // Qb(c) (the chain waves only take part)
+    const int c_nx = uniform(min(c + 1, c1 - 1));
+    const int n_tok0 = PASS_B ? chunk_tok0[c_nx] : 0, n_len = PASS_B ? chunk_len[c_nx] : 0;
     X8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+    X8 fq[EARLY_Q ? 2 * (KT / 16) : 1];
     X8 ft[6];              // T (stage 2), P (output)
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
@@ -1046,6 +1098,18 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
     lds_fence();
     lds_barrier();  // B(c): every operand that comes from the k, v and T tiles of chunk c is in registers
     dtot *= dec;
+    float qs0 = 0.0f, qs1 = 0.0f;
+    if constexpr (EARLY_Q) {  // batch: Q rows, P fragments, output factors (in flight during the state update)
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < KT / 16; ++ks) fq[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh)
+                                        : op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+#pragma unroll
+      for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
+      qs0 = s_qs[ln];
+      qs1 = s_qs[32 + ln];
+    }
 #pragma unroll
     for (int km = 0; km < KT / 32; ++km) {  // S <- dec S + K^T (dk v_new)
 #pragma unroll
@@ -1054,15 +1118,17 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int ks = 0; ks < 4; ++ks) S[km] = mfma32(fk[km * 4 + ks], Vsb[ks], S[km]);
     }
     if constexpr (PASS_B) {
-      // batch: Q rows, P fragments, output factors
+      if constexpr (!EARLY_Q) {  // batch: Q rows, P fragments, output factors
 #pragma unroll
-      for (int tm = 0; tm < 2; ++tm)
+        for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh)
-                                        : op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
+          for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh)
+                                          : op_ld_kappa<OT>(s_q, SK, 32 * tm + ln, 16 * ks, hh);
 #pragma unroll
-      for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
-      const float qs0 = s_qs[ln], qs1 = s_qs[32 + ln];  // scale e^{gamma_i} rq_i of this lane's token in either row tile
+        for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
+        qs0 = s_qs[ln];  // scale e^{gamma_i} rq_i of this lane's token in either row tile
+        qs1 = s_qs[32 + ln];
+      }
       lds_fence();
       lds_barrier();  // C(c): the q and P operands of chunk c are in registers
       // o^T = S_old^T (qs Q)^T + v_new^T P^T: the state and v_new, which this wave holds in accumulator layout (lane =
@@ -1075,7 +1141,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       for (int tm = 0; tm < 2; ++tm) {
         f32x16 a1 = zero16(), a2 = zero16();
 #pragma unroll
-        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(Sb[ks], fk[tm * (KT / 16) + ks], a1);
+        for (int ks = 0; ks < KT / 16; ++ks) a1 = mfma32(Sb[ks], (EARLY_Q ? fq : fk)[tm * (KT / 16) + ks], a1);
 #pragma unroll
         for (int ks = 0; ks < 2 * (tm + 1); ++ks) a2 = mfma32(Vb[ks], ft[2 * tm + ks], a2);
         const float qsv = tm ? qs1 : qs0;
@@ -1090,7 +1156,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
       }
       lds_fence();
       {
-        const int cu = uniform(c), tok0 = chunk_tok0[cu], len = chunk_len[cu];
+        const int tok0 = o_tok0, len = o_len;
         T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
         const int rs = HV * VT;
 #pragma unroll
@@ -1106,6 +1172,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), 2)
           if (row < len) __builtin_nontemporal_store(nv, reinterpret_cast<nt_u32x4*>(ob + row * rs + 32 * vslab + 8 * part));
         }
       }
+      o_tok0 = n_tok0;
+      o_len = n_len;
     }
   }
 
