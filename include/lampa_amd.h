@@ -290,6 +290,26 @@ int lampa_gdr_bwd(const void* q, const void* k, const void* v, const float* g, c
                   int64_t total_tokens, int n_seq, int n_seg, int H, int HV, int K, int V, int dtype, float scale,
                   int l2norm, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same gradients in the chunked (WY) form on the matrix cores, the form of the reference's own backward pass
+ * (chunk_gated_delta_rule_bwd, models/hattention/gated_delta_rule_ori.py:83-160: chunk_bwd_dv_local chunk_o.py:372,
+ * chunk_gated_delta_rule_bwd_dhu chunk_delta_h.py:209, chunk_bwd_dqkwg chunk_o.py:128, prepare_wy_repr_bwd wy_fast.py:27;
+ * l2norm_bwd gated_delta_rule_ori.py:205-233): per chunk of 64 tokens the affine map of the state (forwards) and of its
+ * gradient (backwards), a scan over the maps in three levels of groups of 8, then every gradient of a chunk from its tiles
+ * and the two states. For K = V = 64, HV = H, dtype LAMPA_BF16 / LAMPA_FP16 (LAMPA_ERR_UNSUPPORTED otherwise: use
+ * lampa_gdr_bwd); every intermediate operand is rounded to the input type, as in the forward pass, so all gradients
+ * carry the rounding of that type. g <= 0 is assumed (the forward's masking of positive exponents is not differentiated).
+ * Shapes as for lampa_gdr_bwd. plan: lampa_gdr_bwd_chunk_plan_fill's tables of the sequence boundaries
+ * (cu_seqlens_host: int64 [n_seq+1]), the same int32 array in host and in device memory.
+ * workspace: lampa_gdr_bwd_chunk_workspace_bytes(plan_host, HV): about 64 KiB per (chunk, head), 0.49 GB for one
+ * sequence of 60 000 tokens with 8 heads. */
+int64_t lampa_gdr_bwd_chunk_plan_size(const int64_t* cu_seqlens_host, int n_seq);
+int lampa_gdr_bwd_chunk_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int32_t* plan_host);
+int64_t lampa_gdr_bwd_chunk_workspace_bytes(const int32_t* plan_host, int HV);
+int lampa_gdr_bwd_chunk(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* h0,
+                        const void* dout, const float* dht, void* dq, void* dk, void* dv, float* dg, float* dbeta,
+                        float* dh0, const int32_t* plan_host, const int32_t* plan_dev, int H, int HV, int K, int V,
+                        int dtype, float scale, int l2norm, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Chunk / segment tables of the chunkwise forward, built on the host from the sequence boundaries.
  * Replaces prepare_chunk_indices / prepare_chunk_offsets (models/hattention/index.py:69-83).
  * cu_seqlens_host: int64 [n_seq+1]; chunks_per_segment: length of a segment of the split-sequence scan in

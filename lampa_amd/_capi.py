@@ -62,6 +62,10 @@ _SIGNATURES = {
                                                  _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),
     "lampa_gdr_bwd_workspace_bytes": (_i64, [_i64, _i32, _i32, _i32, _i32, _i32]),
     "lampa_gdr_bwd": (_i32, [_vp] * 18 + [_i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),
+    "lampa_gdr_bwd_chunk_plan_size": (_i64, [_vp, _i32]),
+    "lampa_gdr_bwd_chunk_plan_fill": (_i32, [_vp, _i32, _vp]),
+    "lampa_gdr_bwd_chunk_workspace_bytes": (_i64, [_vp, _i32]),
+    "lampa_gdr_bwd_chunk": (_i32, [_vp] * 16 + [_i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i64, _vp]),
     "lampa_profile_begin": (_i32, []),
     "lampa_profile_end": (_i32, [_i32, _vp, _vp]),
     "lampa_gdr_traffic_probe": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),

@@ -236,9 +236,65 @@ def _backward_tables(cu_host, seg_len: int, device):
     return tables
 
 
+# Backward pass in the chunked form on the matrix cores (``lampa_gdr_bwd_chunk``) where it is built: 16-bit inputs,
+# K = V = 64, one value head per q/k head. False sends everything to the fp32 token-serial form (``lampa_gdr_bwd``).
+CHUNKED_BACKWARD = True
+
+_backward_plan_cache = {}
+
+
+def _backward_chunk_plan(cu_host, device):
+    """Host + device copies of the chunk tables of ``lampa_gdr_bwd_chunk`` for these sequence boundaries (cached)."""
+    key = (tuple(cu_host), str(device))
+    hit = _backward_plan_cache.get(key)
+    if hit is not None:
+        return hit
+    lib = _capi.lib()
+    cu = (ctypes.c_int64 * len(cu_host))(*cu_host)
+    n_seq = len(cu_host) - 1
+    size = check(lib.lampa_gdr_bwd_chunk_plan_size(cu, n_seq), "lampa_gdr_bwd_chunk_plan_size")
+    host = torch.empty(size, dtype=torch.int32)
+    check(lib.lampa_gdr_bwd_chunk_plan_fill(cu, n_seq, ctypes.c_void_p(host.data_ptr())), "lampa_gdr_bwd_chunk_plan_fill")
+    dev = host.to(device)
+    if len(_backward_plan_cache) > 64:
+        _backward_plan_cache.clear()
+    _backward_plan_cache[key] = (host, dev)
+    return host, dev
+
+
+def _backward_chunk_supported(q, v) -> bool:
+    return (CHUNKED_BACKWARD and q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] == 64 and v.shape[-1] == 64
+            and q.shape[2] == v.shape[2])
+
+
+def _backward_chunk_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, do, dht):
+    """Gradients (dq, dk, dv, dg, dbeta, dh0) through ``lampa_gdr_bwd_chunk``."""
+    B, T, H, K = q.shape
+    HV, V = v.shape[2], v.shape[3]
+    q, k, v, do = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
+    cu_host = _sequence_bounds(cu_seqlens, B, T)
+    plan_host, plan_dev = _backward_chunk_plan(cu_host, q.device)
+    lib = _capi.lib()
+    ws_bytes = check(lib.lampa_gdr_bwd_chunk_workspace_bytes(ctypes.c_void_p(plan_host.data_ptr()), HV),
+                     "lampa_gdr_bwd_chunk_workspace_bytes")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dg, dbeta = torch.empty_like(g), torch.empty_like(beta)
+    h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+    dht = None if dht is None else dht.to(torch.float32).contiguous()
+    dh0 = None if h0 is None else torch.empty_like(h0)
+    check(lib.lampa_gdr_bwd_chunk(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(do), ptr(dht), ptr(dq), ptr(dk),
+                                  ptr(dv), ptr(dg), ptr(dbeta), ptr(dh0), ctypes.c_void_p(plan_host.data_ptr()),
+                                  ptr(plan_dev), H, HV, K, V, _DTYPES[q.dtype], float(scale), l2norm, ptr(ws), ws_bytes,
+                                  stream_of(q)), "lampa_gdr_bwd_chunk")
+    return dq, dk, dv, dg, dbeta, dh0
+
+
 def _backward_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, do, dht):
     """Gradients (dq, dk, dv, dg, dbeta, dh0) through ``lampa_gdr_bwd``. Head sizes that are not multiples of 4 are
     zero-padded (zero columns of q, k and v change neither the function nor the other columns' gradients)."""
+    if _backward_chunk_supported(q, v) and q.shape[0] * q.shape[1] > 0:
+        return _backward_chunk_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, do, dht)
     B, T, H, K = q.shape
     HV, V = v.shape[2], v.shape[3]
     if K > 128:
