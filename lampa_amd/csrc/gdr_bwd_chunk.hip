@@ -305,7 +305,7 @@ __device__ __forceinline__ void gb_store_mprime(unsigned char* out, int tr, int 
 // grid (chunks, HV), 256 threads. REV false: M' = -(D Kh)^T W, N = (D Kh)^T U. REV true: M'^T and
 // N' = scale (E Qh)^T dO - W^T (scale P^T dO), stored at the chunk's reverse item.
 template <typename T, bool REV>
-__global__ void __launch_bounds__(GB_THREADS, 2)
+__global__ void __launch_bounds__(GB_THREADS, 3)
     gdrb_maps_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const T* __restrict__ dout,
                      const unsigned char* __restrict__ recs, const int32_t* __restrict__ chunk_tok0,
                      const int32_t* __restrict__ chunk_len, const int32_t* __restrict__ chunk_item,
@@ -319,8 +319,8 @@ __global__ void __launch_bounds__(GB_THREADS, 2)
   OT* b_bk = b_t + GB_TILE;     // beta e^gamma kh, later e^{gamma_L - gamma} kh
   OT* b_w = b_bk + GB_TILE;     // W
   OT* b_u = b_w + GB_TILE;      // fwd: U;                rev: dO
-  OT* b_y = b_u + GB_TILE;      // rev: -scale P^T dO
-  float* fbase = reinterpret_cast<float*>(b_y + (REV ? GB_TILE : 0));
+  OT* b_y = b_bk;               // rev: -scale P^T dO, over the scaled k tile once M'^T is done
+  float* fbase = reinterpret_cast<float*>(b_u + GB_TILE);
   GbFactors f{fbase, fbase + 64, fbase + 128, fbase + 192, fbase + 256, fbase + 320};
 
   const int chunk = blockIdx.x, hv = blockIdx.y, h = hv / (HV / H);
@@ -429,6 +429,7 @@ __global__ void __launch_bounds__(GB_THREADS, 2)
     f32x16 y = gb_mm<OT, true, true>(b_t, 32 * tr, b_u, 32 * tc, 32 * tr, 64, zero16(), lane);
 #pragma unroll
     for (int r = 0; r < 16; ++r) y[r] = -y[r];
+    __syncthreads();  // every wave is past its reads of the scaled k tile (M'^T) and of qh (P)
     gb_store<OT>(b_y, 32 * tr, 32 * tc, y, lane);
     // scale e^gamma qh in place (every wave is past its reads of qh: P was stored behind the barrier above)
     {
@@ -477,8 +478,10 @@ __device__ __forceinline__ void gdrb_load_n(const unsigned char* Ncomp, size_t s
 
 // The state in front of every item of a "sequence" of the level. Start state: [n, HV, K, V] rows (H0_SLABS false, may
 // be NULL) or the fp32 slabs the level above left at slot `seq`.
+// grid (1, sequences of the level, HV), 4 waves: waves 2 vn, 2 vn + 1 own the 32-column slab vn (both slabs in one
+// workgroup read the same M' fragments, which then come from the CU's L1 the second time).
 template <typename OT, bool H0_SLABS, bool N16, bool OUT16>
-__global__ void __launch_bounds__(128) gdrb_scan_kernel(const int32_t* __restrict__ seg0s, const int32_t* __restrict__ nsegs,
+__global__ void __launch_bounds__(256) gdrb_scan_kernel(const int32_t* __restrict__ seg0s, const int32_t* __restrict__ nsegs,
                                                         const unsigned char* __restrict__ Mcomp,
                                                         const unsigned char* __restrict__ Ncomp,
                                                         const float* __restrict__ Dcomp, const float* __restrict__ h0,
@@ -487,13 +490,14 @@ __global__ void __launch_bounds__(128) gdrb_scan_kernel(const int32_t* __restric
   using X4 = typename OpVec<OT>::x4;
   constexpr int KT = 64, VT = 64, NKS = KT / 16, DEPTH = 4;
   constexpr int M_BYTES = KT * KT * 2;
-  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
-  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  __shared__ __align__(16) unsigned char s_xx[2][2][NKS * 1024];
+  const int vn = threadIdx.x >> 7, seq = blockIdx.y, hv = blockIdx.z;
   const int seg0 = seg0s[seq], nseg = nsegs[seq];
   if (nseg <= 0) return;
   const int nsteps = nseg - 1;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int tid = threadIdx.x & 127, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
   const int col = 32 * vn + ln;
+  unsigned char (*s_x)[NKS * 1024] = s_xx[vn];
   f32x16 S = zero16();
   if (H0_SLABS) {
     const f32x4* src = reinterpret_cast<const f32x4*>(h0 + (((size_t)seq * HV + hv) * (VT / 32) + vn) * (KT * 32));
@@ -565,24 +569,26 @@ __global__ void __launch_bounds__(128) gdrb_scan_kernel(const int32_t* __restric
 
 // Composite of every full group of GB_G items of a sequence but the last (which nothing follows): the step applied to
 // the 64 + 64 columns [P_M | P_N] from [I | 0]; stored like an item (D = the product of the decays, M' = P_M - D I as
-// 16-bit A-operand fragments, N = P_N in fp32) at slot seq * gmax + group. grid (4 * gmax, n_seq, HV).
+// 16-bit A-operand fragments, N = P_N in fp32) at slot seq * gmax + group.
+// grid (gmax, n_seq, HV), 8 waves: waves 2 b, 2 b + 1 own the 32-column block b of [P_M | P_N].
 template <typename OT, bool N16>
-__global__ void __launch_bounds__(128) gdrb_group_kernel(const int32_t* __restrict__ seg0s, const int32_t* __restrict__ nsegs,
+__global__ void __launch_bounds__(512, 4) gdrb_group_kernel(const int32_t* __restrict__ seg0s, const int32_t* __restrict__ nsegs,
                                                          const unsigned char* __restrict__ Msrc,
                                                          const unsigned char* __restrict__ Nsrc,
                                                          const float* __restrict__ Dsrc, unsigned char* __restrict__ Mout,
                                                          float* __restrict__ Nout, float* __restrict__ Dout, int HV,
                                                          int gmax) {
   using X8 = typename OpVec<OT>::x8;
-  constexpr int KT = 64, VT = 64, NKS = KT / 16, DEPTH = 4, G = GB_G;
+  constexpr int KT = 64, VT = 64, NKS = KT / 16, DEPTH = 2, G = GB_G;  // (two items in flight: 128 registers)
   constexpr int M_BYTES = KT * KT * 2;
-  __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
-  const int vn = blockIdx.x % 4, j = blockIdx.x / 4, seq = blockIdx.y, hv = blockIdx.z;
+  __shared__ __align__(16) unsigned char s_xx[4][2][NKS * 1024];
+  const int vn = threadIdx.x >> 7, j = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
   const int seg0 = seg0s[seq], nseg = nsegs[seq];
   const int ngroups = (nseg + G - 1) / G;
   if (j >= ngroups - 1) return;
   const int item0 = seg0 + j * G;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  const int tid = threadIdx.x & 127, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
+  unsigned char (*s_x)[NKS * 1024] = s_xx[vn];
   const bool is_pm = vn < KT / 32;
   const int nblk = max(vn - KT / 32, 0);
   f32x16 S = zero16();
@@ -1026,25 +1032,25 @@ static void gbc_scan(const int32_t* ph, const int32_t* pd, const GbcWorkspace& w
   unsigned char* M1 = ws + w.c1m; unsigned char* N1 = ws + w.c1n; float* D1 = (float*)(ws + w.c1d);
   unsigned char* M2 = ws + w.c2m; unsigned char* N2 = ws + w.c2n; float* D2 = (float*)(ws + w.c2d);
   float* S2 = (float*)(ws + w.s2); float* S1 = (float*)(ws + w.s1);
-  const dim3 blk(128);
+  const dim3 blk(256);
   if (g1 > 1) {
-    hipLaunchKernelGGL((gdrb_group_kernel<OT, true>), dim3(4 * g1, n_seq, HV), blk, 0, s, pd + ph[BP_OFF_L1G],
+    hipLaunchKernelGGL((gdrb_group_kernel<OT, true>), dim3(g1, n_seq, HV), dim3(512), 0, s, pd + ph[BP_OFF_L1G],
                        pd + ph[BP_OFF_L1G] + n_seq, M0, N0, D0, M1, (float*)N1, D1, HV, g1);
     LAMPA_PROF(s, "gdrb_group_kernel<items>");
   }
   if (g2 > 1) {
-    hipLaunchKernelGGL((gdrb_group_kernel<OT, false>), dim3(4 * g2, n_seq, HV), blk, 0, s, pd + ph[BP_OFF_L2G],
+    hipLaunchKernelGGL((gdrb_group_kernel<OT, false>), dim3(g2, n_seq, HV), dim3(512), 0, s, pd + ph[BP_OFF_L2G],
                        pd + ph[BP_OFF_L2G] + n_seq, M1, N1, D1, M2, (float*)N2, D2, HV, g2);
     LAMPA_PROF(s, "gdrb_group_kernel<groups>");
   }
   // the state in front of every supergroup, of every group, of every item
-  hipLaunchKernelGGL((gdrb_scan_kernel<OT, false, false, false>), dim3(2, n_seq, HV), blk, 0, s, pd + ph[BP_OFF_TOP],
+  hipLaunchKernelGGL((gdrb_scan_kernel<OT, false, false, false>), dim3(1, n_seq, HV), blk, 0, s, pd + ph[BP_OFF_TOP],
                      pd + ph[BP_OFF_TOP] + n_seq, M2, N2, D2, h0, (void*)S2, HV, n_seq * g2);
   LAMPA_PROF(s, "gdrb_scan_kernel<supergroups>");
-  hipLaunchKernelGGL((gdrb_scan_kernel<OT, true, false, false>), dim3(2, n_seq * g2, HV), blk, 0, s, pd + ph[BP_OFF_LEAF2],
+  hipLaunchKernelGGL((gdrb_scan_kernel<OT, true, false, false>), dim3(1, n_seq * g2, HV), blk, 0, s, pd + ph[BP_OFF_LEAF2],
                      pd + ph[BP_OFF_LEAF2] + n_seq * g2, M1, N1, D1, (const float*)S2, (void*)S1, HV, n_seq * g1);
   LAMPA_PROF(s, "gdrb_scan_kernel<groups>");
-  hipLaunchKernelGGL((gdrb_scan_kernel<OT, true, true, true>), dim3(2, n_seq * g1, HV), blk, 0, s, pd + ph[BP_OFF_LEAF1],
+  hipLaunchKernelGGL((gdrb_scan_kernel<OT, true, true, true>), dim3(1, n_seq * g1, HV), blk, 0, s, pd + ph[BP_OFF_LEAF1],
                      pd + ph[BP_OFF_LEAF1] + n_seq * g1, M0, N0, D0, (const float*)S1, (void*)S_items, HV, items);
   LAMPA_PROF(s, "gdrb_scan_kernel<items>");
 }
@@ -1056,7 +1062,7 @@ static int gbc_run(const void* q, const void* k, const void* v, const float* g, 
                    hipStream_t s) {
   const int n_seq = ph[BP_N_SEQ], chunks = ph[BP_CHUNKS];
   const GbcWorkspace w = gbc_workspace(chunks, ph[BP_ITEMS], n_seq, ph[BP_GMAX1], ph[BP_GMAX2], HV);
-  constexpr int smem_maps_f = 6 * GB_TILE * 2 + 6 * 64 * 4, smem_maps_r = 7 * GB_TILE * 2 + 6 * 64 * 4;
+  constexpr int smem_maps_f = 6 * GB_TILE * 2 + 6 * 64 * 4, smem_maps_r = smem_maps_f;
   constexpr int smem_grads = 9 * GB_TILE * 2 + (6 * 64 + 64 + 64 + 16) * 4;
   static bool attr_set[64] = {};
   static std::mutex attr_lock;
