@@ -256,6 +256,10 @@ def main():
         "hbm_frac": round(LAYER_BYTES_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "mfma_frac": round(LAYER_FLOP_PER_TOKEN_HEAD * token_heads / (layer_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "kernel_us": {n: round(u, 2) for n, u in stage_us.items()},
+        "kernel_us_sum": round(sum(stage_us.values()), 2),
+        "kernel_us_note": "HIP-event intervals of a separate pass: each holds the kernel and the gap to the next launch, "
+                          "and recording the events slows the pipeline by a few us, so their sum exceeds us_per_layer; "
+                          "the kernel-trace durations are in profiles/",
     }
 
     # ---- LSH stage (config 1): ids + keys + stable sort + feature gather, 3 tables ----
@@ -470,28 +474,54 @@ def main():
                "note": "algorithmic work per token-head: 1032 B and 182.9 kFLOP"}
     del d4
 
-    # ---- backward pass of the layer (lampa_gdr_bwd) at the headline shape and at the reference model's head sizes ----
+    # ---- backward pass of the layer at the headline shape and at the reference model's head sizes: the chunked form on
+    #      the MFMA (lampa_gdr_bwd_chunk) and, beside it, the fp32 token-serial form (lampa_gdr_bwd) ----
     def backward_leg(T_, H_, K_, V_, dtype_):
         qb, kb, vb, gb_, bb = (x.to(dev) for x in synth.gdr_inputs(1, T_, H_, K_, V_, dtype_, seed=0))
         dob = torch.randn_like(vb)
         fn = lambda: gd._backward_launch(qb, kb, vb, gb_, bb, K_ ** -0.5, None, None, gd.L2_CHUNK, dob, None)
-        us = time_us(fn, n=5, w=2)
-        _capi.profile_begin()
-        fn()
-        stage = {}
-        for name, ms in _capi.profile_end(max_entries=64):
-            if name != "start":
-                stage[name] = stage.get(name, 0.0) + 1e3 * ms
-        return {"workload": f"gradients of one gated-delta layer, B=1 H={H_} T={T_} K={K_} V={V_}, "
-                            f"{str(dtype_).split('.')[-1]} q/k/v/do, fp32 arithmetic",
-                "us": round(us, 1), "hits_per_s": round(T_ / (us * 1e-6), 1),
-                "kernel_us": {n: round(v_, 1) for n, v_ in stage.items()}}
+        out_ = {"workload": f"gradients of one gated-delta layer, B=1 H={H_} T={T_} K={K_} V={V_}, "
+                            f"{str(dtype_).split('.')[-1]} q/k/v/do"}
+        for form, flag in (("chunked", True), ("token_serial", False)):
+            gd.CHUNKED_BACKWARD = flag
+            try:
+                us = time_us(fn, n=10 if flag else 5, w=3)
+                _capi.profile_begin()
+                fn()
+                stage = {}
+                for name, ms in _capi.profile_end(max_entries=64):
+                    if name != "start":
+                        stage[name] = stage.get(name, 0.0) + 1e3 * ms
+            finally:
+                gd.CHUNKED_BACKWARD = True
+            out_[form] = {"us": round(us, 1), "hits_per_s": round(T_ / (us * 1e-6), 1),
+                          "kernel_us": {n: round(v_, 1) for n, v_ in stage.items()}}
+        out_["us"] = out_["chunked"]["us"]  # what chunk_gated_delta_rule's autograd takes
+        return out_
 
     backward = {"config2_shape": backward_leg(T, H, K, V, torch.bfloat16),
                 "reference_model_heads": backward_leg(30016, 6, 16, 32, torch.float16),
-                "note": "token-serial inside parallel segments, fp32: forward maps and scan, reverse maps and scan, then "
-                        "every segment forwards (a state kept every 8 tokens) and backwards block by block; dq, dk, dv, "
-                        "dg, dbeta out, q/k normalisation included"}
+                "note": "chunked: per-chunk affine maps of the state (forwards) and of its gradient (backwards) on the "
+                        "MFMA, a three-level scan over the maps, then every gradient of a chunk from its tiles and the "
+                        "two states; operands in the input type (heads below 64 x 64 zero-padded). token_serial: fp32, "
+                        "parallel segments, a state kept every 8 tokens. Both: dq, dk, dv, dg, dbeta out, q/k "
+                        "normalisation included"}
+
+    # ---- the reference layer's own head sizes (d_k = 16, d_v = 32, H = 6, fp16, T = 30000): the chunk operator
+    #      (zero-padded 32 x 32 heads) against the token-serial operator in parallel segments and as one run per head ----
+    qs, ks, vs, gs, bs = (x.to(dev) for x in synth.gdr_inputs(1, 30000, 6, 16, 32, torch.float16, seed=48, g_scale=0.05))
+    sm_chunk = time_us(lambda: gd.chunk_gated_delta_rule(qs, ks, vs, gs, bs), n=10, w=3)
+    sm_seg = time_us(lambda: gd.fused_recurrent_gated_delta_rule(qs, ks, vs, gs, bs), n=10, w=3)
+    keep = gd.SEGMENT_MIN_TOKENS
+    gd.SEGMENT_MIN_TOKENS = None
+    try:
+        sm_loop = time_us(lambda: gd.fused_recurrent_gated_delta_rule(qs, ks, vs, gs, bs), n=1, w=1)
+    finally:
+        gd.SEGMENT_MIN_TOKENS = keep
+    small_heads = {"workload": "B=1 H=6 T=30000 K=16 V=32 fp16 (the reference layer's head sizes)",
+                   "chunk_us": round(sm_chunk, 1), "token_serial_segments_us": round(sm_seg, 1),
+                   "token_serial_one_run_per_head_us": round(sm_loop, 1)}
+    del qs, ks, vs, gs, bs
 
     # ---- CPU baseline (reported, not a target): the reference's pure-PyTorch path on this box's host cores ----
     cpu = None
@@ -529,7 +559,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config2: chunk gated-delta forward, B=1 H=8 T=60000 K=V=64 C=64, bf16 q/k/v, fp32 "
                                "g/beta/state, LSH-sorted token order of a config-1 event"},
-        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0, "config4": config4, "backward": backward,
+        "roofline": roofline, "cpu_baseline": cpu, "layer": layer, "lsh": lsh_info, "block": block_info, "hgdn": hgdn_info, "config0": config0, "config4": config4, "backward": backward, "small_heads": small_heads,
     }
     print(json.dumps(out))
 

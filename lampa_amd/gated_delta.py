@@ -263,14 +263,28 @@ def _backward_chunk_plan(cu_host, device):
 
 
 def _backward_chunk_supported(q, v) -> bool:
-    return (CHUNKED_BACKWARD and q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] == 64 and v.shape[-1] == 64
-            and q.shape[2] == v.shape[2])
+    """16-bit inputs with K, V <= 64: smaller heads are zero-padded to 64 x 64 (as in the forward pass: zero columns of
+    q, k and v change neither the function nor the other columns' gradients), and grouped value heads (HV > H) run with
+    q and k repeated per value head, their gradients summed over each group afterwards."""
+    return (CHUNKED_BACKWARD and q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] <= 64 and v.shape[-1] <= 64
+            and q.data_ptr() % 16 == 0)
 
 
 def _backward_chunk_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, do, dht):
-    """Gradients (dq, dk, dv, dg, dbeta, dh0) through ``lampa_gdr_bwd_chunk``."""
+    """Gradients (dq, dk, dv, dg, dbeta, dh0) through ``lampa_gdr_bwd_chunk`` (built for K = V = 64, HV = H)."""
     B, T, H, K = q.shape
     HV, V = v.shape[2], v.shape[3]
+    pad = torch.nn.functional.pad
+    if K < 64:
+        q, k = pad(q, (0, 64 - K)), pad(k, (0, 64 - K))
+    if V < 64:
+        v, do = pad(v, (0, 64 - V)), pad(do, (0, 64 - V))
+    if (K, V) != (64, 64):
+        initial_state = None if initial_state is None else pad(initial_state.to(torch.float32), (0, 64 - V, 0, 64 - K))
+        dht = None if dht is None else pad(dht.to(torch.float32), (0, 64 - V, 0, 64 - K))
+    rep = HV // H
+    if rep > 1:
+        q, k = q.repeat_interleave(rep, dim=2), k.repeat_interleave(rep, dim=2)
     q, k, v, do = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
     cu_host = _sequence_bounds(cu_seqlens, B, T)
     plan_host, plan_dev = _backward_chunk_plan(cu_host, q.device)
@@ -285,8 +299,14 @@ def _backward_chunk_launch(q, k, v, g, beta, scale, initial_state, cu_seqlens, l
     dh0 = None if h0 is None else torch.empty_like(h0)
     check(lib.lampa_gdr_bwd_chunk(ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(do), ptr(dht), ptr(dq), ptr(dk),
                                   ptr(dv), ptr(dg), ptr(dbeta), ptr(dh0), ctypes.c_void_p(plan_host.data_ptr()),
-                                  ptr(plan_dev), H, HV, K, V, _DTYPES[q.dtype], float(scale), l2norm, ptr(ws), ws_bytes,
+                                  ptr(plan_dev), HV, HV, 64, 64, _DTYPES[q.dtype], float(scale), l2norm, ptr(ws), ws_bytes,
                                   stream_of(q)), "lampa_gdr_bwd_chunk")
+    if rep > 1:  # the value heads of a group share their q / k head
+        dq = dq.view(B, T, H, rep, 64).float().sum(3).to(q.dtype)
+        dk = dk.view(B, T, H, rep, 64).float().sum(3).to(k.dtype)
+    if (K, V) != (64, 64):
+        dq, dk, dv = dq[..., :K].contiguous(), dk[..., :K].contiguous(), dv[..., :V].contiguous()
+        dh0 = None if dh0 is None else dh0[..., :K, :V].contiguous()
     return dq, dk, dv, dg, dbeta, dh0
 
 

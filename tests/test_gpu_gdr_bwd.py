@@ -46,7 +46,10 @@ def _gpu_grads(device, q, k, v, g, beta, do, h0, dht, cu, l2, scale=None):
     return [a.grad for a in args] + [None if h0d is None else h0d.grad]
 
 
-def _check(got, want, dtype, chunked=False):
+def _check(got, want, dtype, chunked=None):
+    """chunked: the gradients came from the chunked form (default: every 16-bit case while ``gd.CHUNKED_BACKWARD``)."""
+    if chunked is None:
+        chunked = dtype != torch.float32 and gd.CHUNKED_BACKWARD
     for name, a, b in zip(NAMES, got, want):
         if b is None:
             assert a is None, name
@@ -75,11 +78,15 @@ def test_gradients_fp32_match_oracle(device, K, V, H, HV, l2):
     _check(_gpu_grads(device, q, k, v, g, beta, do, h0, dht, None, l2, scale=0.37), want, torch.float32)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-def test_gradients_varlen_segments(device, dtype, monkeypatch):
+@pytest.mark.parametrize("dtype,chunked", [(torch.float32, False), (torch.bfloat16, False), (torch.float16, False),
+                                           (torch.bfloat16, True), (torch.float16, True)])
+def test_gradients_varlen_segments(device, dtype, chunked, monkeypatch):
     """Packed sequences (an empty one, one shorter than a block, lengths off the block and segment sizes), cut into
-    segments of 64 tokens so that the reverse maps and the reverse scan carry the state gradient over many segments."""
+    segments of 64 tokens so that the reverse maps and the reverse scan carry the state gradient over many segments.
+    16-bit inputs through both forms: token-serial, and chunked with the 32 x 32 heads zero-padded to 64 x 64 and the
+    two value heads of a group sharing their q / k head."""
     monkeypatch.setattr(gd, "BACKWARD_UNITS", 1 << 20)
+    monkeypatch.setattr(gd, "CHUNKED_BACKWARD", chunked)
     lens = [0, 5, 333, 64, 1, 500, 97]
     T = sum(lens)
     (q, k, v, g, beta, do), gen = _inputs(1, T, 2, 4, 32, 32, dtype, 7, unit=False)
@@ -134,7 +141,16 @@ def test_gradients_without_states_and_with_unused_output(device):
 
 def test_gradients_long_sequence_weak_decay(device):
     """4 096 tokens with g of the order of -0.003 per token: the state and its gradient carry over hundreds of tokens
-    and through every segment."""
+    and through every segment (token-serial form; the chunked form has its own case below)."""
+    gd_chunked = gd.CHUNKED_BACKWARD
+    gd.CHUNKED_BACKWARD = False
+    try:
+        _weak_decay_case(device)
+    finally:
+        gd.CHUNKED_BACKWARD = gd_chunked
+
+
+def _weak_decay_case(device):
     (q, k, v, g, beta, do), gen = _inputs(1, 4096, 1, 2, 64, 64, torch.bfloat16, 11, unit=False, g_scale=0.003)
     h0 = 0.5 * torch.randn(1, 2, 64, 64, generator=gen)
     dht = torch.randn(1, 2, 64, 64, generator=gen)
