@@ -117,6 +117,7 @@ class LshgdBlock(nn.Module):
         # kept as bit patterns so that module.to(bfloat16) leaves the float32 hash parameters alone
         self.register_buffer("lsh_alpha_bits", alpha.view(torch.int32))
         self.register_buffer("lsh_beta_bits", beta.view(torch.int32))
+        self._flags_host = None  # pinned copy of the LSH stage's flag fields (one per table), made on first use
 
     @property
     def lsh_alpha(self) -> torch.Tensor:
@@ -127,30 +128,55 @@ class LshgdBlock(nn.Module):
         return self.lsh_beta_bits.view(torch.float32)
 
     @torch.no_grad()
-    def order(self, coords: torch.Tensor) -> torch.Tensor:
-        """Sequence order of the hits: the stable bucket-sort permutation of the first hash table (int32 [N]). The flag
-        field of the stage is read once per event (one small copy to the host): when a workgroup of the one-launch
-        kernel gave up a wait (``lsh.META_GAVE_UP``) the stage runs again as separate kernels, which wait for nothing; a
-        key that does not fit 32 bits raises."""
+    def order(self, coords: torch.Tensor, check: bool = True):
+        """Sequence order of the hits: the stable bucket-sort permutation of the first hash table (int32 [N]).
+        ``check=True`` reads the flag field of the stage at once (one host synchronisation): when a workgroup of the
+        one-launch kernel gave up a wait (``lsh.META_GAVE_UP``) the stage runs again as separate kernels, which wait for
+        nothing; a key that does not fit 32 bits raises. ``check=False`` returns ``(perm, pending)`` instead and leaves
+        the flags to ``_flags_of(pending)``: they are copied to pinned host memory behind the kernel, so that the caller
+        can queue its other launches first and look at them without draining the stream."""
         args = (coords.float(), self.lsh_alpha, self.lsh_beta, self.bucket_width, self.n_tables, self.n_proj)
         out = lsh.lsh_bucket_sort(*args, return_ids=False)
+        if not check:
+            if self._flags_host is None:
+                self._flags_host = torch.empty(self.n_tables, dtype=torch.int32, pin_memory=True)
+            self._flags_host.copy_(out["meta"][..., -1], non_blocking=True)
+            done = torch.cuda.Event()
+            done.record()
+            return out["perm"][0], done
         flags = lsh.decode_meta_flags(out["meta"])
         if bool(flags["gave_up"].any()):
-            lsh.one_launch_config(enabled=False)
-            try:
-                out = lsh.lsh_bucket_sort(*args, return_ids=False, strict=True)
-            finally:
-                lsh.one_launch_config(enabled=True)
-        elif bool(flags["key_overflow"][0]):
+            return self._order_with_separate_kernels(args)
+        if bool(flags["key_overflow"][0]):
             raise lsh.LampaError("LshgdBlock: the bucket key of the first hash table does not fit 32 bits; the "
                                  "sequence order would be meaningless")
         return out["perm"][0]
 
+    def _order_with_separate_kernels(self, args):
+        lsh.one_launch_config(enabled=False)
+        try:
+            return lsh.lsh_bucket_sort(*args, return_ids=False, strict=True)["perm"][0]
+        finally:
+            lsh.one_launch_config(enabled=True)
+
+    def _flags_of(self, done) -> int:
+        """The flag fields of the last ``order(check=False)`` call, OR-ed over the tables (waits for that kernel only)."""
+        done.synchronize()
+        flags = 0
+        for f in self._flags_host.tolist():
+            flags |= f
+        return flags
+
     @torch.no_grad()
-    def forward(self, feats: torch.Tensor, coords: torch.Tensor) -> torch.Tensor:
-        """feats [N, in_dim], coords [N, coord_dim] -> [N, out_dim] in the parameters' dtype, in the input hit order."""
+    def forward(self, feats: torch.Tensor, coords: torch.Tensor, perm: torch.Tensor = None) -> torch.Tensor:
+        """feats [N, in_dim], coords [N, coord_dim] -> [N, out_dim] in the parameters' dtype, in the input hit order.
+        The LSH stage's flag field is looked at once per event, after every launch of the block has been queued: a
+        one-launch kernel that gave up a wait (its permutation is then all -1) makes the block run again with the order
+        from the separate kernels; a key overflow raises."""
         dtype = self.input.weight.dtype
-        perm = self.order(coords)
+        pending = None
+        if perm is None:
+            perm, pending = self.order(coords, check=False)
         x = self.input(feats.to(dtype))
         x = lsh.gather_rows(x[None], perm[None])                                 # [1, N, hidden], LSH order
         h, residual = self.norms[0](x, None, True)                               # residual = x, h = norm(x)
@@ -158,4 +184,13 @@ class LshgdBlock(nn.Module):
             next_norm = self.norms[i + 1] if i + 1 < len(self.layers) else self.norm_f
             (h, residual), _ = layer(h, residual=residual, next_norm=next_norm)
         h = lsh.scatter_rows(h, perm[None])[0]                                   # back to the input order
-        return self.head(h)
+        out = self.head(h)
+        if pending is not None:
+            flags = self._flags_of(pending)
+            if flags & lsh.META_GAVE_UP:
+                args = (coords.float(), self.lsh_alpha, self.lsh_beta, self.bucket_width, self.n_tables, self.n_proj)
+                return self.forward(feats, coords, perm=self._order_with_separate_kernels(args))
+            if self._flags_host[0].item() & lsh.META_KEY_OVERFLOW:
+                raise lsh.LampaError("LshgdBlock: the bucket key of the first hash table does not fit 32 bits; the "
+                                     "sequence order would be meaningless")
+        return out

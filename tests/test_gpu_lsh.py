@@ -313,6 +313,14 @@ def test_one_launch_give_up_path_poisons_the_outputs(device):
         order = blk.order(cd)
         blk_alpha, blk_beta = blk.lsh_alpha.cpu().numpy(), blk.lsh_beta.cpu().numpy()
         assert np.array_equal(_np(order), ol.bucket_sort(coords.numpy(), blk_alpha, blk_beta, 0.5, 3, 4)["perm"][0])
+        # the whole block: it looks at the flags after queuing its launches and runs again with that order
+        torch.manual_seed(2)
+        blk16 = lb.LshgdBlock().to(device).to(torch.bfloat16)
+        lsh.one_launch_config()
+        want_out = blk16(fd, cd)
+        lsh.one_launch_config(wait_limit=0)
+        got_out = blk16(fd, cd)
+        assert torch.equal(got_out, want_out) and bool(torch.isfinite(got_out.float()).all())
     finally:
         lsh.one_launch_config()
     again = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, fd, strict=True)
