@@ -282,7 +282,9 @@ int lampa_gdr_recurrent_segmented_fwd(const void* q, const void* k, const void* 
  * the tables of the pass that runs backwards: seq_seg0_rev device int32 [n_seq+1] = seq_seg0[s] + s, and seg_rev device
  * int32 [n_seg] = seq_seg0_rev[s] + (last segment of s) - p for segment p of sequence s.
  * K <= 128, K and V multiples of 4, q and k 16-byte aligned, at most 64 value heads per q/k head, n_seq <= 65535
- * (LAMPA_ERR_UNSUPPORTED otherwise). workspace: lampa_gdr_bwd_workspace_bytes(total_tokens, n_seq, n_seg, HV, K, V). */
+ * (LAMPA_ERR_UNSUPPORTED otherwise). workspace: lampa_gdr_bwd_workspace_bytes(total_tokens, n_seq, n_seg, HV, K, V);
+ * it grows with the tokens (the state kept at every 8th token) and with the segments: 1.9 GB for one sequence of
+ * 60 000 tokens with 8 heads of 64 x 64 cut into 2048 units. */
 int64_t lampa_gdr_bwd_workspace_bytes(int64_t total_tokens, int n_seq, int n_seg, int HV, int K, int V);
 int lampa_gdr_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* h0,
                   const void* dout, const float* dht, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
@@ -300,8 +302,9 @@ int lampa_gdr_bwd(const void* q, const void* k, const void* v, const float* g, c
  * carry the rounding of that type. g <= 0 is assumed (the forward's masking of positive exponents is not differentiated).
  * Shapes as for lampa_gdr_bwd. plan: lampa_gdr_bwd_chunk_plan_fill's tables of the sequence boundaries
  * (cu_seqlens_host: int64 [n_seq+1]), the same int32 array in host and in device memory.
- * workspace: lampa_gdr_bwd_chunk_workspace_bytes(plan_host, HV): about 64 KiB per (chunk, head), 0.49 GB for one
- * sequence of 60 000 tokens with 8 heads. */
+ * workspace: lampa_gdr_bwd_chunk_workspace_bytes(plan_host, HV): about 41 KiB per (chunk, head) -- the chunk's record,
+ * its two map parts and the state and state gradient it starts from, all in the 16-bit input type, plus the maps and
+ * states of the groups -- 0.33 GB for one sequence of 60 000 tokens with 8 heads (lampa_gdr_bwd: 1.9 GB there). */
 int64_t lampa_gdr_bwd_chunk_plan_size(const int64_t* cu_seqlens_host, int n_seq);
 int lampa_gdr_bwd_chunk_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int32_t* plan_host);
 int64_t lampa_gdr_bwd_chunk_workspace_bytes(const int32_t* plan_host, int HV);

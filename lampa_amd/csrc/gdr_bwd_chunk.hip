@@ -15,10 +15,11 @@
 // Both state sequences are affine recurrences over the chunks (S' = M S + N forwards, dS = M^T G' + N' backwards, with the
 // same M = e^{gamma_L} I - (D Kh)^T W), so nothing here is serial in the tokens and only a short scan is serial in the
 // chunks:
-//   maps   one workgroup per (chunk, head): the chunk's map (M - dI as 16-bit MFMA A-operand fragments, N in fp32), once
-//          for the forward direction and once for the reverse one;
+//   maps   one workgroup per (chunk, head): the chunk's map (M - dI as 16-bit MFMA A-operand fragments, N in the 16-bit
+//          operand type, the decay d in fp32), once for the forward direction and once for the reverse one;
 //   scan   the states entering every chunk (forwards) and the gradients leaving every chunk (backwards) by a scan
-//          over the maps in three levels of groups of 8, with the scan kernels of the forward pass;
+//          over the maps in three levels of groups of 8 (the step of the forward pass's scan kernels; the maps of the
+//          groups keep N and the states in fp32, the states in front of the chunks are stored in the operand type);
 //   grads  one workgroup per (chunk, head): every gradient of the chunk from its tiles, S and G'.
 #include "gdr_chunk_kernels.h"
 #include <mutex>
