@@ -328,6 +328,11 @@ int lampa_gdr_chunk_fwd(const void* q, const void* k, const void* v, const float
                         const float* h0, float* ht, const int32_t* plan_host, const int32_t* plan_dev, int H, int HV,
                         int K, int V, int dtype, float scale, int l2norm, void* workspace, int64_t workspace_bytes,
                         void* stream);
+/* Process-wide choice of the output pass's form (no counterpart in the reference; for A/B measurements). The pass
+ * exists with 32 value columns per recurrence wave (32x32x16 MFMA) and, for K >= 64, with 16 ("narrow": 16x16x32 MFMA,
+ * twice the waves, each with half the dependent chain of a chunk). narrow_output 0: never the narrow form; 1 (default):
+ * where it is the faster one, i.e. for heads wider than 64 x 64; 2: wherever it is built. Results agree to rounding. */
+int lampa_gdr_chunk_config(int narrow_output);
 
 /* Hierarchical (level-weighted) chunkwise forward. Replaces chunk_h_gated_delta_rule -> hattention_kernel ->
  * chunkwise_fwd (models/hattention/gated_delta_rule_apis.py:21-91, kernel.py:338-374, chunkwise_hgdn.py:565-791;

@@ -74,6 +74,7 @@ _SIGNATURES = {
     "lampa_gdr_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),
     "lampa_gdr_chunk_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                    _f32, _i32, _vp, _i64, _vp]),
+    "lampa_gdr_chunk_config": (_i32, [_i32]),
     "lampa_hgdn_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),
     "lampa_hgdn_chunk_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32,
                                     _i32, _i32, _f32, _i32, _vp, _i64, _vp]),

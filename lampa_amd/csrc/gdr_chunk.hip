@@ -1,6 +1,7 @@
 // Host side of the chunkwise gated-delta-rule forward: workspace layout, launch sequence and the C entry points.
 // The kernels (and the description of the algorithm) are in gdr_chunk_kernels.h.
 #include "gdr_chunk_kernels.h"
+#include <atomic>
 #include <mutex>
 
 struct GdrWorkspace {
@@ -24,6 +25,15 @@ static GdrWorkspace gdr_workspace(int64_t chunks, int64_t segs, int HV, int K, i
   return w;
 }
 
+// Output pass with narrow chain waves (16 value columns per wave on the 16x16x32 MFMA; built for K >= 64).
+// 0: never, 1: where it is the faster form (heads wider than 64 x 64), 2: wherever it is built.
+static std::atomic<int> gdr_narrow_output{1};
+extern "C" int lampa_gdr_chunk_config(int narrow_output) {
+  if (narrow_output < 0 || narrow_output > 2) return LAMPA_ERR_INVALID;
+  gdr_narrow_output.store(narrow_output);
+  return LAMPA_OK;
+}
+
 static bool gdr_chunk_supported(int K, int V) {
   return ((K == 64 || K == 128) && (V == 64 || V == 128)) || (K == 32 && V == 32);
 }
@@ -45,6 +55,8 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   float* Dc = (float*)(ws + w.off_d);
   float* Si = (float*)(ws + w.off_sinit);
   constexpr int smem_a = GdrSegSmem<KT, VT, false>::BYTES, smem_b = GdrSegSmem<KT, VT, true>::BYTES;
+  constexpr int CWN = KT >= 64 ? 16 : 32;  // chain-wave width of the narrow output pass (K = 32 has none)
+  constexpr int smem_n = GdrSegSmem<KT, VT, true, false, GdrSegShape<KT, VT, true, CWN>::DOUBLE_Q ? 2 : 1>::BYTES;
   // the dynamic LDS limit is a per-device attribute of a kernel: set once per device and instantiation
   static bool attr_set[64] = {};
   static std::mutex attr_lock;  // (several host threads may call at once)
@@ -55,7 +67,9 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
     if (hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem_a) != hipSuccess ||
         hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, true>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_b) != hipSuccess ||
+        hipFuncSetAttribute((const void*)gdr_segment_kernel<T, KT, VT, true, false, T, CWN>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem_n) != hipSuccess)
       return LAMPA_ERR_LAUNCH;
     attr_set[dev] = true;
   }
@@ -97,6 +111,13 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
                        pv, Mc, Nc, Dc, h0, Si, HV, segs);
     LAMPA_PROF(s, "gdr_scan_kernel");
   }
+  const int narrow = gdr_narrow_output.load();
+  if (CWN == 16 && (narrow == 2 || (narrow == 1 && KT + VT > 128)))
+    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true, false, T, CWN>), dim3(segs, HV),
+                       dim3(64 * GdrSegShape<KT, VT, true, CWN>::WAVES), smem_n, s, (const T*)q, (const T*)k, (const T*)v, g, beta,
+                       pv, pv.chunk_tok0, pv.chunk_len, tf, Si, Mc, Nc, Dc, (T*)o, ht, H, HV, scale, l2norm,
+                       (const unsigned char*)Gm, (const unsigned char*)Gn, (const float*)Gd, h0, walk_in_output ? gmax : 0);
+  else
   hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
                      (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, Mc, Nc, Dc, (T*)o, ht, H, HV, scale,
                      l2norm, (const unsigned char*)Gm, (const unsigned char*)Gn, (const float*)Gd, h0, walk_in_output ? gmax : 0);

@@ -503,7 +503,8 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
 //   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
 //                                                          -> the stagers may write q(c+1)
 // Global loads are issued about one chunk period before their data is staged.
-template <int KT, int VT, bool PASS_B, bool SCALED = !PASS_B>
+// NQ: copies of the q tile, the P fragments and the q factor rows (2: by chunk parity, like the tile sets)
+template <int KT, int VT, bool PASS_B, bool SCALED = !PASS_B, int NQ = 1>
 struct GdrSegSmem {
   static constexpr int SK = KT + 8;  // row stride of the k / q tiles (bf16 elements)
   static constexpr int SV = VT + 8;  // row stride of the v and o tiles
@@ -516,11 +517,12 @@ struct GdrSegSmem {
   static constexpr int N_FACT = 6;  // beta, ek, dk, gamma, rk, misc
   static constexpr int T_OFF_KD = T_OFF_F + N_FACT * 64 * 4;  // PASS_A: second scaled copy of the k tile
   static constexpr int TILE_BYTES = T_OFF_KD + (SCALED ? 64 * SK * 2 : 0);
+  static constexpr int Q_BYTES = 64 * SK * 2, P_BYTES = 6 * 1024, QF_BYTES = 2 * 64 * 4;
   static constexpr int OFF_Q = 2 * TILE_BYTES;
-  static constexpr int OFF_P = OFF_Q + (PASS_B ? 64 * SK * 2 : 0);
-  static constexpr int OFF_O = OFF_P + (PASS_B ? 6 * 1024 : 0);
+  static constexpr int OFF_P = OFF_Q + (PASS_B ? NQ * Q_BYTES : 0);
+  static constexpr int OFF_O = OFF_P + (PASS_B ? NQ * P_BYTES : 0);
   static constexpr int OFF_QF = OFF_O + (PASS_B ? 64 * SV * 2 : 0);  // qs, rq
-  static constexpr int BYTES = OFF_QF + (PASS_B ? 2 * 64 * 4 : 0);
+  static constexpr int BYTES = OFF_QF + (PASS_B ? NQ * QF_BYTES : 0);
 };
 
 // pointers into one of the two tile sets
@@ -535,20 +537,33 @@ struct GdrTilesT {
   float *beta, *ek, *dk, *gamma, *rk, *misc;  // ek = e^{gamma_i} rk_i, dk = e^{gamma_last - gamma_i} rk_i, misc[0] = e^{gamma_last}
 };
 
-template <int KT, int VT, bool PASS_B>
+// CW: columns of the state per chain wave. 32: products on the 32x32x16 MFMA. 16 (output pass, K >= 64): "narrow" chain
+// waves on the 16x16x32 MFMA -- twice as many waves, each with half the dependent MFMA -> convert -> MFMA chain of a chunk
+// and half the state registers (K / 4 per lane).
+template <int KT, int VT, bool PASS_B, int CW = 32>
 struct GdrSegShape {
-  static constexpr int SLABS = PASS_B ? VT / 32 : (KT + VT) / 32;  // chain waves
-  static constexpr int WAVES = SLABS + 2;                          // + two stager waves
+  static_assert(CW == 32 || (CW == 16 && PASS_B && KT >= 64), "narrow chain waves: output pass, K >= 64");
+  static constexpr int SLABS = PASS_B ? VT / CW : (KT + VT) / 32;  // chain waves
+  // + the stager waves: two (each stages half the rows of every tile and builds part of P), or, beside narrow chain
+  // waves, two pairs -- one for k, v, T and the per-token factors, one for q and P -- so that neither role needs more
+  // registers than four waves per SIMD leave
+  static constexpr int STAGERS = CW == 16 ? 4 : 2;
+  static constexpr bool DOUBLE_Q = CW == 16 && KT + VT > 128;  // q tile and P fragments double-buffered (LDS allows it)
+  static constexpr int WAVES = SLABS + STAGERS;
   // The k and q tiles are stored swizzled (op_swizzle16 in gdr_ops.h: one conflict-free 16-byte LDS read per operand
   // fragment instead of two 8-byte reads). It pays in the output pass of the 128-wide heads (-10 %); at K = V = 64
   // the output pass times the same and the composite pass loses: the wider reads cost it 24 registers, and two of
   // its six-wave workgroups only share a CU below 128 (the hardware deals a workgroup's waves out to the SIMDs in a
   // fixed rotation and starts the next workgroup one step further on, so one SIMD carries four of the twelve waves).
-  static constexpr bool SWIZZLED = PASS_B && (KT > 64 || VT > 64);
+  // (the composite pass of the 128-wide heads, whose LDS is 90 % busy with half of it bank conflicts, gets slower with
+  // swizzled scaled tiles: 814 -> 909 us at config 4 -- the swizzled 16-byte reads cost it registers it does not have)
+  static constexpr bool SWIZZLED = CW == 32 && PASS_B && (KT > 64 || VT > 64);
   // Waves per SIMD the register allocation has to leave room for (the second argument of the launch bounds). The
   // composite pass at K = V = 64 runs two six-wave workgroups per CU, and the hardware's rotation puts four of those
   // twelve waves on one SIMD: 128 registers each.
-  static constexpr int WAVES_PER_SIMD = (!PASS_B && KT + VT <= 128) ? 4 : 2;  // (with the scaled k tiles)
+  // Narrow output pass: K = V = 64 runs two eight-wave workgroups per CU (four waves per SIMD), the wider heads one
+  // workgroup of up to twelve waves (three per SIMD).
+  static constexpr int WAVES_PER_SIMD = CW == 16 ? (KT + VT <= 128 ? 4 : 3) : (!PASS_B && KT + VT <= 128) ? 4 : 2;
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -577,8 +592,9 @@ __device__ __forceinline__ bf16x8 ld_kappa_tr(const __bf16* arr, int stride, int
   return out;
 }
 
-template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B, typename OT = T>
-__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SCALED_K ? GdrSegShape<KT, VT, PASS_B>::WAVES_PER_SIMD : 2))
+template <typename T, int KT, int VT, bool PASS_B, bool SCALED_K = !PASS_B, typename OT = T, int CW = 32>
+__global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
+                                  ((SCALED_K || CW == 16) ? GdrSegShape<KT, VT, PASS_B, CW>::WAVES_PER_SIMD : 2))
     gdr_segment_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                        const float* __restrict__ g, const float* __restrict__ beta, const GdrPlanView pv,
                        const int32_t* __restrict__ chunk_tok0, const int32_t* __restrict__ chunk_len,
@@ -593,13 +609,22 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
   using X8 = typename OpVec<OT>::x8;
   using X4 = typename OpVec<OT>::x4;
   constexpr bool SCALED = !PASS_B && SCALED_K;
-  constexpr bool SWZ = GdrSegShape<KT, VT, PASS_B>::SWIZZLED;
+  constexpr bool SWZ = GdrSegShape<KT, VT, PASS_B, CW>::SWIZZLED;
+  // narrow chain waves: the k, q and T tiles keep every 32 columns in the order of op_perm32 (gdr_ops.h)
+  constexpr bool P16 = CW == 16;
+  // The narrow form keeps the k, q and T tiles in op_perm32 order (one 16-byte read per operand fragment). With the
+  // tiles in plain order and two 8-byte reads per fragment the output pass is slower: 71.0 against 68.2 us at
+  // K = V = 64, 1 463 against 1 290 us at K = V = 128 (config 4).
+  constexpr bool PERM = P16;
   // Output pass at K <= 64: a stager builds the P tiles of the q rows it staged itself (stager 0 the tile (0,0),
   // stager 1 the tiles (1,0) and (1,1)), so no barrier separates staging q from building P. At K = 128 a P tile is
   // twice the work, the two stagers share the middle tile, and the barrier Qb(c) (q(c) is staged) comes back.
-  constexpr bool OWN_Q = KT <= 64;
-  using SM = GdrSegSmem<KT, VT, PASS_B, SCALED>;
-  constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B>::SLABS;
+  constexpr bool OWN_Q = KT <= 64 || CW == 16;  // (the narrow form's q / P stagers have registers of their own to spare)
+  // Narrow form of the heads wider than 64 x 64 (one workgroup per CU, LDS to spare): q, P and the q factor rows exist
+  // twice, so the q / P stagers stage q(c + 1) while the chain waves still read q(c) and P(c).
+  constexpr bool DBQ = GdrSegShape<KT, VT, PASS_B, CW>::DOUBLE_Q;
+  using SM = GdrSegSmem<KT, VT, PASS_B, SCALED, DBQ ? 2 : 1>;
+  constexpr int NSLAB = GdrSegShape<KT, VT, PASS_B, CW>::SLABS;
   constexpr int SK = SM::SK, SV = SM::SV, ST = SM::ST;
   extern __shared__ __align__(16) unsigned char smem[];
   auto tiles = [&](int par) {
@@ -617,11 +642,17 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
     t.misc = t.beta + 320;
     return t;
   };
-  OT* s_q = reinterpret_cast<OT*>(smem + SM::OFF_Q);
-  unsigned char* s_P = smem + SM::OFF_P;
+  OT* const s_q0 = reinterpret_cast<OT*>(smem + SM::OFF_Q);
+  unsigned char* const s_P0 = smem + SM::OFF_P;
   T* s_o = reinterpret_cast<T*>(smem + SM::OFF_O);
-  float* s_qs = reinterpret_cast<float*>(smem + SM::OFF_QF);  // scale e^{gamma_i} rq_i
-  float* s_rq = s_qs + 64;
+  float* const s_qs0 = reinterpret_cast<float*>(smem + SM::OFF_QF);  // scale e^{gamma_i} rq_i, then rq_i
+  // the copy of the q tile / the P fragments / the factor rows that belongs to a chunk of parity par
+#define GDR_Q_BUFFERS(par)                                                          \
+  OT* const s_q = s_q0 + (DBQ ? (par) : 0) * (SM::Q_BYTES / 2);                     \
+  unsigned char* const s_P = s_P0 + (DBQ ? (par) : 0) * SM::P_BYTES;                \
+  float* const s_qs = s_qs0 + (DBQ ? (par) : 0) * (SM::QF_BYTES / 4);               \
+  float* const s_rq = s_qs + 64;                                                    \
+  (void)s_q; (void)s_P; (void)s_qs; (void)s_rq
 
   const int seg = blockIdx.x, hv = blockIdx.y;
   const int h = hv / (HV / H);
@@ -636,7 +667,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
   if (wave >= NSLAB) {
     // ================================================ stager ================================================
     constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
-    const int stid = tid - 64 * NSLAB, sw = wave - NSLAB;
+    // (narrow form: pair 0 = waves NSLAB, NSLAB + 1 stages k, v, T and the factors, pair 1 = the next two q and P; a
+    // pair is the 128 threads the staging code is written for)
+    const int spair = P16 ? (wave - NSLAB) >> 1 : 0;
+    const int stid = tid - 64 * (NSLAB + 2 * spair), sw = (wave - NSLAB) & 1;
     const int srow = stid >> 1, spart = stid & 1;
     // PASS_A keeps the raw k rows of two chunks (sets by chunk parity): the scaled tiles are written from the
     // registers after the row norms are known, and the next k loads must already be on their way by then
@@ -654,10 +688,23 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
       int row, part;
       const int da = stid, db = 128 + (stid & 31);  // indices among the 160 packed pieces (T11: 0 .. 79, T22: 80 .. 159)
       tri_piece(da < T_DIAG_PIECES ? da : da - T_DIAG_PIECES, row, part);
-      ta_off = ((da < T_DIAG_PIECES ? 0 : 2) * 32 + row) * ST + 8 * part;
+      ta_off = ((da < T_DIAG_PIECES ? 0 : 2) * 32 + row) * ST + (PERM ? op_perm32_piece(part) : 8 * part);
       tri_piece(db - T_DIAG_PIECES, row, part);
-      tb_off = (2 * 32 + row) * ST + 8 * part;
+      tb_off = (2 * 32 + row) * ST + (PERM ? op_perm32_piece(part) : 8 * part);
     }
+    const int t21_off = (1 * 32 + (stid >> 2)) * ST + (PERM ? op_perm32_piece(stid & 3) : 8 * (stid & 3));
+    // a 16-byte piece of T into a tile: as it is, or (P16) its two halves 8 elements apart
+    auto put_t = [&](OT* at, X8 v) __attribute__((always_inline)) {
+      if constexpr (PERM) {
+        X4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { lo[e] = v[e]; hi[e] = v[4 + e]; }
+        *reinterpret_cast<X4*>(at) = lo;
+        *reinterpret_cast<X4*>(at + 8) = hi;
+      } else {
+        *reinterpret_cast<X8*>(at) = v;
+      }
+    };
     if (stid < 128 - T_DIAG_PIECES) {
       int ur, up;
       tri_upper_piece(stid, ur, up);
@@ -667,8 +714,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
 #pragma unroll
       for (int par = 0; par < 2; ++par) {
         OT* tt = tiles(par).t;
-        *reinterpret_cast<X8*>(&tt[(0 * 32 + ur) * ST + 8 * up]) = z8;
-        *reinterpret_cast<X8*>(&tt[(2 * 32 + ur) * ST + 8 * up]) = z8;
+        put_t(&tt[(0 * 32 + ur) * ST + (PERM ? op_perm32_piece(up) : 8 * up)], z8);
+        put_t(&tt[(2 * 32 + ur) * ST + (PERM ? op_perm32_piece(up) : 8 * up)], z8);
       }
     }
     // Loads are unconditional (rows past the end of a partial chunk read its last row and are zeroed when staged):
@@ -723,12 +770,25 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
       const GdrTilesT<OT> tl = tiles(par);
       zero_dead_rows(len, rk_, KU);
       zero_dead_rows(len, rv_, VU);
-      *reinterpret_cast<X8*>(&tl.t[(1 * 32 + (stid >> 2)) * ST + 8 * (stid & 3)]) = rt_[0];
-      *reinterpret_cast<X8*>(&tl.t[ta_off]) = rt_[1];
-      *reinterpret_cast<X8*>(&tl.t[tb_off]) = rt_[2];
+      put_t(&tl.t[t21_off], rt_[0]);
+      put_t(&tl.t[ta_off], rt_[1]);
+      put_t(&tl.t[tb_off], rt_[2]);
       kss = 0.0f;
+      if constexpr (PERM) {
 #pragma unroll
-      for (int u = 0; u < KU; u += 2) {
+        for (int u = 0; u < KU; u += 4) {  // (a thread's half row is one or two groups of 32 columns)
+          X8 p0 = raw_to_op<T, OT>(rk_[u], kss, want_ss), p1 = raw_to_op<T, OT>(rk_[u + 1], kss, want_ss);
+          X8 p2 = raw_to_op<T, OT>(rk_[u + 2], kss, want_ss), p3 = raw_to_op<T, OT>(rk_[u + 3], kss, want_ss);
+          op_perm32<OT>(p0, p1, p2, p3);
+          OT* at = &tl.k[srow * SK + spart * (KT / 2) + 8 * u];
+          *reinterpret_cast<X8*>(at) = p0;
+          *reinterpret_cast<X8*>(at + 8) = p1;
+          *reinterpret_cast<X8*>(at + 16) = p2;
+          *reinterpret_cast<X8*>(at + 24) = p3;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < (PERM ? 0 : KU); u += 2) {
         X8 pa = raw_to_op<T, OT>(rk_[u], kss, want_ss), pb = raw_to_op<T, OT>(rk_[u + 1], kss, want_ss);
         if constexpr (!SCALED) {
           if constexpr (SWZ) op_swizzle16<OT>(pa, pb);
@@ -774,29 +834,57 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
         if (srow == 0) {
           tl.misc[0] = __builtin_amdgcn_exp2f(g_last);
           tl.misc[1] = (PASS_B && pfast) ? 1.0f : 0.0f;
+          tl.misc[2] = ghalf;
         }
       }
       if constexpr (SCALED) {  // the two scaled k tiles, from the raw row that is still in registers
 #pragma unroll
-        for (int u = 0; u < KU; ++u) {
-          const typename Raw8<T>::type piece = rk_[u];  // (dead rows were zeroed by stage_data)
-          X8 pe, pd;
+        for (int u = 0; u < KU; u += 2) {
+          X8 pe[2], pd[2];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float f = (float)piece[e];
-            pe[e] = (OT)(f * ekr);
-            pd[e] = (OT)(f * dkr);
+          for (int h = 0; h < 2; ++h) {
+            const typename Raw8<T>::type piece = rk_[u + h];  // (dead rows were zeroed by stage_data)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float f = (float)piece[e];
+              pe[h][e] = (OT)(f * ekr);
+              pd[h][e] = (OT)(f * dkr);
+            }
           }
-          *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * u]) = pe;
-          *reinterpret_cast<X8*>(&tl.kd[srow * SK + spart * (KT / 2) + 8 * u]) = pd;
+          if constexpr (SWZ) { op_swizzle16<OT>(pe[0], pe[1]); op_swizzle16<OT>(pd[0], pd[1]); }
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<X8*>(&tl.k[srow * SK + spart * (KT / 2) + 8 * (u + h)]) = pe[h];
+            *reinterpret_cast<X8*>(&tl.kd[srow * SK + spart * (KT / 2) + 8 * (u + h)]) = pd[h];
+          }
         }
       }
     };
-    auto stage_q = [&](int len, typename Raw8<T>::type* rq_) {
+    auto stage_q = [&](int len, typename Raw8<T>::type* rq_, int par = 0) {
+      GDR_Q_BUFFERS(par);
+      if constexpr (P16) {  // the factors of this chunk were derived by the other pair of stagers
+        const GdrTilesT<OT> tl = tiles(par);
+        grow = tl.gamma[srow];
+        pfast = tl.misc[1] != 0.0f;
+        ghalf = tl.misc[2];
+      }
       zero_dead_rows(len, rq_, KU);
       float qss = 0.0f;
+      if constexpr (PERM) {
 #pragma unroll
-      for (int u = 0; u < KU; u += 2) {
+        for (int u = 0; u < KU; u += 4) {
+          X8 p0 = raw_to_op<T, OT>(rq_[u], qss, want_ss), p1 = raw_to_op<T, OT>(rq_[u + 1], qss, want_ss);
+          X8 p2 = raw_to_op<T, OT>(rq_[u + 2], qss, want_ss), p3 = raw_to_op<T, OT>(rq_[u + 3], qss, want_ss);
+          op_perm32<OT>(p0, p1, p2, p3);
+          OT* at = &s_q[srow * SK + spart * (KT / 2) + 8 * u];
+          *reinterpret_cast<X8*>(at) = p0;
+          *reinterpret_cast<X8*>(at + 8) = p1;
+          *reinterpret_cast<X8*>(at + 16) = p2;
+          *reinterpret_cast<X8*>(at + 24) = p3;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < (PERM ? 0 : KU); u += 2) {
         X8 pa = raw_to_op<T, OT>(rq_[u], qss, want_ss), pb = raw_to_op<T, OT>(rq_[u + 1], qss, want_ss);
         if constexpr (SWZ) op_swizzle16<OT>(pa, pb);
         *reinterpret_cast<X8*>(&s_q[srow * SK + spart * (KT / 2) + 8 * u]) = pa;
@@ -812,6 +900,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
 
     auto build_p = [&](int par) {
       if constexpr (PASS_B) {
+        GDR_Q_BUFFERS(par);
         const GdrTilesT<OT> tl = tiles(par);
         // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero. Stager 0 takes tile 0, stager 1 tile 2,
         // and they share tile 1: both run its four MFMAs, each finishes and stores one of its two fragments.
@@ -836,6 +925,35 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
           f32x16 acc = zero16();
 #pragma unroll
           for (int ks = 0; ks < KT / 16; ++ks) acc = mfma32(fa[ks], fb[ks], acc);
+          if constexpr (P16) {
+            // Narrow chain waves read P as the B operand of the 16x16x32 shape: lane 16 g + i' of fragment (tt, ts)
+            // holds P[token 16 tt + i'][32 ts + 4 g .. + 3 and 32 ts + 16 + 4 g .. + 3]. Of this tile (columns = tokens
+            // 32 tn + ln, rows j = 32 jm + 8 b + 4 hh + e in register 4 b + e) a lane therefore holds two pieces:
+            // registers {0-3, 8-11} for g = hh and {4-7, 12-15} for g = hh + 2, both of fragment (2 tn + ln / 16, jm).
+            const int tt = 2 * tn + (ln >> 4), f16 = tt < 2 ? tt : 2 + 2 * (tt - 2) + jm;
+#pragma unroll
+            for (int pc = 0; pc < 2; ++pc) {
+              if (half >= 0 && half != pc) continue;
+              X8 piece;
+              if (fast) {  // (one branch per piece, not per element)
+#pragma unroll
+                for (int x = 0; x < 8; ++x) {
+                  const int r = (x < 4 ? 0 : 8) + 4 * pc + (x & 3);
+                  const float t = acc[r] * (fi * rj[r / 4][r % 4]);
+                  piece[x] = (OT)((jm != tn || ln >= acc_row(r, hh)) ? t : 0.0f);
+                }
+              } else {
+#pragma unroll
+                for (int x = 0; x < 8; ++x) {
+                  const int r = (x < 4 ? 0 : 8) + 4 * pc + (x & 3);
+                  const int j = 32 * jm + acc_row(r, hh);
+                  piece[x] = (OT)(acc[r] * (fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f)));
+                }
+              }
+              op_frag_store<OT>(s_P, f16, 16 * (hh + 2 * pc) + (ln & 15), piece);
+            }
+            return;
+          }
           const int f0 = tn == 0 ? 0 : 2 + 2 * jm;  // fragments: tm=0 -> 0,1 ; tm=1 -> 2..5
 #pragma unroll
           for (int part = 0; part < 2; ++part) {
@@ -856,6 +974,62 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
             op_frag_store<OT>(s_P, f0 + part, lane, acc_to_op<OT>(acc, 8 * part));
           }
         };
+        if constexpr (P16 && KT <= 64) {
+          // Narrow form (the P builders are on the critical path there): one batch of operand reads for all tiles of the
+          // wave -- stager 1's two tiles share their q rows --, the tiles' MFMA chains interleaved, the column factors
+          // requested behind the MFMAs. Fragment layout as in p_tile.
+          const int tn = sw;
+          const int i = 32 * tn + ln;
+          X8 fb[KT / 16], fa0[KT / 16], fa1[KT / 16];
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) {
+            fb[ks] = *reinterpret_cast<const X8*>(&s_q[(32 * tn + ln) * SK + 16 * ks + 8 * hh]);
+            fa0[ks] = *reinterpret_cast<const X8*>(&tl.k[ln * SK + 16 * ks + 8 * hh]);
+            if (sw == 1) fa1[ks] = *reinterpret_cast<const X8*>(&tl.k[(32 + ln) * SK + 16 * ks + 8 * hh]);
+          }
+          const float gi = fast ? 0.0f : tl.gamma[i], fi = scale * s_rq[i];
+          lds_fence();
+          f32x16 acc0 = zero16(), acc1 = zero16();
+#pragma unroll
+          for (int ks = 0; ks < KT / 16; ++ks) {
+            acc0 = mfma32(fa0[ks], fb[ks], acc0);
+            if (sw == 1) acc1 = mfma32(fa1[ks], fb[ks], acc1);
+          }
+          asm volatile("" ::: "memory");
+          auto finish = [&](const f32x16& acc, int jm) __attribute__((always_inline)) {
+            f32x4 gj[4], rj[4];
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+              if (!fast) gj[b4] = *reinterpret_cast<const f32x4*>(&tl.gamma[32 * jm + 8 * b4 + 4 * hh]);
+              rj[b4] = *reinterpret_cast<const f32x4*>(&tl.rk[32 * jm + 8 * b4 + 4 * hh]);
+            }
+            const int tt = 2 * tn + (ln >> 4), f16 = tt < 2 ? tt : 2 + 2 * (tt - 2) + jm;
+            f32x16 val;
+            if (fast) {  // (one branch for the tile: inside the element loop it becomes a branch per element)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const float t = acc[r] * (fi * rj[r / 4][r % 4]);
+                val[r] = (jm != tn || ln >= acc_row(r, hh)) ? t : 0.0f;
+              }
+            } else {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int j = 32 * jm + acc_row(r, hh);
+                val[r] = acc[r] * (fi * rj[r / 4][r % 4] * safe_exp2(i >= j ? gi - gj[r / 4][r % 4] : 1.0f));
+              }
+            }
+#pragma unroll
+            for (int pc = 0; pc < 2; ++pc) {
+              X8 piece;
+#pragma unroll
+              for (int x = 0; x < 8; ++x) piece[x] = (OT)val[(x < 4 ? 0 : 8) + 4 * pc + (x & 3)];
+              op_frag_store<OT>(s_P, f16, 16 * (hh + 2 * pc) + (ln & 15), piece);
+            }
+          };
+          finish(acc0, 0);
+          if (sw == 1) finish(acc1, 1);
+          return;
+        }
         // P^T tiles (0,0), (0,1), (1,1) -> P fragments; tile (1,0) is zero.
         if constexpr (OWN_Q) {  // a stager builds the tiles whose q rows it staged itself
           if (sw == 0) p_tile(0, -1);
@@ -870,6 +1044,79 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
     // every iteration issues the same loads: with conditional issues the compiler could not count the loads in
     // flight any more and would drain the queue at every wait. q(c) / q(c+2) share a register set.
     const int cl = c1 - 1;
+    if constexpr (P16) {
+      if (nc > 0) {
+        const int ca = uniform(c0), cb = uniform(min(c0 + 1, cl)), cc = uniform(min(c0 + 2, cl));
+        const int tk0 = chunk_tok0[ca], ln0 = chunk_len[ca], tk1 = chunk_tok0[cb], ln1 = chunk_len[cb];
+        int ln_c = ln0, ln_c1 = ln1, tk_c1 = tk1, tk_c2 = chunk_tok0[cc], ln_c2 = chunk_len[cc];
+        if (spair == 0) {
+          // ---- k, v, T and the factors: tiles and factors (c + 1) are staged and the loads (c + 2) issued before B(c)
+          issue_tiles(c0, tk0, ln0, rk0_);
+          issue_gb(c0);
+          stage_data(ln0, 0, rk0_);
+          stage_factors(c0, 0, rk0_);
+          issue_tiles(min(c0 + 1, cl), tk1, ln1, rk0_);
+          issue_gb(min(c0 + 1, cl));
+          lds_barrier();  // tiles (c0) are ready
+          for (int c = c0; c < c1; ++c) {
+            const int par = (c - c0) & 1;
+            const int cn = uniform(min(c + 3, cl));
+            const int tk_n = chunk_tok0[cn], ln_n = chunk_len[cn];
+            if constexpr (!OWN_Q) lds_barrier();  // Qb(c) (this pair only takes part)
+            if (c + 1 < c1) {
+              stage_data(ln_c1, par ^ 1, rk0_);
+              stage_factors(c + 1, par ^ 1, rk0_);  // (that set's factor rows are free since B(c - 1))
+            }
+            issue_tiles(min(c + 2, cl), tk_c2, ln_c2, rk0_);
+            issue_gb(min(c + 2, cl));
+            lds_barrier();  // B(c)
+            lds_barrier();  // C(c)
+            ln_c = ln_c1; ln_c1 = ln_c2; tk_c2 = tk_n; ln_c2 = ln_n;
+          }
+        } else {
+          // ---- q and P: q(c) staged and P(c) built before B(c) (from the k tile and the factors of chunk c, complete
+          //      since C(c - 1)); the loads of q(c + 1) follow the staging of q(c) into the same registers
+          issue_q(tk0, ln0, rq0_);
+          lds_barrier();  // tiles (c0) are ready
+          if constexpr (DBQ) {
+            // q and P exist twice: q(c + 1) is staged between B(c) and C(c) (its factors are complete at B(c), its buffer
+            // free since C(c - 1)), P(c + 1) is built after C(c) -- so only the P products sit between C(c) and B(c + 1)
+            stage_q(ln_c, rq0_, 0);
+            issue_q(tk_c1, ln_c1, rq0_);
+            lds_fence();
+            build_p(0);
+            for (int c = c0; c < c1; ++c) {
+              const int par = (c - c0) & 1;
+              const int cn = uniform(min(c + 3, cl));
+              const int tk_n = chunk_tok0[cn], ln_n = chunk_len[cn];
+              lds_barrier();  // B(c)
+              if (c + 1 < c1) {
+                stage_q(ln_c1, rq0_, par ^ 1);
+                issue_q(tk_c2, ln_c2, rq0_);
+              }
+              lds_barrier();  // C(c)
+              if (c + 1 < c1) build_p(par ^ 1);
+              ln_c = ln_c1; tk_c1 = tk_c2; ln_c1 = ln_c2; tk_c2 = tk_n; ln_c2 = ln_n;
+            }
+          } else
+          for (int c = c0; c < c1; ++c) {
+            const int par = (c - c0) & 1;
+            const int cn = uniform(min(c + 3, cl));
+            const int tk_n = chunk_tok0[cn], ln_n = chunk_len[cn];
+            stage_q(ln_c, rq0_, par);
+            issue_q(tk_c1, ln_c1, rq0_);
+            if constexpr (OWN_Q) lds_fence();  // this wave's own q rows are in LDS (it builds P from no others)
+            else lds_barrier();                // Qb(c)
+            build_p(par);
+            lds_barrier();  // B(c)
+            lds_barrier();  // C(c)
+            ln_c = ln_c1; tk_c1 = tk_c2; ln_c1 = ln_c2; tk_c2 = tk_n; ln_c2 = ln_n;
+          }
+        }
+        lds_barrier();  // the o tile of the last chunk is complete (the chain waves' last flush)
+      }
+      return;
+    }
     if (nc > 0) {
       typename Raw8<T>::type* const rkA = rk0_;
       typename Raw8<T>::type* const rkB = SCALED ? rk1_ : rk0_;
@@ -916,6 +1163,272 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
     }
     return;
   }
+
+  if constexpr (CW == 16) {
+    // ============================================ narrow chain wave ============================================
+    // Wave w owns the 16 value columns 16 w .. + 15 and all K rows of them: S as K / 16 accumulator tiles of the
+    // 16x16x32 shape (lane 16 g + i: rows 16 km + 4 g + r, column i). Same stages and barriers as the 32-column chain
+    // wave below; every operand fragment from memory is one 16-byte LDS read (tiles in op_perm32 order).
+    constexpr int NKM = KT / 16, NKS = KT / 32, NF = 4 * NKS;  // state tiles, contraction steps over K, k / q fragments
+    const int g4 = lane >> 4, li = lane & 15;
+    const int col = 16 * wave + li;
+    f32x4 S[NKM];
+    // where this lane's part of a state tile sits in the 32-column accumulator order the scan kernels use: tile
+    // (column slab wave / 2, row block km / 2), plane 2 (km % 2) + g / 2, lane 32 (g % 2) + 16 (wave % 2) + i
+    const int lane32 = 32 * (g4 & 1) + 16 * (wave & 1) + li;
+    auto slab_piece = [&](int km) { return ((km >> 1) * 4 + 2 * (km & 1) + (g4 >> 1)) * 64 + lane32; };
+    bool walked = false;
+    if constexpr (KT == 64) if (gmax > 0) {
+      walked = true;
+      // second level of the two-level scan (see the 32-column chain wave): the composites of the groups before this
+      // segment's group, then of the segments before it inside its group
+      constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
+      const int seq = pv.seg_seq[seg], local = seg - pv.seq_seg0[seq];
+      const int lead = local / GDR_SCAN_GROUP, nst = lead + local % GDR_SCAN_GROUP;
+      const int item0 = seg - local % GDR_SCAN_GROUP;
+#pragma unroll
+      for (int km = 0; km < NKM; ++km)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          S[km][r] = h0 ? h0[(((size_t)seq * HV + hv) * KT + 16 * km + 4 * g4 + r) * VT + col] : 0.0f;
+      X8 rm[2][NKM * NKS];
+      f32x4 rn[2][NKM];
+      float rd[2];
+      // M' is stored as A-operand fragments of the 32x32x16 shape: element (row, c) in fragment (row / 32, c / 16), lane
+      // 32 ((c % 16 / 4) & 1) + row % 32, slot 4 (c % 16 / 8) + c % 4. This lane's share of the step ks (columns
+      // 32 ks + 4 g .. and 32 ks + 16 + 4 g ..) of rows 16 km + i: the 8-byte half g / 2 of lane 32 (g % 2) + (16 km + i) % 32
+      // in the fragments (km / 2, 2 ks) and (km / 2, 2 ks + 1).
+      auto issue = [&](int p, X8* m, f32x4* n, float& d) __attribute__((always_inline)) {
+        p = uniform(max(0, min(p, nst - 1)));
+        const bool top = p < lead;
+        const size_t sh = (size_t)(top ? seq * gmax + p : item0 + (p - lead)) * HV + hv;
+        const unsigned char* M = (top ? Mgrp : Mcomp) + sh * M_BYTES;
+        const f32x4* N = reinterpret_cast<const f32x4*>((top ? Ngrp : Ncomp) + (sh * (VT / 32) + (wave >> 1)) * N_BYTES);
+#pragma unroll
+        for (int km = 0; km < NKM; ++km)
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const int l32 = 32 * (g4 & 1) + 16 * (km & 1) + li;
+            const unsigned char* f = M + ((size_t)((km >> 1) * (KT / 16) + 2 * ks) * 64 + l32) * 16 + 8 * (g4 >> 1);
+            const X4 lo = *reinterpret_cast<const X4*>(f), hi = *reinterpret_cast<const X4*>(f + 1024);
+            X8 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+            m[km * NKS + ks] = v;
+          }
+#pragma unroll
+        for (int km = 0; km < NKM; ++km) n[km] = N[slab_piece(km)];
+        d = (top ? Dgrp : Dcomp)[sh];
+      };
+      auto step = [&](const X8* m, const f32x4* n, float d) __attribute__((always_inline)) {
+        X8 Sb[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc2_to_op<OT>(S[2 * ks], S[2 * ks + 1]);
+#pragma unroll
+        for (int km = 0; km < NKM; ++km) {
+          f32x4 acc;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(d, S[km][e], n[km][e]);
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) acc = mfma16(m[km * NKS + ks], Sb[ks], acc);
+          S[km] = acc;
+        }
+      };
+      if (nst > 0) {
+        issue(0, rm[0], rn[0], rd[0]);
+        issue(1, rm[1], rn[1], rd[1]);
+        for (int p = 0; p < nst; p += 2) {
+          step(rm[0], rn[0], rd[0]);
+          issue(p + 2, rm[0], rn[0], rd[0]);
+          if (p + 1 < nst) step(rm[1], rn[1], rd[1]);
+          issue(p + 3, rm[1], rn[1], rd[1]);
+        }
+      }
+    }
+    if (!walked) {  // the scan leaves every segment's initial state as 32-column slabs in accumulator order
+      const f32x4* si = reinterpret_cast<const f32x4*>(Sinit + (((size_t)seg * HV + hv) * (VT / 32) + (wave >> 1)) * (KT * 32));
+#pragma unroll
+      for (int km = 0; km < NKM; ++km) S[km] = si[slab_piece(km)];
+    }
+
+    // this wave's rows of the o tile -> HBM: 64 / NSLAB whole rows of V values, two 16-byte pieces per lane (piece
+    // lane + 64 j of the wave's rows: the same part of a row 64 / PPR rows further down)
+    constexpr int RW = 64 / NSLAB, PPR = VT / 8;
+    const int fo_row = wave * RW + lane / PPR;
+    const T* fo_lds = s_o + fo_row * SV + 8 * (lane % PPR);
+    const unsigned fo_off = (unsigned)(fo_row * (HV * VT) + 8 * (lane % PPR));  // elements, from the chunk's first o row
+    auto flush_o = [&](int tok0, int len) __attribute__((always_inline)) {
+      T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets
+      const uint4 v0 = *reinterpret_cast<const uint4*>(fo_lds);
+      const uint4 v1 = *reinterpret_cast<const uint4*>(fo_lds + (64 / PPR) * SV);
+      // (o is written once and not read again by this pipeline: non-temporal, see the 32-column chain wave)
+      typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+      nt_u32x4 n0, n1;
+      n0[0] = v0.x; n0[1] = v0.y; n0[2] = v0.z; n0[3] = v0.w;
+      n1[0] = v1.x; n1[1] = v1.y; n1[2] = v1.z; n1[3] = v1.w;
+      if (fo_row < len) __builtin_nontemporal_store(n0, reinterpret_cast<nt_u32x4*>(ob + fo_off));
+      if (fo_row + 64 / PPR < len)
+        __builtin_nontemporal_store(n1, reinterpret_cast<nt_u32x4*>(ob + fo_off + (unsigned)((64 / PPR) * (HV * VT))));
+    };
+    // A-operand fragment of a row-major tile: row `row`, the 32-wide contraction step that starts at column c32, in
+    // the slot order of the narrow shape (columns 4 g .. + 3 and 16 + 4 g .. + 3): one 16-byte piece of a tile in
+    // op_perm32 order, two 8-byte pieces otherwise
+    auto row_frag = [&](const OT* arr, int stride, int row, int c32) __attribute__((always_inline)) {
+      if constexpr (PERM) {
+        return *reinterpret_cast<const X8*>(&arr[row * stride + c32 + 8 * g4]);
+      } else {
+        const X4 lo = *reinterpret_cast<const X4*>(&arr[row * stride + c32 + 4 * g4]);
+        const X4 hi = *reinterpret_cast<const X4*>(&arr[row * stride + c32 + 16 + 4 * g4]);
+        X8 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { out[e] = lo[e]; out[4 + e] = hi[e]; }
+        return out;
+      }
+    };
+    // T fragment (tm, ts): rows 16 tm + i of the block T11 (tm < 2) or of T21 / T22 (tm >= 2, ts = 0 / 1)
+    auto t_frag = [&](const OT* tt, int tm, int ts) {
+      const int blk = tm < 2 ? 0 : 1 + ts;
+      return row_frag(tt, ST, blk * 32 + 16 * (tm & 1) + li, 0);
+    };
+
+    int o_tok0 = 0, o_len = 0, p_tok0 = 0, p_len = 0;  // table entries of this chunk and of the one before it
+    if (nc > 0) { o_tok0 = chunk_tok0[uniform(c0)]; o_len = chunk_len[uniform(c0)]; }
+    if (nc > 0) lds_barrier();  // tiles (c0) are ready
+    for (int c = c0; c < c1; ++c) {
+      const GdrTilesT<OT> tl = tiles((c - c0) & 1);
+      GDR_Q_BUFFERS((c - c0) & 1);
+      if constexpr (!OWN_Q) lds_barrier();  // Qb(c) (the chain waves only take part)
+      const int c_nx = uniform(min(c + 1, c1 - 1));
+      const int n_tok0 = chunk_tok0[c_nx], n_len = chunk_len[c_nx];
+      // Registers: four waves share a SIMD at K = V = 64 (128 registers each), so every batch of LDS reads is requested
+      // behind the MFMAs whose operands it replaces (an MFMA has read its operands once it is issued), not a stage ahead;
+      // the MFMAs in flight and the epilogue arithmetic cover the reads. (The empty asm statements keep the compiler from
+      // hoisting the reads back up.)
+      X8 fk[NF];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+      X8 ft[6];   // T (stage 2), P (output)
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+          fk[tm * NKS + ks] = row_frag(tl.k, SK, 16 * tm + li, 32 * ks);
+      X8 Sb[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) Sb[ks] = acc2_to_op<OT>(S[2 * ks], S[2 * ks + 1]);
+      lds_fence();
+      f32x4 R[4];
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) {  // K S
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) acc = mfma16(fk[tm * NKS + ks], Sb[ks], acc);
+        R[tm] = acc;
+      }
+      asm volatile("" ::: "memory");
+      // the per-token factors and the v tile (in accumulator layout) of stage 1's epilogue, then the T fragments
+      f32x4 be[4], ek[4];
+      X4 vv[4];
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) {
+        be[tm] = *reinterpret_cast<const f32x4*>(&tl.beta[16 * tm + 4 * g4]);
+        ek[tm] = *reinterpret_cast<const f32x4*>(&tl.ek[16 * tm + 4 * g4]);
+        vv[tm] = op_lds_read_tr4<OT>(tl.v + (16 * tm + 4 * g4 + (li >> 2)) * SV + 16 * wave + 4 * (li & 3));
+      }
+      ft[0] = t_frag(tl.t, 0, 0); ft[1] = t_frag(tl.t, 1, 0); ft[2] = t_frag(tl.t, 2, 0);
+      ft[3] = t_frag(tl.t, 2, 1); ft[4] = t_frag(tl.t, 3, 0); ft[5] = t_frag(tl.t, 3, 1);
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm)  // R = beta (v - ek (K S))
+#pragma unroll
+        for (int e = 0; e < 4; ++e) R[tm][e] = be[tm][e] * ((float)vv[tm][e] - ek[tm][e] * R[tm][e]);
+      X8 Rb[2];
+      Rb[0] = acc2_to_op<OT>(R[0], R[1]);
+      Rb[1] = acc2_to_op<OT>(R[2], R[3]);
+      f32x4 Vn[4];
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) {  // v_new = T R (T is lower triangular: rows 32 .. 63 need both steps)
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        acc = mfma16(ft[tm < 2 ? tm : 2 * tm - 2], Rb[0], acc);
+        if (tm >= 2) acc = mfma16(ft[2 * tm - 1], Rb[1], acc);
+        Vn[tm] = acc;
+      }
+      asm volatile("" ::: "memory");
+      // K^T fragments (transposing reads of the row-major k tile) and the decay factors of the state update
+#pragma unroll
+      for (int km = 0; km < NKM; ++km)
+#pragma unroll
+        for (int ts = 0; ts < 2; ++ts) fk[km * 2 + ts] = op_ld_tr16<OT, PERM>(tl.k, SK, 16 * km, 32 * ts, lane);
+      f32x4 dk[4];
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) dk[tm] = *reinterpret_cast<const f32x4*>(&tl.dk[16 * tm + 4 * g4]);
+      const float dec = tl.misc[0];
+      X8 Vb[2], Vsb[2];
+#pragma unroll
+      for (int ts = 0; ts < 2; ++ts) {
+        Vb[ts] = acc2_to_op<OT>(Vn[2 * ts], Vn[2 * ts + 1]);
+        f32x4 a = Vn[2 * ts], b = Vn[2 * ts + 1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { a[e] *= dk[2 * ts][e]; b[e] *= dk[2 * ts + 1][e]; }
+        Vsb[ts] = acc2_to_op<OT>(a, b);
+      }
+      lds_fence();
+      lds_barrier();  // B(c): every operand that comes from the k, v and T tiles of chunk c is in registers; the o
+                      // tile of chunk c - 1 is complete
+#pragma unroll
+      for (int km = 0; km < NKM; ++km) {  // S <- dec S + K^T (dk v_new)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[km][e] *= dec;
+#pragma unroll
+        for (int ts = 0; ts < 2; ++ts) S[km] = mfma16(fk[km * 2 + ts], Vsb[ts], S[km]);
+      }
+      asm volatile("" ::: "memory");
+      if (c > c0) flush_o(p_tok0, p_len);  // (behind the MFMAs of the state update, where few registers are live)
+      asm volatile("" ::: "memory");
+      // Q rows, P fragments, output factors
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+          fk[tt * NKS + ks] = row_frag(s_q, SK, 16 * tt + li, 32 * ks);
+#pragma unroll
+      for (int f = 0; f < 6; ++f) ft[f] = op_frag_load<OT>(s_P, f, lane);
+      float qsv[4];
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) qsv[tt] = s_qs[16 * tt + li];  // scale e^{gamma} rq of this lane's token per row tile
+      lds_fence();
+      lds_barrier();  // C(c): the q and P operands of chunk c are in registers, the o tile of chunk c - 1 has been read
+      // o^T = S_old^T (qs Q)^T + v_new^T P^T (computed transposed: the lane holds a token and four value columns, see
+      // the 32-column chain wave): tile tt = tokens 16 tt .. + 15, rows of the result = this wave's 16 value columns
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        f32x4 a1 = {0.0f, 0.0f, 0.0f, 0.0f}, a2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) a1 = mfma16(Sb[ks], fk[tt * NKS + ks], a1);
+        a2 = mfma16(Vb[0], ft[tt < 2 ? tt : 2 * tt - 2], a2);
+        if (tt >= 2) a2 = mfma16(Vb[1], ft[2 * tt - 1], a2);
+        typedef T T4 __attribute__((ext_vector_type(4)));
+        T4 pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk[e] = GdrElem<T>::from_float(__builtin_fmaf(qsv[tt], a1[e], a2[e]));
+        *reinterpret_cast<T4*>(&s_o[(16 * tt + li) * SV + 16 * wave + 4 * g4]) = pk;
+      }
+      p_tok0 = o_tok0; p_len = o_len;
+      o_tok0 = n_tok0; o_len = n_len;
+    }
+    if (nc > 0) {
+      lds_barrier();  // the o tile of the last chunk is complete
+      flush_o(p_tok0, p_len);
+    }
+    int late = 0;  // (keeps the compiler from computing these addresses before the loop)
+    asm volatile("" : "+v"(late));
+    if (ht && (flags & SEG_LAST)) {
+      const int seq = pv.seg_seq[seg];
+      float* out = ht + ((size_t)seq * HV + hv) * KT * VT + late;
+#pragma unroll
+      for (int km = 0; km < NKM; ++km)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) out[(16 * km + 4 * g4 + r) * VT + col] = S[km][r];
+    }
+    return;
+  } else {
 
   // ================================================== chain ==================================================
   // this wave's 32 columns: PASS_B value columns; PASS_A columns of [M | N]
@@ -1003,6 +1516,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
       for (int r = 0; r < 16; ++r) S[km][r] = (is_m && 32 * km + acc_row(r, hh) == 32 * wave + ln) ? 1.0f : 0.0f;
   }
 
+  GDR_Q_BUFFERS(0);
   float dtot = 1.0f;  // product of the chunks' decays over the segment (PASS_A)
   // The LDS operand reads of a stage are issued as one batch one stage ahead of the MFMAs that use them
   // (lds_fence() pins that order); left alone the compiler fetches each fragment right before its MFMA and
@@ -1218,6 +1732,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B>::WAVES), (SC
         reinterpret_cast<f32x4*>(out)[(km * 4 + q4) * 64 + lane] = t;
       }
   }
+  }  // (the 32-column chain wave)
+#undef GDR_Q_BUFFERS
 }
 
 // ---- scan ---------------------------------------------------------------------------------------------------------

@@ -107,6 +107,68 @@ __device__ __forceinline__ typename OpVec<T>::x8 op_ld_kappa_tr(const T* arr, in
   return out;
 }
 
+// ---- 16 x 16 x 32 products ("narrow" chain waves: 16 columns of the state per wave) ------------------------------------
+// D = A (16 x 32) * B (32 x 16) + C on one wave. Lane l = 16 g + i supplies A[row i][k 8 g .. 8 g + 7] and
+// B[k 8 g .. 8 g + 7][col i]; accumulator register r of lane l is element (row 4 g + r, col i).
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// Two accumulator tiles that cover rows 0-15 and 16-31 of a 32-row block, rounded to T: the lane's share of an operand
+// whose 32-wide contraction step visits those rows in the order slot s -> row 16 (s / 4) + 4 g + s % 4 ("slot order
+// of the narrow shape"). Read as the B operand it is the block itself (the lane's column = operand column), read as the
+// A operand its transpose (operand row = the lane's column).
+template <typename T>
+__device__ __forceinline__ typename OpVec<T>::x8 acc2_to_op(const f32x4& lo, const f32x4& hi) {
+  typename OpVec<T>::x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = (T)lo[s]; out[4 + s] = (T)hi[s]; }
+  return out;
+}
+
+// Row-major tiles that feed such products from memory keep every group of 32 columns in the order
+// [0-3 | 16-19 | 4-7 | 20-23 | 8-11 | 24-27 | 12-15 | 28-31]: the lane's share of a 32-wide step in the slot order above
+// (columns 4 g .. + 3 and 16 + 4 g .. + 3) is then ONE aligned 16-byte piece at position 8 g of the group. A writer that
+// holds the four 8-element pieces of a group renames registers:
+template <typename T>
+__device__ __forceinline__ void op_perm32(typename OpVec<T>::x8& p0, typename OpVec<T>::x8& p1, typename OpVec<T>::x8& p2,
+                                          typename OpVec<T>::x8& p3) {
+  typename OpVec<T>::x8 d0, d1, d2, d3;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    d0[s] = p0[s];     d0[4 + s] = p2[s];
+    d1[s] = p0[4 + s]; d1[4 + s] = p2[4 + s];
+    d2[s] = p1[s];     d2[4 + s] = p3[s];
+    d3[s] = p1[4 + s]; d3[4 + s] = p3[4 + s];
+  }
+  p0 = d0; p1 = d1; p2 = d2; p3 = d3;
+}
+// position (in elements) inside such a tile row of the 4-column group that starts at logical column c (c % 4 == 0)
+__device__ __forceinline__ int op_perm32_col(int c) {
+  const int q = (c >> 2) & 7;  // group within its 32
+  return (c & ~31) + 4 * (q < 4 ? 2 * q : 2 * (q - 4) + 1);
+}
+// where the two 8-byte halves of the 8-column piece `part` (0..3) of a 32-column group go: the first at 4 * slot, the
+// second 8 elements further on
+__device__ __forceinline__ int op_perm32_piece(int part) { return 4 * (part < 2 ? 4 * part : 4 * (part - 2) + 1); }
+
+// Fragment of the TRANSPOSE of such a tile for the narrow shape: operand row (A) = tile column col0 + i, contraction
+// over the tile rows row0 .. row0 + 31 in the slot order above. PERM: the tile's columns are stored in the order above.
+template <typename T, bool PERM>
+__device__ __forceinline__ typename OpVec<T>::x8 op_ld_tr16(const T* arr, int stride, int col0, int row0, int lane) {
+  const int L = lane & 15, g = lane >> 4;
+  const int c = col0 + 4 * (L & 3);
+  const T* p = arr + (row0 + 4 * g + (L >> 2)) * stride + (PERM ? op_perm32_col(c) : c);
+  const typename OpVec<T>::x4 lo = op_lds_read_tr4<T>(p), hi = op_lds_read_tr4<T>(p + 16 * stride);
+  typename OpVec<T>::x8 out;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { out[s] = lo[s]; out[4 + s] = hi[s]; }
+  return out;
+}
+
 // sum of squares of a 16-byte piece of the input type, accumulated in fp32
 template <typename T>
 __device__ __forceinline__ float op_sumsq(typename OpVec<T>::x8 v, float ss) {

@@ -85,6 +85,13 @@ def _plan(cu_host, device, n_value_heads: int, head_dims):
     return host, dev
 
 
+def output_pass_config(narrow: int = 1) -> None:
+    """Process-wide form of the chunk forward's output pass (``lampa_gdr_chunk_config``): 0 = 32 value columns per
+    recurrence wave everywhere, 1 = 16 columns ("narrow" waves on the 16x16x32 MFMA) for heads wider than 64 x 64, where
+    it is the faster form (the default), 2 = narrow wherever it is built (K >= 64). For A/B measurements and tests."""
+    check(_capi.lib().lampa_gdr_chunk_config(int(narrow)), "lampa_gdr_chunk_config")
+
+
 # Token-serial operator: sequences at least this long are cut into segments that run in parallel when the launch
 # would otherwise occupy less than a quarter of the chip (None: never).
 SEGMENT_MIN_TOKENS: Optional[int] = 512

@@ -239,6 +239,35 @@ def test_chunk_bf16_matches_oracle(device, T, g_scale):
     _assert_bf16_close(s, want_s, f"state T={T}")
 
 
+@pytest.fixture
+def output_pass_form():
+    """Lets a test force one form of the output pass; the default choice is restored afterwards."""
+    yield gd.output_pass_config
+    gd.output_pass_config(1)
+
+
+@pytest.mark.parametrize("narrow", [0, 2])
+@pytest.mark.parametrize("K,V,dtype", [(64, 64, torch.bfloat16), (128, 128, torch.bfloat16), (64, 128, torch.float16),
+                                       (128, 64, torch.bfloat16)])
+def test_both_forms_of_the_output_pass(device, K, V, dtype, narrow, output_pass_form, monkeypatch):
+    """The output pass with 32 value columns per recurrence wave and with 16 (narrow waves, 16x16x32 MFMA), each forced
+    at every head size it is built for: packed sequences with partial chunks and an empty one, initial states, the norm in
+    the kernel, weak decay, one chunk per segment (so that at K = 64 the walk over the group composites runs inside the
+    pass) -- against the token loop."""
+    output_pass_form(narrow)
+    monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", 1)
+    lens = [64 * 27 - 5, 0, 130, 64]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int64)
+    total = int(cu[-1])
+    q, k, v, g, beta = synth.gdr_inputs(1, total, 2, K, V, dtype, seed=K + V + narrow, g_scale=0.003)
+    h0 = 0.5 * torch.randn(len(lens), 2, K, V, generator=torch.Generator().manual_seed(5))
+    want_o, want_s = og.recurrent_c(q, k, v, g, beta, initial_state=h0, cu_seqlens=cu, l2=og.L2_CHUNK)
+    o, s = gd.chunk_gated_delta_rule(*_to(device, q, k, v, g, beta), initial_state=h0.to(device), output_final_state=True,
+                                     cu_seqlens=cu.to(device), use_qk_l2norm_in_kernel=True)
+    _assert_bf16_close(o, want_o, f"o narrow={narrow}")
+    _assert_bf16_close(s, want_s, f"state narrow={narrow}")
+
+
 @pytest.mark.parametrize("cps", [1, 3, 16])
 def test_chunk_segment_split_is_invisible(device, cps, monkeypatch):
     monkeypatch.setattr(gd, "CHUNKS_PER_SEGMENT", cps)
