@@ -616,6 +616,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
   // tiles in plain order and two 8-byte reads per fragment the output pass is slower: 71.0 against 68.2 us at
   // K = V = 64, 1 463 against 1 290 us at K = V = 128 (config 4).
   constexpr bool PERM = P16;
+  // 32-column output pass: the o tile of a chunk is written to HBM by the STAGER waves (after the next chunk's barrier
+  // B, whole rows), so the read-back and the stores are off the recurrence waves' chain.
+  constexpr bool STAGER_FLUSH = PASS_B && CW == 32 && KT + VT <= 128;  // (the wider heads have no registers for it)
   // Output pass at K <= 64: a stager builds the P tiles of the q rows it staged itself (stager 0 the tile (0,0),
   // stager 1 the tiles (1,0) and (1,1)), so no barrier separates staging q from building P. At K = 128 a P tile is
   // twice the work, the two stagers share the middle tile, and the barrier Qb(c) (q(c) is staged) comes back.
@@ -1124,6 +1127,27 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
       const int ca = uniform(c0), cb = uniform(min(c0 + 1, cl)), cc = uniform(min(c0 + 2, cl));
       const int tk0 = chunk_tok0[ca], ln0 = chunk_len[ca], tk1 = chunk_tok0[cb], ln1 = chunk_len[cb];
       int ln_c = ln0, ln_c1 = ln1, tk_c2 = chunk_tok0[cc], ln_c2 = chunk_len[cc];  // of chunks c, c + 1, c + 2 (clamped)
+      int tk_c = tk0, tk_c1 = tk1, tk_p = 0, ln_p = 0;                              // (tk_p, ln_p: of chunk c - 1)
+      // the o tile (rows of chunk `tok0`) -> HBM, 16-byte pieces, whole rows (non-temporal: o is not read again here)
+      auto stager_flush = [&](int tok0, int len) __attribute__((always_inline)) {
+        constexpr int PPR = VT / 8, NP = 64 * PPR / 128;
+        T* ob = o + ((size_t)tok0 * HV + hv) * VT;
+        uint4 val[NP];
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+          const int x = stid + 128 * j;
+          val[j] = *reinterpret_cast<const uint4*>(&s_o[(x / PPR) * SV + 8 * (x % PPR)]);
+        }
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+          const int x = stid + 128 * j, row = x / PPR, part = x % PPR;
+          typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+          nt_u32x4 nv;
+          nv[0] = val[j].x; nv[1] = val[j].y; nv[2] = val[j].z; nv[3] = val[j].w;
+          if (row < len)
+            __builtin_nontemporal_store(nv, reinterpret_cast<nt_u32x4*>(ob + (unsigned)(row * (HV * VT) + 8 * part)));
+        }
+      };
       issue_tiles(c0, tk0, ln0, rkA);
       issue_gb(c0);
       if constexpr (PASS_B) { issue_q(tk0, ln0, rq0_); issue_q(tk1, ln1, rq1_); }
@@ -1146,6 +1170,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
           else lds_barrier();                // Qb(c)
           build_p(par);
           lds_barrier();  // B(c)
+          if constexpr (STAGER_FLUSH) {
+            if (c > c0) stager_flush(tk_p, ln_p);  // o(c - 1): written after C(c - 1), next written after C(c)
+          }
           if (c + 1 < c1) stage_factors(c + 1, par ^ 1, rk_next);
           issue_gb(min(c + 2, cl));
           lds_barrier();  // C(c)
@@ -1154,11 +1181,16 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
           issue_gb(min(c + 2, cl));
           lds_barrier();  // B(c)
         }
+        tk_p = tk_c; ln_p = ln_c; tk_c = tk_c1; tk_c1 = tk_c2;
         ln_c = ln_c1; ln_c1 = ln_c2; tk_c2 = tk_n; ln_c2 = ln_n;
       };
       for (int c = c0; c < c1; c += 2) {
         one_chunk(c, 0, rq0_, rkB, rkA);
         if (c + 1 < c1) one_chunk(c + 1, 1, rq1_, rkA, rkB);
+      }
+      if constexpr (STAGER_FLUSH) {
+        lds_barrier();  // the o tile of the last chunk is complete
+        stager_flush(tk_p, ln_p);
       }
     }
     return;
@@ -1668,8 +1700,8 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
           *reinterpret_cast<T4*>(&s_o[(32 * tm + ln) * SV + 32 * vslab + 8 * b4 + 4 * hh]) = pk;
         }
       }
-      lds_fence();
-      {
+      if constexpr (!STAGER_FLUSH) {
+        lds_fence();
         const int tok0 = o_tok0, len = o_len;
         T* ob = o + ((size_t)tok0 * HV + hv) * VT;  // uniform base; per-lane 32-bit offsets below
         const int rs = HV * VT;
@@ -1691,6 +1723,9 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
     }
   }
 
+  if constexpr (STAGER_FLUSH) {
+    if (nc > 0) lds_barrier();  // the o tile of the last chunk is complete (the stagers write it out)
+  }
   // epilogue; the opaque zero keeps the compiler from computing all these addresses before the loop
   int late = 0;
   asm volatile("" : "+v"(late));
