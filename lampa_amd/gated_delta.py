@@ -39,6 +39,13 @@ def _sequence_bounds(cu_seqlens, B: int, T: int):
     keep uninitialised outputs and gradients."""
     if cu_seqlens is None:
         return [i * T for i in range(B + 1)]
+    # Reading a device tensor on the host drains the stream, so the validated list is remembered for the tensor OBJECT it
+    # was read from (and the version counter that in-place writes bump), as the reference's `tensor_cache` does for its
+    # `prepare_chunk_indices` (models/hattention/fla_utils.py:88-125, index.py:69-83): a loop that passes the same `cu_seqlens`
+    # tensor every step pays the copy once.
+    for ref, version, key, cached in _bounds_cache:
+        if ref is cu_seqlens and version == cu_seqlens._version and key == (B, T):
+            return cached
     cu = [int(c) for c in cu_seqlens.tolist()]
     if len(cu) < 2:
         raise ValueError(f"cu_seqlens must hold at least two entries (one sequence), got {len(cu)}")
@@ -46,7 +53,12 @@ def _sequence_bounds(cu_seqlens, B: int, T: int):
         raise ValueError(f"cu_seqlens must start at 0, be non-decreasing and end at the number of tokens ({B * T}); "
                          f"got first = {cu[0]}, last = {cu[-1]}"
                          + ("" if all(b >= a for a, b in zip(cu[:-1], cu[1:])) else ", not monotone"))
+    _bounds_cache.insert(0, (cu_seqlens, cu_seqlens._version, (B, T), cu))
+    del _bounds_cache[4:]
     return cu
+
+
+_bounds_cache = []  # (tensor, its version when read, (B, T), validated list), most recent first
 
 
 def _default_chunks_per_segment(chunks_per_seq, n_value_heads: int, slots: int) -> int:

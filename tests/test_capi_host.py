@@ -241,3 +241,15 @@ def test_sequence_boundaries_are_validated_on_the_host():
     import inspect
     for launcher in (gd._chunk_launch, gd._recurrent_launch, gd._backward_launch):
         assert "_sequence_bounds" in inspect.getsource(launcher)
+    # the validated list is remembered per tensor object and version: the same tensor is not read again (reading a device
+    # tensor drains the stream), an in-place change is seen, another token count is checked afresh
+    cu = torch.tensor([0, 4, 10])
+    first = gd._sequence_bounds(cu, 1, 10)
+    assert gd._sequence_bounds(cu, 1, 10) is first
+    with pytest.raises(ValueError, match="cu_seqlens"):
+        gd._sequence_bounds(cu, 1, 12)
+    cu[1] = 11
+    with pytest.raises(ValueError, match="cu_seqlens"):
+        gd._sequence_bounds(cu, 1, 10)
+    cu[1] = 7
+    assert gd._sequence_bounds(cu, 1, 10) == [0, 7, 10]
