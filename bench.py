@@ -222,7 +222,32 @@ def main():
         "kernel_over_twin": round(stage_us.get("gdr_segment_kernel<output>", float("nan")) / probe_us, 3),
         "note": "the output pass's loads and stores with no arithmetic (lampa_gdr_traffic_probe), 100 launches with "
                 "HIP events: the practical floor of that kernel on this memory system"}
-    del rec, o_probe
+    # the same twin with the reads of the walk over the earlier composites that the output pass does before its first chunk
+    # (the second level of the two-level scan runs inside that kernel): the floor of the kernel as it is now
+    n_seg_probe = (n_chunks_probe + cps_probe - 1) // cps_probe
+    comp = torch.zeros((n_seg_probe + (n_seg_probe + 7) // 8) * H * 24576, dtype=torch.uint8, device=dev)
+
+    def probe_walk():
+        _capi.check(_capi.lib().lampa_gdr_traffic_probe_walk(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), rec.data_ptr(),
+                                                             comp.data_ptr(), o_probe.data_ptr(), n_chunks_probe, H,
+                                                             cps_probe, torch.cuda.current_stream().cuda_stream),
+                    "traffic probe (walk)")
+    for _ in range(20):
+        probe_walk()
+    ev0.record()
+    for _ in range(100):
+        probe_walk()
+    ev1.record()
+    torch.cuda.synchronize()
+    walk_us = 1e3 * ev0.elapsed_time(ev1) / 100
+    walk_steps = sum(s_ // 8 + s_ % 8 for s_ in range(n_seg_probe))
+    walk_bytes = probe_bytes + walk_steps * H * 24576
+    roofline["memory_only_twin_with_walk"] = {
+        "us": round(walk_us, 2), "bytes": walk_bytes, "GB/s": round(walk_bytes / (walk_us * 1e-6) / 1e9, 1),
+        "kernel_over_twin": round(stage_us.get("gdr_segment_kernel<output>", float("nan")) / walk_us, 3),
+        "note": "the twin above plus the composites the kernel reads for the scan's second level before its first chunk "
+                "(lampa_gdr_traffic_probe_walk: per step and wave 8 KiB of M' and 8 KiB of N, two steps ahead)"}
+    del rec, o_probe, comp
     # ---- per-step distribution (HIP events on the launch stream, one pair per step) and a cold variant that rotates
     #      among input sets totalling more than 512 MB, so that no step finds its inputs in the memory-side cache ----
     def event_times(fn, n):

@@ -384,6 +384,13 @@ int lampa_profile_end(int max_entries, float* ms, const char** names);
  * overwritten. Its duration is what that access pattern costs on the memory system alone. */
 int lampa_gdr_traffic_probe(const void* q, const void* k, const void* v, const void* records, void* o, int n_chunks,
                             int H, int chunks_per_segment, void* stream);
+/* The same twin with the reads of the walk that the output pass does before its first chunk when the scan runs in two
+ * levels (the composites of the groups of 8 segments before the workgroup's group, then of the segments before it inside
+ * the group: 8 KiB of M' and 8 KiB of N per step and wave). composites: (segments + ceil(segments / 8)) * H * 24576
+ * bytes of any content. */
+int lampa_gdr_traffic_probe_walk(const void* q, const void* k, const void* v, const void* records,
+                                 const void* composites, void* o, int n_chunks, int H, int chunks_per_segment,
+                                 void* stream);
 
 #ifdef __cplusplus
 }

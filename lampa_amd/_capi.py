@@ -69,6 +69,7 @@ _SIGNATURES = {
     "lampa_profile_begin": (_i32, []),
     "lampa_profile_end": (_i32, [_i32, _vp, _vp]),
     "lampa_gdr_traffic_probe": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "lampa_gdr_traffic_probe_walk": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "lampa_gdr_plan_size": (_i64, [_vp, _i32, _i32]),
     "lampa_gdr_plan_fill": (_i32, [_vp, _i32, _i32, _vp]),
     "lampa_gdr_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),

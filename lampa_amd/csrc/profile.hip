@@ -60,10 +60,16 @@ extern "C" int lampa_profile_end(int max_entries, float* ms, const char** names)
 typedef unsigned int prof_u32x4 __attribute__((ext_vector_type(4)));
 #define PROBE_REC_U4 336  // 5376-byte record of a chunk and head, in 16-byte units (the first 288 are read: T)
 
+// WALK: before its first chunk the workgroup also reads what the output pass reads for the second level of the two-level
+// scan -- the composites of the groups of 8 segments before its group, then of the segments before it inside its group:
+// per step and wave the 8 KiB of M' and the wave's 8 KiB slab of N, two steps ahead, as the kernel does.
+#define PROBE_COMP_U4 1536  // composite of a segment (or group) and head: M' 8 KiB, then N 16 KiB, in 16-byte units
+template <bool WALK>
 __global__ void __launch_bounds__(256, 2)
     gdr_traffic_probe_kernel(const prof_u32x4* __restrict__ q, const prof_u32x4* __restrict__ k,
                              const prof_u32x4* __restrict__ v, const prof_u32x4* __restrict__ rec,
-                             prof_u32x4* __restrict__ o, int n_chunks, int H, int cps) {
+                             const prof_u32x4* __restrict__ comp, prof_u32x4* __restrict__ o, int n_chunks, int H,
+                             int cps) {
   const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int c0 = seg * cps, c1 = min(c0 + cps, n_chunks);
   if (tid < 128) {
@@ -88,6 +94,33 @@ __global__ void __launch_bounds__(256, 2)
     if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) o[0] = acc;  // keeps the loads alive; never true in practice
   } else {
     const int t = tid - 128;
+    if constexpr (WALK) {
+      const int segs = gridDim.x, lane = t & 63, slab = t >> 6;
+      const int lead = seg / 8, nst = lead + seg % 8, item0 = seg - seg % 8;
+      prof_u32x4 ring[2][16], acc = {0, 0, 0, 0};
+      auto issue = [&](int p, prof_u32x4* r) __attribute__((always_inline)) {
+        p = max(0, min(p, nst - 1));
+        const int item = p < lead ? segs + p : item0 + (p - lead);  // (the groups' composites follow the segments')
+        const prof_u32x4* base = comp + ((size_t)item * H + h) * PROBE_COMP_U4;
+#pragma unroll
+        for (int f = 0; f < 8; ++f) { r[f] = base[f * 64 + lane]; r[8 + f] = base[512 + slab * 512 + f * 64 + lane]; }
+      };
+      if (nst > 0) {
+        issue(0, ring[0]);
+        issue(1, ring[1]);
+        for (int p = 0; p < nst; p += 2) {
+#pragma unroll
+          for (int f = 0; f < 16; ++f) acc += ring[0][f];
+          issue(p + 2, ring[0]);
+          if (p + 1 < nst) {
+#pragma unroll
+            for (int f = 0; f < 16; ++f) acc += ring[1][f];
+          }
+          issue(p + 3, ring[1]);
+        }
+      }
+      if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) o[1] = acc;  // keeps the loads alive; never true in practice
+    }
     for (int c = c0; c < c1; ++c) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -106,8 +139,23 @@ extern "C" int lampa_gdr_traffic_probe(const void* q, const void* k, const void*
                                        int n_chunks, int H, int chunks_per_segment, void* stream) {
   if (!q || !k || !v || !records || !o || n_chunks < 1 || H < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
   const int segs = (n_chunks + chunks_per_segment - 1) / chunks_per_segment;
-  hipLaunchKernelGGL(gdr_traffic_probe_kernel, dim3(segs, H), dim3(256), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(gdr_traffic_probe_kernel<false>, dim3(segs, H), dim3(256), 0, (hipStream_t)stream,
                      (const prof_u32x4*)q, (const prof_u32x4*)k, (const prof_u32x4*)v, (const prof_u32x4*)records,
-                     (prof_u32x4*)o, n_chunks, H, chunks_per_segment);
+                     (const prof_u32x4*)nullptr, (prof_u32x4*)o, n_chunks, H, chunks_per_segment);
+  return hipGetLastError() == hipSuccess ? LAMPA_OK : LAMPA_ERR_LAUNCH;
+}
+
+// The same with the reads of the walk over the earlier composites that the output pass does before its first chunk when
+// the scan runs in two levels. composites: (segments + ceil(segments / 8)) * H * 24576 bytes of any content (the
+// segments' composites, then the groups').
+extern "C" int lampa_gdr_traffic_probe_walk(const void* q, const void* k, const void* v, const void* records,
+                                            const void* composites, void* o, int n_chunks, int H,
+                                            int chunks_per_segment, void* stream) {
+  if (!q || !k || !v || !records || !composites || !o || n_chunks < 1 || H < 1 || chunks_per_segment < 1)
+    return LAMPA_ERR_INVALID;
+  const int segs = (n_chunks + chunks_per_segment - 1) / chunks_per_segment;
+  hipLaunchKernelGGL(gdr_traffic_probe_kernel<true>, dim3(segs, H), dim3(256), 0, (hipStream_t)stream,
+                     (const prof_u32x4*)q, (const prof_u32x4*)k, (const prof_u32x4*)v, (const prof_u32x4*)records,
+                     (const prof_u32x4*)composites, (prof_u32x4*)o, n_chunks, H, chunks_per_segment);
   return hipGetLastError() == hipSuccess ? LAMPA_OK : LAMPA_ERR_LAUNCH;
 }

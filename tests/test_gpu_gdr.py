@@ -558,3 +558,17 @@ def test_traffic_probe_writes_every_output_row(device):
     assert torch.equal(words, want)
     assert _capi.lib().lampa_gdr_traffic_probe(None, k.data_ptr(), v.data_ptr(), rec.data_ptr(), o.data_ptr(), n_chunks, H,
                                                cps, None) == -1
+    # the form that also reads the composites of the walk (27 one-chunk segments: four groups, walks of up to 3 + 7 steps)
+    n2 = 27
+    q2, k2, v2 = (torch.zeros(64 * n2, H, 64, dtype=torch.bfloat16, device=device) for _ in range(3))
+    rec2 = torch.zeros(n2 * H * 6656, dtype=torch.uint8, device=device)
+    comp = torch.zeros((n2 + 4) * H * 24576, dtype=torch.uint8, device=device)
+    o2 = torch.full((64 * n2, H, 64), -1.0, dtype=torch.bfloat16, device=device)
+    _capi.check(_capi.lib().lampa_gdr_traffic_probe_walk(q2.data_ptr(), k2.data_ptr(), v2.data_ptr(), rec2.data_ptr(),
+                                                         comp.data_ptr(), o2.data_ptr(), n2, H, 1,
+                                                         torch.cuda.current_stream().cuda_stream), "probe walk")
+    torch.cuda.synchronize()
+    words2 = o2.view(torch.int32).reshape(n2, 64, H, 8, 4).cpu()
+    assert torch.equal(words2[..., 0], torch.arange(n2).view(-1, 1, 1, 1).expand(n2, 64, H, 8).int())
+    assert _capi.lib().lampa_gdr_traffic_probe_walk(q2.data_ptr(), k2.data_ptr(), v2.data_ptr(), rec2.data_ptr(), None,
+                                                    o2.data_ptr(), n2, H, 1, None) == -1
