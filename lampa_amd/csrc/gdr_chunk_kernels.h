@@ -503,6 +503,10 @@ __global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ 
 //   C(c)  (PASS_B) the chain waves hold the q and P operands of chunk c, factors (c+1) are complete
 //                                                          -> the stagers may write q(c+1)
 // Global loads are issued about one chunk period before their data is staged.
+// Output pass of the heads up to 64 x 64: the chain waves only write their slab of the o tile; the stagers carry the
+// tile of chunk c - 1 to HBM after B(c) (whole rows), and one more barrier after the last chunk lets them write the last.
+// Narrow form of the output pass (CW = 16, GdrSegShape): chain waves of 16 columns on the 16x16x32 MFMA, two PAIRS of
+// stager waves (k / v / T / factors and q / P), the same barriers; for heads wider than 64 x 64 q and P exist twice.
 // NQ: copies of the q tile, the P fragments and the q factor rows (2: by chunk parity, like the tile sets)
 template <int KT, int VT, bool PASS_B, bool SCALED = !PASS_B, int NQ = 1>
 struct GdrSegSmem {
