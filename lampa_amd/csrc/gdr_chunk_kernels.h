@@ -1562,20 +1562,28 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
   constexpr bool EARLY_Q = PASS_B && KT <= 64;
   int o_tok0 = 0, o_len = 0;  // table entries of the chunk whose o rows are stored, fetched a chunk ahead
   if (PASS_B && nc > 0) { o_tok0 = chunk_tok0[uniform(c0)]; o_len = chunk_len[uniform(c0)]; }
+  // Output pass at K <= 64: the K rows of chunk c + 1 are requested behind the barrier C(c), in front of the output's
+  // MFMAs (the fragment registers are free from the state update on, and the tiles of chunk c + 1 are complete since
+  // B(c)), so the next chunk does not start with an LDS round trip.
+  constexpr bool EARLY_K = EARLY_Q && KT == 64;  // (the 32 x 32 form has no registers for it)
+  X8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
+  auto load_k_rows = [&](const GdrTilesT<OT>& tx) __attribute__((always_inline)) {
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(tx.k, SK, 32 * tm + ln, 16 * ks, hh)
+                                        : op_ld_kappa<OT>(tx.k, SK, 32 * tm + ln, 16 * ks, hh);
+  };
   if (nc > 0) lds_barrier();  // tiles (c0) are ready
+  if constexpr (EARLY_K) load_k_rows(tiles(0));
   for (int c = c0; c < c1; ++c) {
     const GdrTilesT<OT> tl = tiles((c - c0) & 1);
     if constexpr (PASS_B && !OWN_Q) lds_barrier();  // Qb(c) (the chain waves only take part)
     const int c_nx = uniform(min(c + 1, c1 - 1));
     const int n_tok0 = PASS_B ? chunk_tok0[c_nx] : 0, n_len = PASS_B ? chunk_len[c_nx] : 0;
-    X8 fk[2 * (KT / 16)];  // K rows (stage 1), K^T rows (stage 3), Q rows (output)
     X8 fq[EARLY_Q ? 2 * (KT / 16) : 1];
     X8 ft[6];              // T (stage 2), P (output)
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-      for (int ks = 0; ks < KT / 16; ++ks) fk[tm * (KT / 16) + ks] = SWZ ? op_ld_kappa_swz<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh)
-                                        : op_ld_kappa<OT>(tl.k, SK, 32 * tm + ln, 16 * ks, hh);
+    if constexpr (!EARLY_K) load_k_rows(tl);
     X8 Sb[KT / 16];
 #pragma unroll
     for (int ks = 0; ks < KT / 16; ++ks) Sb[ks] = acc_to_op<OT>(S[ks / 2], 8 * (ks % 2));
@@ -1681,6 +1689,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
       }
       lds_fence();
       lds_barrier();  // C(c): the q and P operands of chunk c are in registers
+      if constexpr (EARLY_K) load_k_rows(tiles((c + 1 - c0) & 1));  // (after the last chunk: read and dropped)
       // o^T = S_old^T (qs Q)^T + v_new^T P^T: the state and v_new, which this wave holds in accumulator layout (lane =
       // value column), are read as the A operands (operand row = value column), the Q and P fragments as the B
       // operands (operand column = token). The result tile has the TOKEN in the lane and 16 value columns (four runs
