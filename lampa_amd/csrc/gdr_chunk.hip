@@ -107,7 +107,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
       LAMPA_PROF(s, "gdr_scan2_kernel<leaf>");
     }
   } else {
-    hipLaunchKernelGGL((gdr_scan_kernel<T, KT, VT, 4>), dim3(VT / 32, n_seq, HV), dim3(64 * (KT / 32)), 0, s,
+    hipLaunchKernelGGL((gdr_scan_kernel<T, KT, VT, 4>), dim3(n_seq, HV, VT / 32), dim3(64 * (KT / 32)), 0, s,
                        pv, Mc, Nc, Dc, h0, Si, HV, segs);
     LAMPA_PROF(s, "gdr_scan_kernel");
   }

@@ -1785,7 +1785,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
 }
 
 // ---- scan ---------------------------------------------------------------------------------------------------------
-// grid (VT/32, n_seq, HV), KT/32 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column
+// grid (n_seq, HV, VT/32), KT/32 waves. S_{p+1} = M_p S_p + N_p over the segments of one sequence for a 32-column
 // slab of the state; Sinit receives the state every segment starts from, as 32-column slabs in accumulator order
 // (the layout the output pass loads with 16-byte reads).
 // The composite pass stores M_p as d_p I + M'_p (d_p = the segment's total decay, exact in fp32) with M' in bf16
@@ -1807,7 +1807,10 @@ __global__ void __launch_bounds__(64 * (KT / 32)) gdr_scan_kernel(const GdrPlanV
   constexpr int NKS = KT / 16;
   constexpr int M_BYTES = KT * KT * 2, N_BYTES = KT * 32 * 4;
   __shared__ __align__(16) unsigned char s_x[2][NKS * 1024];
-  const int vn = blockIdx.x, seq = blockIdx.y, hv = blockIdx.z;
+  // grid (n_seq, HV, VT / 32): workgroups go to the 8 XCDs round robin by their linear id, so with the column slab as the
+  // SLOWEST index the slabs of one (sequence, head) -- which all read the same M' -- sit n_seq * HV ids apart, on one XCD
+  // whenever that is a multiple of 8, and its L2 serves M' to all but the first of them
+  const int seq = blockIdx.x, hv = blockIdx.y, vn = blockIdx.z;
   const int seg0 = pv.seq_seg0[seq], nseg = pv.seq_nseg[seq];
   const int nsteps = nseg - 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, hh = lane >> 5, ln = lane & 31;
