@@ -294,20 +294,42 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         for (int w = 0; w < LF_WAVES; ++w) s_bin[w][d] = 0;
       }
       __syncthreads();
+      {
+        // Ranks within the wave. Lanes with the same digit find each other through two tables of the wave in LDS
+        // (s_tot and s_base are free at this point): every lane writes its number to tab[d] and reads back the one
+        // that stayed (the group's speaker), sets its bit in the speaker's 64-bit word, reads the word (= the group)
+        // and clears it; the speaker then adds the group's size to the wave's count of the digit. The LDS executes
+        // the instructions of one wave in order, so the steps need no wait between them, and the relaxed atomic
+        // accesses keep the compiler from forwarding a lane's own store to its load. (Eleven wavefront ballots per
+        // key did the same in three times the instructions: 62.3 -> 58.7 us for one event.) A hit beyond the event's
+        // end carries the largest digit and comes last in (item, lane) order: it changes no rank, only the count of
+        // the largest digit in the segment's last tile, which no other key's position depends on.
+        uint8_t* tab = reinterpret_cast<uint8_t*>(s_tot) + wave * LF_MAX_BINS;
+        unsigned long long* grp = reinterpret_cast<unsigned long long*>(s_base) + wave * 64;
+        grp[lane] = 0ull;
+        const unsigned long long bit = 1ull << lane;
+        uint32_t dd[ITEMS], spk[ITEMS], old[ITEMS];
+        uint64_t peers[ITEMS];
 #pragma unroll
-      for (int k = 0; k < ITEMS; ++k) {
-        const uint32_t d = (key[k] >> shift) & mask;
-        uint64_t peers = __ballot(inside[k]);
-        for (int b = 0; b < nbits; ++b) {
-          const uint64_t bal = __ballot((d >> b) & 1u);
-          peers &= ((d >> b) & 1u) ? bal : ~bal;
+        for (int k = 0; k < ITEMS; ++k) {
+          dd[k] = (key[k] >> shift) & mask;
+          __hip_atomic_store(&tab[dd[k]], (uint8_t)lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+          spk[k] = __hip_atomic_load(&tab[dd[k]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
         }
-        if (!inside[k]) peers = 0;
-        const int leader = peers ? (__ffsll((unsigned long long)peers) - 1) : lane;
-        uint32_t old = 0;
-        if (inside[k] && lane == leader) old = atomicAdd(&s_bin[wave][d], (uint32_t)__popcll(peers));
-        old = __shfl(old, leader);
-        rank[k] = old + (uint32_t)__popcll(peers & lt_mask);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+          __hip_atomic_fetch_or(&grp[spk[k]], bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+          peers[k] = __hip_atomic_load(&grp[spk[k]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+          __hip_atomic_store(&grp[spk[k]], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+          old[k] = 0;
+          if ((uint32_t)lane == spk[k]) old[k] = atomicAdd(&s_bin[wave][dd[k]], (uint32_t)__popcll(peers[k]));
+        }
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+          rank[k] = (uint32_t)__shfl((int)old[k], (int)spk[k]) + (uint32_t)__popcll(peers[k] & lt_mask);
       }
       __syncthreads();
       // the tile's digit counts for the other tiles of the segment

@@ -183,13 +183,22 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __
   uint32_t key[RS_ITEMS], rank[RS_ITEMS];
   int32_t val[RS_ITEMS];
   bool valid[RS_ITEMS];
-  if (dg.first) {  // the caller's keys and payload (or the position)
+  if (dg.first) {  // the caller's keys and payload (or the position): every load is requested before the key mapping
+                   // (whose branches on the key kind would otherwise sit between the loads and wait for each of them)
 #pragma unroll
     for (int i = 0; i < RS_ITEMS; ++i) {
       const int64_t idx = wbase + i * 64 + lane;
       valid[i] = idx < n;
-      key[i] = valid[i] ? rs_ordered(keys_orig[sbase + idx], kind_orig) : 0xFFFFFFFFu;
-      val[i] = valid[i] ? (vals_orig ? vals_orig[sbase + idx] : (int32_t)idx) : 0;
+      key[i] = valid[i] ? keys_orig[sbase + idx] : 0xFFFFFFFFu;
+      val[i] = (int32_t)idx;
+    }
+    if (vals_orig) {
+#pragma unroll
+      for (int i = 0; i < RS_ITEMS; ++i) val[i] = valid[i] ? vals_orig[sbase + wbase + i * 64 + lane] : 0;
+    }
+    if (kind_orig != KEY_U32) {
+#pragma unroll
+      for (int i = 0; i < RS_ITEMS; ++i) key[i] = valid[i] ? rs_ordered(key[i], kind_orig) : 0xFFFFFFFFu;
     }
   } else {  // (ordered key, payload) pairs of the previous pass
 #pragma unroll
