@@ -319,6 +319,12 @@ int lampa_gdr_bwd_chunk(const void* q, const void* k, const void* v, const float
  * 64-token chunks. plan[1] = number of chunks, plan[2] = number of segments. */
 int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment);
 int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment, int32_t* plan_host);
+/* The same tables with total_segments segments over all sequences, dealt out so that the longest segment is as short
+ * as possible (a sequence's segments differ by at most one chunk; every sequence owns at least one segment, and no
+ * segment is cut below one chunk). For batches whose (segment, head) workgroups take several rounds on the chip: with
+ * segments of one fixed length the last round is partly empty. plan[3] (chunks per segment) is 0 in such a plan. */
+int64_t lampa_gdr_plan_size_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments);
+int lampa_gdr_plan_fill_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments, int32_t* plan_host);
 
 /* Chunkwise forward (chunk = 64 tokens). Replaces chunk_gated_delta_rule_fwd and the seven Triton kernels it
  * launches (models/hattention/gated_delta_rule_ori.py:29-80). Shapes as above with H <= HV; K, V in {64, 128} or K = V = 32;

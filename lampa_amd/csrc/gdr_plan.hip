@@ -1,43 +1,69 @@
 // Host-side construction of the plan (see gdr_plan.h). No device code.
 #include "gdr_plan.h"
+#include <vector>
 
-static int64_t plan_counts(const int64_t* cu, int n_seq, int cps, int64_t* n_chunks, int64_t* n_segments) {
+// Segments per sequence. cps > 0: segments of cps chunks (the last one of a sequence may be shorter).
+// cps == 0: `target` segments in all, dealt out so that the longest segment is as short as possible (every sequence
+// starts with one segment and the next segment always goes to the sequence whose segments are longest); a sequence's
+// segments then differ by at most one chunk. An empty sequence still owns one (empty) segment.
+static int plan_segments(const int64_t* cu, int n_seq, int cps, int64_t target, std::vector<int64_t>& ns,
+                         int64_t* n_chunks, int64_t* n_segments) {
+  ns.assign(n_seq, 1);
   int64_t chunks = 0, segs = 0;
+  std::vector<int64_t> nc(n_seq);
   for (int s = 0; s < n_seq; ++s) {
     const int64_t len = cu[s + 1] - cu[s];
     if (len < 0) return -1;
-    const int64_t nc = (len + GDR_C - 1) / GDR_C;
-    chunks += nc;
-    segs += nc == 0 ? 1 : (nc + cps - 1) / cps;  // an empty sequence still owns one (empty) segment
+    nc[s] = (len + GDR_C - 1) / GDR_C;
+    chunks += nc[s];
+    if (cps > 0 && nc[s] > 0) ns[s] = (nc[s] + cps - 1) / cps;
+    segs += ns[s];
+  }
+  if (cps == 0) {
+    for (; segs < target; ++segs) {
+      int best = -1;
+      for (int s = 0; s < n_seq; ++s) {  // longest segments = largest nc / ns, compared without division
+        if (nc[s] <= ns[s]) continue;    // already one chunk per segment
+        if (best < 0 || nc[s] * ns[best] > nc[best] * ns[s]) best = s;
+      }
+      if (best < 0) break;
+      ++ns[best];
+    }
   }
   *n_chunks = chunks;
   *n_segments = segs;
   return 0;
 }
 
-// Number of int32 entries of the plan for these sequences (negative on error).
-extern "C" int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment) {
-  if (!cu_seqlens_host || n_seq < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
+static int64_t plan_size(const int64_t* cu, int n_seq, int cps, int64_t target) {
+  std::vector<int64_t> ns;
   int64_t chunks, segs;
-  if (plan_counts(cu_seqlens_host, n_seq, chunks_per_segment, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
-  if (cu_seqlens_host[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
+  if (plan_segments(cu, n_seq, cps, target, ns, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
+  if (cu[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
   return PLAN_HEADER + 2 * chunks + 4 * segs + 2 * (int64_t)n_seq;
 }
 
-// Fills plan_host (lampa_gdr_plan_size entries). The caller copies it to the device and passes that pointer on.
-extern "C" int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment,
-                                   int32_t* plan_host) {
-  if (!plan_host) return LAMPA_ERR_INVALID;
-  const int64_t size = lampa_gdr_plan_size(cu_seqlens_host, n_seq, chunks_per_segment);
-  if (size < 0) return (int)size;
+// Number of int32 entries of the plan for these sequences (negative on error).
+extern "C" int64_t lampa_gdr_plan_size(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment) {
+  if (!cu_seqlens_host || n_seq < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
+  return plan_size(cu_seqlens_host, n_seq, chunks_per_segment, 0);
+}
+extern "C" int64_t lampa_gdr_plan_size_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments) {
+  if (!cu_seqlens_host || n_seq < 1 || total_segments < 1) return LAMPA_ERR_INVALID;
+  return plan_size(cu_seqlens_host, n_seq, 0, total_segments);
+}
+
+static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t target, int32_t* plan_host) {
+  std::vector<int64_t> seq_ns;
   int64_t chunks, segs;
-  plan_counts(cu_seqlens_host, n_seq, chunks_per_segment, &chunks, &segs);
+  if (plan_segments(cu_seqlens_host, n_seq, cps, target, seq_ns, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
+  if (cu_seqlens_host[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
   int32_t* p = plan_host;
   for (int i = 0; i < PLAN_HEADER; ++i) p[i] = 0;
   p[PLAN_N_SEQ] = n_seq;
   p[PLAN_TOTAL_CHUNKS] = (int32_t)chunks;
   p[PLAN_N_SEGMENTS] = (int32_t)segs;
-  p[PLAN_CHUNKS_PER_SEGMENT] = chunks_per_segment;
+  p[PLAN_CHUNKS_PER_SEGMENT] = cps;  // 0: segments of unequal length
   p[PLAN_TOTAL_TOKENS] = (int32_t)cu_seqlens_host[n_seq];
   int64_t off = PLAN_HEADER;
   p[PLAN_OFF_CHUNK_TOK0] = (int32_t)off; off += chunks;
@@ -52,16 +78,19 @@ extern "C" int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, in
   for (int s = 0; s < n_seq; ++s) {
     const int64_t bos = cu_seqlens_host[s], len = cu_seqlens_host[s + 1] - bos;
     const int64_t nc = (len + GDR_C - 1) / GDR_C;
-    const int64_t ns = nc == 0 ? 1 : (nc + chunks_per_segment - 1) / chunks_per_segment;
+    const int64_t ns = seq_ns[s];
     p[p[PLAN_OFF_SEQ_SEG0] + s] = (int32_t)g;
     p[p[PLAN_OFF_SEQ_NSEG] + s] = (int32_t)ns;
+    // segments of cps chunks, or (cps == 0) the first nc % ns segments one chunk longer than the others
+    const int64_t lo = nc / ns, longer = nc % ns;
+    int64_t c0 = 0;
     for (int64_t i = 0; i < ns; ++i) {
-      const int64_t c0 = i * chunks_per_segment;
-      const int64_t cn = nc - c0 < chunks_per_segment ? nc - c0 : chunks_per_segment;
+      int64_t cn = cps > 0 ? (nc - c0 < cps ? nc - c0 : cps) : lo + (i < longer ? 1 : 0);
       p[p[PLAN_OFF_SEG_CHUNK0] + g] = (int32_t)(c + c0);
       p[p[PLAN_OFF_SEG_NCHUNKS] + g] = (int32_t)(cn < 0 ? 0 : cn);
       p[p[PLAN_OFF_SEG_SEQ] + g] = s;
       p[p[PLAN_OFF_SEG_FLAGS] + g] = (i == 0 ? SEG_FIRST : 0) | (i == ns - 1 ? SEG_LAST : 0);
+      c0 += cn < 0 ? 0 : cn;
       ++g;
     }
     for (int64_t i = 0; i < nc; ++i) {
@@ -73,3 +102,16 @@ extern "C" int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, in
   return LAMPA_OK;
 }
 
+// Fills plan_host (lampa_gdr_plan_size entries). The caller copies it to the device and passes that pointer on.
+extern "C" int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_per_segment,
+                                   int32_t* plan_host) {
+  if (!plan_host || !cu_seqlens_host || n_seq < 1 || chunks_per_segment < 1) return LAMPA_ERR_INVALID;
+  return plan_fill(cu_seqlens_host, n_seq, chunks_per_segment, 0, plan_host);
+}
+// The same tables with total_segments segments of nearly equal length over all sequences (more when there are more
+// sequences than that, fewer when there are fewer chunks): for batches whose workgroups take several rounds on the chip.
+extern "C" int lampa_gdr_plan_fill_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments,
+                                            int32_t* plan_host) {
+  if (!plan_host || !cu_seqlens_host || n_seq < 1 || total_segments < 1) return LAMPA_ERR_INVALID;
+  return plan_fill(cu_seqlens_host, n_seq, 0, total_segments, plan_host);
+}

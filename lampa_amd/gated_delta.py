@@ -67,29 +67,49 @@ def _default_chunks_per_segment(chunks_per_seq, n_value_heads: int, slots: int) 
     (``slots`` = workgroups the chip holds), and the scan in between is serial in the segments per sequence:
     the shortest segments that still fit are best."""
     cps = 4
-    while cps < 64 and sum((n + cps - 1) // cps for n in chunks_per_seq) * n_value_heads > slots:
+    while cps < MAX_CHUNKS_PER_SEGMENT and sum((n + cps - 1) // cps for n in chunks_per_seq) * n_value_heads > slots:
         cps += 1
     return cps
 
 
+MAX_CHUNKS_PER_SEGMENT = 64
+
+
+def _default_segmentation(chunks_per_seq, n_value_heads: int, slots: int):
+    """(chunks per segment, 0) for segments of one length, or (0, total segments) for a balanced plan.
+
+    When even segments of MAX_CHUNKS_PER_SEGMENT chunks give more workgroups than the chip holds, the workgroups run in
+    rounds, and with one fixed length the last round is partly empty while every round lasts a full segment (config 4:
+    1 064 workgroups on 256 slots = 4.2 rounds that take the time of 5). The plan then deals out a whole number of rounds
+    of segments of nearly equal length instead (4 rounds of 63-64 chunks there)."""
+    cps = _default_chunks_per_segment(chunks_per_seq, n_value_heads, slots)
+    if sum(max(1, (n + cps - 1) // cps) for n in chunks_per_seq) * n_value_heads <= slots:
+        return cps, 0
+    work = sum(chunks_per_seq) * n_value_heads
+    rounds = (work + slots * MAX_CHUNKS_PER_SEGMENT - 1) // (slots * MAX_CHUNKS_PER_SEGMENT)
+    return 0, max(1, rounds * slots // n_value_heads)
+
+
 def _plan(cu_host, device, n_value_heads: int, head_dims):
     """Host + device copies of the chunk/segment tables for these sequence boundaries (cached)."""
-    cps = CHUNKS_PER_SEGMENT
+    cps, balanced = CHUNKS_PER_SEGMENT, 0
     if not cps:
         cus = torch.cuda.get_device_properties(device).multi_processor_count
         per_cu = 2 if max(head_dims) <= 64 else 1  # workgroups of the segment kernels a CU holds (LDS, registers)
         chunks_per_seq = [(b - a + 63) // 64 for a, b in zip(cu_host[:-1], cu_host[1:])]
-        cps = _default_chunks_per_segment(chunks_per_seq, n_value_heads, per_cu * cus)
-    key = (tuple(cu_host), cps, str(device))
+        cps, balanced = _default_segmentation(chunks_per_seq, n_value_heads, per_cu * cus)
+    key = (tuple(cu_host), cps, balanced, str(device))
     hit = _plan_cache.get(key)
     if hit is not None:
         return hit
     lib = _capi.lib()
     cu = (ctypes.c_int64 * len(cu_host))(*cu_host)
     n_seq = len(cu_host) - 1
-    size = check(lib.lampa_gdr_plan_size(cu, n_seq, cps), "lampa_gdr_plan_size")
+    size_fn, fill_fn, arg = ((lib.lampa_gdr_plan_size_balanced, lib.lampa_gdr_plan_fill_balanced, balanced) if balanced
+                             else (lib.lampa_gdr_plan_size, lib.lampa_gdr_plan_fill, cps))
+    size = check(size_fn(cu, n_seq, arg), "lampa_gdr_plan_size")
     host = torch.empty(size, dtype=torch.int32)
-    check(lib.lampa_gdr_plan_fill(cu, n_seq, cps, ctypes.c_void_p(host.data_ptr())), "lampa_gdr_plan_fill")
+    check(fill_fn(cu, n_seq, arg, ctypes.c_void_p(host.data_ptr())), "lampa_gdr_plan_fill")
     dev = host.to(device)
     if len(_plan_cache) > 64:
         _plan_cache.clear()

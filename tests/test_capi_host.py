@@ -87,6 +87,61 @@ def test_plan_tables(lib):
     assert p[12] == cu[-1]
 
 
+def test_balanced_plan_tables(lib):
+    """Segments of nearly equal length over all sequences: the greedy deal minimises the longest segment (checked
+    against brute force over the segment counts), a sequence's segments differ by at most one chunk and tile it in
+    order, empty sequences keep their one empty segment, and the default segmentation of a batch that needs several
+    rounds of workgroups asks for a whole number of rounds."""
+    import itertools
+    from lampa_amd import gated_delta as gd
+
+    def plan(cu, total):
+        arr = (ctypes.c_int64 * len(cu))(*cu)
+        size = lib.lampa_gdr_plan_size_balanced(arr, len(cu) - 1, total)
+        assert size > 0
+        p = torch.zeros(size, dtype=torch.int32)
+        assert lib.lampa_gdr_plan_fill_balanced(arr, len(cu) - 1, total, ctypes.c_void_p(p.data_ptr())) == 0
+        return p.tolist()
+
+    cu = [0, 5, 69, 69, 1000, 60199, 60200]
+    lens = [b - a for a, b in zip(cu[:-1], cu[1:])]
+    nc = [(l + 63) // 64 for l in lens]
+    for total in (1, 6, 7, 13, 40, 5000):
+        p = plan(cu, total)
+        n_seq, chunks, segs, cps = p[0:4]
+        assert (n_seq, chunks, cps) == (6, sum(nc), 0)
+        assert segs == min(max(total, n_seq), sum(max(c, 1) for c in nc))
+        seg_c0, seg_nc = p[p[6]:p[6] + segs], p[p[7]:p[7] + segs]
+        seg_seq, seg_flags = p[p[8]:p[8] + segs], p[p[9]:p[9] + segs]
+        seq_seg0, seq_nseg = p[p[10]:p[10] + n_seq], p[p[11]:p[11] + n_seq]
+        c = 0
+        for s in range(n_seq):
+            mine = list(range(seq_seg0[s], seq_seg0[s] + seq_nseg[s]))
+            assert [g for g in range(segs) if seg_seq[g] == s] == mine
+            assert seg_flags[mine[0]] & 1 and seg_flags[mine[-1]] & 2
+            assert all(not (seg_flags[g] & 3) for g in mine[1:-1])
+            sizes = [seg_nc[g] for g in mine]
+            assert sum(sizes) == nc[s] and max(sizes) - min(sizes) <= 1 and sizes == sorted(sizes, reverse=True)
+            for g in mine:  # in order, without gaps
+                assert seg_c0[g] == c
+                c += seg_nc[g]
+        if segs <= 13:  # brute force: no other split of `segs` segments has a shorter longest segment
+            longest = max(seg_nc)
+            live = [i for i in range(n_seq) if nc[i] > 0]
+            best = min(max(-(-nc[i] // k) for i, k in zip(live, ks))
+                       for ks in itertools.product(range(1, segs + 1), repeat=len(live))
+                       if sum(ks) + (n_seq - len(live)) == segs and all(k <= nc[i] for i, k in zip(live, ks)))
+            assert longest == best
+    assert lib.lampa_gdr_plan_size_balanced((ctypes.c_int64 * 2)(0, 10), 1, 0) == -1
+    assert lib.lampa_gdr_plan_size_balanced((ctypes.c_int64 * 3)(0, 10, 5), 2, 4) == -1
+    # default segmentation: one round -> one fixed length; several rounds -> whole rounds of balanced segments
+    assert gd._default_segmentation([938], 8, 512) == (15, 0)
+    nc4 = [819, 830, 564, 635, 735, 659, 314, 205, 404, 189, 231, 755, 500, 434, 203, 655]
+    assert gd._default_segmentation(nc4, 8, 256) == (0, 128)
+    assert gd._default_segmentation([300] * 4, 8, 256) == (38, 0)   # one round of 38-chunk segments holds it
+    assert gd._default_segmentation([600] * 4, 8, 256) == (0, 64)   # 1.2 rounds of 64 chunks -> 2 rounds of 37-38
+
+
 def test_plan_rejects_bad_input(lib):
     bad = (ctypes.c_int64 * 3)(0, 10, 5)
     assert lib.lampa_gdr_plan_size(bad, 2, 4) == -1
