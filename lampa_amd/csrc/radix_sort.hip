@@ -99,13 +99,40 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_histogram_kernel(const uint32_t* 
   for (int d = threadIdx.x; d < bins; d += RS_BLOCK) s_hist[d] = 0;
   __syncthreads();
   const int64_t base = (int64_t)seg * n, first = (int64_t)tile * RS_TILE;
+  // a whole tile of a 16-byte aligned segment is read 16 bytes per lane (the order inside a tile does not matter here)
+  const bool wide = (n & 3) == 0 && first + RS_TILE <= n &&
+                    ((dg.first ? (uintptr_t)keys_orig : (uintptr_t)pairs_buf) & 15) == 0;
+  if (wide && dg.first) {
+    const uint4* src = reinterpret_cast<const uint4*>(keys_orig + base + first);
+    uint4 v[RS_ITEMS / 4];
 #pragma unroll
-  for (int i = 0; i < RS_ITEMS; ++i) {
-    const int64_t idx = first + i * RS_BLOCK + threadIdx.x;
-    if (idx < n) {
-      // the ping-pong buffers hold (ordered key, payload) pairs
-      const uint32_t k = dg.first ? rs_ordered(keys_orig[base + idx], kind_orig) : pairs_buf[base + idx].x;
-      atomicAdd(&s_hist[(k >> dg.shift) & mask], 1u);
+    for (int i = 0; i < RS_ITEMS / 4; ++i) v[i] = src[i * RS_BLOCK + threadIdx.x];
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS / 4; ++i) {
+      atomicAdd(&s_hist[(rs_ordered(v[i].x, kind_orig) >> dg.shift) & mask], 1u);
+      atomicAdd(&s_hist[(rs_ordered(v[i].y, kind_orig) >> dg.shift) & mask], 1u);
+      atomicAdd(&s_hist[(rs_ordered(v[i].z, kind_orig) >> dg.shift) & mask], 1u);
+      atomicAdd(&s_hist[(rs_ordered(v[i].w, kind_orig) >> dg.shift) & mask], 1u);
+    }
+  } else if (wide) {
+    const uint4* src = reinterpret_cast<const uint4*>(pairs_buf + base + first);  // two (key, payload) pairs
+    uint4 v[RS_ITEMS / 2];
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS / 2; ++i) v[i] = src[i * RS_BLOCK + threadIdx.x];
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS / 2; ++i) {
+      atomicAdd(&s_hist[(v[i].x >> dg.shift) & mask], 1u);
+      atomicAdd(&s_hist[(v[i].z >> dg.shift) & mask], 1u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      const int64_t idx = first + i * RS_BLOCK + threadIdx.x;
+      if (idx < n) {
+        // the ping-pong buffers hold (ordered key, payload) pairs
+        const uint32_t k = dg.first ? rs_ordered(keys_orig[base + idx], kind_orig) : pairs_buf[base + idx].x;
+        atomicAdd(&s_hist[(k >> dg.shift) & mask], 1u);
+      }
     }
   }
   __syncthreads();
@@ -127,12 +154,15 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_offsets_kernel(const int32_t* bit
   if (d >= (1 << dg.nbits)) return;
   uint32_t* hcol = hist + (int64_t)seg * n_tiles * RS_MAX_BINS + d;
   uint32_t run = 0;
-  for (int t0 = 0; t0 < n_tiles; t0 += 8) {
-    uint32_t c[8];
+  // 32 tiles at a time, every load requested before the first is used: a segment of 60 000 keys (30 tiles) is one
+  // round trip to memory instead of four
+  constexpr int OB = 32;
+  for (int t0 = 0; t0 < n_tiles; t0 += OB) {
+    uint32_t c[OB];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) c[u] = hcol[(int64_t)min(t0 + u, n_tiles - 1) * RS_MAX_BINS];
+    for (int u = 0; u < OB; ++u) c[u] = hcol[(int64_t)min(t0 + u, n_tiles - 1) * RS_MAX_BINS];
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < OB; ++u)
       if (t0 + u < n_tiles) {
         hcol[(int64_t)(t0 + u) * RS_MAX_BINS] = run;
         run += c[u];
