@@ -7,7 +7,7 @@
 //
 // Each pass = a histogram kernel (LDS histogram per tile of 2048 keys, written to HBM per tile), an offsets kernel
 // (per digit: prefix of the tile counts over the tiles of the segment, and the digit's total) and a scatter kernel
-// (scan of the digit totals, per-wave ranks from wavefront ballots, both added to the tile's offsets).  The number of
+// (scan of the digit totals, per-wave ranks through a match table in LDS, both added to the tile's offsets).  The number of
 // passes is fixed by the host; the digit width of a segment is at most 11 bits. key_bits may live in device memory
 // (written by the key-packing kernel) so that no host synchronisation is needed: then the host launches the worst
 // case and each segment uses only the launches its keys need (see rs_digit).
@@ -173,6 +173,17 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_offsets_kernel(const int32_t* bit
 
 // 1-D grid of rs_grid_blocks(n_tiles, S) blocks. Element order inside a tile: wave w owns [w*512, (w+1)*512), item i
 // of lane l is at w*512 + i*64 + l, so (item, lane) order within a wave is input order and the scatter is stable.
+//
+// A key's output position = (keys of the segment with a smaller digit) + (keys with its digit in earlier tiles)
+// [s_base, 32 bits per digit] + (keys with its digit in earlier waves of the tile) [s_cnt, 16 bits per wave and digit:
+// a wave holds 512 keys, a tile 2048] + its rank among the wave's keys with its digit. Ranks: lanes of a wave with the
+// same digit find each other through two small tables of the wave in LDS -- every lane writes its number to tab[d] and
+// reads back the one that stayed (the group's speaker), sets its bit in the speaker's 64-bit word, reads the word
+// (= the group) and clears it; the speaker adds the group's size to the wave's 16-bit count of the digit and hands the
+// old count to the group. The LDS executes the instructions of one wave in order, so these steps need no waits between
+// them; relaxed atomic accesses keep the compiler from forwarding a lane's own store to its load. A key beyond the
+// segment's end carries the largest digit and comes last in (wave, item, lane) order: it changes no rank and only
+// counts that no real key's position depends on.
 __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __restrict__ keys_orig,
                                                              const int32_t* __restrict__ vals_orig,
                                                              const uint2* __restrict__ pairs_in, int64_t n,
@@ -182,9 +193,10 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __
                                                              const uint32_t* __restrict__ tot,
                                                              uint2* __restrict__ pairs_out,
                                                              int32_t* __restrict__ vals_out) {
-  // Row 0 starts at the number of keys of the segment with a smaller digit, the other rows at zero; after the
-  // ranking the rows become the output bases of the waves.
-  __shared__ uint32_t s_bin[RS_WAVES][RS_MAX_BINS];
+  __shared__ uint32_t s_base[RS_MAX_BINS];
+  __shared__ uint32_t s_cnt[RS_WAVES][RS_MAX_BINS / 2];  // two 16-bit counts per word: digits 2j (low half) and 2j + 1
+  __shared__ uint8_t s_tab[RS_WAVES][RS_MAX_BINS];
+  __shared__ unsigned long long s_grp[RS_WAVES][64];
   __shared__ uint32_t s_wsum[RS_WAVES];
   int seg, tile;
   if (!rs_block_to_tile(n_tiles, n_segments, seg, tile)) return;
@@ -240,16 +252,18 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __
       val[i] = (int32_t)kv.y;
     }
   }
-  // this tile's offsets within each digit (written by rs_offsets_kernel); used after the ranking
+  // this tile's offsets within each digit (written by rs_offsets_kernel), for the digit pairs of the words this thread
+  // turns into bases after the ranking: words t, t + 256, ...
+  constexpr int WPT = RS_MAX_BINS / 2 / RS_BLOCK;
   const uint32_t* hrow = hist + ((int64_t)seg * n_tiles + tile) * RS_MAX_BINS;
-  uint32_t hoff[DPT];
+  uint2 hoff[WPT];
 #pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = threadIdx.x + j * RS_BLOCK;
-    hoff[j] = d < bins ? hrow[d] : 0u;
+  for (int j = 0; j < WPT; ++j) {
+    const int w2 = threadIdx.x + j * RS_BLOCK;
+    hoff[j] = 2 * w2 < bins ? *reinterpret_cast<const uint2*>(hrow + 2 * w2) : make_uint2(0u, 0u);
   }
 
-  // exclusive scan of the digit totals over the block -> row 0 of s_bin; rows 1.. start at zero
+  // exclusive scan of the digit totals over the block -> s_base; the waves' counts start at zero
   {
     uint32_t mine = 0;
 #pragma unroll
@@ -261,63 +275,82 @@ __global__ void __launch_bounds__(RS_BLOCK) rs_scatter_kernel(const uint32_t* __
       if (lane >= off) incl += up;
     }
     if (lane == 63) s_wsum[wave] = incl;
-    for (int d = threadIdx.x; d < bins; d += RS_BLOCK) {
+    for (int w2 = threadIdx.x; 2 * w2 < bins; w2 += RS_BLOCK) {
 #pragma unroll
-      for (int w = 1; w < RS_WAVES; ++w) s_bin[w][d] = 0;
+      for (int w = 0; w < RS_WAVES; ++w) s_cnt[w][w2] = 0;
     }
+    s_grp[wave][lane] = 0ull;
     __syncthreads();
     uint32_t run = incl - mine;
 #pragma unroll
     for (int w = 0; w < RS_WAVES; ++w) run += w < wave ? s_wsum[w] : 0u;
 #pragma unroll
     for (int j = 0; j < DPT; ++j) {
-      if ((int)threadIdx.x * DPT + j < bins) s_bin[0][threadIdx.x * DPT + j] = run;
+      if ((int)threadIdx.x * DPT + j < bins) s_base[threadIdx.x * DPT + j] = run;
       run += dt[j];
     }
   }
-  __syncthreads();
 
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  uint32_t dd[RS_ITEMS];
+  {
+    uint8_t* tab = s_tab[wave];
+    unsigned long long* grp = s_grp[wave];
+    uint32_t* cnt = s_cnt[wave];
+    const unsigned long long bit = 1ull << lane;
+    uint32_t spk[RS_ITEMS], old[RS_ITEMS];
+    uint64_t peers[RS_ITEMS];
 #pragma unroll
-  for (int i = 0; i < RS_ITEMS; ++i) {
-    const uint32_t d = (key[i] >> dg.shift) & mask;
-    uint64_t peers = __ballot(valid[i]);
-    for (int b = 0; b < dg.nbits; ++b) {
-      const uint64_t bal = __ballot((d >> b) & 1u);
-      peers &= ((d >> b) & 1u) ? bal : ~bal;
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      dd[i] = (key[i] >> dg.shift) & mask;
+      __hip_atomic_store(&tab[dd[i]], (uint8_t)lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      spk[i] = __hip_atomic_load(&tab[dd[i]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
     }
-    if (!valid[i]) peers = 0;
-    const int leader = peers ? (__ffsll((unsigned long long)peers) - 1) : lane;
-    uint32_t old = 0;
-    if (valid[i] && lane == leader) old = atomicAdd(&s_bin[wave][d], (uint32_t)__popcll(peers));
-    old = __shfl(old, leader);
-    rank[i] = old + (uint32_t)__popcll(peers & lt_mask);
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      __hip_atomic_fetch_or(&grp[spk[i]], bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      peers[i] = __hip_atomic_load(&grp[spk[i]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      __hip_atomic_store(&grp[spk[i]], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    }
+    // in item order: the value a speaker gets back is the number of the wave's earlier keys with this digit
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i) {
+      const int sh = 16 * (dd[i] & 1u);
+      old[i] = 0;
+      if ((uint32_t)lane == spk[i])
+        old[i] = (atomicAdd(&cnt[dd[i] >> 1], (uint32_t)__popcll(peers[i]) << sh) >> sh) & 0xFFFFu;
+    }
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i)
+      rank[i] = (uint32_t)__shfl((int)old[i], (int)spk[i]) + (uint32_t)__popcll(peers[i] & lt_mask);
   }
   __syncthreads();
 
-  // output base of every wave of the tile for every digit: tile offset, then the waves in order. Row 0 holds
-  // (smaller digits + keys of wave 0), which carries the digit base into the running sum.
+  // the waves' counts become the keys of the tile's earlier waves with the digit (both halves of a word at once: no
+  // sum exceeds the 2048 keys of a tile); the tile's offset joins the digit's base
 #pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = threadIdx.x + j * RS_BLOCK;
-    if (d < bins) {
-      uint32_t run = hoff[j];
+  for (int j = 0; j < WPT; ++j) {
+    const int w2 = threadIdx.x + j * RS_BLOCK;
+    if (2 * w2 < bins) {
+      uint32_t run = 0;
 #pragma unroll
       for (int w = 0; w < RS_WAVES; ++w) {
-        const uint32_t c = s_bin[w][d];
-        s_bin[w][d] = run;
+        const uint32_t c = s_cnt[w][w2];
+        s_cnt[w][w2] = run;
         run += c;
       }
+      s_base[2 * w2] += hoff[j].x;
+      if (2 * w2 + 1 < bins) s_base[2 * w2 + 1] += hoff[j].y;
     }
   }
   __syncthreads();
 
   // one scattered store per key: an 8-byte (key, payload) pair between passes, the payload alone after the last
+  const uint16_t* wpre = reinterpret_cast<const uint16_t*>(s_cnt[wave]);
 #pragma unroll
   for (int i = 0; i < RS_ITEMS; ++i) {
     if (valid[i]) {
-      const uint32_t d = (key[i] >> dg.shift) & mask;
-      const int64_t pos = sbase + s_bin[wave][d] + rank[i];
+      const int64_t pos = sbase + s_base[dd[i]] + wpre[dd[i]] + rank[i];
       if (pairs_out) pairs_out[pos] = make_uint2(key[i], (uint32_t)val[i]);
       else vals_out[pos] = val[i];
     }
