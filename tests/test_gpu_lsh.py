@@ -118,6 +118,27 @@ def test_stable_argsort_per_segment_device_bits(device):
         assert torch.equal(got.cpu().long(), want), passes
 
 
+def test_stable_argsort_device_bits_many_segments(device):
+    """Many segments (40 x 15 tiles, spread over the XCDs by segment) with ties: segments that skip the launches only
+    wide keys need and segments that need them (23 .. 32 bits) in one call, three and four launches."""
+    gen = torch.Generator().manual_seed(11)
+    n, bits = 30000, [9, 19, 22, 23, 27, 30, 31, 32] * 5
+    rows = []
+    for b in bits:
+        r = torch.randint(0, 1 << min(b, 31), (n,), generator=gen, dtype=torch.int64)
+        if b == 32:
+            r = r * 2 + torch.randint(0, 2, (n,), generator=gen, dtype=torch.int64)
+        r[::7] = r[0]  # ties, so that stability is tested
+        rows.append(r)
+    keys64 = torch.stack(rows)
+    keys = (keys64 - ((keys64 >> 31) << 32)).to(torch.int32)
+    want = torch.sort(keys64, dim=-1, stable=True).indices
+    bits_dev = torch.tensor(bits, dtype=torch.int32, device=device)
+    for passes in (0, 4):
+        got = lsh.stable_argsort(keys.to(device), key_bits_dev=bits_dev, n_passes=passes, unsigned=True)
+        assert torch.equal(got.cpu().long(), want), passes
+
+
 def test_gather_scatter_invert_roundtrip(device):
     gen = torch.Generator().manual_seed(1)
     for d, dtype in ((24, torch.float32), (5, torch.float32), (3, torch.int16), (64, torch.bfloat16)):
