@@ -37,7 +37,7 @@
 // Device pointers to the tables of the plan (resolved on the host, so that a kernel reaches an entry with one
 // load instead of a dependent pair).
 struct GdrPlanView {
-  const int32_t *chunk_tok0, *chunk_len, *seg_chunk0, *seg_nchunks, *seg_seq, *seg_flags, *seq_seg0, *seq_nseg;
+  const int32_t *chunk_tok0, *chunk_len, *seg_chunk0, *seg_nchunks, *seg_seq, *seg_flags, *seq_seg0, *seq_nseg, *seg_order;
 };
 static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_dev) {
   GdrPlanView pv;
@@ -49,6 +49,7 @@ static GdrPlanView gdr_plan_view(const int32_t* plan_host, const int32_t* plan_d
   pv.seg_flags = plan_dev + plan_host[PLAN_OFF_SEG_FLAGS];
   pv.seq_seg0 = plan_dev + plan_host[PLAN_OFF_SEQ_SEG0];
   pv.seq_nseg = plan_dev + plan_host[PLAN_OFF_SEQ_NSEG];
+  pv.seg_order = plan_dev + plan_host[PLAN_OFF_SEG_ORDER];
   return pv;
 }
 
@@ -661,7 +662,7 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
   float* const s_rq = s_qs + 64;                                                    \
   (void)s_q; (void)s_P; (void)s_qs; (void)s_rq
 
-  const int seg = blockIdx.x, hv = blockIdx.y;
+  const int seg = pv.seg_order[blockIdx.x], hv = blockIdx.y;  // long segments first (see the plan)
   const int h = hv / (HV / H);
   const int flags = pv.seg_flags[seg];
   if (!PASS_B && (flags & SEG_LAST)) return;  // nothing follows the last segment of a sequence

@@ -23,6 +23,7 @@ enum {
   PLAN_OFF_SEQ_SEG0 = 10,
   PLAN_OFF_SEQ_NSEG = 11,
   PLAN_TOTAL_TOKENS = 12,
+  PLAN_OFF_SEG_ORDER = 13,  // the segments from the longest to the shortest: the order the segment kernels take them in
   PLAN_HEADER = 16
 };
 #define SEG_FIRST 1

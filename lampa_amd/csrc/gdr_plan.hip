@@ -1,5 +1,6 @@
 // Host-side construction of the plan (see gdr_plan.h). No device code.
 #include "gdr_plan.h"
+#include <algorithm>
 #include <vector>
 
 // Segments per sequence. cps > 0: segments of cps chunks (the last one of a sequence may be shorter).
@@ -40,7 +41,7 @@ static int64_t plan_size(const int64_t* cu, int n_seq, int cps, int64_t target) 
   int64_t chunks, segs;
   if (plan_segments(cu, n_seq, cps, target, ns, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
   if (cu[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
-  return PLAN_HEADER + 2 * chunks + 4 * segs + 2 * (int64_t)n_seq;
+  return PLAN_HEADER + 2 * chunks + 5 * segs + 2 * (int64_t)n_seq;
 }
 
 // Number of int32 entries of the plan for these sequences (negative on error).
@@ -74,6 +75,7 @@ static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t
   p[PLAN_OFF_SEG_FLAGS] = (int32_t)off; off += segs;
   p[PLAN_OFF_SEQ_SEG0] = (int32_t)off; off += n_seq;
   p[PLAN_OFF_SEQ_NSEG] = (int32_t)off; off += n_seq;
+  p[PLAN_OFF_SEG_ORDER] = (int32_t)off; off += segs;
   int64_t c = 0, g = 0;
   for (int s = 0; s < n_seq; ++s) {
     const int64_t bos = cu_seqlens_host[s], len = cu_seqlens_host[s + 1] - bos;
@@ -99,6 +101,13 @@ static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t
       ++c;
     }
   }
+  // Workgroups start in the order of their index, and a batch may need several rounds of them: with the long segments
+  // first and the short ones last, the workgroups of the last round end together (the first free slots, those of the
+  // shortest segments, take the longest of the next head).
+  int32_t* order = p + p[PLAN_OFF_SEG_ORDER];
+  const int32_t* len = p + p[PLAN_OFF_SEG_NCHUNKS];
+  for (int64_t i = 0; i < segs; ++i) order[i] = (int32_t)i;
+  std::stable_sort(order, order + segs, [len](int32_t a, int32_t b) { return len[a] > len[b]; });
   return LAMPA_OK;
 }
 

@@ -85,6 +85,10 @@ def test_plan_tables(lib):
         assert seg_flags[mine[0]] & 1 and seg_flags[mine[-1]] & 2
         assert all(seg_nc[g] <= 16 for g in mine) and sum(seg_nc[g] for g in mine) == want_chunks[s]
     assert p[12] == cu[-1]
+    # the order the segment kernels take the segments in: every segment once, the longest first, ties in plan order
+    order = p[p[13]:p[13] + segs]
+    assert sorted(order) == list(range(segs))
+    assert order == sorted(range(segs), key=lambda g: -seg_nc[g])
 
 
 def test_balanced_plan_tables(lib):
@@ -125,6 +129,8 @@ def test_balanced_plan_tables(lib):
             for g in mine:  # in order, without gaps
                 assert seg_c0[g] == c
                 c += seg_nc[g]
+        order = p[p[13]:p[13] + segs]
+        assert order == sorted(range(segs), key=lambda g: -seg_nc[g])
         if segs <= 13:  # brute force: no other split of `segs` segments has a shorter longest segment
             longest = max(seg_nc)
             live = [i for i in range(n_seq) if nc[i] > 0]
