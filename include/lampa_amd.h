@@ -325,6 +325,11 @@ int lampa_gdr_plan_fill(const int64_t* cu_seqlens_host, int n_seq, int chunks_pe
  * segments of one fixed length the last round is partly empty. plan[3] (chunks per segment) is 0 in such a plan. */
 int64_t lampa_gdr_plan_size_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments);
 int lampa_gdr_plan_fill_balanced(const int64_t* cu_seqlens_host, int n_seq, int total_segments, int32_t* plan_host);
+/* The same tables with the caller's own segment lengths: seg_chunks[n_segments] in 64-token chunks, the segments of
+ * sequence 0 first; every sequence's lengths must add up to its chunks (an empty sequence takes one segment of 0). */
+int64_t lampa_gdr_plan_size_lengths(const int64_t* cu_seqlens_host, int n_seq, const int32_t* seg_chunks, int n_segments);
+int lampa_gdr_plan_fill_lengths(const int64_t* cu_seqlens_host, int n_seq, const int32_t* seg_chunks, int n_segments,
+                                int32_t* plan_host);
 
 /* Chunkwise forward (chunk = 64 tokens). Replaces chunk_gated_delta_rule_fwd and the seven Triton kernels it
  * launches (models/hattention/gated_delta_rule_ori.py:29-80). Shapes as above with H <= HV; K, V in {64, 128} or K = V = 32;

@@ -74,6 +74,8 @@ _SIGNATURES = {
     "lampa_gdr_plan_fill": (_i32, [_vp, _i32, _i32, _vp]),
     "lampa_gdr_plan_size_balanced": (_i64, [_vp, _i32, _i32]),
     "lampa_gdr_plan_fill_balanced": (_i32, [_vp, _i32, _i32, _vp]),
+    "lampa_gdr_plan_size_lengths": (_i64, [_vp, _i32, _vp, _i32]),
+    "lampa_gdr_plan_fill_lengths": (_i32, [_vp, _i32, _vp, _i32, _vp]),
     "lampa_gdr_chunk_workspace_bytes": (_i64, [_i64, _i64, _i32, _i32, _i32]),
     "lampa_gdr_chunk_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                    _f32, _i32, _vp, _i64, _vp]),

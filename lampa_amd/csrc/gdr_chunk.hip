@@ -80,7 +80,7 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
                        pv.chunk_tok0, pv.chunk_len, tf, chunks, H, HV, l2norm);
     LAMPA_PROF(s, "gdr_local_kernel");
     if (segs > n_seq) {
-      hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
+      hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, false>), dim3(segs * HV), dim3(64 * GdrSegShape<KT, VT, false>::WAVES), smem_a, s,
                          (const T*)q, (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, (const float*)nullptr, Mc, Nc, Dc,
                          (T*)nullptr, (float*)nullptr, H, HV, scale, l2norm, (const unsigned char*)nullptr,
                          (const unsigned char*)nullptr, (const float*)nullptr, (const float*)nullptr, 0);
@@ -113,12 +113,12 @@ static int gdr_chunk_launch(const void* q, const void* k, const void* v, const f
   }
   const int narrow = gdr_narrow_output.load();
   if (CWN == 16 && (narrow == 2 || (narrow == 1 && KT + VT > 128)))
-    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true, false, T, CWN>), dim3(segs, HV),
+    hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true, false, T, CWN>), dim3(segs * HV),
                        dim3(64 * GdrSegShape<KT, VT, true, CWN>::WAVES), smem_n, s, (const T*)q, (const T*)k, (const T*)v, g, beta,
                        pv, pv.chunk_tok0, pv.chunk_len, tf, Si, Mc, Nc, Dc, (T*)o, ht, H, HV, scale, l2norm,
                        (const unsigned char*)Gm, (const unsigned char*)Gn, (const float*)Gd, h0, walk_in_output ? gmax : 0);
   else
-  hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs, HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
+  hipLaunchKernelGGL((gdr_segment_kernel<T, KT, VT, true>), dim3(segs * HV), dim3(64 * GdrSegShape<KT, VT, true>::WAVES), smem_b, s, (const T*)q,
                      (const T*)k, (const T*)v, g, beta, pv, pv.chunk_tok0, pv.chunk_len, tf, Si, Mc, Nc, Dc, (T*)o, ht, H, HV, scale,
                      l2norm, (const unsigned char*)Gm, (const unsigned char*)Gn, (const float*)Gd, h0, walk_in_output ? gmax : 0);
   LAMPA_PROF(s, "gdr_segment_kernel<output>");

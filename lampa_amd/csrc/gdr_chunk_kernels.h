@@ -662,7 +662,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
   float* const s_rq = s_qs + 64;                                                    \
   (void)s_q; (void)s_P; (void)s_qs; (void)s_rq
 
-  const int seg = pv.seg_order[blockIdx.x], hv = blockIdx.y;  // long segments first (see the plan)
+  // long segments first (see the plan). Grid (segments, heads), or one row of segments x heads workgroups in which the
+  // heads of a segment are neighbours, so that the order holds over all heads
+  const int seg = pv.seg_order[gridDim.y > 1 ? blockIdx.x : blockIdx.x / HV];
+  const int hv = gridDim.y > 1 ? blockIdx.y : blockIdx.x % HV;
   const int h = hv / (HV / H);
   const int flags = pv.seg_flags[seg];
   if (!PASS_B && (flags & SEG_LAST)) return;  // nothing follows the last segment of a sequence

@@ -7,9 +7,32 @@
 // cps == 0: `target` segments in all, dealt out so that the longest segment is as short as possible (every sequence
 // starts with one segment and the next segment always goes to the sequence whose segments are longest); a sequence's
 // segments then differ by at most one chunk. An empty sequence still owns one (empty) segment.
+// cps < 0: the caller's own segment lengths (`lens`, `target` of them: sequence after sequence, every sequence's
+// lengths adding up to its chunks; an empty sequence takes one length of 0).
 static int plan_segments(const int64_t* cu, int n_seq, int cps, int64_t target, std::vector<int64_t>& ns,
-                         int64_t* n_chunks, int64_t* n_segments) {
+                         int64_t* n_chunks, int64_t* n_segments, const int32_t* lens = nullptr) {
   ns.assign(n_seq, 1);
+  if (cps < 0) {
+    int64_t chunks = 0, at = 0;
+    for (int s = 0; s < n_seq; ++s) {
+      const int64_t len = cu[s + 1] - cu[s];
+      if (len < 0) return -1;
+      const int64_t nc = (len + GDR_C - 1) / GDR_C;
+      int64_t sum = 0, cnt = 0;
+      do {
+        if (at >= target || lens[at] < 0 || (nc > 0 && lens[at] == 0)) return -1;
+        sum += lens[at++];
+        ++cnt;
+      } while (sum < nc);
+      if (sum != nc) return -1;
+      ns[s] = cnt;
+      chunks += nc;
+    }
+    if (at != target) return -1;
+    *n_chunks = chunks;
+    *n_segments = target;
+    return 0;
+  }
   int64_t chunks = 0, segs = 0;
   std::vector<int64_t> nc(n_seq);
   for (int s = 0; s < n_seq; ++s) {
@@ -54,17 +77,18 @@ extern "C" int64_t lampa_gdr_plan_size_balanced(const int64_t* cu_seqlens_host, 
   return plan_size(cu_seqlens_host, n_seq, 0, total_segments);
 }
 
-static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t target, int32_t* plan_host) {
+static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t target, int32_t* plan_host,
+                     const int32_t* lens = nullptr) {
   std::vector<int64_t> seq_ns;
   int64_t chunks, segs;
-  if (plan_segments(cu_seqlens_host, n_seq, cps, target, seq_ns, &chunks, &segs) != 0) return LAMPA_ERR_INVALID;
+  if (plan_segments(cu_seqlens_host, n_seq, cps, target, seq_ns, &chunks, &segs, lens) != 0) return LAMPA_ERR_INVALID;
   if (cu_seqlens_host[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
   int32_t* p = plan_host;
   for (int i = 0; i < PLAN_HEADER; ++i) p[i] = 0;
   p[PLAN_N_SEQ] = n_seq;
   p[PLAN_TOTAL_CHUNKS] = (int32_t)chunks;
   p[PLAN_N_SEGMENTS] = (int32_t)segs;
-  p[PLAN_CHUNKS_PER_SEGMENT] = cps;  // 0: segments of unequal length
+  p[PLAN_CHUNKS_PER_SEGMENT] = cps > 0 ? cps : 0;  // 0: segments of unequal length
   p[PLAN_TOTAL_TOKENS] = (int32_t)cu_seqlens_host[n_seq];
   int64_t off = PLAN_HEADER;
   p[PLAN_OFF_CHUNK_TOK0] = (int32_t)off; off += chunks;
@@ -87,7 +111,7 @@ static int plan_fill(const int64_t* cu_seqlens_host, int n_seq, int cps, int64_t
     const int64_t lo = nc / ns, longer = nc % ns;
     int64_t c0 = 0;
     for (int64_t i = 0; i < ns; ++i) {
-      int64_t cn = cps > 0 ? (nc - c0 < cps ? nc - c0 : cps) : lo + (i < longer ? 1 : 0);
+      int64_t cn = cps > 0 ? (nc - c0 < cps ? nc - c0 : cps) : cps < 0 ? lens[g] : lo + (i < longer ? 1 : 0);
       p[p[PLAN_OFF_SEG_CHUNK0] + g] = (int32_t)(c + c0);
       p[p[PLAN_OFF_SEG_NCHUNKS] + g] = (int32_t)(cn < 0 ? 0 : cn);
       p[p[PLAN_OFF_SEG_SEQ] + g] = s;
@@ -123,4 +147,20 @@ extern "C" int lampa_gdr_plan_fill_balanced(const int64_t* cu_seqlens_host, int 
                                             int32_t* plan_host) {
   if (!plan_host || !cu_seqlens_host || n_seq < 1 || total_segments < 1) return LAMPA_ERR_INVALID;
   return plan_fill(cu_seqlens_host, n_seq, 0, total_segments, plan_host);
+}
+// The same tables with the caller's own segment lengths: seg_chunks[n_segments], the segments of sequence 0 first, every
+// sequence's lengths adding up to its number of 64-token chunks (an empty sequence takes one segment of 0 chunks).
+extern "C" int64_t lampa_gdr_plan_size_lengths(const int64_t* cu_seqlens_host, int n_seq, const int32_t* seg_chunks,
+                                               int n_segments) {
+  if (!cu_seqlens_host || !seg_chunks || n_seq < 1 || n_segments < n_seq) return LAMPA_ERR_INVALID;
+  std::vector<int64_t> ns;
+  int64_t chunks, segs;
+  if (plan_segments(cu_seqlens_host, n_seq, -1, n_segments, ns, &chunks, &segs, seg_chunks) != 0) return LAMPA_ERR_INVALID;
+  if (cu_seqlens_host[n_seq] > INT32_MAX) return LAMPA_ERR_UNSUPPORTED;
+  return PLAN_HEADER + 2 * chunks + 5 * segs + 2 * (int64_t)n_seq;
+}
+extern "C" int lampa_gdr_plan_fill_lengths(const int64_t* cu_seqlens_host, int n_seq, const int32_t* seg_chunks,
+                                           int n_segments, int32_t* plan_host) {
+  if (!plan_host || !cu_seqlens_host || !seg_chunks || n_seq < 1 || n_segments < n_seq) return LAMPA_ERR_INVALID;
+  return plan_fill(cu_seqlens_host, n_seq, -1, n_segments, plan_host, seg_chunks);
 }

@@ -140,12 +140,50 @@ def test_balanced_plan_tables(lib):
             assert longest == best
     assert lib.lampa_gdr_plan_size_balanced((ctypes.c_int64 * 2)(0, 10), 1, 0) == -1
     assert lib.lampa_gdr_plan_size_balanced((ctypes.c_int64 * 3)(0, 10, 5), 2, 4) == -1
-    # default segmentation: one round -> one fixed length; several rounds -> whole rounds of balanced segments
-    assert gd._default_segmentation([938], 8, 512) == (15, 0)
+    # default segmentation: several rounds -> whole rounds of balanced segments; one round with one workgroup per CU ->
+    # one fixed length; one round with two per CU -> the first half of a sequence's segments longer than the second
+    assert gd._default_segmentation([938], 8, 256, 1) == ("cps", 30)
     nc4 = [819, 830, 564, 635, 735, 659, 314, 205, 404, 189, 231, 755, 500, 434, 203, 655]
-    assert gd._default_segmentation(nc4, 8, 256) == (0, 128)
-    assert gd._default_segmentation([300] * 4, 8, 256) == (38, 0)   # one round of 38-chunk segments holds it
-    assert gd._default_segmentation([600] * 4, 8, 256) == (0, 64)   # 1.2 rounds of 64 chunks -> 2 rounds of 37-38
+    assert gd._default_segmentation(nc4, 8, 256, 1) == ("balanced", 128)
+    assert gd._default_segmentation([300] * 4, 8, 256, 1) == ("cps", 38)       # one round of 38-chunk segments holds it
+    assert gd._default_segmentation([600] * 4, 8, 256, 1) == ("balanced", 64)  # 1.2 rounds of 64 chunks -> 2 of 37-38
+    kind, lens = gd._default_segmentation([938], 8, 512, 2)
+    assert kind == "lengths" and len(lens) == 64 and sum(lens) == 938
+    assert lens[:32] == [17] * 32 and set(lens[32:]) == {12, 13} and lens[32:] == sorted(lens[32:], reverse=True)
+    kind, lens = gd._default_segmentation([235, 0, 700], 8, 512, 2)
+    assert kind == "lengths" and len(lens) == 64 and min(lens[:16]) > 0 and lens[16] == 0
+    assert sum(lens[:16]) == 235 and sum(lens[17:]) == 700
+    assert gd._default_segmentation([3, 0, 7], 8, 512, 2) == ("cps", 4)      # short sequences: 4-chunk segments
+
+
+def test_plan_with_given_segment_lengths(lib):
+    cu = [0, 64 * 10, 64 * 10, 64 * 10 + 1000]
+    nc = [10, 0, 16]
+
+    def plan(lens):
+        arr = (ctypes.c_int64 * len(cu))(*cu)
+        la = (ctypes.c_int32 * len(lens))(*lens)
+        size = lib.lampa_gdr_plan_size_lengths(arr, 3, la, len(lens))
+        if size < 0:
+            return size
+        p = torch.zeros(size, dtype=torch.int32)
+        assert lib.lampa_gdr_plan_fill_lengths(arr, 3, la, len(lens), ctypes.c_void_p(p.data_ptr())) == 0
+        return p.tolist()
+
+    lens = [4, 3, 3, 0, 7, 5, 4]
+    p = plan(lens)
+    n_seq, chunks, segs, cps = p[0:4]
+    assert (n_seq, chunks, segs, cps) == (3, 26, 7, 0)
+    assert p[p[7]:p[7] + segs] == lens
+    assert p[p[6]:p[6] + segs] == [0, 4, 7, 10, 10, 17, 22]
+    assert p[p[8]:p[8] + segs] == [0, 0, 0, 1, 2, 2, 2]
+    assert p[p[9]:p[9] + segs] == [1, 0, 2, 3, 1, 0, 2]
+    assert p[p[10]:p[10] + 3] == [0, 3, 4] and p[p[11]:p[11] + 3] == [3, 1, 3]
+    assert p[p[13]:p[13] + segs] == [4, 5, 0, 6, 1, 2, 3]  # longest first, ties in plan order
+    # lengths that do not tile the sequences are refused
+    for bad in ([4, 3, 4, 0, 7, 5, 4], [4, 3, 3, 7, 5, 4], [4, 3, 3, 0, 7, 5, 3], [4, 3, 3, 0, 7, 5, 4, 1], [10, 0, 0, 16],
+                [4, 3, 3, 0, 7, -1, 10]):
+        assert plan(bad) == -1, bad
 
 
 def test_plan_rejects_bad_input(lib):
