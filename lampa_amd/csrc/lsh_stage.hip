@@ -501,7 +501,8 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
 #define LF_MAX_DEVICES 64
 struct LfDevice {
   int state;             // 0 unknown, 1 known
-  int capacity[2][2];    // workgroups the GPU holds at once: [generic dim, dim 4][ITEMS 8, 4]
+  int cus;               // compute units
+  int capacity[2][2];    // workgroups the GPU holds at once: [generic dim, dim 4][ITEMS 4, 3]
 };
 static LfDevice lf_dev[LF_MAX_DEVICES];
 static std::mutex lf_lock;
@@ -513,7 +514,7 @@ static uint32_t lf_next_generation() {
   static std::atomic<uint32_t> counter{(uint32_t)std::chrono::steady_clock::now().time_since_epoch().count()};
   return counter.fetch_add(1) + 1;
 }
-static const int lf_items[2] = {8, 4};
+static const int lf_items[2] = {4, 3};
 
 // Process-wide switches of the one-launch form (lampa_lsh_one_launch_config): whether it is used at all, and the
 // number of polls a tile spends in one wait (< 0: LF_SPIN_LIMIT).
@@ -521,7 +522,7 @@ static std::atomic<int> lf_enabled{1};
 static std::atomic<int64_t> lf_wait_limit{-1};
 
 extern "C" int lampa_lsh_one_launch_config(int enabled, int64_t wait_limit) {
-  lf_enabled.store(enabled ? 1 : 0);
+  lf_enabled.store(enabled == 3 || enabled == 4 ? enabled : (enabled ? 1 : 0));
   lf_wait_limit.store(wait_limit);
   return LAMPA_OK;
 }
@@ -549,8 +550,9 @@ static const LfDevice* lf_device() {
       (void)hipGetLastError();
       return nullptr;
     }
-    d.capacity[0][0] = cus * lf_occupancy<0, 8>(); d.capacity[0][1] = cus * lf_occupancy<0, 4>();
-    d.capacity[1][0] = cus * lf_occupancy<4, 8>(); d.capacity[1][1] = cus * lf_occupancy<4, 4>();
+    d.cus = cus;
+    d.capacity[0][0] = cus * lf_occupancy<0, 4>(); d.capacity[0][1] = cus * lf_occupancy<0, 3>();
+    d.capacity[1][0] = cus * lf_occupancy<4, 4>(); d.capacity[1][1] = cus * lf_occupancy<4, 3>();
     d.state = 1;
   }
   return &d;
@@ -568,8 +570,8 @@ static int64_t lf_tiles(int64_t n_hits, int items) {
 // Workspace of the fused kernel: flags | partials | digit counts and totals | two pair buffers, sized for the
 // smallest tile. Zero when the call is too large for the fused kernel.
 int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables) {
-  const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, 4);
-  if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 8) > 4096) return 0;
+  const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, 3);
+  if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 4) > 4096) return 0;
   return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256) +
          lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256) +
          lampa_align_up(segs * 4, 256);
@@ -594,11 +596,25 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   if (workspace_bytes < need) return LAMPA_ERR_WORKSPACE;
   const LfDevice* d = lf_device();
   if (!d) return 1;
-  // the smaller tile (more workgroups, shorter steps) when the whole call is then still on the GPU at once
+  // Tiles of 768 hits when that gives at most one workgroup per CU, else tiles of 1 024 hits when those give at most
+  // 1.4 per CU, else the separate kernels: every step of this kernel is latency bound, and a CU that runs two tiles
+  // takes 1.3-1.7 times as long for each. Measured (us per call; separate kernels | tiles of 2 048 | 1 024 | 768 hits):
+  //   60 000 hits x 1 / 2 / 3 / 4 events: 64.7 | 74.1 | 59.1 | 56.2,  73.5 | 76.3 | 73.9 | 79.0,  83.1 | 86.8 | 86.6 | 97.9,
+  //                                       91.3 | 97.5 | 102.7 | -
+  //   30 000 hits x 1 / 2 / 3 / 4 events: 59.4 | 76.5 | 57.1 | 50.3,  62.4 | 77.0 | 58.9 | 54.0,  67.8 | 79.4 | 63.9 | 67.0,
+  //                                       72.3 | 79.9 | 72.9 | 71.9
+  // (tiles of 2 048 hits never won and are not built). lampa_lsh_one_launch_config(3 or 4) forces a tile size.
   const int dsel = dim == 4 ? 1 : 0;
+  const int forced = lf_enabled.load();
   int pick = -1;
-  for (int i = 1; i >= 0 && pick < 0; --i)
-    if (segs * lf_tiles(n_hits, lf_items[i]) <= d->capacity[dsel][i]) pick = i;
+  const int64_t wg4 = segs * lf_tiles(n_hits, 4), wg3 = segs * lf_tiles(n_hits, 3);
+  if (forced == 1) {
+    if (wg3 <= d->cus && wg3 <= d->capacity[dsel][1]) pick = 1;
+    else if (5 * wg4 <= 7 * (int64_t)d->cus && wg4 <= d->capacity[dsel][0]) pick = 0;
+  } else {
+    for (int i = 1; i >= 0 && pick < 0; --i)
+      if (segs * lf_tiles(n_hits, lf_items[i]) <= d->capacity[dsel][i] && forced == lf_items[i]) pick = i;
+  }
   if (pick < 0) return 1;
   const int items = lf_items[pick];
   const int64_t tiles = lf_tiles(n_hits, items);
@@ -623,9 +639,9 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   LAMPA_PROF(s, "start");
 #define LF_LAUNCH(DIM, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, ITEMS>), grid, block, 0, s, a)
   if (dim == 4) {
-    if (items == 8) LF_LAUNCH(4, 8); else LF_LAUNCH(4, 4);
+    if (items == 4) LF_LAUNCH(4, 4); else LF_LAUNCH(4, 3);
   } else {
-    if (items == 8) LF_LAUNCH(0, 8); else LF_LAUNCH(0, 4);
+    if (items == 4) LF_LAUNCH(0, 4); else LF_LAUNCH(0, 3);
   }
 #undef LF_LAUNCH
   LAMPA_PROF(s, "lsh_fused_kernel");

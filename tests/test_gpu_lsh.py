@@ -264,13 +264,21 @@ def test_one_launch_and_separate_kernels_agree(device):
     f25 = torch.cat([fd, fd[:, :1]], dim=1)
     odd = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, f25, strict=True)
     assert torch.equal(odd["perm"], one["perm"]) and torch.equal(odd["feats"][..., :24], one["feats"])
-    four = lsh.lsh_bucket_sort(cd[None].expand(4, -1, -1).contiguous(), ad, bd, 0.5, 3, 4,
-                               fd[None].expand(4, -1, -1).contiguous(), n_valid=torch.tensor([n, 17, 0, 2049]),
-                               strict=True)  # 12 tables in one launch, padded events
-    for e, nv in enumerate([n, 17, 0, 2049]):
-        w = ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy(), n_valid=nv)
-        for name in ("ids", "meta", "keys", "perm", "feats"):
-            assert np.array_equal(_np(four[name][e]), w[name]), (name, e)
+    # 12 tables of padded events: by itself the library sends this size to the separate kernels (1.4 workgroups per CU
+    # or more); with a forced tile it is one launch of 480 (tiles of 768 hits) or 360 workgroups
+    wants = [ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy(), n_valid=nv)
+             for nv in [n, 17, 0, 2049]]
+    try:
+        for tile in (0, 3, 4):
+            lsh.one_launch_config(tile=tile)
+            four = lsh.lsh_bucket_sort(cd[None].expand(4, -1, -1).contiguous(), ad, bd, 0.5, 3, 4,
+                                       fd[None].expand(4, -1, -1).contiguous(), n_valid=torch.tensor([n, 17, 0, 2049]),
+                                       strict=True)
+            for e, w in enumerate(wants):
+                for name in ("ids", "meta", "keys", "perm", "feats"):
+                    assert np.array_equal(_np(four[name][e]), w[name]), (tile, name, e)
+    finally:
+        lsh.one_launch_config()
 
 
 def test_one_launch_generic_dim_and_wide_keys(device):
