@@ -78,8 +78,8 @@ int lampa_lsh_bucket_keys(const float* coords, int64_t n_hits, int64_t n_valid, 
  * Replaces the hash -> argsort -> sort_to_buckets sequence of models/attention/hept.py:127-143.
  * perm_out [n_tables, n_hits] int32; feats [n_hits, feat_row_bytes] -> feats_out [n_tables, n_hits, feat_row_bytes].
  * n_passes: 0 (automatic), 3 or 4 sort launches for the 32-bit keys.
- * A call (this one or the batch form) of at most 64 tables whose tiles (768 or 1 024 hits) come to at most about 1.4
- * workgroups per CU (one or two events of 60 000 hits on 256 CUs), with feature rows made of 16-byte pieces, runs as ONE
+ * A call (this one or the batch form) of at most 64 tables whose tiles of 1 024 hits come to at most two workgroups
+ * per CU (one or two events of 60 000 hits on 256 CUs), with feature rows made of 16-byte pieces, runs as ONE
  * kernel whose workgroups wait for the other workgroups of their table (flags in the
  * workspace; no host-visible state); any other call runs as separate kernels. The results are the same bits. The waits
  * are bounded: should one run out (two such kernels sharing one GPU at the same time can starve each other), bit 1 of the
@@ -376,9 +376,10 @@ int lampa_hgdn_step(const void* q, const void* k, const void* v, const float* g,
 
 /* Process-wide switches of the one-launch form of lampa_lsh_bucket_sort[_batch] (no counterpart in the reference).
  * enabled = 0: every call takes the separate kernels (what a caller retries with after a call came back with bit 1 of
- * an overflow field set); 1: the library chooses (tiles of 768 hits when that is at most one workgroup per CU, else
- * tiles of 1 024 hits up to about 1.4 workgroups per CU, else the separate kernels); 3 / 4: tiles of 768 / 1 024 hits
- * for every call whose workgroups fit the GPU at once. wait_limit: polls a workgroup spends in one wait for the other workgroups of its table
+ * an overflow field set); 1: the library chooses (workgroups of 768 threads on tiles of 768 hits when that is at most
+ * one workgroup per CU and 48 tiles per table, else workgroups of 512 threads on tiles of 1 024 hits when they fit the
+ * GPU at once, else the separate kernels); 100 / 101: the 512- / 768-thread form for every call that fits.
+ * wait_limit: polls a workgroup spends in one wait for the other workgroups of its table
  * before it gives up; < 0 = the built-in bound; 0 = give up at once, which lets a test reach the give-up path from the
  * host with every kernel still ending normally. */
 int lampa_lsh_one_launch_config(int enabled, int64_t wait_limit);

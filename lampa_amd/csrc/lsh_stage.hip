@@ -26,8 +26,6 @@
 #include <chrono>
 #include <mutex>
 
-#define LF_BLOCK 256
-#define LF_WAVES (LF_BLOCK / 64)
 #define LF_MAX_DIGIT_BITS 11
 #define LF_MAX_BINS (1 << LF_MAX_DIGIT_BITS)
 #define LF_SPIN_LIMIT (1 << 22)
@@ -108,24 +106,29 @@ __device__ __forceinline__ uint32_t lf_wave_inclusive(uint32_t v, int lane) {
 }
 
 // grid = segments * n_tiles workgroups: workgroup b is tile b % n_tiles of segment b / n_tiles (segment =
-// event * n_tables + table). A tile is 256 * ITEMS hits; element order inside a tile as in the radix sort: wave w owns
-// a quarter of the tile, item k of lane l is at quarter * w + k * 64 + l. Small ITEMS = more, smaller tiles: more CUs
-// and more waves per hit, which is what the latency of one event needs.
-template <int DIM, int ITEMS>
-__global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs a) {
-  __shared__ uint32_t s_bin[LF_WAVES][LF_MAX_BINS];  // per-wave digit counts, later the waves' output bases
-  __shared__ uint32_t s_base[LF_MAX_BINS];           // keys of the segment with a smaller digit
+// event * n_tables + table). A tile is BLOCK * ITEMS hits; element order inside a tile as in the radix sort: wave w owns
+// 64 * ITEMS consecutive hits, item k of lane l is at 64 * ITEMS * w + k * 64 + l. Every step of the kernel is latency
+// bound: small tiles (more CUs) and many waves per tile (less serial work per thread) are what one event needs.
+template <int DIM, int BLOCK, int ITEMS>
+__global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) {
+  constexpr int WAVES = BLOCK / 64;
+  // per-wave digit counts, later the keys of the tile's earlier waves with the digit: 16 bits each (a wave holds
+  // 64 * ITEMS keys, a tile at most 2048), digits 2j and 2j + 1 in one word
+  __shared__ uint32_t s_cnt[WAVES][LF_MAX_BINS / 2];
+  __shared__ uint32_t s_base[LF_MAX_BINS];           // keys of the segment with a smaller digit (+ of earlier tiles)
   __shared__ uint32_t s_tot[LF_MAX_BINS];            // digit totals of the segment; later the tile's permutation
-  __shared__ int32_t s_mm[LF_WAVES][LF_PARTIAL_STRIDE];
+  __shared__ uint8_t s_tab[WAVES][LF_MAX_BINS];      // the ranking's match tables (see below)
+  __shared__ unsigned long long s_grp[WAVES][64];
+  __shared__ int32_t s_mm[WAVES][LF_PARTIAL_STRIDE];
   __shared__ int32_t s_lo[LSH_MAX_PROJ], s_hi[LSH_MAX_PROJ];
   __shared__ uint32_t s_stride[LSH_MAX_PROJ];
   __shared__ float s_alpha[LSH_MAX_DIM][LSH_MAX_PROJ], s_beta[LSH_MAX_PROJ];  // the table's projections
   __shared__ uint32_t s_total;
   __shared__ int s_bits, s_over;
-  __shared__ uint32_t s_wsum[LF_WAVES];
+  __shared__ uint32_t s_wsum[WAVES];
   constexpr int XD = DIM ? DIM : LSH_MAX_DIM;
-  constexpr int DPT = LF_MAX_BINS / LF_BLOCK;
-  constexpr int TILE = LF_BLOCK * ITEMS;
+  constexpr int DPT = (LF_MAX_BINS + BLOCK - 1) / BLOCK;
+  constexpr int TILE = BLOCK * ITEMS;
   static_assert(TILE <= LF_MAX_BINS, "the tile's permutation is staged in s_tot");
 
   const int tile = blockIdx.x % a.n_tiles, seg = blockIdx.x / a.n_tiles;
@@ -139,7 +142,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
   uint2* pairs[2] = {a.pairs0 + (int64_t)seg * n_hits, a.pairs1 + (int64_t)seg * n_hits};
   uint64_t phase = (uint64_t)a.gen << 32;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  const int ibase = tile * TILE + wave * (TILE / LF_WAVES) + lane;
+  const int ibase = tile * TILE + wave * (TILE / WAVES) + lane;
 
   {
     const int ev = seg / T, table = seg - ev * T;
@@ -199,7 +202,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       const int q = threadIdx.x;
       int32_t v = s_mm[0][q];
 #pragma unroll
-      for (int w = 1; w < LF_WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
+      for (int w = 1; w < WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
       lf_store(partial + tile * LF_PARTIAL_STRIDE + q, v);
     }
     healthy = lf_sync(++phase);
@@ -210,7 +213,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       int32_t v = (q & 1) ? INT32_MIN : INT32_MAX;
       if (q < 2 * J) {
 #pragma unroll 8
-        for (int p = threadIdx.x >> 4; p < n_tiles; p += LF_BLOCK / 16) {
+        for (int p = threadIdx.x >> 4; p < n_tiles; p += BLOCK / 16) {
           const int32_t o = lf_load(partial + p * LF_PARTIAL_STRIDE + q);
           v = (q & 1) ? max(v, o) : min(v, o);
         }
@@ -224,7 +227,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       if ((int)threadIdx.x < 2 * J) {
         v = s_mm[0][q];
 #pragma unroll
-        for (int w = 1; w < LF_WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
+        for (int w = 1; w < WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
         if (n_valid == 0) v = 0;
         if (q & 1) s_hi[q >> 1] = v; else s_lo[q >> 1] = v;
       }
@@ -289,14 +292,14 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       const int shift = e * width, nbits = min(width, bits - shift), bins = 1 << nbits;
       const uint32_t mask = (uint32_t)bins - 1u;
       const bool last = e == eff - 1;
-      for (int d = threadIdx.x; d < bins; d += LF_BLOCK) {
+      for (int d2 = threadIdx.x; 2 * d2 < bins; d2 += BLOCK) {
 #pragma unroll
-        for (int w = 0; w < LF_WAVES; ++w) s_bin[w][d] = 0;
+        for (int w = 0; w < WAVES; ++w) s_cnt[w][d2] = 0;
       }
       __syncthreads();
       {
-        // Ranks within the wave. Lanes with the same digit find each other through two tables of the wave in LDS
-        // (s_tot and s_base are free at this point): every lane writes its number to tab[d] and reads back the one
+        // Ranks within the wave. Lanes with the same digit find each other through two tables of the wave in LDS:
+        // every lane writes its number to tab[d] and reads back the one
         // that stayed (the group's speaker), sets its bit in the speaker's 64-bit word, reads the word (= the group)
         // and clears it; the speaker then adds the group's size to the wave's count of the digit. The LDS executes
         // the instructions of one wave in order, so the steps need no wait between them, and the relaxed atomic
@@ -304,8 +307,8 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         // key did the same in three times the instructions: 62.3 -> 58.7 us for one event.) A hit beyond the event's
         // end carries the largest digit and comes last in (item, lane) order: it changes no rank, only the count of
         // the largest digit in the segment's last tile, which no other key's position depends on.
-        uint8_t* tab = reinterpret_cast<uint8_t*>(s_tot) + wave * LF_MAX_BINS;
-        unsigned long long* grp = reinterpret_cast<unsigned long long*>(s_base) + wave * 64;
+        uint8_t* tab = s_tab[wave];
+        unsigned long long* grp = s_grp[wave];
         grp[lane] = 0ull;
         const unsigned long long bit = 1ull << lane;
         uint32_t dd[ITEMS], spk[ITEMS], old[ITEMS];
@@ -324,8 +327,10 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         }
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
+          const int sh = 16 * (dd[k] & 1u);
           old[k] = 0;
-          if ((uint32_t)lane == spk[k]) old[k] = atomicAdd(&s_bin[wave][dd[k]], (uint32_t)__popcll(peers[k]));
+          if ((uint32_t)lane == spk[k])
+            old[k] = (atomicAdd(&s_cnt[wave][dd[k] >> 1], (uint32_t)__popcll(peers[k]) << sh) >> sh) & 0xFFFFu;
         }
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
@@ -333,10 +338,10 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       }
       __syncthreads();
       // the tile's digit counts for the other tiles of the segment
-      for (int d = threadIdx.x; d < bins; d += LF_BLOCK) {
+      for (int d = threadIdx.x; d < bins; d += BLOCK) {
         uint32_t c = 0;
 #pragma unroll
-        for (int w = 0; w < LF_WAVES; ++w) c += s_bin[w][d];
+        for (int w = 0; w < WAVES; ++w) c += (s_cnt[w][d >> 1] >> (16 * (d & 1))) & 0xFFFFu;
         lf_store(rows + tile * LF_MAX_BINS + d, c);
       }
       healthy = lf_sync(++phase);
@@ -345,14 +350,14 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       // takes a digit, its lanes the tiles (128 at a time); four digits per wave are in flight, all loads first.
       {
         const int per = (bins + n_tiles - 1) / n_tiles, d0 = tile * per;
-        const int steps = (per + LF_WAVES - 1) / LF_WAVES;
+        const int steps = (per + WAVES - 1) / WAVES;
         for (int s0 = 0; s0 < steps; s0 += 4) {
           uint32_t carry[4] = {0, 0, 0, 0};
           for (int p0 = 0; p0 < n_tiles; p0 += 128) {
             uint32_t c[4][2];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-              const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+              const int dd = (s0 + u) * WAVES + wave, d = d0 + dd;
 #pragma unroll
               for (int h = 0; h < 2; ++h) {
                 const int p = p0 + 64 * h + lane;
@@ -361,7 +366,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-              const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+              const int dd = (s0 + u) * WAVES + wave, d = d0 + dd;
 #pragma unroll
               for (int h = 0; h < 2; ++h) {
                 const int p = p0 + 64 * h + lane;
@@ -373,7 +378,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
           }
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
-            const int dd = (s0 + u) * LF_WAVES + wave, d = d0 + dd;
+            const int dd = (s0 + u) * WAVES + wave, d = d0 + dd;
             if (lane == 0 && dd < per && d < bins) lf_store(totals + d, carry[u]);
           }
         }
@@ -383,7 +388,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       uint32_t excl[DPT];
 #pragma unroll
       for (int j = 0; j < DPT; ++j) {
-        const int d = threadIdx.x + j * LF_BLOCK;
+        const int d = threadIdx.x + j * BLOCK;
         excl[j] = d < bins ? lf_load(rows + tile * LF_MAX_BINS + d) : 0u;
         if (d < bins) s_tot[d] = lf_load(totals + d);
       }
@@ -406,7 +411,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         __syncthreads();
         uint32_t run = incl - mine;
 #pragma unroll
-        for (int w = 0; w < LF_WAVES; ++w) run += w < wave ? s_wsum[w] : 0u;
+        for (int w = 0; w < WAVES; ++w) run += w < wave ? s_wsum[w] : 0u;
 #pragma unroll
         for (int j = 0; j < DPT; ++j) {
           const int d = threadIdx.x * DPT + j;
@@ -416,14 +421,16 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       }
       __syncthreads();
 #pragma unroll
-      for (int j = 0; j < DPT; ++j) {  // output base of every wave of the tile for every digit
-        const int d = threadIdx.x + j * LF_BLOCK;
+      for (int j = 0; j < DPT; ++j) {  // per digit: the tile's base, and the keys of the tile's earlier waves
+        const int d = threadIdx.x + j * BLOCK;
         if (d < bins) {
-          uint32_t run = s_base[d] + excl[j];
+          s_base[d] += excl[j];
+          uint32_t run = 0;
 #pragma unroll
-          for (int w = 0; w < LF_WAVES; ++w) {
-            const uint32_t c = s_bin[w][d];
-            s_bin[w][d] = run;
+          for (int w = 0; w < WAVES; ++w) {
+            uint16_t* half = reinterpret_cast<uint16_t*>(s_cnt[w]) + d;
+            const uint32_t c = *half;
+            *half = (uint16_t)run;
             run += c;
           }
         }
@@ -433,7 +440,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
       for (int k = 0; k < ITEMS; ++k) {
         if (inside[k]) {
           const uint32_t d = (key[k] >> shift) & mask;
-          const uint32_t pos = s_bin[wave][d] + rank[k];
+          const uint32_t pos = s_base[d] + reinterpret_cast<const uint16_t*>(s_cnt[wave])[d] + rank[k];
           if (pos < (uint32_t)n_hits) {  // always, unless a wait was abandoned
             if (last) { if (healthy) lf_store(perm + pos, val[k]); }
             else lf_store_pair(pairs[e & 1] + pos, key[k], (uint32_t)val[k]);
@@ -461,22 +468,22 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
     const bool poisoned = !healthy || lf_load(a.failed + seg) == a.gen;
     const int row0 = tile * TILE, n_rows = max(0, min(TILE, n_hits - row0));
     if (poisoned)
-      for (int r = threadIdx.x; r < n_hits; r += LF_BLOCK) lf_store(perm + r, (int32_t)-1);
+      for (int r = threadIdx.x; r < n_hits; r += BLOCK) lf_store(perm + r, (int32_t)-1);
 
     // ---- the hit features in sorted order: rows tile*TILE .. of the segment's output ----
     if (a.feats) {
-      for (int r = threadIdx.x; r < n_rows; r += LF_BLOCK)
+      for (int r = threadIdx.x; r < n_rows; r += BLOCK)
         s_tot[r] = poisoned ? 0xFFFFFFFFu : (uint32_t)lf_load(perm + row0 + r);
       __syncthreads();
       const int vpr = a.vec_per_row, items = n_rows * vpr;
       const uint4* src = reinterpret_cast<const uint4*>(a.feats) + (int64_t)ev * n_hits * vpr;
       uint4* dst = reinterpret_cast<uint4*>(a.feats_out) + ((int64_t)seg * n_hits + row0) * vpr;
       constexpr int GU = 12;  // 16-byte loads in flight per thread: the reads are random rows, a memory latency each
-      for (int it0 = 0; it0 < items; it0 += GU * LF_BLOCK) {
+      for (int it0 = 0; it0 < items; it0 += GU * BLOCK) {
         uint4 v[GU];
 #pragma unroll
         for (int u = 0; u < GU; ++u) {
-          const int it = it0 + u * LF_BLOCK + threadIdx.x;
+          const int it = it0 + u * BLOCK + threadIdx.x;
           v[u] = make_uint4(0, 0, 0, 0);
           if (it < items) {
             const int r = it / vpr, piece = it - r * vpr;
@@ -486,7 +493,7 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
         }
 #pragma unroll
         for (int u = 0; u < GU; ++u) {
-          const int it = it0 + u * LF_BLOCK + threadIdx.x;
+          const int it = it0 + u * BLOCK + threadIdx.x;
           if (it < items) dst[it] = v[u];
         }
       }
@@ -499,10 +506,15 @@ __global__ void __launch_bounds__(LF_BLOCK) lsh_fused_kernel(const LshFusedArgs 
 
 // ---- host side ---------------------------------------------------------------------------------------------------
 #define LF_MAX_DEVICES 64
+// The forms of the kernel that are built: threads per workgroup x hits per thread (tile = their product).
+struct LfForm { int block, items; };
+static const LfForm lf_forms[] = {{512, 2}, {768, 1}};
+#define LF_FORMS ((int)(sizeof(lf_forms) / sizeof(lf_forms[0])))
+#define LF_MIN_TILE 768
 struct LfDevice {
-  int state;             // 0 unknown, 1 known
-  int cus;               // compute units
-  int capacity[2][2];    // workgroups the GPU holds at once: [generic dim, dim 4][ITEMS 4, 3]
+  int state;                    // 0 unknown, 1 known
+  int cus;                      // compute units
+  int capacity[2][LF_FORMS];    // workgroups the GPU holds at once: [generic dim, dim 4][form]
 };
 static LfDevice lf_dev[LF_MAX_DEVICES];
 static std::mutex lf_lock;
@@ -514,23 +526,22 @@ static uint32_t lf_next_generation() {
   static std::atomic<uint32_t> counter{(uint32_t)std::chrono::steady_clock::now().time_since_epoch().count()};
   return counter.fetch_add(1) + 1;
 }
-static const int lf_items[2] = {4, 3};
 
-// Process-wide switches of the one-launch form (lampa_lsh_one_launch_config): whether it is used at all, and the
-// number of polls a tile spends in one wait (< 0: LF_SPIN_LIMIT).
+// Process-wide switches of the one-launch form (lampa_lsh_one_launch_config): whether it is used at all (0 / 1, or
+// 100 + i: form i for every call that fits), and the number of polls a tile spends in one wait (< 0: LF_SPIN_LIMIT).
 static std::atomic<int> lf_enabled{1};
 static std::atomic<int64_t> lf_wait_limit{-1};
 
 extern "C" int lampa_lsh_one_launch_config(int enabled, int64_t wait_limit) {
-  lf_enabled.store(enabled == 3 || enabled == 4 ? enabled : (enabled ? 1 : 0));
+  lf_enabled.store(enabled >= 100 && enabled < 100 + LF_FORMS ? enabled : (enabled ? 1 : 0));
   lf_wait_limit.store(wait_limit);
   return LAMPA_OK;
 }
 
-template <int DIM, int ITEMS>
+template <int DIM, int BLOCK, int ITEMS>
 static int lf_occupancy() {
   int occ = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, lsh_fused_kernel<DIM, ITEMS>, LF_BLOCK, 0) != hipSuccess) {
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, lsh_fused_kernel<DIM, BLOCK, ITEMS>, BLOCK, 0) != hipSuccess) {
     (void)hipGetLastError();
     occ = 0;
   }
@@ -551,17 +562,14 @@ static const LfDevice* lf_device() {
       return nullptr;
     }
     d.cus = cus;
-    d.capacity[0][0] = cus * lf_occupancy<0, 4>(); d.capacity[0][1] = cus * lf_occupancy<0, 3>();
-    d.capacity[1][0] = cus * lf_occupancy<4, 4>(); d.capacity[1][1] = cus * lf_occupancy<4, 3>();
+    d.capacity[0][0] = cus * lf_occupancy<0, 512, 2>(); d.capacity[1][0] = cus * lf_occupancy<4, 512, 2>();
+    d.capacity[0][1] = cus * lf_occupancy<0, 768, 1>(); d.capacity[1][1] = cus * lf_occupancy<4, 768, 1>();
     d.state = 1;
   }
   return &d;
 }
 
-static int64_t lf_tiles(int64_t n_hits, int items) {
-  const int64_t tile = (int64_t)LF_BLOCK * items;
-  return n_hits > 0 ? (n_hits + tile - 1) / tile : 1;
-}
+static int64_t lf_tiles(int64_t n_hits, int tile) { return n_hits > 0 ? (n_hits + tile - 1) / tile : 1; }
 
 // The fused kernel is for calls of at most this many segments (events x tables): beyond it the call cannot fit the
 // GPU at once whatever the event size.
@@ -570,8 +578,8 @@ static int64_t lf_tiles(int64_t n_hits, int items) {
 // Workspace of the fused kernel: flags | partials | digit counts and totals | two pair buffers, sized for the
 // smallest tile. Zero when the call is too large for the fused kernel.
 int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables) {
-  const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, 3);
-  if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 4) > 4096) return 0;
+  const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, LF_MIN_TILE);
+  if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 1024) > 4096) return 0;
   return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256) +
          lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256) +
          lampa_align_up(segs * 4, 256);
@@ -596,28 +604,33 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   if (workspace_bytes < need) return LAMPA_ERR_WORKSPACE;
   const LfDevice* d = lf_device();
   if (!d) return 1;
-  // Tiles of 768 hits when that gives at most one workgroup per CU, else tiles of 1 024 hits when those give at most
-  // 1.4 per CU, else the separate kernels: every step of this kernel is latency bound, and a CU that runs two tiles
-  // takes 1.3-1.7 times as long for each. Measured (us per call; separate kernels | tiles of 2 048 | 1 024 | 768 hits):
-  //   60 000 hits x 1 / 2 / 3 / 4 events: 64.7 | 74.1 | 59.1 | 56.2,  73.5 | 76.3 | 73.9 | 79.0,  83.1 | 86.8 | 86.6 | 97.9,
-  //                                       91.3 | 97.5 | 102.7 | -
-  //   30 000 hits x 1 / 2 / 3 / 4 events: 59.4 | 76.5 | 57.1 | 50.3,  62.4 | 77.0 | 58.9 | 54.0,  67.8 | 79.4 | 63.9 | 67.0,
-  //                                       72.3 | 79.9 | 72.9 | 71.9
-  // (tiles of 2 048 hits never won and are not built). lampa_lsh_one_launch_config(3 or 4) forces a tile size.
+  // Which form, if any. Every step of this kernel is latency bound: more waves per tile shorten the steps (a tile of
+  // 1 024 hits: 60.5 us with 256 threads, 49.7 us with 512, for one event of 60 000 hits), smaller tiles do too as long as
+  // a CU runs one of them and a table does not get too many (the barriers run over a table's tiles), and a CU that runs
+  // two tiles takes 1.3-1.7 times as long for each, while the separate kernels grow by only 0.145 us per 1 000 hits.
+  // Measured, us per call: separate kernels | 256 threads x 4 hits | 256 x 3 | 512 x 2 | 1 024 x 1 | 768 x 1 (- = the
+  // workgroups do not fit the GPU at once):
+  //   60 000 hits x 1 event   65.7 | 60.5 | 56.2 | 49.7 | 50.0 | 51.1      30 000 x 1   60.3 | 58.6 | 51.0 | 45.5 | 43.7 | 43.4
+  //            x 2 events     72.4 | 74.8 | 77.7 | 69.1 |  -   |  -                x 2   62.3 | 61.1 | 55.1 | 50.1 | 48.7 | 48.5
+  //            x 3            82.5 | 87.1 | 99.6 |  -   |  -   |  -                x 3   67.4 | 64.9 | 67.0 | 57.3 |  -   |  -
+  //            x 4            90.9 | 102.9 | -   |  -   |  -   |  -                x 4   72.1 | 72.1 | 71.0 | 66.7 |  -   |  -
+  // Built: 512 x 2 and 768 x 1. The latter when it gives at most one workgroup per CU and at most 48 tiles per table,
+  // else the former when its workgroups fit the GPU at once (two per CU), else the separate kernels.
+  // lampa_lsh_one_launch_config(100 / 101, ...) forces a form for every call that fits.
   const int dsel = dim == 4 ? 1 : 0;
   const int forced = lf_enabled.load();
   int pick = -1;
-  const int64_t wg4 = segs * lf_tiles(n_hits, 4), wg3 = segs * lf_tiles(n_hits, 3);
-  if (forced == 1) {
-    if (wg3 <= d->cus && wg3 <= d->capacity[dsel][1]) pick = 1;
-    else if (5 * wg4 <= 7 * (int64_t)d->cus && wg4 <= d->capacity[dsel][0]) pick = 0;
+  if (forced >= 100) {
+    const int i = forced - 100;
+    if (segs * lf_tiles(n_hits, lf_forms[i].block * lf_forms[i].items) <= d->capacity[dsel][i]) pick = i;
   } else {
-    for (int i = 1; i >= 0 && pick < 0; --i)
-      if (segs * lf_tiles(n_hits, lf_items[i]) <= d->capacity[dsel][i] && forced == lf_items[i]) pick = i;
+    const int64_t t768 = lf_tiles(n_hits, 768), t1024 = lf_tiles(n_hits, 1024);
+    if (segs * t768 <= d->cus && segs * t768 <= d->capacity[dsel][1] && t768 <= 48) pick = 1;
+    else if (segs * t1024 <= d->capacity[dsel][0]) pick = 0;
   }
   if (pick < 0) return 1;
-  const int items = lf_items[pick];
-  const int64_t tiles = lf_tiles(n_hits, items);
+  const int tile_hits = lf_forms[pick].block * lf_forms[pick].items;
+  const int64_t tiles = lf_tiles(n_hits, tile_hits);
   LshFusedArgs a;
   a.coords = coords; a.n_hits = n_hits; a.n_valid = n_valid; a.n_valid_dev = n_valid_dev; a.dim = dim;
   a.alpha = alpha; a.beta = beta; a.n_tables = n_tables; a.n_proj = n_proj; a.inv_w = 1.0f / w;
@@ -635,14 +648,16 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   a.gen = lf_next_generation();
   const int64_t limit = lf_wait_limit.load();
   a.spin_limit = limit < 0 ? LF_SPIN_LIMIT : (int)(limit > LF_SPIN_LIMIT ? LF_SPIN_LIMIT : limit);
-  const dim3 grid((unsigned)(segs * tiles)), block(LF_BLOCK);
+  const dim3 grid((unsigned)(segs * tiles)), block(lf_forms[pick].block);
   LAMPA_PROF(s, "start");
-#define LF_LAUNCH(DIM, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, ITEMS>), grid, block, 0, s, a)
-  if (dim == 4) {
-    if (items == 4) LF_LAUNCH(4, 4); else LF_LAUNCH(4, 3);
-  } else {
-    if (items == 4) LF_LAUNCH(0, 4); else LF_LAUNCH(0, 3);
+#define LF_LAUNCH(DIM, BLOCK, ITEMS) hipLaunchKernelGGL((lsh_fused_kernel<DIM, BLOCK, ITEMS>), grid, block, 0, s, a)
+#define LF_LAUNCH_DIM(DIM)                                                                        \
+  switch (pick) {                                                                                 \
+    case 0: LF_LAUNCH(DIM, 512, 2); break;                                                        \
+    default: LF_LAUNCH(DIM, 768, 1); break;                                                       \
   }
+  if (dim == 4) { LF_LAUNCH_DIM(4) } else { LF_LAUNCH_DIM(0) }
+#undef LF_LAUNCH_DIM
 #undef LF_LAUNCH
   LAMPA_PROF(s, "lsh_fused_kernel");
   return lampa_launch_status();

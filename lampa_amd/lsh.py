@@ -277,12 +277,11 @@ def decode_meta_flags(meta) -> dict:
 def one_launch_config(enabled: bool = True, wait_limit: int = -1, tile: int = 0) -> None:
     """Process-wide switches of the one-launch form of the stage (``lampa_lsh_one_launch_config``): ``enabled=False``
     sends every call to the separate kernels; ``wait_limit`` is the number of polls a workgroup spends in one wait
-    before it gives up (< 0: the built-in bound; 0: give up at once, for tests of the give-up path); ``tile`` = 3 or 4
-    forces tiles of 768 / 1 024 hits for every call that fits the GPU at once (0: the library chooses, and sends calls
-    that would put more than about 1.4 workgroups on a CU to the separate kernels)."""
-    assert tile in (0, 3, 4)
-    check(_capi.lib().lampa_lsh_one_launch_config((tile or 1) if enabled else 0, int(wait_limit)),
-          "lampa_lsh_one_launch_config")
+    before it gives up (< 0: the built-in bound; 0: give up at once, for tests of the give-up path); ``tile`` = 1024
+    or 768 forces that form of the kernel (512 threads x 2 hits, 768 threads x 1 hit) for every call whose workgroups fit
+    the GPU at once (0: the library chooses between them and the separate kernels)."""
+    code = {0: 1, 1024: 100, 768: 101}[tile]
+    check(_capi.lib().lampa_lsh_one_launch_config(code if enabled else 0, int(wait_limit)), "lampa_lsh_one_launch_config")
 
 
 def _raise_on_overflow(meta: torch.Tensor, strict: bool):
@@ -315,8 +314,8 @@ def lsh_bucket_sort(coords, alpha, beta, w, n_tables, n_proj, feats: Optional[to
     then sets ``meta[..., -1]`` (overflow) and the order of that table is meaningless. ``strict=True`` reads the flag
     (one host synchronisation) and raises ``LampaError``; otherwise the caller has to look at the flag.
 
-    A call of at most 64 tables in total whose tiles come to at most about 1.4 workgroups per CU (one or two events of
-    60 000 hits do, four of 30 000) runs as ONE kernel whose workgroups wait for each other; larger calls run as separate kernels. The waits of the
+    A call of at most 64 tables in total whose tiles of 1 024 hits come to at most two workgroups per CU (one or two
+    events of 60 000 hits do, four of 30 000) runs as ONE kernel whose workgroups wait for each other; larger calls run as separate kernels. The waits of the
     one-launch kernel are bounded: should one run out (two such kernels sharing a GPU can starve each other) bit 1 of
     ``meta[..., -1]`` is set, the table's ``perm`` is all -1 and its ``feats`` all zero; ``strict=True`` raises for it as
     well (``decode_meta_flags`` reads the field). Calls that may run at the same time on one GPU (different streams,

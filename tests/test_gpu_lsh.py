@@ -264,12 +264,12 @@ def test_one_launch_and_separate_kernels_agree(device):
     f25 = torch.cat([fd, fd[:, :1]], dim=1)
     odd = lsh.lsh_bucket_sort(cd, ad, bd, 0.5, 3, 4, f25, strict=True)
     assert torch.equal(odd["perm"], one["perm"]) and torch.equal(odd["feats"][..., :24], one["feats"])
-    # 12 tables of padded events: by itself the library sends this size to the separate kernels (1.4 workgroups per CU
-    # or more); with a forced tile it is one launch of 480 (tiles of 768 hits) or 360 workgroups
+    # 12 tables of padded events: one launch of 360 workgroups of 512 threads (the library's own choice; the 768-thread
+    # form does not hold 480 workgroups at once and leaves the call to the separate kernels)
     wants = [ol.bucket_sort(coords.numpy(), alpha.numpy(), beta.numpy(), 0.5, 3, 4, feats.numpy(), n_valid=nv)
              for nv in [n, 17, 0, 2049]]
     try:
-        for tile in (0, 3, 4):
+        for tile in (0, 768, 1024):
             lsh.one_launch_config(tile=tile)
             four = lsh.lsh_bucket_sort(cd[None].expand(4, -1, -1).contiguous(), ad, bd, 0.5, 3, 4,
                                        fd[None].expand(4, -1, -1).contiguous(), n_valid=torch.tensor([n, 17, 0, 2049]),
