@@ -109,14 +109,15 @@ def cpu_baseline_lsh(coords, feats, alpha, offsets):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults long enough for the GPU clocks to settle (a layer is ~0.16 ms: 50 + 200 steps take 40 ms)
+    # (a layer is ~0.12 ms: 50 + 200 steps take 30 ms; the clocks are settled by the untimed steps of --prewarm-ms)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192,
                     help="prefix of the workload the CPU baseline is timed on (median of 5 passes, scaled linearly)")
-    ap.add_argument("--prewarm-ms", type=float, default=150.0,
-                    help="untimed steps run before the warm-up until this much wall clock has passed, so that the GPU "
-                         "clocks have settled whatever --warmup is")
+    ap.add_argument("--prewarm-ms", type=float, default=1000.0,
+                    help="untimed steps run before the warm-up until this much wall clock has passed AND five batches "
+                         "of 20 steps in a row agree within 2 % (at most three times as long), so that the clocks of a "
+                         "GPU that was idle have settled whatever --warmup is")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (for profiler runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run one plain device copy of 256 MiB, the known-size kernel that scales a counter run")
@@ -157,15 +158,38 @@ def main():
     def step():
         return gd.chunk_gated_delta_rule(qd, kd, vd, gd_, bd, output_final_state=True)
 
+    def settle(fn, ms=60.0):
+        """Untimed calls of a leg's step for `ms` of wall clock before its own warm-up: every leg prepares its inputs on
+        the host first, the GPU idles meanwhile, and for about 30 ms after an idle spell everything runs up to a third
+        slower (clocks)."""
+        t_ = time.perf_counter()
+        while 1e3 * (time.perf_counter() - t_) < ms:
+            fn()
+            fn()
+            torch.cuda.synchronize()
+
     # ---- clock settling (untimed, stated in the output), then W warm-up steps, then the timed region: exactly K steps ----
+    # (On a box whose GPU had been idle, the first 20-step region timed 150 ms after the first launch read 146-150 us per
+    # step twice where every later process read 120-123: the region is 2.4 ms long, and one power-state change of the
+    # memory system inside it is a fifth of it. Hence the longer settling and the check that the step time is steady.)
     t_pre = time.perf_counter()
     n_pre = 0
-    while 1e3 * (time.perf_counter() - t_pre) < args.prewarm_ms:
+    recent = []
+    while True:
+        tb = time.perf_counter()
         for _ in range(20):
             step()
         torch.cuda.synchronize()
         n_pre += 20
+        recent = (recent + [time.perf_counter() - tb])[-5:]
+        spent = 1e3 * (time.perf_counter() - t_pre)
+        steady = len(recent) == 5 and max(recent) <= 1.02 * min(recent)
+        if (spent >= args.prewarm_ms and steady) or spent >= 3 * args.prewarm_ms:
+            break
     prewarm_ms = 1e3 * (time.perf_counter() - t_pre)
+    import gc
+    gc.disable()  # no collector pause inside the timed region (and no collection here: while the host is busy the GPU
+                  # idles, its clocks drop, and the next ~200 steps are up to a third slower)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -174,6 +198,7 @@ def main():
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    gc.enable()
     ms_per_step = 1e3 * elapsed / args.steps
     hits_per_s = T / (elapsed / args.steps)
 
@@ -291,6 +316,7 @@ def main():
     def lsh_step():
         return lsh.lsh_bucket_sort(coords_d, alpha_d, beta_hd, W_BUCKET, N_TABLES, N_PROJ, feats_d)
 
+    settle(lsh_step)
     for _ in range(args.warmup):
         lsh_step()
     torch.cuda.synchronize()
@@ -331,6 +357,7 @@ def main():
     def lsh_batch_step():
         return lsh.lsh_bucket_sort(bc_d, alpha_d, beta_hd, W_BUCKET, N_TABLES, N_PROJ, bf_d)
 
+    settle(lsh_batch_step)
     for _ in range(3):
         lsh_batch_step()
     torch.cuda.synchronize()
@@ -352,6 +379,7 @@ def main():
     from lampa_amd import block as lblock
     torch.manual_seed(2)
     blk = lblock.LshgdBlock().to(dev).to(torch.bfloat16)
+    settle(lambda: blk(feats_d, coords_d))
     for _ in range(3):
         blk(feats_d, coords_d)
     torch.cuda.synchronize()
@@ -445,6 +473,8 @@ def main():
     d0 = [x.to(dev) for x in (q0, k0, v0, g0, b0)]
 
     def time_us(fn, n=20, w=3):
+        if w > 1:
+            settle(fn)
         for _ in range(w):
             fn()
         torch.cuda.synchronize()
