@@ -2,14 +2,16 @@
 // event, or of a few, in ONE kernel launch on gfx950.
 //
 // Why one kernel: for one event of 60 000 hits every step is a few microseconds of work, and a dependent kernel
-// launch costs about as much as the step itself. Here the steps of a segment (a table of an event: its own key
-// ranges, its own sort) are separated by barriers over the segment's tiles instead (a flag per tile; one to two
-// microseconds), and a segment's keys go from the packing step into the first sort pass in registers. What tiles hand
-// to each other (min / max partials, digit counts, the scattered pairs, the permutation) moves through device-scope
-// relaxed atomic stores and loads: such a store is written through, such a load never reads a CU's L1, and the
-// producer waits for its stores to complete before it raises its flag. No fence is used: on this GPU a device-scope
-// release writes back a whole L2 and an acquire invalidates one, several microseconds each (measured), which is more
-// than a step costs.
+// launch costs about as much as the step itself. Here the tiles of a segment (a table of an event: its own key
+// ranges, its own sort) hand their results to each other inside the kernel instead, and a segment's keys go from the
+// packing step into the first sort pass in registers. Everything that is handed over moves through device-scope relaxed
+// atomic stores and loads: such a store is written through, such a load never reads a CU's L1. Small values (min / max
+// partials, digit counts, prefixes, totals) are 64-bit words that carry a tag of the launch and the step, and the reader
+// polls the word itself (lf_put / lf_get): one trip to memory per exchange. The scattered (key, payload) pairs and the
+// permutation have no room for a tag: after each radix pass's scatter there is a barrier over the segment's tiles (a
+// flag per tile, raised after the tile's stores have completed; two to four microseconds). No fence is used: on this
+// GPU a device-scope release writes back a whole L2 and an acquire invalidates one, several microseconds each
+// (measured), which is more than a step costs.
 //
 // Every tile of every segment of the call is a workgroup, and all of them must be on the GPU at once (a tile waits
 // for the other tiles of its segment): the launcher checks the grid against what the GPU holds and otherwise leaves
@@ -37,7 +39,7 @@ struct LshFusedArgs {
   int32_t* ids; int32_t* keys; int32_t* meta; int32_t* perm;
   const char* feats; int vec_per_row; char* feats_out;   // rows of vec_per_row 16-byte pieces
   int n_events; int n_tiles;
-  uint64_t* flags; int32_t* partial; uint32_t* rows; uint32_t* totals; uint2* pairs0; uint2* pairs1;
+  uint64_t* flags; uint64_t* partial; uint64_t* rows; uint64_t* totals; uint2* pairs0; uint2* pairs1;
   uint32_t* failed;     // one word per segment: holds `gen` once a tile of the segment has given up a wait in this call
   uint32_t gen;
   int spin_limit;       // polls a tile spends in one wait before it gives up
@@ -65,6 +67,26 @@ __device__ __forceinline__ uint2 lf_load_pair(const uint2* p) {
 }
 __device__ __forceinline__ void lf_store_pair(uint2* p, uint32_t key, uint32_t val) {
   lf_store(reinterpret_cast<uint64_t*>(p), (uint64_t)key | ((uint64_t)val << 32));
+}
+
+// Small values that tiles hand to each other (min / max partials, digit counts, prefixes, totals) travel as 64-bit
+// words that carry their own tag: value | tag << 32, the tag naming the launch and the step. The reader polls the word
+// itself until the tag is there, so such an exchange costs one trip to memory instead of the three of "stores, wait for
+// them, raise a flag | poll the flag, load" -- five of the kernel's seven barriers became exchanges of this kind.
+// The waits are bounded as the barriers' are: `budget` polls per thread and wait (none at all when the limit is 0 or the
+// tile has already given up: the value is then meaningless and `ok` false).
+__device__ __forceinline__ void lf_put(uint64_t* p, uint32_t tag, uint32_t value) {
+  lf_flag_store(p, (uint64_t)value | ((uint64_t)tag << 32));
+}
+__device__ __forceinline__ uint32_t lf_get(const uint64_t* p, uint32_t tag, int limit, bool healthy, bool& ok) {
+  uint64_t v = lf_flag_load(p);
+  if (!healthy || limit <= 0) { ok = false; return (uint32_t)v; }
+  for (int spins = 0; (uint32_t)(v >> 32) != tag; ++spins) {
+    if (spins >= limit) { ok = false; break; }
+    __builtin_amdgcn_s_sleep(1);
+    v = lf_flag_load(p);
+  }
+  return (uint32_t)v;
 }
 
 // Barrier over the n_tiles workgroups of a segment: a flag per tile, every tile polls all of them. Before the flag is
@@ -136,9 +158,9 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
   const int n_hits = (int)a.n_hits, dim = DIM ? DIM : a.dim;
   const int wave = threadIdx.x >> 6, lane = lane_id();
   uint64_t* gf = a.flags + (int64_t)seg * n_tiles;
-  int32_t* partial = a.partial + (int64_t)seg * n_tiles * LF_PARTIAL_STRIDE;
-  uint32_t* rows = a.rows + (int64_t)seg * n_tiles * LF_MAX_BINS;
-  uint32_t* totals = a.totals + (int64_t)seg * LF_MAX_BINS;
+  uint64_t* partial = a.partial + (int64_t)seg * n_tiles * LF_PARTIAL_STRIDE;
+  uint64_t* rows = a.rows + (int64_t)seg * n_tiles * LF_MAX_BINS;
+  uint64_t* totals = a.totals + (int64_t)seg * LF_MAX_BINS;
   uint2* pairs[2] = {a.pairs0 + (int64_t)seg * n_hits, a.pairs1 + (int64_t)seg * n_hits};
   uint64_t phase = (uint64_t)a.gen << 32;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -155,6 +177,14 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
       const bool ok = lf_barrier(gf, tile, n_tiles, want, a.spin_limit, healthy);
       if (healthy && !ok && threadIdx.x == 0) lf_store(a.failed + seg, a.gen);
       return ok;
+    };
+    // tag of the words of exchange k (0 .. 3) of radix pass e (the partials: pass 0, exchange 3)
+    auto lf_tag = [&](int e, int k) -> uint32_t { return (a.gen << 4) | (uint32_t)(e << 2 | k); };
+    // closes an exchange: did every thread of the tile get its words? (workgroup barrier inside)
+    auto lf_got = [&](bool ok) -> bool {
+      const bool all = __syncthreads_and(ok ? 1 : 0) != 0;
+      if (healthy && !all && threadIdx.x == 0) lf_store(a.failed + seg, a.gen);
+      return healthy && all;
     };
 
     // ---- hash the tile's hits for this table: min / max of every projection's bucket id ----
@@ -203,21 +233,22 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
       int32_t v = s_mm[0][q];
 #pragma unroll
       for (int w = 1; w < WAVES; ++w) v = (q & 1) ? max(v, s_mm[w][q]) : min(v, s_mm[w][q]);
-      lf_store(partial + tile * LF_PARTIAL_STRIDE + q, v);
+      lf_put(partial + tile * LF_PARTIAL_STRIDE + q, lf_tag(0, 3), (uint32_t)v);
     }
-    healthy = lf_sync(++phase);
 
     // ---- ranges, mixed-radix strides, key width (every tile computes them; tile 0 writes the meta row) ----
     {  // thread t reduces value t % 16 over tiles t / 16, t / 16 + 16, ...: independent loads, one round trip
       const int q = threadIdx.x & 15;
       int32_t v = (q & 1) ? INT32_MIN : INT32_MAX;
+      bool got = true;
       if (q < 2 * J) {
-#pragma unroll 8
+#pragma unroll 4
         for (int p = threadIdx.x >> 4; p < n_tiles; p += BLOCK / 16) {
-          const int32_t o = lf_load(partial + p * LF_PARTIAL_STRIDE + q);
+          const int32_t o = (int32_t)lf_get(partial + p * LF_PARTIAL_STRIDE + q, lf_tag(0, 3), a.spin_limit, healthy, got);
           v = (q & 1) ? max(v, o) : min(v, o);
         }
       }
+      healthy = lf_got(got);
       int32_t o = __shfl_xor(v, 16);
       v = (q & 1) ? max(v, o) : min(v, o);
       o = __shfl_xor(v, 32);
@@ -342,15 +373,15 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
         uint32_t c = 0;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) c += (s_cnt[w][d >> 1] >> (16 * (d & 1))) & 0xFFFFu;
-        lf_store(rows + tile * LF_MAX_BINS + d, c);
+        lf_put(rows + tile * LF_MAX_BINS + d, lf_tag(e, 0), c);
       }
-      healthy = lf_sync(++phase);
       // Tile t turns the counts of digits t*per .. (t+1)*per - 1 of ALL tiles into prefixes over the tiles (in place)
       // and their sum into the segment's totals: every tile reads n_tiles * per words instead of n_tiles rows. A wave
       // takes a digit, its lanes the tiles (128 at a time); four digits per wave are in flight, all loads first.
       {
         const int per = (bins + n_tiles - 1) / n_tiles, d0 = tile * per;
         const int steps = (per + WAVES - 1) / WAVES;
+        bool got = true;
         for (int s0 = 0; s0 < steps; s0 += 4) {
           uint32_t carry[4] = {0, 0, 0, 0};
           for (int p0 = 0; p0 < n_tiles; p0 += 128) {
@@ -361,7 +392,8 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
 #pragma unroll
               for (int h = 0; h < 2; ++h) {
                 const int p = p0 + 64 * h + lane;
-                c[u][h] = (dd < per && d < bins && p < n_tiles) ? lf_load(rows + p * LF_MAX_BINS + d) : 0u;
+                c[u][h] = (dd < per && d < bins && p < n_tiles)
+                              ? lf_get(rows + p * LF_MAX_BINS + d, lf_tag(e, 0), a.spin_limit, healthy, got) : 0u;
               }
             }
 #pragma unroll
@@ -371,7 +403,8 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
               for (int h = 0; h < 2; ++h) {
                 const int p = p0 + 64 * h + lane;
                 const uint32_t incl = lf_wave_inclusive(c[u][h], lane);
-                if (dd < per && d < bins && p < n_tiles) lf_store(rows + p * LF_MAX_BINS + d, carry[u] + incl - c[u][h]);
+                if (dd < per && d < bins && p < n_tiles)
+                  lf_put(rows + p * LF_MAX_BINS + d, lf_tag(e, 1), carry[u] + incl - c[u][h]);
                 carry[u] += __shfl(incl, 63);
               }
             }
@@ -379,20 +412,23 @@ __global__ void __launch_bounds__(BLOCK) lsh_fused_kernel(const LshFusedArgs a) 
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int dd = (s0 + u) * WAVES + wave, d = d0 + dd;
-            if (lane == 0 && dd < per && d < bins) lf_store(totals + d, carry[u]);
+            if (lane == 0 && dd < per && d < bins) lf_put(totals + d, lf_tag(e, 1), carry[u]);
           }
         }
+        healthy = lf_got(got);
       }
-      healthy = lf_sync(++phase);
-      // thread t owns digits t, t + 256, ...: keys of the digit in the tiles before this one, and in the segment
+      // thread t owns digits t, t + BLOCK, ...: keys of the digit in the tiles before this one, and in the segment
       uint32_t excl[DPT];
+      {
+        bool got = true;
 #pragma unroll
-      for (int j = 0; j < DPT; ++j) {
-        const int d = threadIdx.x + j * BLOCK;
-        excl[j] = d < bins ? lf_load(rows + tile * LF_MAX_BINS + d) : 0u;
-        if (d < bins) s_tot[d] = lf_load(totals + d);
+        for (int j = 0; j < DPT; ++j) {
+          const int d = threadIdx.x + j * BLOCK;
+          excl[j] = d < bins ? lf_get(rows + tile * LF_MAX_BINS + d, lf_tag(e, 1), a.spin_limit, healthy, got) : 0u;
+          if (d < bins) s_tot[d] = lf_get(totals + d, lf_tag(e, 1), a.spin_limit, healthy, got);
+        }
+        healthy = lf_got(got);
       }
-      __syncthreads();
       {  // exclusive scan of the digit totals: thread t scans digits 8t .. 8t+7
         uint32_t dt[DPT], mine = 0;
 #pragma unroll
@@ -580,8 +616,8 @@ static int64_t lf_tiles(int64_t n_hits, int tile) { return n_hits > 0 ? (n_hits 
 int64_t lsh_fused_workspace_bytes(int n_events, int64_t n_hits, int n_tables) {
   const int64_t segs = (int64_t)n_events * n_tables, tiles = lf_tiles(n_hits, LF_MIN_TILE);
   if (segs > LF_MAX_SEGMENTS || segs * lf_tiles(n_hits, 1024) > 4096) return 0;
-  return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256) +
-         lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256) +
+  return lampa_align_up(segs * tiles * 8, 256) + lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 8, 256) +
+         lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 8, 256) + 2 * lampa_align_up(segs * n_hits * 8, 256) +
          lampa_align_up(segs * 4, 256);
 }
 
@@ -639,9 +675,9 @@ int lsh_fused_launch(const float* coords, int n_events, int64_t n_hits, int64_t 
   a.n_events = n_events; a.n_tiles = (int)tiles;
   char* p = (char*)workspace;
   a.flags = (uint64_t*)p;   p += lampa_align_up(segs * tiles * 8, 256);
-  a.partial = (int32_t*)p;  p += lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 4, 256);
-  a.rows = (uint32_t*)p;    a.totals = a.rows + segs * tiles * LF_MAX_BINS;
-  p += lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 4, 256);
+  a.partial = (uint64_t*)p; p += lampa_align_up(segs * tiles * LF_PARTIAL_STRIDE * 8, 256);
+  a.rows = (uint64_t*)p;    a.totals = a.rows + segs * tiles * LF_MAX_BINS;
+  p += lampa_align_up(segs * (tiles + 1) * LF_MAX_BINS * 8, 256);
   a.pairs0 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
   a.pairs1 = (uint2*)p;     p += lampa_align_up(segs * n_hits * 8, 256);
   a.failed = (uint32_t*)p;
