@@ -352,3 +352,26 @@ def test_sequence_boundaries_are_validated_on_the_host():
         gd._sequence_bounds(cu, 1, 10)
     cu[1] = 7
     assert gd._sequence_bounds(cu, 1, 10) == [0, 7, 10]
+
+
+def test_bench_reads_the_traffic_table_of_the_committed_profile():
+    """bench.py takes `roofline.traffic` from the counter summary under profiles/: the four kernels of the layer must
+    be in its table, with a commit stamp, and every summary must say which commit it was measured at."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    table, commit = bench.measured_traffic()
+    assert re.fullmatch(r"[0-9a-f]{7,40}", commit or ""), commit
+    for kernel in ("gdr_local_kernel", "gdr_segment_kernel<composite>", "gdr_scan2_kernel<group>",
+                   "gdr_segment_kernel<output>"):
+        assert table.get(kernel, 0) > 1e6, (kernel, table)
+    # the output pass moves at least its algorithmic bytes (520 B per token and head at the headline shape)
+    assert table["gdr_segment_kernel<output>"] >= 520 * 60000 * 8
+    prof = os.path.join(ROOT, "profiles")
+    for name in sorted(os.listdir(prof)):
+        if name.endswith(".md"):
+            text = open(os.path.join(prof, name)).read()
+            assert re.search(r"^commit: [0-9a-f]{7,40}\b", text, flags=re.M), name
+            assert "rocprofv3" in text, name
