@@ -281,6 +281,34 @@ def test_one_launch_and_separate_kernels_agree(device):
         lsh.one_launch_config()
 
 
+def test_one_launch_kernel_on_changing_sizes_shares_one_workspace(device):
+    """The words that the tiles of the one-launch kernel hand to each other carry the launch and the step in their
+    upper half and are never cleared: launches of different sizes, event counts and tile forms, one after the other
+    on the same workspace memory, must each give the bits of the separate kernels."""
+    import random
+
+    rnd = random.Random(5)
+    alpha, beta = synth.lsh_params(4, 3, 4, 1.0, 1)
+    ad, bd = alpha.to(device), beta.to(device)
+    sizes = [1, 63, 65, 767, 768, 769, 1023, 1025, 2048, 5000, 12345, 30000, 45000, 60000, 61234]
+    try:
+        for it in range(48):
+            n = rnd.choice(sizes)
+            ev = rnd.choice([1, 1, 2]) if n <= 45000 else 1
+            gen = torch.Generator().manual_seed(it)
+            coords = (torch.randn(ev, n, 4, generator=gen) * rnd.choice([0.3, 1.0, 3.0])).to(device)
+            feats = torch.randn(ev, n, 24, generator=gen).to(device)
+            tile = rnd.choice([0, 0, 768, 1024])
+            lsh.one_launch_config(True, tile=tile)
+            one = lsh.lsh_bucket_sort(coords, ad, bd, 1.0, 3, 4, feats, strict=True)
+            lsh.one_launch_config(False)
+            sep = lsh.lsh_bucket_sort(coords, ad, bd, 1.0, 3, 4, feats, strict=True)
+            for name in ("ids", "meta", "keys", "perm", "feats"):
+                assert torch.equal(one[name], sep[name]), (it, n, ev, tile, name)
+    finally:
+        lsh.one_launch_config()
+
+
 def test_one_launch_generic_dim_and_wide_keys(device):
     """dim 3 (the generic coordinate path) and a bucket width that makes the keys need three radix passes."""
     n = 9000
