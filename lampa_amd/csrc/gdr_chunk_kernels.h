@@ -206,10 +206,11 @@ __device__ __forceinline__ f32x4 lds_ld_n(const float* p) {
 // steps) and two levels of MFMA merges T21 = -T22 (A21 T11), each product a single fp16 instruction (T is rounded to
 // the operand type OT afterwards, the coarser or an equal rounding). LDS holds the two diagonal 32x32 blocks in fp32
 // and the per-token factor rows, all wave-private. Output: the record of the chunk and head.
+// Built for four waves per SIMD (128 registers; its 10.5 KB of LDS then allow 15 of these one-wave workgroups per CU).
 static inline int gdr_local_grid(int n_chunks, int HV) { return 8 * ((n_chunks + 7) / 8) * HV; }
 
 template <typename T, typename OT, int KT>
-__global__ void __launch_bounds__(64, 3) gdr_local_kernel(const T* __restrict__ k, const float* __restrict__ g,
+__global__ void __launch_bounds__(64, 4) gdr_local_kernel(const T* __restrict__ k, const float* __restrict__ g,
                                                           const float* __restrict__ beta,
                                                           const int32_t* __restrict__ chunk_tok0,
                                                           const int32_t* __restrict__ chunk_len,
@@ -677,6 +678,10 @@ __global__ void __launch_bounds__((64 * GdrSegShape<KT, VT, PASS_B, CW>::WAVES),
 
   if (wave >= NSLAB) {
     // ================================================ stager ================================================
+    // Narrow output pass: with eight or more chain waves beside them the four stagers are the longer pole, so they get
+    // the SIMDs' issue slots first (config 4: output pass 1 168 -> 993 - 1 012 us). In the other forms the chain is
+    // the longer pole and a raised priority on either side changes nothing or costs a little.
+    if constexpr (PASS_B && CW == 16) __builtin_amdgcn_s_setprio(3);
     constexpr int KU = KT / 16, VU = VT / 16;  // 16-byte pieces per thread: half a row of k / q, of v
     // (narrow form: pair 0 = waves NSLAB, NSLAB + 1 stages k, v, T and the factors, pair 1 = the next two q and P; a
     // pair is the 128 threads the staging code is written for)
